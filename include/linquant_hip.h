@@ -1,0 +1,205 @@
+/* C ABI of liblinquant_hip.so: MI355X (gfx950) INT8 chunkwise linear-recurrence prefill.
+ *
+ * Every entry point takes a pointer to a plain args struct (device pointers, sizes, element
+ * strides, scalars, flags) and the HIP stream to launch on, and returns 0 or a negative code:
+ *   LQ_E_NULL  (-14) a required pointer is missing
+ *   LQ_E_SHAPE (-22) unsupported size / stride / alignment / flag
+ *   LQ_E_LAUNCH (-5) hipGetLastError() reported a launch failure
+ * Entry points never allocate, never synchronise, never throw and keep no mutable global state:
+ * the caller owns every buffer (inputs, outputs, intermediates) and may call concurrently on
+ * different streams.  All strides are in elements of the tensor's dtype.  "device float*" scalars
+ * (dt_scale, A_log_scale, D_scale) are 0-dim device tensors read inside the kernel, as in the
+ * reference, so no host synchronisation is needed to obtain them.
+ *
+ * Each declaration cites the reference (ntumm120/LinQuant) interface it replaces.
+ */
+#ifndef LINQUANT_HIP_H
+#define LINQUANT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef __HIP__
+#ifndef HIP_INCLUDE_HIP_HIP_RUNTIME_API_H
+typedef struct ihipStream_t* hipStream_t;
+#endif
+#endif
+
+#define LQ_E_NULL (-14)
+#define LQ_E_SHAPE (-22)
+#define LQ_E_LAUNCH (-5)
+
+/* element types accepted for the raw dt input */
+#define LQ_DT_F16 0
+#define LQ_DT_F32 1
+#define LQ_DT_I8 2
+
+/* ABI version; bumped whenever a struct layout changes. */
+int lq_abi_version(void);
+/* sizeof() of the named args struct as compiled into the library (negative if unknown); lets a binding
+ * check its own struct layout before the first call. */
+int lq_args_size(const char* name);
+
+/* ------------------------------------------------------------------------------------------
+ * Mamba-2 SSD pipeline (SSDi8 lineage).  Layouts: x (B,L,H,P) fp16 with arbitrary batch/seq/head
+ * strides and unit P stride (a view of xBC); B/C (B,L,G,N); dt, dA_cumsum (B,H,nc,Q) fp32
+ * contiguous; chunk states (B,nc,H,P,N) int8 contiguous.
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces _quant_chunk_cumsum_fwd, linquant/kernels/mamba2/chunk_cumsum.py:77-100 (kernel :27-74) */
+typedef struct {
+  const void* dt;            /* (B,L,H) raw dt, dtype dt_dtype, strides below */
+  int32_t dt_dtype;          /* LQ_DT_* */
+  int64_t dt_stride_b, dt_stride_l, dt_stride_h;
+  const float* dt_scale;     /* device scalar */
+  const int8_t* A_log;       /* (H,) int8 */
+  int64_t A_log_stride_h;
+  const float* A_log_scale;  /* device scalar */
+  const float* dt_bias;      /* (H,) fp32 or NULL */
+  int64_t dt_bias_stride_h;
+  float* dt_out;             /* (B,H,nc,Q) fp32 contiguous */
+  float* dA_cumsum;          /* (B,H,nc,Q) fp32 contiguous */
+  int32_t batch, seqlen, nheads, chunk_size;
+  int32_t dt_softplus;
+  float dt_min, dt_max;
+} lq_chunk_cumsum_args;
+int lq_chunk_cumsum(const lq_chunk_cumsum_args* args, hipStream_t stream);
+
+/* replaces _quant_chunk_state_fwd_xfp_static_int8, linquant/kernels/mamba2/chunk_state.py:258-349
+ * (kernel :72-255): value-side absorption, x quantized per tile with alpha_hp against INT8 B. */
+typedef struct {
+  const void* x;             /* (B,L,H,P) fp16, unit P stride */
+  int64_t x_stride_b, x_stride_l, x_stride_h;
+  const int8_t* B;           /* (B,L,G,N) int8, unit N stride */
+  int64_t B_stride_b, B_stride_l, B_stride_g;
+  const float* dt;           /* (B,H,nc,Q) fp32 contiguous */
+  const float* dA_cumsum;    /* (B,H,nc,Q) fp32 contiguous */
+  const float* alpha_hp;     /* (H,P) view; stride_p == 0 means one scalar per head */
+  int64_t alpha_stride_h, alpha_stride_p;
+  const float* bscale_g;     /* (G,) */
+  int64_t bscale_stride_g;
+  const float* out_qscale;   /* (H,P) view, stride_p may be 0 */
+  int64_t oqs_stride_h, oqs_stride_p;
+  int8_t* states;            /* (B,nc,H,P,N) int8 contiguous */
+  int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+} lq_chunk_state_value_args;
+int lq_chunk_state_value(const lq_chunk_state_value_args* args, hipStream_t stream);
+
+/* replaces _chunk_state_keyside_fwd, linquant/kernels/mamba2/chunk_state_keyside.py:342-424
+ * (kernel :163-330): key-side absorption, x quantized with x_scale_hp, fp16 B weighted by the gate
+ * and quantized in-loop with the raw-amax b_gate_scale (codes = rint(gate*B*127/b_gate)). */
+typedef struct {
+  const void* x;             /* (B,L,H,P) fp16, unit P stride */
+  int64_t x_stride_b, x_stride_l, x_stride_h;
+  const void* B;             /* (B,L,G,N) fp16, unit N stride */
+  int64_t B_stride_b, B_stride_l, B_stride_g;
+  const float* dt;
+  const float* dA_cumsum;
+  const float* x_scale_hp;   /* (H,P) view */
+  int64_t xs_stride_h, xs_stride_p;
+  const float* out_qscale;   /* (H,P) view */
+  int64_t oqs_stride_h, oqs_stride_p;
+  const float* b_gate_scale; /* 4-D broadcastable (B,nc,H,N); size-1 dims carry stride 0 */
+  int64_t bgs_stride_b, bgs_stride_c, bgs_stride_h, bgs_stride_n;
+  int8_t* states;            /* (B,nc,H,P,N) int8 contiguous */
+  int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+} lq_chunk_state_key_args;
+int lq_chunk_state_key(const lq_chunk_state_key_args* args, hipStream_t stream);
+
+/* replaces _fixedpoint_state_passing_fwd, linquant/kernels/mamba2/state_passing.py:96-121
+ * (kernel :25-93). out[:,0] = 0, out[:,c+1] = state after chunk c, final = state after the last. */
+typedef struct {
+  const int8_t* states;      /* (B,nc,H,dim) int8 */
+  int64_t states_stride_b, states_stride_c, states_stride_h, states_stride_d;
+  const float* dA_chunk_cumsum; /* (B,H,nc) view: last cumsum entry of every chunk */
+  int64_t dA_stride_b, dA_stride_h, dA_stride_c;
+  int8_t* out;               /* (B,nc,H,dim) int8 */
+  int64_t out_stride_b, out_stride_c, out_stride_h, out_stride_d;
+  int8_t* final_states;      /* (B,H,dim) int8 or NULL */
+  int64_t final_stride_b, final_stride_h, final_stride_d;
+  int32_t batch, nchunks, nheads, dim;
+  int32_t gate_shift;        /* fractional bits of the fixed-point gate, 0..15 (reference: 7) */
+  int32_t vec_hint;          /* 0 = auto; 4/8/16 = bytes per thread to try first */
+} lq_state_passing_args;
+int lq_state_passing(const lq_state_passing_args* args, hipStream_t stream);
+
+/* replaces _quant_bmm_chunk_fwd, linquant/kernels/mamba2/bmm_chunk.py:142-217 (kernel :49-139):
+ * CB_i8 = clamp(rint(C_i8 . B_i8^T * (sC*sB/S_cb)), +-127) per (batch, chunk, group). */
+typedef struct {
+  const int8_t* a;           /* C: (B,L,G,N) int8, unit N stride */
+  int64_t a_stride_b, a_stride_l, a_stride_g;
+  const void* b;             /* B: (B,L,G,N) int8, or fp16 when b_is_fp */
+  int64_t b_stride_b, b_stride_l, b_stride_g;
+  const float* a_scale;      /* (G,) */
+  const float* b_scale;      /* (G,) */
+  const float* cb_scale;     /* (G,) static output scale */
+  int8_t* out;               /* (B,nc,G,Q,Q) int8 contiguous */
+  int32_t batch, seqlen, ngroups, dstate, chunk_size;
+  int32_t b_is_fp;
+} lq_bmm_chunk_args;
+int lq_bmm_chunk(const lq_bmm_chunk_args* args, hipStream_t stream);
+
+/* replaces _quant_chunk_scan_fwd, linquant/kernels/mamba2/chunk_scan_v2.py:259-366 (kernel :56-256). */
+typedef struct {
+  const int8_t* cb;          /* (B,nc,G,Q,Q) int8 contiguous */
+  const void* x;             /* (B,L,H,P) fp16, unit P stride */
+  int64_t x_stride_b, x_stride_l, x_stride_h;
+  const float* dt;           /* (B,H,nc,Q) */
+  const float* dA_cumsum;    /* (B,H,nc,Q) */
+  const int8_t* C;           /* (B,L,G,N) int8, unit N stride */
+  int64_t C_stride_b, C_stride_l, C_stride_g;
+  const float* C_scale;      /* (G,) */
+  const int8_t* states;      /* (B,nc,H,P,N) int8 contiguous: state entering each chunk */
+  const float* states_scale; /* (H,P) view, stride_p may be 0 */
+  int64_t ss_stride_h, ss_stride_p;
+  const int8_t* D;           /* (H,) or (H,P) int8, or NULL */
+  int64_t D_stride_h;
+  int32_t D_has_hdim;
+  const float* D_scale;      /* device scalar (ignored when D is NULL) */
+  const float* cb_scale;     /* (G,) */
+  void* out;                 /* (B,L,H,P) fp16 contiguous */
+  int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+} lq_chunk_scan_args;
+int lq_chunk_scan(const lq_chunk_scan_args* args, hipStream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Rotation + quantize prologue.
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces fused_split_rotate_quant_xBC, linquant/kernels/mamba2/fused_split_rotate_xBC.py:236-329
+ * (kernel :31-227): B and C lanes of xBC -> [*dqk, fp16] -> signs -> H2 (x) H_{N/2} -> fp16 ->
+ * clamp(rint(y*inv_scale), -128, 127).  x is returned by the caller as a view, never touched here. */
+typedef struct {
+  const void* xBC;           /* (B,T,d_ssm+2*G*N) fp16, unit last stride */
+  int64_t xBC_stride_b, xBC_stride_t;
+  int8_t* qB;                /* (B,T,G,N) int8 contiguous */
+  int8_t* qC;                /* (B,T,G,N) int8 contiguous */
+  const void* signs;         /* (G,N) +-1 values of dtype signs_dtype, or NULL for no rotation */
+  int32_t signs_dtype;       /* LQ_DT_F16 / LQ_DT_F32 / LQ_DT_I8 */
+  const float* B_inv_scale;  /* (G,) */
+  const float* C_inv_scale;  /* (G,) */
+  const float* dqk_b;        /* (G*N,) fp32 holding fp16-rounded values, or NULL */
+  const float* dqk_c;
+  int32_t batch, seqlen, d_ssm, ngroups, dstate;
+} lq_split_rotate_quant_xBC_args;
+int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* args, hipStream_t stream);
+
+/* replaces kronecker_hadamard_fwd, linquant/kernels/hadamard.py:141-179 (kernel :38-103):
+ * y = (x * signs) . (H2 (x) H_{D/2}) per head, same dtype out, no quantization. */
+typedef struct {
+  const void* x;             /* (B,T,H,D) fp16, unit D stride */
+  int64_t x_stride_b, x_stride_t, x_stride_h;
+  void* y;                   /* (B,T,H,D) fp16 contiguous */
+  const void* signs;         /* (H,D) */
+  int32_t signs_dtype;
+  int32_t batch, seqlen, nheads, dim;
+} lq_kron_hadamard_args;
+int lq_kron_hadamard(const lq_kron_hadamard_args* args, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LINQUANT_HIP_H */

@@ -1,0 +1,125 @@
+"""Synthetic inputs and absmax calibration of the static scales the INT8 SSD kernels take.
+
+Plain torch reductions that run on whatever device the tensors live on (the GPU in the benchmark, the CPU in
+tests).  Scale semantics follow the reference's calibration collectors:
+  alpha_hp            amax |x * exp(dA_last - dA) * dt| / 127 per (H,P)   scripts/nemotron_h_calibration.py:293-343
+  x_scale_hp          amax |x| / 127 per (H,P)                            scripts/nemotron_h_calibration.py:558-599
+  B_scale / C_scale   amax of the rotated B / C per group / 127           scripts/nemotron_h_calibration.py:346-401
+  bscale_g            max over N of amax |B_rot| / 127 per group          scripts/nemotron_h_calibration.py:404-459
+  b_gate_scale        raw amax |gate * B_rot| per (H,N), shape (1,1,H,N)  scripts/nemotron_h_calibration.py:462-555
+  static_state_scale  amax of the chunk-local fp states / 127 per (H,P)   scripts/nemotron_h_calibration.py:602-651
+  static_cb_scale     amax |C_rot . B_rot^T| / 127 per group              scripts/nemotron_h_w4a8.py:126-169
+  A_log_scale, D_scale  amax / 127 scalars                                scripts/nemotron_h_w4a8.py:474
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as Fn
+
+
+@dataclass
+class Mamba2Shape:
+    batch: int
+    seqlen: int
+    nheads: int
+    headdim: int
+    dstate: int
+    ngroups: int
+    chunk: int
+
+    @property
+    def d_ssm(self):
+        return self.nheads * self.headdim
+
+    @property
+    def xbc_dim(self):
+        return self.d_ssm + 2 * self.ngroups * self.dstate
+
+
+def hadamard(n: int, device=None, dtype=torch.float32) -> torch.Tensor:
+    H = torch.ones(1, 1, dtype=dtype, device=device)
+    while H.shape[0] < n:
+        H = torch.cat([torch.cat([H, H], 1), torch.cat([H, -H], 1)], 0)
+    return H / math.sqrt(n)
+
+
+def mamba2_synthetic(shape: Mamba2Shape, seed: int, device="cpu"):
+    """Seeded synthetic activations of one Mamba-2 SSD layer: xBC ~ N(0,1) fp16, raw dt ~ N(-2, 0.5) fp16
+    (softplus applied in-kernel), drawn on the CPU generator in this order then moved to ``device``."""
+    g = torch.Generator().manual_seed(seed)
+    xBC = torch.randn(shape.batch, shape.seqlen, shape.xbc_dim, generator=g).to(torch.float16)
+    dt_raw = (torch.randn(shape.batch, shape.seqlen, shape.nheads, generator=g) * 0.5 - 2.0).to(torch.float16)
+    return xBC.to(device), dt_raw.to(device)
+
+
+def mamba2_params(shape: Mamba2Shape, seed: int, device="cpu"):
+    """Per-layer parameters: A = -exp(U(log 1, log 16)) as INT8 A_log codes, D ~ N(0,1) as INT8 codes, zero
+    dt_bias, +-1 rotation signs (G,N)."""
+    g = torch.Generator().manual_seed(seed)
+    a_log = torch.rand(shape.nheads, generator=g) * math.log(16.0)
+    D = torch.randn(shape.nheads, generator=g)
+    signs = (torch.randint(0, 2, (shape.ngroups, shape.dstate), generator=g) * 2 - 1).to(torch.float32)
+    A_log_scale = (a_log.abs().amax() / 127.0).clamp_min(1e-8)
+    D_scale = (D.abs().amax() / 127.0).clamp_min(1e-8)
+    return dict(
+        A_log=torch.round(a_log / A_log_scale).clamp(-127, 127).to(torch.int8).to(device),
+        A_log_scale=A_log_scale.float().to(device),
+        D=torch.round(D / D_scale).clamp(-127, 127).to(torch.int8).to(device),
+        D_scale=D_scale.float().to(device),
+        dt_bias=torch.zeros(shape.nheads, dtype=torch.float32, device=device),
+        dt_scale=torch.ones((), dtype=torch.float32, device=device),
+        r_signs=signs.to(device),
+    )
+
+
+@torch.no_grad()
+def calibrate_mamba2(shape: Mamba2Shape, xBC, dt_raw, params, head_block: int = 8):
+    """Static scales from one calibration batch (fp32 math on xBC's device)."""
+    dev = xBC.device
+    B, L, H, P, N, G, Q = shape.batch, shape.seqlen, shape.nheads, shape.headdim, shape.dstate, shape.ngroups, shape.chunk
+    B = xBC.shape[0]
+    nc = L // Q
+    assert L % Q == 0
+    d_ssm, gn = shape.d_ssm, G * N
+    Hn = hadamard(N, dev)
+    signs = params["r_signs"].to(dev).float()
+    Brot = (xBC[..., d_ssm:d_ssm + gn].float().view(B, L, G, N) * signs) @ Hn
+    Crot = (xBC[..., d_ssm + gn:].float().view(B, L, G, N) * signs) @ Hn
+    B_scale = (Brot.abs().amax(dim=(0, 1, 3)) / 127.0).clamp_min(1e-8)
+    C_scale = (Crot.abs().amax(dim=(0, 1, 3)) / 127.0).clamp_min(1e-8)
+    dt = Fn.softplus(dt_raw.float() * params["dt_scale"] + params["dt_bias"])  # (B,L,H)
+    A = -torch.exp(params["A_log_scale"] * params["A_log"].float())  # (H,)
+    dA = (dt * A).view(B, nc, Q, H).cumsum(dim=2)
+    gate = (torch.exp(dA[:, :, -1:, :] - dA) * dt.view(B, nc, Q, H))  # (B,nc,Q,H)
+    cb = torch.einsum("bcqgn,bckgn->bcgqk", Crot.view(B, nc, Q, G, N), Brot.view(B, nc, Q, G, N))
+    static_cb_scale = (cb.abs().amax(dim=(0, 1, 3, 4)) / 127.0).clamp_min(1e-8)
+    del cb
+    alpha = torch.empty(H, P, device=dev)
+    x_scale = torch.empty(H, P, device=dev)
+    b_gate = torch.empty(H, N, device=dev)
+    state_scale = torch.empty(H, P, device=dev)
+    rep = H // G
+    for h0 in range(0, H, head_block):
+        h1 = min(H, h0 + head_block)
+        xh = xBC[..., h0 * P:h1 * P].float().view(B, nc, Q, h1 - h0, P)
+        gh = gate[..., h0:h1]
+        xg = xh * gh[..., None]
+        alpha[h0:h1] = xg.abs().amax(dim=(0, 1, 2)) / 127.0
+        x_scale[h0:h1] = xh.abs().amax(dim=(0, 1, 2)) / 127.0
+        gidx = torch.arange(h0, h1, device=dev) // rep
+        Bh = Brot.view(B, nc, Q, G, N)[:, :, :, gidx]  # (B,nc,Q,hb,N)
+        b_gate[h0:h1] = (Bh * gh[..., None]).abs().amax(dim=(0, 1, 2))
+        st = torch.einsum("bcqhp,bcqhn->bchpn", xg, Bh)
+        state_scale[h0:h1] = st.abs().amax(dim=(0, 1, 4)) / 127.0
+    tiny = 1e-8
+    return dict(
+        B_scale=B_scale.float().contiguous(), C_scale=C_scale.float().contiguous(),
+        B_inv_scale=(1.0 / B_scale).float().contiguous(), C_inv_scale=(1.0 / C_scale).float().contiguous(),
+        bscale_g=B_scale.float().clone(), alpha_hp=alpha.clamp_min(tiny).contiguous(),
+        x_scale_hp=x_scale.clamp_min(tiny).contiguous(), b_gate_scale=b_gate.clamp_min(tiny).view(1, 1, H, N).contiguous(),
+        static_state_scale=state_scale.clamp_min(tiny).contiguous(), static_cb_scale=static_cb_scale.float().contiguous(),
+    )

@@ -1,0 +1,23 @@
+// ABI bookkeeping for liblinquant_hip.so.
+#include <string.h>
+
+#include "lq_common.h"
+#include "../../include/linquant_hip.h"
+
+extern "C" int lq_abi_version(void) { return 1; }
+
+#define LQ_SIZE_OF(T) \
+  if (strcmp(name, #T) == 0) return (int)sizeof(T)
+
+extern "C" int lq_args_size(const char* name) {
+  if (!name) return LQ_ERR_NULL;
+  LQ_SIZE_OF(lq_chunk_cumsum_args);
+  LQ_SIZE_OF(lq_chunk_state_value_args);
+  LQ_SIZE_OF(lq_chunk_state_key_args);
+  LQ_SIZE_OF(lq_state_passing_args);
+  LQ_SIZE_OF(lq_bmm_chunk_args);
+  LQ_SIZE_OF(lq_chunk_scan_args);
+  LQ_SIZE_OF(lq_split_rotate_quant_xBC_args);
+  LQ_SIZE_OF(lq_kron_hadamard_args);
+  return LQ_ERR_SHAPE;
+}

@@ -1,0 +1,88 @@
+// Mamba-2 SSD stage 1: dt pipeline + chunk-local cumulative sum of dt*A.
+// Replaces the reference stage linquant/kernels/mamba2/chunk_cumsum.py:27-74 (launcher :77-100).
+//
+// One wavefront per (head, chunk, batch).  Lane l owns the E = Q/64 consecutive positions
+// l*E .. l*E+E-1 of the chunk.  The prefix sum is: sequential inside the lane, Hillis-Steele
+// inclusive scan of the lane totals over the wave (offsets 1,2,4,...,32, "t = t + up"), then
+// exclusive lane prefix + local prefix.  The CPU checker restates exactly this order.
+#include "lq_common.h"
+#include "../../include/linquant_hip.h"
+
+namespace {
+
+constexpr int kMaxE = 16;  // chunk sizes up to 1024
+
+LQ_DEV float load_dt(const void* p, int64_t off, int dtype) {
+  if (dtype == LQ_DT_F16) return (float)((const _Float16*)p)[off];
+  if (dtype == LQ_DT_F32) return ((const float*)p)[off];
+  return (float)((const int8_t*)p)[off];
+}
+
+__global__ __launch_bounds__(64) void chunk_cumsum_kernel(
+    const void* __restrict__ dt_in, int dt_dtype, int64_t sdt_b, int64_t sdt_l, int64_t sdt_h,
+    const float* __restrict__ dt_scale_p, const int8_t* __restrict__ a_log, int64_t sa_h,
+    const float* __restrict__ a_log_scale_p, const float* __restrict__ dt_bias, int64_t sbias_h,
+    float* __restrict__ dt_out, float* __restrict__ dA_cs, int seqlen, int nheads, int nchunks, int Q,
+    int softplus, float dt_min, float dt_max) {
+  const int h = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
+  const int lane = threadIdx.x;
+  const int E = Q >> 6;
+  const int limit = min(Q, seqlen - c * Q);
+  const float dt_scale = *dt_scale_p;
+  const float A = -lq_expf((*a_log_scale_p) * (float)a_log[(int64_t)h * sa_h]);
+  const float bias = dt_bias ? dt_bias[(int64_t)h * sbias_h] : 0.0f;
+
+  float dtv[kMaxE], pre[kMaxE];
+  float run = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kMaxE; ++i) {
+    if (i < E) {
+      const int pos = lane * E + i;
+      float v = 0.0f;
+      if (pos < limit) {
+        v = dt_scale * load_dt(dt_in, (int64_t)b * sdt_b + (int64_t)(c * Q + pos) * sdt_l + (int64_t)h * sdt_h, dt_dtype);
+        if (dt_bias) v = v + bias;
+        if (softplus) v = (v > 20.0f) ? v : lq_logf(1.0f + lq_expf(v));
+        v = fminf(fmaxf(v, dt_min), dt_max);
+      }
+      dtv[i] = v;
+      const float dA = v * A;
+      run = (i == 0) ? dA : run + dA;
+      pre[i] = run;
+    }
+  }
+  float t = run;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const float up = __shfl_up(t, off, 64);
+    if (lane >= off) t = t + up;
+  }
+  float ex = __shfl_up(t, 1, 64);
+  if (lane == 0) ex = 0.0f;
+  const int64_t base = (((int64_t)b * nheads + h) * nchunks + c) * Q + lane * E;
+#pragma unroll
+  for (int i = 0; i < kMaxE; ++i) {
+    if (i < E) {
+      dt_out[base + i] = dtv[i];
+      dA_cs[base + i] = ex + pre[i];
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int lq_chunk_cumsum(const lq_chunk_cumsum_args* a, hipStream_t stream) {
+  if (!a || !a->dt || !a->dt_scale || !a->A_log || !a->A_log_scale || !a->dt_out || !a->dA_cumsum) return LQ_ERR_NULL;
+  if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0 || a->batch > 65535) return LQ_ERR_SHAPE;
+  const int Q = a->chunk_size;
+  if (Q < 64 || Q % 64 != 0 || Q > 64 * kMaxE) return LQ_ERR_SHAPE;
+  if (a->dt_dtype != LQ_DT_F16 && a->dt_dtype != LQ_DT_F32 && a->dt_dtype != LQ_DT_I8) return LQ_ERR_SHAPE;
+  const int nchunks = (a->seqlen + Q - 1) / Q;
+  if (nchunks > 65535) return LQ_ERR_SHAPE;
+  dim3 grid(a->nheads, nchunks, a->batch);
+  hipLaunchKernelGGL(chunk_cumsum_kernel, grid, dim3(64), 0, stream, a->dt, a->dt_dtype, a->dt_stride_b,
+                     a->dt_stride_l, a->dt_stride_h, a->dt_scale, a->A_log, a->A_log_stride_h, a->A_log_scale,
+                     a->dt_bias, a->dt_bias_stride_h, a->dt_out, a->dA_cumsum, a->seqlen, a->nheads, nchunks, Q,
+                     a->dt_softplus, a->dt_min, a->dt_max);
+  return lq_check_launch();
+}

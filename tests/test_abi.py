@@ -1,0 +1,85 @@
+"""CPU checks of the drop-in boundary: the C-ABI library loads, exports every symbol the public header
+declares, its struct layouts agree with the binding, and the Python wrappers enforce the reference's host-side
+contracts before any launch (no compute call is made here)."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from linquant_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    header = (ROOT / "include" / "linquant_hip.h").read_text()
+    declared = re.findall(r"^\s*int\s+(lq_\w+)\s*\(", header, flags=re.M)
+    assert len(declared) >= 10 and set(declared) == set(_lib.FUNCTIONS)
+    for name in declared:
+        assert getattr(lib, name) is not None, name
+    assert lib.lq_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_layouts_match_the_library():
+    lib = _lib.load()
+    assert len(_lib.STRUCTS) >= 8
+    for name, st in _lib.STRUCTS.items():
+        assert lib.lq_args_size(name.encode()) == ctypes.sizeof(st), name
+    assert lib.lq_args_size(b"no_such_struct") < 0
+
+
+def test_every_declaration_cites_the_reference():
+    header = (ROOT / "include" / "linquant_hip.h").read_text()
+    for m in re.finditer(r"/\*((?:(?!\*/).)*?)\*/\s*typedef struct", header, flags=re.S):
+        assert re.search(r"linquant/kernels/[\w/]+\.py:\d+", m.group(1)), m.group(1)[:80]
+
+
+def test_null_and_shape_errors_without_launch():
+    """Argument validation happens on the host before anything touches a device."""
+    lib = _lib.load()
+    st = _lib.STRUCTS["lq_state_passing_args"]()
+    assert lib.lq_state_passing(ctypes.byref(st), None) == -14  # missing pointers
+    st2 = _lib.STRUCTS["lq_chunk_cumsum_args"]()
+    assert lib.lq_chunk_cumsum(ctypes.byref(st2), None) == -14
+    buf = (ctypes.c_char * 64)()
+    for f in ("dt", "dt_scale", "A_log", "A_log_scale", "dt_out", "dA_cumsum"):
+        setattr(st2, f, ctypes.addressof(buf))
+    st2.batch, st2.seqlen, st2.nheads, st2.chunk_size = 1, 64, 1, 48  # chunk not a multiple of 64
+    assert lib.lq_chunk_cumsum(ctypes.byref(st2), None) == -22
+
+
+def test_wrapper_contracts_raise_assertion_errors():
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2.bmm_chunk import _quant_bmm_chunk_fwd
+    from linquant_amd.kernels.mamba2.chunk_cumsum import _quant_chunk_cumsum_fwd
+    from linquant_amd.kernels.mamba2.chunk_state_keyside import _bgs_strides
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC, prepare_dqk
+
+    one = torch.ones(())
+    with pytest.raises(AssertionError):  # xBC_dim mismatch (fused_split_rotate_xBC.py:270)
+        fused_split_rotate_quant_xBC(torch.zeros(1, 8, 100, dtype=torch.float16), None, 1, 1, 64, 64, one, one)
+    with pytest.raises(AssertionError):  # A_log shape (chunk_cumsum.py:79)
+        _quant_chunk_cumsum_fwd(torch.zeros(1, 64, 2), one, torch.zeros(3, dtype=torch.int8), one, 64)
+    with pytest.raises(AssertionError):  # dt_bias shape (chunk_cumsum.py:81)
+        _quant_chunk_cumsum_fwd(torch.zeros(1, 64, 2), one, torch.zeros(2, dtype=torch.int8), one, 64, dt_bias=torch.zeros(3))
+    with pytest.raises(AssertionError):  # D >= 64 (hadamard.py:152)
+        kronecker_hadamard_fwd(torch.zeros(1, 4, 1, 32, dtype=torch.float16), torch.ones(1, 32), 1)
+    with pytest.raises(AssertionError):  # static_cb_scale shape (bmm_chunk.py:174)
+        _quant_bmm_chunk_fwd(torch.zeros(1, 64, 2, 64, dtype=torch.int8), torch.ones(2), torch.zeros(1, 64, 2, 64, dtype=torch.int8),
+                             torch.ones(2), 64, torch.ones(3))
+    with pytest.raises(AssertionError):  # 4-D b_gate_scale (chunk_state_keyside.py:338)
+        _bgs_strides(torch.ones(2, 64))
+    assert _bgs_strides(torch.ones(1, 1, 4, 64)) == (0, 0, 64, 1)
+    d = prepare_dqk(torch.tensor([[1.0001, 2.0]]))
+    assert d.dtype == torch.float32 and d.shape == (2,) and float(d[0]) == float(torch.tensor(1.0001).half())
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(_lib.LinQuantHipError):
+        _lib.load()

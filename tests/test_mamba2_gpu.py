@@ -1,0 +1,374 @@
+"""GPU parity of the Mamba-2 INT8 SSD HIP kernels against the CPU oracle (through the Python call surface,
+which goes through the C ABI).  Integer tensors must be bit-exact; the fp16 output stage is held to
+max |err| <= 1e-3 * max |ref| against the float64 oracle."""
+
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from linquant_amd.calibration import Mamba2Shape
+from oracle import mamba2_ssd as O
+from tests.mamba2_cases import build_case, npy, oracle_pipeline
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def dev(t, device):
+    return None if t is None else torch.from_numpy(np.ascontiguousarray(t)).to(device)
+
+
+def assert_same_codes(got, ref, name):
+    got, ref = npy(got), np.asarray(ref)
+    assert got.shape == ref.shape, (name, got.shape, ref.shape)
+    bad = np.argwhere(got != ref)
+    assert bad.size == 0, f"{name}: {len(bad)} of {ref.size} codes differ, first at {bad[0]}: got {got[tuple(bad[0])]} ref {ref[tuple(bad[0])]}"
+
+
+def assert_close_out(got, ref, name, tol=1e-3):
+    got, ref = npy(got).astype(np.float64), np.asarray(ref, np.float64)
+    assert np.isfinite(got).all(), name
+    err = np.abs(got - ref).max() / np.abs(ref).max()
+    assert err <= tol, f"{name}: max err / max ref = {err:.3e} > {tol}"
+
+
+SHAPES = [
+    Mamba2Shape(batch=2, seqlen=512, nheads=4, headdim=64, dstate=128, ngroups=1, chunk=256),
+    Mamba2Shape(batch=1, seqlen=256, nheads=8, headdim=64, dstate=64, ngroups=2, chunk=64),
+    Mamba2Shape(batch=2, seqlen=384, nheads=2, headdim=128, dstate=128, ngroups=2, chunk=128),
+]
+
+
+@pytest.fixture(scope="module", params=range(len(SHAPES)))
+def case(request):
+    c = build_case(SHAPES[request.param])
+    c["oracle"] = {False: oracle_pipeline(c, False), True: oracle_pipeline(c, True)}
+    return c
+
+
+def gpu_inputs(case, cuda):
+    p = {k: v.to(cuda) for k, v in case["params"].items()}
+    sc = {k: v.to(cuda) for k, v in case["scales"].items()}
+    return case["xBC"].to(cuda), case["dt_raw"].to(cuda), p, sc
+
+
+def test_chunk_cumsum(case, cuda):
+    from linquant_amd.kernels.mamba2.chunk_cumsum import _quant_chunk_cumsum_fwd
+
+    s = case["shape"]
+    say("chunk_cumsum", s)
+    _, dt_raw, p, _ = gpu_inputs(case, cuda)
+    dA, dt = _quant_chunk_cumsum_fwd(dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], s.chunk, dt_bias=p["dt_bias"],
+                                     dt_softplus=True)
+    torch.cuda.synchronize()
+    ref = case["oracle"][False]
+    assert np.array_equal(npy(dt), ref["dt"]) and np.array_equal(npy(dA), ref["dA_cumsum"])
+
+
+@pytest.mark.parametrize("L,Q,softplus,limit,dtype", [(300, 128, True, (0.001, 0.5), torch.float16),
+                                                      (1000, 256, False, (0.0, float("inf")), torch.float32),
+                                                      (64, 64, True, (0.0, float("inf")), torch.float16),
+                                                      (700, 512, True, (0.0, float("inf")), torch.float16)])
+def test_chunk_cumsum_ragged_strided(cuda, L, Q, softplus, limit, dtype):
+    from linquant_amd.kernels.mamba2.chunk_cumsum import _quant_chunk_cumsum_fwd
+
+    say("chunk_cumsum ragged", L, Q, softplus, limit, dtype)
+    g = torch.Generator().manual_seed(5)
+    B, H = 2, 6
+    wide = (torch.randn(B, L, H + 10, generator=g) * 0.5 - 2).to(dtype)
+    if not softplus:
+        wide = wide.abs() * 0.1
+    bias = torch.randn(H, generator=g) * 0.1
+    a_log = torch.randint(0, 127, (H,), generator=g).to(torch.int8)
+    view = wide.to(cuda)[..., 3:3 + H]  # non-contiguous slice, as the in_proj split produces
+    dA, dt = _quant_chunk_cumsum_fwd(view, torch.tensor(0.9, device=cuda), a_log.to(cuda), torch.tensor(0.02, device=cuda),
+                                     Q, dt_bias=bias.to(cuda), dt_softplus=softplus, dt_limit=limit)
+    torch.cuda.synchronize()
+    rdA, rdt = O.chunk_cumsum(npy(wide[..., 3:3 + H]), np.float32(0.9), npy(a_log), np.float32(0.02), Q, npy(bias), softplus, limit)
+    assert np.array_equal(npy(dt), rdt) and np.array_equal(npy(dA), rdA)
+
+
+def test_prologue_and_rotation(case, cuda):
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    s = case["shape"]
+    say("prologue", s)
+    xBC, _, p, sc = gpu_inputs(case, cuda)
+    x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                             sc["B_inv_scale"], sc["C_inv_scale"])
+    torch.cuda.synchronize()
+    ref = case["oracle"][True]
+    assert x.data_ptr() == xBC.data_ptr() and x.shape == (s.batch, s.seqlen, s.nheads, s.headdim)
+    assert_same_codes(qB, ref["q_B"], "q_B")
+    assert_same_codes(qC, ref["q_C"], "q_C")
+    gn = s.ngroups * s.dstate
+    b_view = xBC[..., s.d_ssm:s.d_ssm + gn].view(s.batch, s.seqlen, s.ngroups, s.dstate)  # strided view
+    y = kronecker_hadamard_fwd(b_view, p["r_signs"], s.ngroups)
+    torch.cuda.synchronize()
+    assert np.array_equal(npy(y).view(np.uint16), ref["b_fp"].view(np.uint16))
+
+
+def test_prologue_dqk_and_no_rotation(cuda):
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC, prepare_dqk
+
+    s = Mamba2Shape(batch=2, seqlen=203, nheads=2, headdim=64, dstate=128, ngroups=2, chunk=64)  # T not a multiple of 16
+    say("prologue dqk / no rotation", s)
+    g = torch.Generator().manual_seed(11)
+    xBC = torch.randn(s.batch, s.seqlen, s.xbc_dim, generator=g).half()
+    signs = (torch.randint(0, 2, (s.ngroups, s.dstate), generator=g) * 2 - 1).float()
+    dq = torch.rand(s.ngroups, s.dstate, generator=g) + 0.5
+    binv, cinv = torch.tensor([20.0, 35.0]), torch.tensor([28.0, 31.0])
+    for use_signs, use_dqk in ((True, True), (False, False), (False, True)):
+        _, qB, qC = fused_split_rotate_quant_xBC(xBC.to(cuda), signs.to(cuda) if use_signs else None, s.nheads, s.ngroups,
+                                                 s.dstate, s.headdim, binv.to(cuda), cinv.to(cuda),
+                                                 dqk_b=(1 / dq).to(cuda) if use_dqk else None, dqk_c=dq.to(cuda) if use_dqk else None)
+        torch.cuda.synchronize()
+        _, rB, rC = O.split_rotate_quant_xBC(npy(xBC), npy(signs) if use_signs else None, s.nheads, s.ngroups, s.dstate,
+                                             s.headdim, npy(binv), npy(cinv),
+                                             npy(prepare_dqk(1 / dq)) if use_dqk else None, npy(prepare_dqk(dq)) if use_dqk else None)
+        assert_same_codes(qB, rB, f"q_B signs={use_signs} dqk={use_dqk}")
+        assert_same_codes(qC, rC, f"q_C signs={use_signs} dqk={use_dqk}")
+
+
+@pytest.mark.parametrize("keyside", [False, True])
+def test_chunk_state(case, cuda, keyside):
+    from linquant_amd.kernels.mamba2.chunk_state import _quant_chunk_state_fwd_xfp_static_int8
+    from linquant_amd.kernels.mamba2.chunk_state_keyside import _chunk_state_keyside_fwd
+
+    s = case["shape"]
+    say("chunk_state", "key" if keyside else "value", s)
+    xBC, _, p, sc = gpu_inputs(case, cuda)
+    ref = case["oracle"][keyside]
+    x = xBC[..., :s.d_ssm].view(s.batch, s.seqlen, s.nheads, s.headdim)
+    dt, dA = dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda)
+    if keyside:
+        st = _chunk_state_keyside_fwd(x, sc["x_scale_hp"], dev(ref["b_fp"], cuda), dt, dA, sc["static_state_scale"],
+                                      sc["b_gate_scale"])
+    else:
+        st = _quant_chunk_state_fwd_xfp_static_int8(x, dev(ref["q_B"], cuda), dt, dA, sc["alpha_hp"], sc["bscale_g"],
+                                                    sc["static_state_scale"])
+    torch.cuda.synchronize()
+    assert_same_codes(st, ref["states"], "states")
+
+
+def test_chunk_state_scalar_scales_and_ragged(cuda):
+    """Per-head scalars passed as stride-0 (H,P) views, sequence length not a multiple of the chunk."""
+    from linquant_amd.kernels.mamba2.chunk_state import _quant_chunk_state_fwd_xfp_static_int8
+
+    s = Mamba2Shape(batch=1, seqlen=384, nheads=2, headdim=64, dstate=64, ngroups=1, chunk=128)
+    say("chunk_state scalar scales + ragged", s)
+    c = build_case(s)
+    L = 300
+    ref = oracle_pipeline(c, False)
+    x = npy(c["xBC"])[:, :L, :s.d_ssm].reshape(1, L, 2, 64)
+    qB = ref["q_B"][:, :L]
+    dA, dt = O.chunk_cumsum(npy(c["dt_raw"])[:, :L], 1.0, npy(c["params"]["A_log"]), float(c["params"]["A_log_scale"]), 128,
+                            None, True)
+    alpha = npy(c["scales"]["alpha_hp"]).max(1, keepdims=True)
+    sout = npy(c["scales"]["static_state_scale"]).max(1, keepdims=True)
+    rs = O.chunk_state_value(x, qB, dt, dA, np.broadcast_to(alpha, (2, 64)), npy(c["scales"]["bscale_g"]),
+                             np.broadcast_to(sout, (2, 64)))
+    xg = c["xBC"][:, :L].to(cuda)[..., :s.d_ssm].view(1, L, 2, 64)
+    st = _quant_chunk_state_fwd_xfp_static_int8(xg, dev(qB, cuda), dev(dt, cuda), dev(dA, cuda),
+                                                dev(alpha, cuda).expand(2, 64), c["scales"]["bscale_g"].to(cuda),
+                                                dev(sout, cuda).expand(2, 64))
+    torch.cuda.synchronize()
+    assert_same_codes(st, rs, "states (scalar scales, ragged)")
+
+
+@pytest.mark.parametrize("dim,shift,nc", [(8192, 7, 32), (4096 + 16, 7, 5), (1000, 7, 9), (999, 5, 3), (64 * 64, 7, 1)])
+def test_state_passing(cuda, dim, shift, nc):
+    from linquant_amd.kernels.mamba2.state_passing import _fixedpoint_state_passing_fwd
+
+    say("state_passing", dim, shift, nc)
+    rng = np.random.default_rng(dim + nc)
+    B, H = 2, 3
+    states = rng.integers(-128, 128, size=(B, nc, H, dim)).astype(np.int8)
+    dA_full = -rng.random((B, H, nc, 4)).astype(np.float32) * 3
+    dA_full[0, 0] = 0.0
+    dA_full[1, 1] = -200.0
+    dA_g = dev(dA_full, cuda)
+    out, fin = _fixedpoint_state_passing_fwd(dev(states, cuda), dA_g[..., -1], gate_shift=shift)
+    torch.cuda.synchronize()
+    rout, rfin = O.state_passing(states, dA_full[..., -1], shift)
+    assert_same_codes(out, rout, "passed")
+    assert_same_codes(fin, rfin, "final")
+
+
+def test_state_passing_noncontiguous(cuda):
+    from linquant_amd.kernels.mamba2.state_passing import _fixedpoint_state_passing_fwd
+
+    say("state_passing non-contiguous")
+    rng = np.random.default_rng(0)
+    wide = rng.integers(-127, 128, size=(2, 6, 3, 200)).astype(np.int8)
+    dA = -rng.random((2, 3, 6)).astype(np.float32)
+    view = dev(wide, cuda)[..., 7:107:2]  # stride 2 on the state axis -> generic kernel
+    out, fin = _fixedpoint_state_passing_fwd(view, dev(dA, cuda))
+    torch.cuda.synchronize()
+    rout, rfin = O.state_passing(np.ascontiguousarray(wide[..., 7:107:2]), dA)
+    assert_same_codes(out, rout, "passed")
+    assert_same_codes(fin, rfin, "final")
+
+
+@pytest.mark.parametrize("keyside", [False, True])
+def test_bmm_chunk(case, cuda, keyside):
+    from linquant_amd.kernels.mamba2.bmm_chunk import _quant_bmm_chunk_fwd
+
+    s = case["shape"]
+    say("bmm_chunk", "key" if keyside else "value", s)
+    _, _, _, sc = gpu_inputs(case, cuda)
+    ref = case["oracle"][keyside]
+    b = dev(ref["b_fp"], cuda) if keyside else dev(ref["q_B"], cuda)
+    cb = _quant_bmm_chunk_fwd(dev(ref["q_C"], cuda), sc["C_scale"], b, sc["B_scale"], s.chunk, sc["static_cb_scale"],
+                              b_is_fp=keyside)
+    torch.cuda.synchronize()
+    assert_same_codes(cb, ref["cb"], "cb")
+
+
+@pytest.mark.parametrize("keyside", [False, True])
+def test_chunk_scan(case, cuda, keyside):
+    from linquant_amd.kernels.mamba2.chunk_scan_v2 import _quant_chunk_scan_fwd
+
+    s = case["shape"]
+    say("chunk_scan", "key" if keyside else "value", s)
+    xBC, _, p, sc = gpu_inputs(case, cuda)
+    ref = case["oracle"][keyside]
+    x = xBC[..., :s.d_ssm].view(s.batch, s.seqlen, s.nheads, s.headdim)
+    out = _quant_chunk_scan_fwd(dev(ref["cb"], cuda), x, dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda),
+                                dev(ref["q_C"], cuda), sc["C_scale"], dev(ref["passed"], cuda), p["D"], p["D_scale"],
+                                sc["static_state_scale"], sc["static_cb_scale"])
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float16 and out.is_contiguous()
+    assert_close_out(out, ref["out"], "out")
+    # without the D residual, with a per-(H,P) D and with a stride-0 state scale
+    out2 = _quant_chunk_scan_fwd(dev(ref["cb"], cuda), x, dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda),
+                                 dev(ref["q_C"], cuda), sc["C_scale"], dev(ref["passed"], cuda), None, None,
+                                 sc["static_state_scale"], sc["static_cb_scale"])
+    r2 = O.chunk_scan(ref["cb"], ref["x"], ref["dt"], ref["dA_cumsum"], ref["q_C"], npy(sc["C_scale"]), ref["passed"],
+                      None, None, npy(sc["static_state_scale"]), npy(sc["static_cb_scale"]))
+    assert_close_out(out2, r2, "out (no D)")
+
+
+@pytest.mark.parametrize("keyside", [False, True])
+def test_pipeline_end_to_end(case, cuda, keyside):
+    """The drop-in path a caller takes: prologue -> (rotation of fp B) -> combined forward."""
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    s = case["shape"]
+    say("pipeline", "key" if keyside else "value", s)
+    xBC, dt_raw, p, sc = gpu_inputs(case, cuda)
+    x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                             sc["B_inv_scale"], sc["C_inv_scale"])
+    kw = {}
+    if keyside:
+        gn = s.ngroups * s.dstate
+        b_fp = xBC[..., s.d_ssm:s.d_ssm + gn].reshape(s.batch, s.seqlen, s.ngroups, s.dstate).contiguous()
+        kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=kronecker_hadamard_fwd(b_fp, p["r_signs"], s.ngroups),
+                  b_gate_scale=sc["b_gate_scale"])
+    seen = {}
+    orig_sp, orig_scan = M._fixedpoint_state_passing_fwd, M._chunk_scan_v2
+
+    def spy_sp(states, dA, gate_shift=7):  # the stage names are re-bindable module attributes
+        seen["states"] = states
+        r = orig_sp(states, dA, gate_shift=gate_shift)
+        seen["passed"] = r[0]
+        return r
+
+    def spy_scan(cb, *a):
+        seen["cb"] = cb
+        return orig_scan(cb, *a)
+
+    M._fixedpoint_state_passing_fwd, M._chunk_scan_v2 = spy_sp, spy_scan
+    try:
+        out, none = M._quant_mamba_chunk_scan_combined_fwd(
+            x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], **kw)
+    finally:
+        M._fixedpoint_state_passing_fwd, M._chunk_scan_v2 = orig_sp, orig_scan
+    torch.cuda.synchronize()
+    ref = case["oracle"][keyside]
+    assert none is None
+    assert_same_codes(seen["states"].reshape(ref["states"].shape), ref["states"], "states")
+    assert_same_codes(seen["passed"].reshape(ref["passed"].shape), ref["passed"], "passed")
+    assert_same_codes(seen["cb"], ref["cb"], "cb")
+    assert_close_out(out, ref["out"], "out")
+
+
+def test_full_size_config5_slices(cuda):
+    """Mamba-2 2.7B-shape layer (B4 L8192 H80 P64 N128 Q256) on the GPU; every integer stage is checked
+    bit-exactly against the oracle on head / batch slices the oracle finishes in seconds, the output on the
+    same slices, and state passing additionally through its zero-gate and copy properties at full size."""
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+    from linquant_amd.kernels.mamba2.state_passing import _fixedpoint_state_passing_fwd
+    from linquant_amd.calibration import calibrate_mamba2, mamba2_params, mamba2_synthetic
+
+    s = Mamba2Shape(batch=4, seqlen=8192, nheads=80, headdim=64, dstate=128, ngroups=1, chunk=256)
+    say("full size", s)
+    p = mamba2_params(s, 42, cuda)
+    cal = Mamba2Shape(batch=1, seqlen=2048, nheads=80, headdim=64, dstate=128, ngroups=1, chunk=256)
+    cx, cdt = mamba2_synthetic(cal, 1, cuda)
+    sc = calibrate_mamba2(cal, cx, cdt, p)
+    del cx, cdt
+    xBC, dt_raw = mamba2_synthetic(s, 0, cuda)
+    x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], 80, 1, 128, 64, sc["B_inv_scale"], sc["C_inv_scale"])
+    b_fp = kronecker_hadamard_fwd(xBC[..., s.d_ssm:s.d_ssm + 128].view(4, 8192, 1, 128), p["r_signs"], 1)
+    seen = {}
+    orig_sp = M._fixedpoint_state_passing_fwd
+
+    def spy_sp(states, dA, gate_shift=7):
+        r = orig_sp(states, dA, gate_shift=gate_shift)
+        seen["states"], seen["passed"], seen["dA_last"] = states, r[0], dA
+        return r
+
+    M._fixedpoint_state_passing_fwd = spy_sp
+    outs = {}
+    try:
+        for keyside in (False, True):
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"]) if keyside else {}
+            out, _ = M._quant_mamba_chunk_scan_combined_fwd(
+                x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+                p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+                static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], **kw)
+            torch.cuda.synchronize()
+            outs[keyside] = (out, seen["states"], seen["passed"])
+    finally:
+        M._fixedpoint_state_passing_fwd = orig_sp
+    # oracle on slices: batch b, heads hs
+    for keyside, b, hs in ((False, 0, [0, 79]), (True, 3, [17, 42])):
+        say("full size slice check", keyside, b, hs)
+        out, states, passed = outs[keyside]
+        hsel = torch.tensor(hs, device=cuda)
+        xs = npy(x[b:b + 1][:, :, hsel])
+        sub = lambda t: npy(t[hsel])  # noqa: E731
+        r = O.ssd_combined(xs, npy(dt_raw[b:b + 1][:, :, hsel]), 1.0, sub(p["A_log"]), float(p["A_log_scale"]),
+                           npy(qB[b:b + 1]), npy(sc["B_scale"]), npy(qC[b:b + 1]), npy(sc["C_scale"]), 256, sub(p["D"]),
+                           float(p["D_scale"]), dt_bias=sub(p["dt_bias"]), dt_softplus=True,
+                           static_state_scale=sub(sc["static_state_scale"]), static_cb_scale=npy(sc["static_cb_scale"]),
+                           alpha_hp=sub(sc["alpha_hp"]), bscale_g=npy(sc["bscale_g"]), keyside=keyside,
+                           x_scale_hp=sub(sc["x_scale_hp"]), b_fp=npy(b_fp[b:b + 1]),
+                           b_gate_scale=npy(sc["b_gate_scale"][:, :, hsel]))
+        st = states.view(4, 32, 80, 64, 128)[b:b + 1][:, :, hsel]
+        ps = passed.view(4, 32, 80, 64, 128)[b:b + 1][:, :, hsel]
+        assert_same_codes(st, r["states"], "states slice")
+        assert_same_codes(ps, r["passed"], "passed slice")
+        assert_close_out(out[b:b + 1][:, :, hsel], r["out"], "out slice")
+    # size-independent properties of state passing at full size
+    states = outs[True][1]
+    zero_gate = torch.full((4, 80, 32), -200.0, device=cuda)
+    o, f = _fixedpoint_state_passing_fwd(states, zero_gate)
+    torch.cuda.synchronize()
+    assert torch.equal(o[:, 1:], states[:, :-1].clamp(-127, 127)) and torch.equal(f, states[:, -1].clamp(-127, 127))
+    assert int(o[:, 0].abs().max()) == 0

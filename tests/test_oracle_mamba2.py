@@ -1,0 +1,312 @@
+"""Pins the CPU oracle of the Mamba-2 INT8 SSD pipeline (oracle/mamba2_ssd.py, oracle/kernel_arith.py).
+
+The reference has no test or fixture for these kernels, so the oracle is pinned by what the mathematics fixes:
+float64 library routines, exact integer arithmetic, brute-force scalar loops on tiny inputs, the structural
+fp32-arithmetic restatement of state passing the reference carries in patches/ssdi8.patch:2515-2562, scipy's
+Hadamard matrix, and the unquantized sequential SSD recurrence.
+"""
+
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import scipy.linalg
+
+from linquant_amd.calibration import Mamba2Shape
+from oracle import kernel_arith as KA
+from oracle import mamba2_ssd as O
+from tests.mamba2_cases import build_case, npy, oracle_pipeline
+
+F = np.float32
+
+
+# ----------------------------------------------------------------------------- arithmetic helpers
+def test_expf_accuracy_and_edges():
+    x = np.concatenate([np.linspace(-85.99, 88.0, 400001), np.linspace(-1, 1, 100001)]).astype(np.float32)
+    got = KA.lq_expf(x).astype(np.float64)
+    ref = np.exp(x.astype(np.float64))
+    assert np.max(np.abs(got - ref) / ref) < 2e-7
+    assert KA.lq_expf(F(0.0)) == F(1.0)
+    assert KA.lq_expf(F(-86.0)) == 0.0 and KA.lq_expf(F(-1000.0)) == 0.0 and KA.lq_expf(F(-np.inf)) == 0.0
+    assert np.isinf(KA.lq_expf(F(88.5))) and np.isnan(KA.lq_expf(F(np.nan)))
+    # every result in range is a normal number (no denormal handling differences between devices)
+    assert np.all(got[x > -86.0] >= np.finfo(np.float32).tiny)
+    # monotone on a fine grid around a reduction boundary
+    g = np.linspace(0.34, 0.36, 20001).astype(np.float32)
+    assert np.all(np.diff(KA.lq_expf(g).astype(np.float64)) >= -1e-7)
+
+
+def test_logf_accuracy():
+    y = np.concatenate([np.linspace(1.0, 4.0, 300001), np.exp(np.linspace(0, 21, 100001))]).astype(np.float32)
+    got = KA.lq_logf(y).astype(np.float64)
+    ref = np.log(y.astype(np.float64))
+    assert np.max(np.abs(got - ref) / np.maximum(ref, 1e-3)) < 3e-7
+    assert KA.lq_logf(F(1.0)) == 0.0
+    # softplus as the kernels evaluate it
+    x = np.linspace(-30, 20, 50001).astype(np.float32)
+    sp = KA.lq_logf(F(1.0) + KA.lq_expf(x)).astype(np.float64)
+    ref = np.log1p(np.exp(x.astype(np.float64)))
+    assert np.max(np.abs(sp - ref)) < 1.5e-7 * np.maximum(1.0, ref).max()
+
+
+def test_round_half_away_exact():
+    """rha against exact rational arithmetic, including every +-x.5 tie. The kernels form y + 0.5 in fp32
+    (linquant/kernels/zoo/simple_gla.py:19, mamba2/chunk_state.py:217): wherever that sum is exact the result
+    is the mathematical round-half-away; the one fp32 value just below 0.5 rounds up to 1 by that formula."""
+    ties = np.concatenate([np.arange(-300, 300) + 0.5, np.arange(-300, 300) * 1.0,
+                           [126.5, -126.5, 1e9, -1e9, 0.25, -0.25, 0.375, -0.375]]).astype(np.float32)
+    for y, g in zip(ties, KA.q_rha(ties, 127)):
+        fr = Fraction(float(y))
+        exact = math.floor(abs(fr) + Fraction(1, 2)) * (1 if fr >= 0 else -1)  # mathematical round-half-away
+        assert g == max(-127, min(127, exact)), (y, g, exact)
+    grid = np.linspace(-200, 200, 40001).astype(np.float32)
+    for y, g in zip(grid, KA.q_rha(grid, 127)):
+        sfl = Fraction(float(F(abs(y)) + F(0.5)))  # the fp32 sum the kernels form, floored exactly
+        exact = math.floor(sfl) * (1 if y >= 0 else -1)
+        assert g == max(-127, min(127, exact)), (y, g, exact)
+    below_half = np.nextafter(F(0.5), F(0.0))
+    assert list(KA.q_rha(np.array([below_half, -below_half], np.float32), 127)) == [1, -1]
+    assert list(KA.q_rint(np.array([0.5, 1.5, 2.5, -0.5, -1.5, 200.0, -200.0], np.float32), -128, 127)) == [0, 2, 2, 0, -2, 127, -128]
+
+
+def test_bf16_round_matches_torch():
+    import torch
+
+    x = np.random.default_rng(0).standard_normal(100000).astype(np.float32) * 37.0
+    ref = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(KA.bf16_round(x), ref)
+
+
+# ----------------------------------------------------------------------------- stage 1
+@pytest.mark.parametrize("Q", [64, 128, 256, 512])
+def test_wave_cumsum(Q):
+    rng = np.random.default_rng(Q)
+    ints = rng.integers(-1000, 1000, size=(3, 5, Q)).astype(np.float32)
+    assert np.array_equal(O.wave_cumsum(ints), np.cumsum(ints.astype(np.int64), -1).astype(np.float32))  # exact sums
+    v = -rng.random((4, 7, Q)).astype(np.float32) * 3
+    got = O.wave_cumsum(v).astype(np.float64)
+    ref = np.cumsum(v.astype(np.float64), -1)
+    assert np.max(np.abs(got - ref) / np.abs(ref)) < 1e-6
+
+
+def test_chunk_cumsum_against_float64():
+    rng = np.random.default_rng(1)
+    B, L, H, Q = 2, 300, 5, 128  # ragged last chunk
+    dt_raw = (rng.standard_normal((B, L, H)) * 0.5 - 2).astype(np.float16)
+    a_log = rng.integers(0, 127, H).astype(np.int8)
+    bias = rng.standard_normal(H).astype(np.float32) * 0.1
+    dA, dt = O.chunk_cumsum(dt_raw, 1.0, a_log, 0.02, Q, bias, True, (0.001, 0.5))
+    nc = math.ceil(L / Q)
+    assert dA.shape == dt.shape == (B, H, nc, Q)
+    v = dt_raw.astype(np.float64) + bias
+    sp = np.clip(np.where(v > 20, v, np.log1p(np.exp(v))), 0.001, 0.5)
+    pad = np.zeros((B, nc * Q - L, H))
+    spc = np.concatenate([sp, pad], 1).reshape(B, nc, Q, H).transpose(0, 3, 1, 2)
+    A = -np.exp(0.02 * a_log.astype(np.float64))
+    ref = np.cumsum(spc * A[None, :, None, None], -1)
+    # log(1 + exp(x)) formed in fp32 carries the absolute rounding of 1 + e (6e-8), as in the reference's kernel
+    assert np.allclose(dt, spc, rtol=3e-7, atol=2e-7)
+    assert np.max(np.abs(dA - ref) / np.maximum(np.abs(ref), 1e-2)) < 5e-6
+    assert np.all(dt[:, :, -1, L - (nc - 1) * Q:] == 0)  # positions past the sequence end
+
+
+# ----------------------------------------------------------------------------- stage 3
+def _state_passing_scalar(states, dA, shift):
+    Bsz, nc, H, dim = states.shape
+    out = np.zeros_like(states)
+    fin = np.zeros((Bsz, H, dim), np.int8)
+    for b in range(Bsz):
+        for h in range(H):
+            for d in range(dim):
+                s = 0
+                for c in range(nc):
+                    g = math.exp(float(dA[b, h, c])) * (1 << shift)
+                    gq = int(max(-127, min(127, math.floor(g + 0.5))))
+                    s = ((s * gq + ((1 << shift) >> 1)) >> shift) + int(states[b, c, h, d])  # python >> is arithmetic
+                    q = max(-127, min(127, s))
+                    if c < nc - 1:
+                        out[b, c + 1, h, d] = q
+                    else:
+                        fin[b, h, d] = q
+    return out, fin
+
+
+@pytest.mark.parametrize("shift", [7, 5])
+def test_state_passing_bruteforce(shift):
+    rng = np.random.default_rng(3)
+    states = rng.integers(-128, 128, size=(2, 9, 3, 11)).astype(np.int8)
+    dA = -rng.random((2, 3, 9)).astype(np.float32) * 2.0
+    dA[0, 0, :] = 0.0  # gate 1.0 saturates to 127/128
+    dA[1, 2, :] = -100.0  # gate 0: plain copy
+    out, fin = O.state_passing(states, dA, shift)
+    rout, rfin = _state_passing_scalar(states, dA, shift)
+    assert np.array_equal(out, rout) and np.array_equal(fin, rfin)
+    assert np.all(out[:, 0] == 0)
+    assert np.array_equal(out[1, 1:, 2], np.clip(states[1, :-1, 2], -127, 127))
+
+
+def test_state_passing_tracks_fp32_arithmetic_restatement():
+    """Gates exactly representable in Q0.7: the fixed-point pass equals the fp32-arithmetic pass
+    (s = gate*s + new, unclamped accumulator, clamp on store) up to the per-step rounding 0.5/(1-gate)."""
+    rng = np.random.default_rng(4)
+    k = rng.integers(1, 120, size=(2, 4, 16))
+    dA = np.log(k / 128.0).astype(np.float32)
+    states = rng.integers(-127, 128, size=(2, 16, 4, 64)).astype(np.int8)
+    out, fin = O.state_passing(states, dA, 7)
+    s = np.zeros((2, 4, 64))
+    bound = np.zeros((2, 4, 1))
+    for c in range(16):
+        g = (k[:, :, c] / 128.0)[..., None]
+        s = g * s + states[:, c]
+        bound = g * bound + 0.5
+        ref = np.clip(np.round(s), -127, 127)
+        got = (fin if c == 15 else out[:, c + 1]).astype(np.float64)
+        assert np.all(np.abs(got - ref) <= np.ceil(bound) + 1)
+
+
+def test_state_passing_geometric_closed_form():
+    """Constant input v=64 and gate 64/128: s_n = floor((s_{n-1}*64+64)/128) + 64 converges to 128 -> stored 127."""
+    states = np.full((1, 12, 1, 4), 64, np.int8)
+    dA = np.full((1, 1, 12), math.log(0.5), np.float32)
+    out, fin = O.state_passing(states, dA, 7)
+    s, exp = 0, []
+    for _ in range(12):
+        s = (s * 64 + 64) // 128 + 64
+        exp.append(min(s, 127))
+    assert list(out[0, 1:, 0, 0]) == exp[:-1] and fin[0, 0, 0] == exp[-1] == 127
+
+
+# ----------------------------------------------------------------------------- stages 2 and 4: brute force
+def _tiny_case():
+    return build_case(Mamba2Shape(batch=1, seqlen=128, nheads=2, headdim=64, dstate=64, ngroups=1, chunk=64))
+
+
+def test_chunk_state_value_scalar_bruteforce():
+    case = _tiny_case()
+    r = oracle_pipeline(case, keyside=False)
+    sc = case["scales"]
+    x, qB, dt, dA = r["x"], r["q_B"], r["dt"], r["dA_cumsum"]
+    alpha, sout, bs = npy(sc["alpha_hp"]), npy(sc["static_state_scale"]), npy(sc["bscale_g"])
+    rng = np.random.default_rng(0)
+    for _ in range(40):
+        c, h, p, n = rng.integers(2), rng.integers(2), rng.integers(64), rng.integers(64)
+        acc = 0
+        for k in range(64):
+            gate = F(KA.lq_expf(F(dA[0, h, c, 63] - dA[0, h, c, k]))) * dt[0, h, c, k]
+            y = F(F(F(x[0, c * 64 + k, h, p]) * F(F(1.0) / alpha[h, p])) * gate)
+            xq = int(np.clip(math.floor(y + F(0.5)) if y >= 0 else math.ceil(y - F(0.5)), -127, 127))
+            acc += xq * int(qB[0, c * 64 + k, 0, n])
+        req = F(F(alpha[h, p] / sout[h, p]) * bs[0])
+        v = F(F(acc) * req)
+        code = int(np.clip(math.floor(v + F(0.5)) if v >= 0 else math.ceil(v - F(0.5)), -127, 127))
+        assert code == r["states"][0, c, h, p, n]
+
+
+def test_chunk_state_key_and_bmm_scalar_bruteforce():
+    case = _tiny_case()
+    r = oracle_pipeline(case, keyside=True)
+    sc = case["scales"]
+    x, bfp, dt, dA = r["x"], r["b_fp"], r["dt"], r["dA_cumsum"]
+    xs, sout, bg = npy(sc["x_scale_hp"]), npy(sc["static_state_scale"]), npy(sc["b_gate_scale"])[0, 0]
+    rng = np.random.default_rng(1)
+    for _ in range(40):
+        c, h, p, n = rng.integers(2), rng.integers(2), rng.integers(64), rng.integers(64)
+        acc = 0
+        for k in range(64):
+            gate = F(KA.lq_expf(F(dA[0, h, c, 63] - dA[0, h, c, k]))) * dt[0, h, c, k]
+            xq = int(np.clip(np.rint(F(F(x[0, c * 64 + k, h, p]) * F(F(1.0) / max(xs[h, p], F(1e-10))))), -127, 127))
+            bq = int(np.clip(np.rint(F(F(F(bfp[0, c * 64 + k, 0, n]) * gate) * F(F(127.0) / bg[h, n]))), -127, 127))
+            acc += xq * bq
+        v = F(F(F(acc) * F(bg[h, n] / F(127.0))) * F(xs[h, p] / sout[h, p]))
+        assert int(np.clip(np.rint(v), -127, 127)) == r["states"][0, c, h, p, n]
+    # C.B^T with in-loop key quantization
+    qC, sC, sB, scb = r["q_C"], npy(sc["C_scale"]), npy(sc["B_scale"]), npy(sc["static_cb_scale"])
+    for _ in range(40):
+        c, m, k = rng.integers(2), rng.integers(64), rng.integers(64)
+        acc = 0
+        for n in range(64):
+            bq = int(np.clip(np.rint(F(F(bfp[0, c * 64 + k, 0, n]) * F(F(1.0) / sB[0]))), -127, 127))
+            acc += int(qC[0, c * 64 + m, 0, n]) * bq
+        v = F(F(acc) * F(F(sC[0] * sB[0]) / scb[0]))
+        assert int(np.clip(np.rint(v), -127, 127)) == r["cb"][0, c, 0, m, k]
+
+
+# ----------------------------------------------------------------------------- rotation
+@pytest.mark.parametrize("N", [64, 128])
+def test_kron_rotation_is_signed_hadamard(N):
+    rng = np.random.default_rng(N)
+    Hn = scipy.linalg.hadamard(N).astype(np.float64)
+    H2, Hh = scipy.linalg.hadamard(2), scipy.linalg.hadamard(N // 2)
+    assert np.array_equal(np.kron(H2, Hh), Hn)  # H2 (x) H_{N/2} is the Sylvester H_N
+    signs = rng.integers(0, 2, N) * 2.0 - 1.0
+    b = rng.standard_normal((50, N)).astype(np.float16).astype(np.float32)
+    got = O.kron_rotate(b, signs[None]).astype(np.float64)
+    # exact evaluation of the reference's definition: bf16 operand, bf16 H block, exact sums
+    hb = float(KA.bf16_round(F(1.0) / np.sqrt(F(N // 2))))
+    v = KA.bf16_round(b * signs[None].astype(np.float32)).astype(np.float64)
+    w0, w1 = (v[:, :N // 2] @ Hh) * hb, (v[:, N // 2:] @ Hh) * hb
+    ref = np.concatenate([w0 + w1, w0 - w1], 1) * float(F(1.0 / math.sqrt(2.0)))
+    assert np.max(np.abs(got - ref)) <= 4e-7 * np.abs(ref).max()
+    # and it is the orthogonal rotation diag(s) H_N / sqrt(N) up to the bf16 rounding of the operand
+    ideal = (b.astype(np.float64) * signs[None]) @ Hn / math.sqrt(N)
+    assert np.max(np.abs(got - ideal)) < 2 ** -8 * np.abs(b).max() * math.sqrt(N)
+    R = np.diag(signs) @ Hn / math.sqrt(N)
+    assert np.allclose(R @ R.T, np.eye(N), atol=1e-12)
+
+
+def test_prologue_codes_vs_exact_definition():
+    """INT8 codes of the fused prologue against an exact float64 evaluation of the definition: identical except
+    where an fp32 rounding of the butterfly straddles an fp16/INT8 rounding boundary (rare, +-1)."""
+    case = build_case(Mamba2Shape(batch=1, seqlen=256, nheads=2, headdim=64, dstate=128, ngroups=1, chunk=64))
+    s, p, sc = case["shape"], case["params"], case["scales"]
+    _, qB, qC = O.split_rotate_quant_xBC(npy(case["xBC"]), npy(p["r_signs"]), 2, 1, 128, 64, npy(sc["B_inv_scale"]),
+                                         npy(sc["C_inv_scale"]))
+    xBC = npy(case["xBC"]).astype(np.float32)
+    Hh = scipy.linalg.hadamard(64).astype(np.float64)
+    signs = npy(p["r_signs"]).astype(np.float32)
+    for q, off, inv in ((qB, 128, npy(sc["B_inv_scale"])), (qC, 256, npy(sc["C_inv_scale"]))):
+        b = xBC[0, :, off:off + 128]
+        v = KA.bf16_round(b * signs).astype(np.float64)
+        w0, w1 = v[:, :64] @ Hh * 0.125, v[:, 64:] @ Hh * 0.125
+        y = (np.concatenate([w0 + w1, w0 - w1], 1).astype(np.float32) * F(1 / math.sqrt(2))).astype(np.float16)
+        ref = np.clip(np.rint(y.astype(np.float32) * inv[0]), -128, 127)
+        diff = np.abs(ref - q[0, :, 0].astype(np.float64))
+        assert diff.max() <= 1 and (diff > 0).mean() < 1e-3
+
+
+# ----------------------------------------------------------------------------- whole pipeline vs unquantized SSD
+def _ssd_sequential(case):
+    """h_t = exp(dt_t A) h_{t-1} + dt_t x_t B_t^T ; y_t = h_t C_t + D x_t in float64, rotated B/C (exact rotation)."""
+    s, p = case["shape"], case["params"]
+    xBC = npy(case["xBC"]).astype(np.float64)
+    Bsz, L, H, P, N, G = s.batch, s.seqlen, s.nheads, s.headdim, s.dstate, s.ngroups
+    x = xBC[..., :s.d_ssm].reshape(Bsz, L, H, P)
+    R = np.diag(npy(p["r_signs"])[0].astype(np.float64)) @ scipy.linalg.hadamard(N) / math.sqrt(N)
+    Bm = xBC[..., s.d_ssm:s.d_ssm + N] @ R
+    Cm = xBC[..., s.d_ssm + N:] @ R
+    dt = np.log1p(np.exp(npy(case["dt_raw"]).astype(np.float64)))
+    A = -np.exp(float(p["A_log_scale"]) * npy(p["A_log"]).astype(np.float64))
+    D = float(p["D_scale"]) * npy(p["D"]).astype(np.float64)
+    y = np.zeros((Bsz, L, H, P))
+    h = np.zeros((Bsz, H, P, N))
+    for t in range(L):
+        h = h * np.exp(dt[:, t] * A)[..., None, None] + (dt[:, t, :, None] * x[:, t])[..., None] * Bm[:, t, None, None, :]
+        y[:, t] = np.einsum("bhpn,bn->bhp", h, Cm[:, t]) + D[None, :, None] * x[:, t]
+    return y
+
+
+@pytest.mark.parametrize("keyside", [False, True])
+def test_pipeline_matches_unquantized_recurrence(keyside):
+    case = build_case(Mamba2Shape(batch=1, seqlen=512, nheads=2, headdim=64, dstate=128, ngroups=1, chunk=128))
+    r = oracle_pipeline(case, keyside)
+    ref = _ssd_sequential(case)
+    err = np.abs(r["out"] - ref)
+    # INT8 noise floor: ~2 % mean / rms; the maximum sits at chunk starts of slowly forgetting heads, where the
+    # carried state saturates its chunk-local scale (the lineage's calibration convention), hence the loose max
+    assert err.mean() / np.abs(ref).mean() < 0.03 and np.sqrt((err ** 2).mean() / (ref ** 2).mean()) < 0.04
+    assert err.max() / np.abs(ref).max() < 0.2
+    # dequantized chunk-local states track the fp chunk states
+    sc = npy(case["scales"]["static_state_scale"])
+    assert np.abs(r["states"]).max() <= 127 and (np.abs(r["states"]) == 127).mean() < 0.02
+    assert r["passed"].shape == r["states"].shape and np.all(r["passed"][:, 0] == 0) and sc.shape == (2, 64)
