@@ -1,0 +1,209 @@
+"""Benchmark of the INT8 chunkwise linear-recurrence prefill on one MI355X.
+
+Workload (the configuration the metric is quoted on): Mamba-2 2.7B-shape SSD layer, INT8 prefill, batch 4,
+seqlen 8192, 80 heads x headdim 64, d_state 128, 1 group, chunk 256, key-side absorption. One step = the whole
+hot path over one batch resident in HBM: split/rotate/quantize prologue of B and C, rotation of the fp16 B
+used by the key-side chunk state, then cumsum -> chunk state -> INT8 state passing -> C.B^T -> chunk scan.
+
+Prints ONE JSON line: the whole-step throughput, a per-stage breakdown measured with HIP events on the
+launch stream, the roofline of the dominant kernel, and the CPU oracle timed on a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0
+
+
+def stage_bytes(s, keyside):
+    """Algorithmic HBM bytes per stage: every tensor a stage must read or write, counted once."""
+    B, L, H, P, N, G, Q = s.batch, s.seqlen, s.nheads, s.headdim, s.dstate, s.ngroups, s.chunk
+    nc = L // Q
+    x = B * L * H * P * 2
+    bc_i8 = B * L * G * N
+    dtda = 2 * B * H * nc * Q * 4
+    states = B * nc * H * P * N
+    cb = B * nc * G * Q * Q
+    return {
+        "prologue": 2 * bc_i8 * 2 + 2 * bc_i8,
+        "rotate_b_fp": (bc_i8 * 2 * 2) if keyside else 0,
+        "chunk_cumsum": B * L * H * 2 + dtda,
+        "chunk_state": x + (bc_i8 * 2 if keyside else bc_i8) + dtda + states,
+        "state_passing": 2 * states + B * H * P * N,
+        "bmm_chunk": bc_i8 + (bc_i8 * 2 if keyside else bc_i8) + cb,
+        "chunk_scan": states + x + x + bc_i8 + cb + dtda,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--value-side", action="store_true", help="value-side absorption instead of key-side")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-heads", type=int, default=8, help="heads of the CPU-oracle sample (batch 1)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards over batch x head "
+              "with no communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from linquant_amd import _lib
+    from linquant_amd.calibration import Mamba2Shape, calibrate_mamba2, mamba2_params, mamba2_synthetic
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    if not _lib.LIB_PATH.exists():
+        from linquant_amd.build import build
+
+        build()
+    _lib.load()
+    dev = torch.device("cuda:0")
+    keyside = not args.value_side
+    s = Mamba2Shape(batch=4, seqlen=8192, nheads=80, headdim=64, dstate=128, ngroups=1, chunk=256)
+    p = mamba2_params(s, 42, dev)
+    cal = Mamba2Shape(batch=1, seqlen=2048, nheads=s.nheads, headdim=s.headdim, dstate=s.dstate, ngroups=s.ngroups, chunk=s.chunk)
+    cx, cdt = mamba2_synthetic(cal, 1, dev)
+    sc = calibrate_mamba2(cal, cx, cdt, p)
+    del cx, cdt
+    xBC, dt_raw = mamba2_synthetic(s, 0, dev)
+    gn = s.ngroups * s.dstate
+    torch.cuda.synchronize()
+
+    def step():
+        x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                 sc["B_inv_scale"], sc["C_inv_scale"])
+        kw = {}
+        if keyside:
+            b_view = xBC[..., s.d_ssm:s.d_ssm + gn].view(s.batch, s.seqlen, s.ngroups, s.dstate)
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=kronecker_hadamard_fwd(b_view, p["r_signs"], s.ngroups),
+                      b_gate_scale=sc["b_gate_scale"])
+        out, _ = M._quant_mamba_chunk_scan_combined_fwd(
+            x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], **kw)
+        return out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    tokens = s.batch * s.seqlen
+
+    # ---- per-stage durations: HIP events on the launch stream around every stage call (separate pass)
+    names = {"_quant_chunk_cumsum_fwd": "chunk_cumsum", "_chunk_state_keyside_fwd": "chunk_state",
+             "_quant_chunk_state_fwd_xfp_static_int8": "chunk_state", "_fixedpoint_state_passing_fwd": "state_passing",
+             "_quant_bmm_chunk_fwd": "bmm_chunk", "_chunk_scan_v2": "chunk_scan"}
+    records = {}
+
+    def timed(fn, label):
+        def wrapper(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            records.setdefault(label, []).append((e0, e1))
+            return r
+        return wrapper
+
+    import linquant_amd.kernels.hadamard as Hm
+    import linquant_amd.kernels.mamba2.fused_split_rotate_xBC as Fs
+
+    saved = {n: getattr(M, n) for n in names}
+    for n, label in names.items():
+        setattr(M, n, timed(saved[n], label))
+    fused_t, rot_t = timed(Fs.fused_split_rotate_quant_xBC, "prologue"), timed(Hm.kronecker_hadamard_fwd, "rotate_b_fp")
+
+    def step_staged():
+        x, qB, qC = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"], sc["C_inv_scale"])
+        kw = {}
+        if keyside:
+            b_view = xBC[..., s.d_ssm:s.d_ssm + gn].view(s.batch, s.seqlen, s.ngroups, s.dstate)
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=rot_t(b_view, p["r_signs"], s.ngroups),
+                      b_gate_scale=sc["b_gate_scale"])
+        M._quant_mamba_chunk_scan_combined_fwd(
+            x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], **kw)
+
+    try:
+        for _ in range(max(10, args.steps)):
+            step_staged()
+        torch.cuda.synchronize()
+    finally:
+        for n, f in saved.items():
+            setattr(M, n, f)
+    nbytes = stage_bytes(s, keyside)
+    stages = {}
+    for label, evs in records.items():
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        med = statistics.median(ts)
+        stages[label] = {"ms": round(med, 4), "p25": round(ts[len(ts) // 4], 4), "p75": round(ts[(3 * len(ts)) // 4], 4),
+                         "MB": round(nbytes[label] / 1e6, 1), "GBps": round(nbytes[label] / 1e6 / med, 1),
+                         "hbm_frac": round(nbytes[label] / 1e6 / med / HBM_PEAK_GBS, 4)}
+    dom = max(stages, key=lambda k: stages[k]["ms"])
+    avg_dom = statistics.mean(a.elapsed_time(b) for a, b in records[dom])
+    achieved = nbytes[dom] / 1e6 / avg_dom
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "avg_ms": round(avg_dom, 4),
+                "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
+
+    # ---- CPU baseline: the CPU oracle on a bounded sample (batch 1 x a few heads x full length), same seeds
+    cpu = None
+    if not args.no_cpu_baseline:
+        import numpy as np
+
+        from oracle import mamba2_ssd as O
+
+        nh = min(args.cpu_heads, s.nheads)
+        threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        npy = lambda t: t.detach().cpu().numpy()  # noqa: E731
+        xs = npy(xBC[:1, :, :nh * s.headdim]).reshape(1, s.seqlen, nh, s.headdim)
+        xBC_s = np.concatenate([xs.reshape(1, s.seqlen, -1), npy(xBC[:1, :, s.d_ssm:])], axis=-1)
+        t0 = time.perf_counter()
+        x_o, qB_o, qC_o = O.split_rotate_quant_xBC(xBC_s, npy(p["r_signs"]), nh, s.ngroups, s.dstate, s.headdim,
+                                                   npy(sc["B_inv_scale"]), npy(sc["C_inv_scale"]))
+        bfp_o = O.kron_hadamard(xBC_s[..., nh * s.headdim:nh * s.headdim + gn].reshape(1, s.seqlen, s.ngroups, s.dstate),
+                                npy(p["r_signs"])) if keyside else None
+        O.ssd_combined(x_o, npy(dt_raw[:1, :, :nh]), 1.0, npy(p["A_log"][:nh]), float(p["A_log_scale"]), qB_o,
+                       npy(sc["B_scale"]), qC_o, npy(sc["C_scale"]), s.chunk, npy(p["D"][:nh]), float(p["D_scale"]),
+                       dt_bias=npy(p["dt_bias"][:nh]), dt_softplus=True,
+                       static_state_scale=npy(sc["static_state_scale"][:nh]), static_cb_scale=npy(sc["static_cb_scale"]),
+                       alpha_hp=npy(sc["alpha_hp"][:nh]), bscale_g=npy(sc["bscale_g"]), keyside=keyside,
+                       x_scale_hp=npy(sc["x_scale_hp"][:nh]), b_fp=bfp_o, b_gate_scale=npy(sc["b_gate_scale"][:, :, :nh]))
+        t_cpu = time.perf_counter() - t0
+        frac = nh / (s.batch * s.nheads)
+        cpu = {"value": round(tokens * frac / t_cpu, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+               "sample": f"numpy/BLAS oracle on batch 1 x {nh} of {s.nheads} heads x {s.seqlen} tokens "
+                         f"({frac:.4f} of the layer) in {t_cpu:.2f} s; value = layer-equivalent tokens/s",
+               "host_cpus": os.cpu_count(), "torch_threads": torch.get_num_threads()}
+
+    line = {
+        "metric": "prefill tokens/s per layer at T=8192", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "mamba2-2.7b-shape SSD layer INT8 prefill (BASELINE.json configs[4]): B=4 L=8192 H=80 P=64 "
+                               "N=128 G=1 chunk=256, " + ("key-side" if keyside else "value-side") + " absorption, "
+                               "prologue + 5 SSD stages", "tokens_per_step": tokens},
+        "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

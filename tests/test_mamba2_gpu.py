@@ -129,7 +129,7 @@ def test_prologue_dqk_and_no_rotation(cuda):
     for use_signs, use_dqk in ((True, True), (False, False), (False, True)):
         _, qB, qC = fused_split_rotate_quant_xBC(xBC.to(cuda), signs.to(cuda) if use_signs else None, s.nheads, s.ngroups,
                                                  s.dstate, s.headdim, binv.to(cuda), cinv.to(cuda),
-                                                 dqk_b=(1 / dq).to(cuda) if use_dqk else None, dqk_c=dq.to(cuda) if use_dqk else None)
+                                                 dqk_b=(1 / dq).half().to(cuda) if use_dqk else None, dqk_c=prepare_dqk(dq).to(cuda) if use_dqk else None)
         torch.cuda.synchronize()
         _, rB, rC = O.split_rotate_quant_xBC(npy(xBC), npy(signs) if use_signs else None, s.nheads, s.ngroups, s.dstate,
                                              s.headdim, npy(binv), npy(cinv),
