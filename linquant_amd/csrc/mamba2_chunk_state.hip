@@ -9,16 +9,22 @@
 //               state = clamp(rint(float(acc) * (b_gate[n]/127) * (x_scale[p]/S_out[p])), +-127)
 //   gate[k] = exp(dA_last - dA[k]) * dt[k]
 //
-// One wavefront per (64-row P tile, <=128-col N tile, batch*chunk, head); the whole K = chunk loop runs in
-// registers.  Both operands are stored token-major in HBM while the MFMA wants 16 contraction slots per
-// lane, so each lane loads, for its 16 tokens, the 4 adjacent channels {4*(lane&15)+j}: 16 lanes cover one
-// contiguous 128-byte row, and packing "along tokens" yields the operand of MFMA call j directly.  Tile
-// row i of call j is therefore channel 4*i+j; the accumulator layout then gives every lane 4 adjacent
-// output columns, which are packed into one 32-bit store.
+// One 4-wave workgroup per (64-row P tile, <=128-col N tile, batch*chunk, head).  The per-element
+// quantization is the expensive part (VALU), so it is done exactly once per element: for every 64-token
+// slab the workgroup quantizes the x slab and the B slab cooperatively, writing INT8 codes to LDS already
+// transposed to "channel-major, token-contiguous" rows (each thread handles 4 tokens x 8 channels and emits
+// one dword of 4 token codes per channel), double-buffered against the next slab's global loads.  MFMA
+// operands are then plain 16-byte LDS reads; wave w owns the 16 P rows 16w..16w+15 and all N columns of
+// the tile (transposed product: accumulator rows are N, so each lane holds 4 adjacent N of one P row and
+// stores them as one dword).  The gates of the whole chunk are evaluated once per workgroup.
+// Round-half-even + clamp + int conversion is one fp32 add of 1.5*2^23 after the clamp (the low byte of the
+// sum's bit pattern is the two's-complement code).
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
 namespace {
+
+constexpr int kRS = 80;  // LDS row stride in bytes: 64 token codes + 16 pad (conflict-free 16-byte operand reads)
 
 struct Params {
   const _Float16* x;
@@ -39,167 +45,195 @@ struct Params {
   int batch, seqlen, nheads, P, G, N, Q, nchunks, n_ntiles;
 };
 
-template <bool KEYSIDE, int NH>
-__global__ __launch_bounds__(64) void chunk_state_kernel(Params p) {
-  const int lane = threadIdx.x, rl = lane & 15, kg = lane >> 4;
+// clamp to [-127, 127] then round half even; returns a dword whose low byte is the INT8 code
+LQ_DEV uint32_t rint_code(float y) {
+  const float c = __builtin_amdgcn_fmed3f(y, -127.0f, 127.0f);
+  return __float_as_uint(c + 12582912.0f);
+}
+
+LQ_DEV uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const uint32_t lo = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // {a.b0, b.b0, 0, 0}
+  const uint32_t hi = __builtin_amdgcn_perm(d, c, 0x04000c0cu);  // {0, 0, c.b0, d.b0}
+  return lo | hi;
+}
+
+template <bool KEYSIDE, int NT>
+__global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int Q = p.Q;
+  float* gate_s = (float*)lds_raw;                    // [Q]
+  unsigned char* xq = lds_raw + (size_t)Q * 4;        // [2][64][kRS]
+  unsigned char* bq = xq + 2 * 64 * kRS;              // [2][NT][kRS]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
   const int ptile = blockIdx.x / p.n_ntiles, ntile = blockIdx.x % p.n_ntiles;
   const int b = blockIdx.y / p.nchunks, c = blockIdx.y % p.nchunks;
   const int h = blockIdx.z;
   const int g = h / (p.nheads / p.G);
-  const int p0 = ptile * 64, n0 = ntile * (64 * NH);
-  const int Q = p.Q;
+  const int p0 = ptile * 64, n0 = ntile * NT;
   const int limit = min(Q, p.seqlen - c * Q);
-
-  const _Float16* xp = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0 + 4 * rl;
-  const int64_t tok0 = (int64_t)c * Q;
   const int64_t cs = (((int64_t)b * p.nheads + h) * p.nchunks + c) * Q;
-  const float* dtp = p.dt + cs;
-  const float* dAp = p.dA + cs;
-  const float dA_last = dAp[Q - 1];
 
-  // per-lane operand scales for the 4 channels p0 + 4*rl + j
-  float xinv[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float s = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 4 * rl + j) * p.sxs_p];
-    xinv[j] = KEYSIDE ? 1.0f / fmaxf(s, 1e-10f) : 1.0f / s;
-  }
-  float bgate[NH][4], binv[NH][4];
-  if (KEYSIDE) {
-#pragma unroll
-    for (int hf = 0; hf < NH; ++hf)
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int n = n0 + 64 * hf + 4 * rl + jj;
-        bgate[hf][jj] = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n];
-        binv[hf][jj] = 127.0f / bgate[hf][jj];
-      }
+  // ---- gates of the whole chunk
+  {
+    const float dA_last = p.dA[cs + Q - 1];
+    for (int k = tid; k < Q; k += 256) gate_s[k] = lq_expf(dA_last - p.dA[cs + k]) * p.dt[cs + k];
   }
 
-  lq_v4i acc[4][NH * 4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int q = 0; q < NH * 4; ++q) acc[j][q] = lq_v4i{0, 0, 0, 0};
+  // ---- fixed thread -> (token quad, 8-channel group) mapping of the quantize phase
+  const int kq = tid >> 4;  // for the B slab with NT = 128: 16 token quads x 16 channel groups
+  const int c8b = tid & 15;
+  const int kqx = tid >> 3;  // x slab: 16 token quads x 8 channel groups (threads 0..127)
+  const int c8x = tid & 7;
+  constexpr int kBItems = NT / 8;  // channel groups of the B slab
+  const bool has_b = (NT == 128) || (tid < 16 * kBItems);
+  const int kqb = (NT == 128) ? kq : (tid / kBItems);
+  const int cb8 = (NT == 128) ? c8b : (tid % kBItems);
+  const bool has_x = tid < 128;
 
-  for (int k0 = 0; k0 < Q; k0 += 64) {
-    const int kb = k0 + kg * 16;
-    float gate[16];
+  float xinv[8], binv[8];
+  if (has_x) {
 #pragma unroll
-    for (int t4 = 0; t4 < 4; ++t4) {
-      const float4 a4 = *(const float4*)(dAp + kb + 4 * t4);
-      const float4 d4 = *(const float4*)(dtp + kb + 4 * t4);
-      gate[4 * t4 + 0] = lq_expf(dA_last - a4.x) * d4.x;
-      gate[4 * t4 + 1] = lq_expf(dA_last - a4.y) * d4.y;
-      gate[4 * t4 + 2] = lq_expf(dA_last - a4.z) * d4.z;
-      gate[4 * t4 + 3] = lq_expf(dA_last - a4.w) * d4.w;
+    for (int e = 0; e < 8; ++e) {
+      const float s = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 8 * c8x + e) * p.sxs_p];
+      xinv[e] = KEYSIDE ? 1.0f / fmaxf(s, 1e-10f) : 1.0f / s;
     }
-    // ---- x operand: 16 tokens x 4 channels per lane
-    lq_v2i xw[16];
+  }
+  if (KEYSIDE && has_b) {
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      xw[t] = lq_v2i{0, 0};
-      if (kb + t < limit) xw[t] = *(const lq_v2i*)(xp + (int64_t)(kb + t) * p.sx_l);
+    for (int e = 0; e < 8; ++e) {
+      const int n = n0 + 8 * cb8 + e;
+      binv[e] = 127.0f / p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n];
     }
-    lq_v4i aop[4];
+  }
+
+  const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0 + 8 * c8x;
+  const int64_t tok0 = (int64_t)c * Q;
+  lq_v4i xr[4];  // x: 4 tokens x 8 fp16
+  lq_v4i br[4];  // key side: 4 tokens x 8 fp16; value side: only [t][0..1] used (8 int8)
+
+  auto load_slab = [&](int k0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int code[16];
-#pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        const uint32_t w = (uint32_t)xw[t][j >> 1];
-        const _Float16 hv = __builtin_bit_cast(_Float16, (uint16_t)(j & 1 ? w >> 16 : w & 0xffff));
-        float y = (float)hv * xinv[j];
+    for (int t = 0; t < 4; ++t) {
+      xr[t] = lq_v4i{0, 0, 0, 0};
+      br[t] = lq_v4i{0, 0, 0, 0};
+      const int kx = k0 + 4 * kqx + t;
+      if (has_x && kx < limit) xr[t] = *(const lq_v4i*)(xg + (int64_t)kx * p.sx_l);
+      const int kb = k0 + 4 * kqb + t;
+      if (has_b && kb < limit) {
         if (KEYSIDE) {
-          code[t] = lq_q_rint(y, -127, 127);
+          br[t] = *(const lq_v4i*)((const _Float16*)p.B + (int64_t)b * p.sB_b + (tok0 + kb) * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8);
         } else {
-          y = y * gate[t];
-          code[t] = lq_q_rha(y, 127);
+          const lq_v2i v = *(const lq_v2i*)((const int8_t*)p.B + (int64_t)b * p.sB_b + (tok0 + kb) * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8);
+          br[t][0] = v[0], br[t][1] = v[1];
         }
       }
-#pragma unroll
-      for (int d = 0; d < 4; ++d) aop[j][d] = (int)lq_pack4(code[4 * d], code[4 * d + 1], code[4 * d + 2], code[4 * d + 3]);
     }
-    // ---- B operand per 64-column half
+  };
+
+  lq_v4i acc[NT / 16];
 #pragma unroll
-    for (int hf = 0; hf < NH; ++hf) {
-      lq_v4i bop[4];
-      if (KEYSIDE) {
-        const _Float16* bp = (const _Float16*)p.B + (int64_t)b * p.sB_b + (int64_t)g * p.sB_g + n0 + 64 * hf + 4 * rl;
-        lq_v2i bw[16];
+  for (int q = 0; q < NT / 16; ++q) acc[q] = lq_v4i{0, 0, 0, 0};
+
+  load_slab(0);
+  __syncthreads();  // gates visible
+
+  const int nslab = Q >> 6;
+  for (int s = 0; s < nslab; ++s) {
+    const int k0 = s * 64;
+    unsigned char* xb = xq + (s & 1) * 64 * kRS;
+    unsigned char* bb = bq + (s & 1) * NT * kRS;
+    // ---- quantize this slab into LDS (codes of 4 consecutive tokens of one channel form one dword)
+    if (has_x) {
+      float gt[4];
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-          bw[t] = lq_v2i{0, 0};
-          if (kb + t < limit) bw[t] = *(const lq_v2i*)(bp + (tok0 + kb + t) * p.sB_l);
-        }
+      for (int t = 0; t < 4; ++t) gt[t] = gate_s[k0 + 4 * kqx + t];
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          int code[16];
+      for (int e = 0; e < 8; ++e) {
+        uint32_t cd[4];
 #pragma unroll
-          for (int t = 0; t < 16; ++t) {
-            const uint32_t w = (uint32_t)bw[t][jj >> 1];
-            const _Float16 hv = __builtin_bit_cast(_Float16, (uint16_t)(jj & 1 ? w >> 16 : w & 0xffff));
-            float y = (float)hv * gate[t];
-            y = y * binv[hf][jj];
-            code[t] = lq_q_rint(y, -127, 127);
+        for (int t = 0; t < 4; ++t) {
+          const uint32_t w = (uint32_t)xr[t][e >> 1];
+          const _Float16 hv = __builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
+          float y = (float)hv * xinv[e];
+          if (KEYSIDE) {
+            cd[t] = rint_code(y);
+          } else {
+            y = y * gt[t];
+            cd[t] = (uint32_t)lq_q_rha(y, 127);
           }
+        }
+        *(uint32_t*)(xb + (8 * c8x + e) * kRS + 4 * kqx) = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
+      }
+    }
+    if (has_b) {
+      if (KEYSIDE) {
+        float gt[4];
 #pragma unroll
-          for (int d = 0; d < 4; ++d)
-            bop[jj][d] = (int)lq_pack4(code[4 * d], code[4 * d + 1], code[4 * d + 2], code[4 * d + 3]);
+        for (int t = 0; t < 4; ++t) gt[t] = gate_s[k0 + 4 * kqb + t];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          uint32_t cd[4];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const uint32_t w = (uint32_t)br[t][e >> 1];
+            const _Float16 hv = __builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
+            float y = (float)hv * gt[t];
+            y = y * binv[e];
+            cd[t] = rint_code(y);
+          }
+          *(uint32_t*)(bb + (8 * cb8 + e) * kRS + 4 * kqb) = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
         }
       } else {
-        const int8_t* bp = (const int8_t*)p.B + (int64_t)b * p.sB_b + (int64_t)g * p.sB_g + n0 + 64 * hf + 4 * rl;
-        uint32_t bw[16];
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-          bw[t] = 0;
-          if (kb + t < limit) bw[t] = *(const uint32_t*)(bp + (tok0 + kb + t) * p.sB_l);
+        for (int e = 0; e < 8; ++e) {
+          // byte e of the four token rows -> one dword
+          const uint32_t s0 = (uint32_t)br[0][e >> 2], s1 = (uint32_t)br[1][e >> 2];
+          const uint32_t s2 = (uint32_t)br[2][e >> 2], s3 = (uint32_t)br[3][e >> 2];
+          const uint32_t sel = 0x0c0c0400u + 0x0101u * (e & 3);
+          const uint32_t lo = __builtin_amdgcn_perm(s1, s0, sel);
+          const uint32_t hi = __builtin_amdgcn_perm(s3, s2, sel);
+          *(uint32_t*)(bb + (8 * cb8 + e) * kRS + 4 * kqb) = lo | (hi << 16);
         }
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-          for (int d = 0; d < 4; ++d) {
-            // byte jj of four consecutive tokens -> one operand dword
-            const uint32_t lo = __builtin_amdgcn_perm(bw[4 * d + 1], bw[4 * d + 0], 0x0c0c0400u + 0x0101u * jj);
-            const uint32_t hi = __builtin_amdgcn_perm(bw[4 * d + 3], bw[4 * d + 2], 0x0c0c0400u + 0x0101u * jj);
-            bop[jj][d] = (int)(lo | (hi << 16));
-          }
       }
+    }
+    if (s + 1 < nslab) load_slab(k0 + 64);
+    __syncthreads();
+    // ---- MFMA from LDS: rows = N (this tile), cols = the wave's 16 P rows
+    const lq_v4i xop = *(const lq_v4i*)(xb + (16 * wave + rl) * kRS + 16 * kg);
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) acc[j][hf * 4 + jj] = lq_mfma_i8(aop[j], bop[jj], acc[j][hf * 4 + jj]);
+    for (int q = 0; q < NT / 16; ++q) {
+      const lq_v4i bop = *(const lq_v4i*)(bb + (16 * q + rl) * kRS + 16 * kg);
+      acc[q] = lq_mfma_i8(bop, xop, acc[q]);
     }
   }
 
-  // ---- epilogue: requantize and store 4 adjacent columns per 32-bit store
-  int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P) * p.N;
-  const float bscale = KEYSIDE ? 0.0f : p.bscale_g[(int64_t)g * p.sbs_g];
+  // ---- epilogue: lane holds N = n0 + 16q + 4kg + {0..3} of P row p0 + 16*wave + rl
+  const int pr = p0 + 16 * wave + rl;
+  const float xs = p.xs[(int64_t)h * p.sxs_h + (int64_t)pr * p.sxs_p];
+  const float so = p.oqs[(int64_t)h * p.soq_h + (int64_t)pr * p.soq_p];
+  const float ratio = xs / so;
+  const float req = KEYSIDE ? 0.0f : ratio * p.bscale_g[(int64_t)g * p.sbs_g];
+  int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + pr) * p.N + n0 + 4 * kg;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int q = 0; q < NT / 16; ++q) {
+    uint32_t cd[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int pr = p0 + 16 * kg + 4 * r + j;
-      const float xs = p.xs[(int64_t)h * p.sxs_h + (int64_t)pr * p.sxs_p];
-      const float so = p.oqs[(int64_t)h * p.soq_h + (int64_t)pr * p.soq_p];
-      const float ratio = xs / so;
-#pragma unroll
-      for (int hf = 0; hf < NH; ++hf) {
-        int code[4];
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const float a = (float)acc[j][hf * 4 + jj][r];
-          if (KEYSIDE) {
-            float y = a * (bgate[hf][jj] / 127.0f);
-            y = y * ratio;
-            code[jj] = lq_q_rint(y, -127, 127);
-          } else {
-            code[jj] = lq_q_rha(a * (ratio * bscale), 127);
-          }
-        }
-        *(uint32_t*)(sp + (int64_t)pr * p.N + n0 + 64 * hf + 4 * rl) = lq_pack4(code[0], code[1], code[2], code[3]);
+      const float a = (float)acc[q][r];
+      if (KEYSIDE) {
+        const int n = n0 + 16 * q + 4 * kg + r;
+        const float bg = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n];
+        float y = a * (bg / 127.0f);
+        y = y * ratio;
+        cd[r] = rint_code(y);
+      } else {
+        cd[r] = (uint32_t)lq_q_rha(a * req, 127);
       }
     }
+    *(uint32_t*)(sp + 16 * q) = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
+  }
 }
 
 bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
@@ -207,22 +241,24 @@ bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
 template <bool KEYSIDE>
 int launch(const Params& p, hipStream_t stream) {
   if (p.batch <= 0 || p.seqlen <= 0 || p.nheads <= 0 || p.G <= 0 || p.nheads % p.G != 0) return LQ_ERR_SHAPE;
-  if (p.P % 64 != 0 || p.N % 64 != 0 || p.Q % 64 != 0 || p.Q < 64) return LQ_ERR_SHAPE;
-  if (p.sx_b % 4 || p.sx_l % 4 || p.sx_h % 4 || !al(p.x, 8)) return LQ_ERR_SHAPE;
-  const int balign = KEYSIDE ? 8 : 4;
-  if (p.sB_b % 4 || p.sB_l % 4 || p.sB_g % 4 || !al(p.B, balign)) return LQ_ERR_SHAPE;
-  if (!al(p.dt, 16) || !al(p.dA, 16) || !al(p.states, 4)) return LQ_ERR_SHAPE;
+  if (p.P % 64 != 0 || p.N % 64 != 0 || p.Q % 64 != 0 || p.Q < 64 || p.Q > 4096) return LQ_ERR_SHAPE;
+  if (p.sx_b % 8 || p.sx_l % 8 || p.sx_h % 8 || !al(p.x, 16)) return LQ_ERR_SHAPE;
+  const int bmod = KEYSIDE ? 8 : 8, balign = KEYSIDE ? 16 : 8;
+  if (p.sB_b % bmod || p.sB_l % bmod || p.sB_g % bmod || !al(p.B, balign)) return LQ_ERR_SHAPE;
+  if (!al(p.states, 4)) return LQ_ERR_SHAPE;
   const int64_t by = (int64_t)p.batch * p.nchunks;
   if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
   Params q = p;
   if (p.N % 128 == 0) {
     q.n_ntiles = p.N / 128;
+    const size_t lds = (size_t)p.Q * 4 + 2 * 64 * kRS + 2 * 128 * kRS;
     dim3 grid((p.P / 64) * q.n_ntiles, (unsigned)by, p.nheads);
-    hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 2>), grid, dim3(64), 0, stream, q);
+    hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128>), grid, dim3(256), lds, stream, q);
   } else {
     q.n_ntiles = p.N / 64;
+    const size_t lds = (size_t)p.Q * 4 + 2 * 64 * kRS + 2 * 64 * kRS;
     dim3 grid((p.P / 64) * q.n_ntiles, (unsigned)by, p.nheads);
-    hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 1>), grid, dim3(64), 0, stream, q);
+    hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64>), grid, dim3(256), lds, stream, q);
   }
   return lq_check_launch();
 }
