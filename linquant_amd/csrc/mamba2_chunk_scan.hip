@@ -10,13 +10,14 @@
 // x[2kp+1][p]}) so that an fp16 MFMA operand (8 tokens of one channel) is four 16-byte LDS reads covering the
 // four channels {4*(lane&15)+j} of the four MFMA calls at once, with no register shuffling:
 //   xP : x as stored
-//   xS : x[k] * exp(dA_e(k) - dA_k) * S_cb * dt_k, where e(k) is the last token of k's 64-token block.
-// For 64-token blocks strictly before a wave's rows the causal weight factors as
-//   exp(dA_m - dA_k) = exp(dA_m - dA_e) * exp(dA_e - dA_k),      both exponents <= 0,
-// so those blocks need no per-element exponential: the A operand is the CB code itself (exact int8 -> fp16),
-// the B operand is xS, consecutive blocks are chained Horner-style with the scalar exp(dA_e(J) - dA_e(J-1))
-// on the fp32 accumulator and the row factor exp(dA_m - dA_e(last)) is applied once.  Only the 64-token block
-// that contains the wave's rows evaluates exp(dA_m - dA_k) per element (masked to k <= m).
+//   xS : x[k] * exp(dA_e(k) - dA_k) * S_cb * dt_k, where e(k) is the last token of k's 32-token slab.
+// For 32-token slabs strictly before a wave's rows the causal weight factors as
+//   exp(dA_m - dA_k) = exp(dA_m - dA_E) * exp(dA_E - dA_e) * exp(dA_e - dA_k),   all exponents <= 0,
+// (E = last token before the wave's rows), so those slabs need no per-element exponential: the B operand is
+// xS, the A operand is the CB code times the per-slab scalar exp(dA_E - dA_e), produced by the same packed
+// fp16 instruction that finishes the int8 -> fp16 conversion, and the row factor exp(dA_m - dA_E) is applied
+// once to the slab accumulator.  Only the wave's own 32-token slab evaluates exp(dA_m - dA_k) per element
+// (masked to k <= m).
 // State path: both INT8 operands are N-contiguous (16-byte global loads, INT8 MFMA).
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
@@ -49,13 +50,13 @@ struct ScanParams {
 LQ_DEV float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // 4 int8 codes (one dword) -> 4 exact fp16 values as two packed dwords: 0x6400 | (b ^ 0x80) is 1024 + (b + 128).
-LQ_DEV void i8x4_to_f16x4(uint32_t w, uint32_t& lo, uint32_t& hi) {
+// With (s2, o2) = (s, -1152 s) the result is s * code (one packed fma: exact for s = 1, fp16-rounded otherwise).
+LQ_DEV void i8x4_to_f16x4(uint32_t w, lq_v2h s2, lq_v2h o2, uint32_t& lo, uint32_t& hi) {
   const uint32_t u = w ^ 0x80808080u;
   const uint32_t a = __builtin_amdgcn_perm(0x64646464u, u, 0x05010400u);
   const uint32_t b = __builtin_amdgcn_perm(0x64646464u, u, 0x05030402u);
-  const lq_v2h off = {(_Float16)-1152.0f, (_Float16)-1152.0f};
-  lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(lq_v2h, a) + off);
-  hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(lq_v2h, b) + off);
+  lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(lq_v2h, a), s2, o2));
+  hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(lq_v2h, b), s2, o2));
 }
 
 LQ_DEV uint32_t pack_h2(float a, float b) {
@@ -74,9 +75,11 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  const int p0 = blockIdx.x * 64;
+  // heads vary fastest across consecutive workgroups: the C / CB tiles of a (batch, chunk) are shared by all
+  // heads of a group and stay in L2 while they are swept
+  const int h = blockIdx.x % p.nheads;
+  const int p0 = (blockIdx.x / p.nheads) * 64;
   const int b = blockIdx.y / p.nchunks, c = blockIdx.y % p.nchunks;
-  const int h = blockIdx.z;
   const int g = h / (p.nheads / p.G);
   const int limit = min(Q, p.seqlen - c * Q);
   const int64_t cs = (((int64_t)b * p.nheads + h) * p.nchunks + c) * Q;
@@ -100,20 +103,45 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     if (2 * kp < limit) r0[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp) * p.sx_l + c8 * 8);
     if (2 * kp + 1 < limit) r1[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp + 1) * p.sx_l + c8 * 8);
   }
+  const int mbase = wave * 32;
+  // ---- state path (INT8 MFMA), issued before the staging barrier so its global loads overlap the x tile's
+  lq_v4i ai[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ai[i][j] = lq_v4i{0, 0, 0, 0};
+  if (mbase < limit) {
+    const int8_t* Cp = p.C + (int64_t)b * p.sC_b + (int64_t)c * Q * p.sC_l + (int64_t)g * p.sC_g;
+    const int8_t* Sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P) * p.N;
+    for (int n0 = 0; n0 < p.N; n0 += 64) {
+      const int nn = n0 + kg * 16;
+      lq_v4i cop[2], sop[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int m = min(mbase + 16 * i + rl, limit - 1);
+        cop[i] = *(const lq_v4i*)(Cp + (int64_t)m * p.sC_l + nn);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sop[j] = *(const lq_v4i*)(Sp + (int64_t)(p0 + 4 * rl + j) * p.N + nn);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ai[i][j] = lq_mfma_i8(cop[i], sop[j], ai[i][j]);
+    }
+  }
   __syncthreads();
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int kp = kp_of[it], c8 = c8_of[it];
-    const int k = 2 * kp, ke = (k | 63);
+    const int k = 2 * kp, ke = (k | 31);
     const float ae = dA2_s[ke];
-    const float g0 = fexp2(ae - dA2_s[k]) * w_s[k];
-    const float g1 = fexp2(ae - dA2_s[k + 1]) * w_s[k + 1];
+    const lq_v2h g2 = {(_Float16)(fexp2(ae - dA2_s[k]) * w_s[k]), (_Float16)(fexp2(ae - dA2_s[k + 1]) * w_s[k + 1])};
     lq_v4i plain[2], scaled[2];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const lq_v2h pr = {r0[it][e], r1[it][e]};
       plain[e >> 2][e & 3] = (int)__builtin_bit_cast(uint32_t, pr);
-      scaled[e >> 2][e & 3] = (int)pack_h2((float)r0[it][e] * g0, (float)r1[it][e] * g1);
+      scaled[e >> 2][e & 3] = (int)__builtin_bit_cast(uint32_t, pr * g2);
     }
     uint32_t* d0 = xP + kp * kRow + c8 * 8;
     uint32_t* d1 = xS + kp * kRow + c8 * 8;
@@ -124,130 +152,86 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   }
   __syncthreads();
 
-  const int mbase = wave * 32;
   if (mbase >= limit) return;
 
-  // ---- state path (INT8 MFMA)
+  // ---- state read dequantized and gated: float(acc) * (sC * ss[p]) * exp(dA_m)
   lq_v4f acc[2][4];  // [16-row tile][channel call j]
   {
-    lq_v4i ai[2][4];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ai[i][j] = lq_v4i{0, 0, 0, 0};
-    const int8_t* Cp = p.C + (int64_t)b * p.sC_b + (int64_t)c * Q * p.sC_l + (int64_t)g * p.sC_g;
-    const int8_t* Sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P) * p.N;
-    for (int n0 = 0; n0 < p.N; n0 += 64) {
-      const int nn = n0 + kg * 16;
-      lq_v4i cop[2], sop[4];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int m = mbase + 16 * i + rl;
-        cop[i] = lq_v4i{0, 0, 0, 0};
-        if (m < limit) cop[i] = *(const lq_v4i*)(Cp + (int64_t)m * p.sC_l + nn);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) sop[j] = *(const lq_v4i*)(Sp + (int64_t)(p0 + 4 * rl + j) * p.N + nn);
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) ai[i][j] = lq_mfma_i8(cop[i], sop[j], ai[i][j]);
-    }
     const float gscale = p.C_scale[g];
     float ssv[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) ssv[j] = p.ss[(int64_t)h * p.sss_h + (int64_t)(p0 + 4 * rl + j) * p.sss_p];
+    for (int j = 0; j < 4; ++j) ssv[j] = gscale * p.ss[(int64_t)h * p.sss_h + (int64_t)(p0 + 4 * rl + j) * p.sss_p];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float rg = fexp2(dA2_s[mbase + 16 * i + 4 * kg + r]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float v = (float)ai[i][j][r] * gscale;
-          v = v * ssv[j];
-          acc[i][j][r] = v * rg;
-        }
+        for (int j = 0; j < 4; ++j) acc[i][j][r] = (float)ai[i][j][r] * (ssv[j] * rg);
       }
   }
 
   const int8_t* cbp = p.cb + ((((int64_t)b * p.nchunks + c) * p.G + g) * Q) * Q;
-  const int nblk = mbase >> 6;  // 64-token blocks strictly before this wave's rows
+  const int nslab = mbase >> 5;  // 32-token slabs strictly before this wave's rows
 
-  // ---- blocks before the wave's rows: CB codes x anchor-scaled x, Horner chain on the accumulator
-  if (nblk > 0) {
+  // ---- slabs before the wave's rows: (scaled CB codes) x (anchor-scaled x), row factor applied once
+  if (nslab > 0) {
     lq_v4f off[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) off[i][j] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-    lq_v2i cw[2][2], cwn[2][2];  // [slab][row tile]
+    const float aE = dA2_s[mbase - 1];
+    lq_v2i cw[2], cwn[2];
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2)
+    for (int i = 0; i < 2; ++i) cw[i] = *(const lq_v2i*)(cbp + (int64_t)(mbase + 16 * i + rl) * Q + 8 * kg);
+    for (int J = 0; J < nslab; ++J) {
+      if (J + 1 < nslab) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        cw[s2][i] = *(const lq_v2i*)(cbp + (int64_t)(mbase + 16 * i + rl) * Q + 32 * s2 + 8 * kg);
-    for (int J = 0; J < nblk; ++J) {
-      if (J + 1 < nblk) {
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int i = 0; i < 2; ++i)
-            cwn[s2][i] = *(const lq_v2i*)(cbp + (int64_t)(mbase + 16 * i + rl) * Q + 64 * (J + 1) + 32 * s2 + 8 * kg);
+        for (int i = 0; i < 2; ++i) cwn[i] = *(const lq_v2i*)(cbp + (int64_t)(mbase + 16 * i + rl) * Q + 32 * (J + 1) + 8 * kg);
       }
-      if (J > 0) {
-        const float hs = fexp2(dA2_s[64 * J + 63] - dA2_s[64 * J - 1]);
+      const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
+      const lq_v2h s2 = {sh, sh};
+      const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
+      const int kp0 = 16 * J + 4 * kg;  // token pair index of this lane's first slot
+      lq_v4i xop[4];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+      for (int d = 0; d < 4; ++d) {
+        const lq_v4i v = *(const lq_v4i*)(xS + (kp0 + d) * kRow + 4 * rl);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) off[i][j] = off[i][j] * hs;
-      }
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        const int kp0 = 32 * J + 16 * s2 + 4 * kg;  // token pair index of this lane's first slot
-        lq_v4i xop[4];
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const lq_v4i v = *(const lq_v4i*)(xS + (kp0 + d) * kRow + 4 * rl);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          lq_v4i aw;
-          uint32_t lo, hi;
-          i8x4_to_f16x4((uint32_t)cw[s2][i][0], lo, hi);
-          aw[0] = (int)lo, aw[1] = (int)hi;
-          i8x4_to_f16x4((uint32_t)cw[s2][i][1], lo, hi);
-          aw[2] = (int)lo, aw[3] = (int)hi;
-          const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) off[i][j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[i][j]);
-        }
+        for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
       }
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
+      for (int i = 0; i < 2; ++i) {
+        lq_v4i aw;
+        uint32_t lo, hi;
+        i8x4_to_f16x4((uint32_t)cw[i][0], s2, o2, lo, hi);
+        aw[0] = (int)lo, aw[1] = (int)hi;
+        i8x4_to_f16x4((uint32_t)cw[i][1], s2, o2, lo, hi);
+        aw[2] = (int)lo, aw[3] = (int)hi;
+        const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) cw[s2][i] = cwn[s2][i];
+        for (int j = 0; j < 4; ++j) off[i][j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[i][j]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) cw[i] = cwn[i];
     }
-    const float ae = dA2_s[64 * nblk - 1];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float rf = fexp2(dA2_s[mbase + 16 * i + 4 * kg + r] - ae);
+        const float rf = fexp2(dA2_s[mbase + 16 * i + 4 * kg + r] - aE);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j][r] = fmaf(off[i][j][r], rf, acc[i][j][r]);
       }
   }
 
-  // ---- the 64-token block holding the wave's rows: per-element weights, masked to k <= m
-  float dAm[2];
+  // ---- the wave's own 32-token slab: per-element weights exp2(dA2_m - (dA2_k - log2(S_cb dt_k))), k <= m
+  {
+    float dAm[2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) dAm[i] = dA2_s[mbase + 16 * i + rl];
-  const int kend = min(mbase + 32, limit);
-  for (int k0 = 64 * nblk; k0 < kend; k0 += 32) {
-    const int kb = k0 + 8 * kg;
+    for (int i = 0; i < 2; ++i) dAm[i] = dA2_s[mbase + 16 * i + rl];
+    const int kb = mbase + 8 * kg;
     lq_v4i xop[4];
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
@@ -257,6 +241,12 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     }
     const lq_v4f a0 = *(const lq_v4f*)(dA2_s + kb), a1 = *(const lq_v4f*)(dA2_s + kb + 4);
     const lq_v4f w0 = *(const lq_v4f*)(w_s + kb), w1 = *(const lq_v4f*)(w_s + kb + 4);
+    float akw[8];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      akw[t] = a0[t] - __builtin_amdgcn_logf(w0[t]);
+      akw[4 + t] = a1[t] - __builtin_amdgcn_logf(w1[t]);
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int m = mbase + 16 * i + rl;
@@ -265,9 +255,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
         const float cf = (float)lq_sbyte((uint32_t)cw[t >> 2], t & 3);
-        const float ak = t < 4 ? a0[t & 3] : a1[t & 3];
-        const float wk = t < 4 ? w0[t & 3] : w1[t & 3];
-        v[t] = cf * (fexp2(dAm[i] - ak) * wk);
+        v[t] = cf * fexp2(dAm[i] - akw[t]);
         if (kb + t > m) v[t] = 0.0f;
       }
       lq_v4i aw;
@@ -298,9 +286,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       lq_v4h o;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t wv = (uint32_t)xv[j];
-        const _Float16 xr = __builtin_bit_cast(_Float16, (uint16_t)((m & 1) ? (wv >> 16) : (wv & 0xffffu)));
-        o[j] = (_Float16)(acc[i][j][r] + (float)xr * Dv[j]);
+        const uint32_t wv = (uint32_t)xv[j];  // rows alternate low / high half: m & 1 == r & 1
+        const _Float16 xr = __builtin_bit_cast(_Float16, (uint16_t)((r & 1) ? (wv >> 16) : (wv & 0xffffu)));
+        o[j] = (_Float16)fmaf((float)xr, Dv[j], acc[i][j][r]);
       }
       *(lq_v4h*)(op + (int64_t)m * p.nheads * p.P) = o;
     }
@@ -335,7 +323,7 @@ extern "C" int lq_chunk_scan(const lq_chunk_scan_args* a, hipStream_t stream) {
   const int64_t by = (int64_t)p.batch * p.nchunks;
   if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
   const size_t lds = (size_t)p.Q * kRow * 4 + (size_t)p.Q * 8;  // two [Q/2][kRow] dword tiles + dA2 + w
-  dim3 grid(p.P / 64, (unsigned)by, p.nheads);
+  dim3 grid((p.P / 64) * p.nheads, (unsigned)by, 1);
   // more than 64 KB of dynamic LDS has to be opted into per kernel
 #define LQ_SCAN_LAUNCH(W)                                                                                   \
   do {                                                                                                      \

@@ -11,10 +11,11 @@
 //
 // One 4-wave workgroup per (64-row P tile, <=128-col N tile, batch*chunk, head).  The per-element
 // quantization is the expensive part (VALU), so it is done exactly once per element: for every 64-token
-// slab the workgroup quantizes the x slab and the B slab cooperatively, writing INT8 codes to LDS already
-// transposed to "channel-major, token-contiguous" rows (each thread handles 4 tokens x 8 channels and emits
-// one dword of 4 token codes per channel), double-buffered against the next slab's global loads.  MFMA
-// operands are then plain 16-byte LDS reads; wave w owns the 16 P rows 16w..16w+15 and all N columns of
+// slab the workgroup quantizes the x slab and the B slab cooperatively into LDS, double-buffered against the
+// next slab's global loads.  A thread handles 4 consecutive tokens of a few adjacent channels and emits, per
+// channel, one dword holding the 4 token codes; LDS is laid out [token quad][channel] in dwords, so those
+// stores are contiguous 16-byte writes and an MFMA operand (16 token codes of one channel) is 4 dword reads
+// at consecutive banks across the lanes.  Wave w owns the 16 P rows 16w..16w+15 and all N columns of
 // the tile (transposed product: accumulator rows are N, so each lane holds 4 adjacent N of one P row and
 // stores them as one dword).  The gates of the whole chunk are evaluated once per workgroup.
 // Round-half-even + clamp + int conversion is one fp32 add of 1.5*2^23 after the clamp (the low byte of the
@@ -24,7 +25,8 @@
 
 namespace {
 
-constexpr int kRS = 80;  // LDS row stride in bytes: 64 token codes + 16 pad (conflict-free 16-byte operand reads)
+constexpr int kXW = 64 + 4;    // dwords per token-quad row of the x slab (64 channels + pad: the four lane groups of an
+constexpr int kPad = 4;       // operand read land on bank offsets 0,16,32,48)
 
 struct Params {
   const _Float16* x;
@@ -62,14 +64,19 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int Q = p.Q;
   float* gate_s = (float*)lds_raw;                    // [Q]
-  unsigned char* xq = lds_raw + (size_t)Q * 4;        // [2][64][kRS]
-  unsigned char* bq = xq + 2 * 64 * kRS;              // [2][NT][kRS]
+  float* bdeq_s = gate_s + Q;                         // [NT] b_gate / 127 (key side)
+  constexpr int kBW = NT + kPad;
+  uint32_t* xq = (uint32_t*)(bdeq_s + NT);            // [2][16][kXW]
+  uint32_t* bq = xq + 2 * 16 * kXW;                   // [2][16][kBW]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  const int ptile = blockIdx.x / p.n_ntiles, ntile = blockIdx.x % p.n_ntiles;
+  // heads vary fastest across consecutive workgroups: the B tile of a (batch, chunk) is shared by the heads of
+  // a group and stays in L2 while they are swept
+  const int h = blockIdx.x % p.nheads;
+  const int tile = blockIdx.x / p.nheads;
+  const int ptile = tile / p.n_ntiles, ntile = tile % p.n_ntiles;
   const int b = blockIdx.y / p.nchunks, c = blockIdx.y % p.nchunks;
-  const int h = blockIdx.z;
   const int g = h / (p.nheads / p.G);
   const int p0 = ptile * 64, n0 = ntile * NT;
   const int limit = min(Q, p.seqlen - c * Q);
@@ -78,27 +85,28 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
   // ---- gates of the whole chunk
   {
     const float dA_last = p.dA[cs + Q - 1];
-    for (int k = tid; k < Q; k += 256) gate_s[k] = lq_expf(dA_last - p.dA[cs + k]) * p.dt[cs + k];
+    for (int k = tid; k < Q; k += 256) gate_s[k] = k < limit ? lq_expf(dA_last - p.dA[cs + k]) * p.dt[cs + k] : 0.0f;
+    if (KEYSIDE && tid < NT) {
+      const int n = n0 + tid;
+      bdeq_s[tid] = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n] / 127.0f;
+    }
   }
 
-  // ---- fixed thread -> (token quad, 8-channel group) mapping of the quantize phase
-  const int kq = tid >> 4;  // for the B slab with NT = 128: 16 token quads x 16 channel groups
-  const int c8b = tid & 15;
-  const int kqx = tid >> 3;  // x slab: 16 token quads x 8 channel groups (threads 0..127)
-  const int c8x = tid & 7;
-  constexpr int kBItems = NT / 8;  // channel groups of the B slab
+  // ---- fixed thread -> work mapping of the quantize phase: x slab = 16 token quads x 16 groups of 4 channels
+  // (all 256 threads), B slab = 16 token quads x NT/8 groups of 8 channels.  Tokens past the sequence end
+  // carry a zero gate, which zeroes the gated operand's codes; their loads are redirected to the last valid
+  // token so no access leaves the tensor.
+  const int kqx = tid >> 4, c4x = tid & 15;
+  constexpr int kBItems = NT / 8;
   const bool has_b = (NT == 128) || (tid < 16 * kBItems);
-  const int kqb = (NT == 128) ? kq : (tid / kBItems);
-  const int cb8 = (NT == 128) ? c8b : (tid % kBItems);
-  const bool has_x = tid < 128;
+  const int kqb = (NT == 128) ? (tid >> 4) : (tid / kBItems);
+  const int cb8 = (NT == 128) ? (tid & 15) : (tid % kBItems);
 
-  float xinv[8], binv[8];
-  if (has_x) {
+  float xinv[4], binv[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float s = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 8 * c8x + e) * p.sxs_p];
-      xinv[e] = KEYSIDE ? 1.0f / fmaxf(s, 1e-10f) : 1.0f / s;
-    }
+  for (int e = 0; e < 4; ++e) {
+    const float sc = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 4 * c4x + e) * p.sxs_p];
+    xinv[e] = KEYSIDE ? 1.0f / fmaxf(sc, 1e-10f) : 1.0f / sc;
   }
   if (KEYSIDE && has_b) {
 #pragma unroll
@@ -108,24 +116,24 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
     }
   }
 
-  const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0 + 8 * c8x;
-  const int64_t tok0 = (int64_t)c * Q;
-  lq_v4i xr[4];  // x: 4 tokens x 8 fp16
+  const int last = limit - 1;
+  const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0 + 4 * c4x;
+  const char* bg0 = (const char*)p.B + ((int64_t)b * p.sB_b + (int64_t)c * Q * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8) * (KEYSIDE ? 2 : 1);
+  const int64_t bstep = p.sB_l * (KEYSIDE ? 2 : 1);  // bytes per token
+  lq_v2i xr[4];  // x: 4 tokens x 4 fp16
   lq_v4i br[4];  // key side: 4 tokens x 8 fp16; value side: only [t][0..1] used (8 int8)
 
   auto load_slab = [&](int k0) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      xr[t] = lq_v4i{0, 0, 0, 0};
-      br[t] = lq_v4i{0, 0, 0, 0};
-      const int kx = k0 + 4 * kqx + t;
-      if (has_x && kx < limit) xr[t] = *(const lq_v4i*)(xg + (int64_t)kx * p.sx_l);
-      const int kb = k0 + 4 * kqb + t;
-      if (has_b && kb < limit) {
+      const int kx = min(k0 + 4 * kqx + t, last);
+      xr[t] = *(const lq_v2i*)(xg + (int64_t)kx * p.sx_l);
+      if (has_b) {
+        const int kb = min(k0 + 4 * kqb + t, last);
         if (KEYSIDE) {
-          br[t] = *(const lq_v4i*)((const _Float16*)p.B + (int64_t)b * p.sB_b + (tok0 + kb) * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8);
+          br[t] = *(const lq_v4i*)(bg0 + (int64_t)kb * bstep);
         } else {
-          const lq_v2i v = *(const lq_v2i*)((const int8_t*)p.B + (int64_t)b * p.sB_b + (tok0 + kb) * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8);
+          const lq_v2i v = *(const lq_v2i*)(bg0 + (int64_t)kb * bstep);
           br[t][0] = v[0], br[t][1] = v[1];
         }
       }
@@ -142,15 +150,16 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
   const int nslab = Q >> 6;
   for (int s = 0; s < nslab; ++s) {
     const int k0 = s * 64;
-    unsigned char* xb = xq + (s & 1) * 64 * kRS;
-    unsigned char* bb = bq + (s & 1) * NT * kRS;
+    uint32_t* xb = xq + (s & 1) * 16 * kXW;
+    uint32_t* bb = bq + (s & 1) * 16 * kBW;
     // ---- quantize this slab into LDS (codes of 4 consecutive tokens of one channel form one dword)
-    if (has_x) {
+    {
       float gt[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) gt[t] = gate_s[k0 + 4 * kqx + t];
+      lq_v4i xo;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 4; ++e) {
         uint32_t cd[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -164,10 +173,12 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
             cd[t] = (uint32_t)lq_q_rha(y, 127);
           }
         }
-        *(uint32_t*)(xb + (8 * c8x + e) * kRS + 4 * kqx) = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
+        xo[e] = (int)pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
       }
+      *(lq_v4i*)(xb + kqx * kXW + 4 * c4x) = xo;
     }
     if (has_b) {
+      lq_v4i bo[2];
       if (KEYSIDE) {
         float gt[4];
 #pragma unroll
@@ -183,7 +194,7 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
             y = y * binv[e];
             cd[t] = rint_code(y);
           }
-          *(uint32_t*)(bb + (8 * cb8 + e) * kRS + 4 * kqb) = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
+          bo[e >> 2][e & 3] = (int)pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
         }
       } else {
 #pragma unroll
@@ -194,17 +205,24 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
           const uint32_t sel = 0x0c0c0400u + 0x0101u * (e & 3);
           const uint32_t lo = __builtin_amdgcn_perm(s1, s0, sel);
           const uint32_t hi = __builtin_amdgcn_perm(s3, s2, sel);
-          *(uint32_t*)(bb + (8 * cb8 + e) * kRS + 4 * kqb) = lo | (hi << 16);
+          bo[e >> 2][e & 3] = (int)(lo | (hi << 16));
         }
       }
+      uint32_t* dst = bb + kqb * kBW + 8 * cb8;
+      *(lq_v4i*)dst = bo[0];
+      *(lq_v4i*)(dst + 4) = bo[1];
     }
     if (s + 1 < nslab) load_slab(k0 + 64);
     __syncthreads();
     // ---- MFMA from LDS: rows = N (this tile), cols = the wave's 16 P rows
-    const lq_v4i xop = *(const lq_v4i*)(xb + (16 * wave + rl) * kRS + 16 * kg);
+    lq_v4i xop;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xop[i] = (int)xb[(4 * kg + i) * kXW + 16 * wave + rl];
 #pragma unroll
     for (int q = 0; q < NT / 16; ++q) {
-      const lq_v4i bop = *(const lq_v4i*)(bb + (16 * q + rl) * kRS + 16 * kg);
+      lq_v4i bop;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bop[i] = (int)bb[(4 * kg + i) * kBW + 16 * q + rl];
       acc[q] = lq_mfma_i8(bop, xop, acc[q]);
     }
   }
@@ -223,9 +241,7 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
     for (int r = 0; r < 4; ++r) {
       const float a = (float)acc[q][r];
       if (KEYSIDE) {
-        const int n = n0 + 16 * q + 4 * kg + r;
-        const float bg = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n];
-        float y = a * (bg / 127.0f);
+        float y = a * bdeq_s[16 * q + 4 * kg + r];
         y = y * ratio;
         cd[r] = rint_code(y);
       } else {
@@ -242,7 +258,7 @@ template <bool KEYSIDE>
 int launch(const Params& p, hipStream_t stream) {
   if (p.batch <= 0 || p.seqlen <= 0 || p.nheads <= 0 || p.G <= 0 || p.nheads % p.G != 0) return LQ_ERR_SHAPE;
   if (p.P % 64 != 0 || p.N % 64 != 0 || p.Q % 64 != 0 || p.Q < 64 || p.Q > 4096) return LQ_ERR_SHAPE;
-  if (p.sx_b % 8 || p.sx_l % 8 || p.sx_h % 8 || !al(p.x, 16)) return LQ_ERR_SHAPE;
+  if (p.sx_b % 4 || p.sx_l % 4 || p.sx_h % 4 || !al(p.x, 8)) return LQ_ERR_SHAPE;
   const int bmod = KEYSIDE ? 8 : 8, balign = KEYSIDE ? 16 : 8;
   if (p.sB_b % bmod || p.sB_l % bmod || p.sB_g % bmod || !al(p.B, balign)) return LQ_ERR_SHAPE;
   if (!al(p.states, 4)) return LQ_ERR_SHAPE;
@@ -251,13 +267,13 @@ int launch(const Params& p, hipStream_t stream) {
   Params q = p;
   if (p.N % 128 == 0) {
     q.n_ntiles = p.N / 128;
-    const size_t lds = (size_t)p.Q * 4 + 2 * 64 * kRS + 2 * 128 * kRS;
-    dim3 grid((p.P / 64) * q.n_ntiles, (unsigned)by, p.nheads);
+    const size_t lds = (size_t)p.Q * 4 + 128 * 4 + (2 * 16 * kXW + 2 * 16 * (128 + kPad)) * 4;
+    dim3 grid((p.P / 64) * q.n_ntiles * p.nheads, (unsigned)by, 1);
     hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128>), grid, dim3(256), lds, stream, q);
   } else {
     q.n_ntiles = p.N / 64;
-    const size_t lds = (size_t)p.Q * 4 + 2 * 64 * kRS + 2 * 64 * kRS;
-    dim3 grid((p.P / 64) * q.n_ntiles, (unsigned)by, p.nheads);
+    const size_t lds = (size_t)p.Q * 4 + 64 * 4 + (2 * 16 * kXW + 2 * 16 * (64 + kPad)) * 4;
+    dim3 grid((p.P / 64) * q.n_ntiles * p.nheads, (unsigned)by, 1);
     hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64>), grid, dim3(256), lds, stream, q);
   }
   return lq_check_launch();
