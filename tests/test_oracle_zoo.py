@@ -1,0 +1,155 @@
+"""Pins the float64 zoo oracle (oracle/zoo_reference.py) against the reference's own golden vectors
+(tests/golden/zoo_golden.npz, written by tests/golden/make_zoo_golden.py from linquant/reference.py), against
+brute-force token-by-token recurrences, and against the invariances the reference's test suite holds
+(/root/reference tests/test_reference.py:74-228)."""
+
+import ast
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import zoo_reference as Z
+from tests.golden.make_zoo_golden import B, C, CELLS, H, K, T, V, make_inputs
+
+GOLD = np.load(Path(__file__).parent / "golden" / "zoo_golden.npz")
+N_CASES = int(GOLD["n_cases"])
+
+
+def _run_case(i):
+    p = f"c{i:02d}_"
+    cs = ast.literal_eval(str(GOLD[p + "meta"]))
+    fam, dec = CELLS[cs["cell"]]
+    q, k, v, g, beta = make_inputs(cs["cell"], seed=100 + i)
+    sums = np.array([t.double().abs().sum().item() for t in (q, k, v, g, beta) if t is not None])
+    assert np.allclose(sums, GOLD[p + "input_sum"], rtol=1e-12), "seeded input generator drifted"
+    qz = Z.ZooQuantizer.kernel_profile(cs["policy"], cs["bits"])
+    rq = torch.from_numpy(GOLD[p + "rot_qk"]) if "rot_qk" in cs else None
+    rv = torch.from_numpy(GOLD[p + "rot_v"]) if "rot_v" in cs else None
+    kw = dict(family=fam, decay=dec, scale=K ** -0.5, qz=qz, eta=cs["eta"], rho=cs["rho"], tau=cs["tau"], read_post=True,
+              C=C, rot_qk=rq, rot_v=rv, storage=cs.get("storage", "rotated"), out_dtype=torch.float64)
+    qz.calibrating = True
+    Z.chunk_forward(q, k, v, g, beta, **kw)
+    qz.finalize()
+    qz.trace = []
+    o = Z.chunk_forward(q, k, v, g, beta, **kw)
+    return cs, qz, o, p
+
+
+@pytest.mark.parametrize("i", range(N_CASES))
+def test_golden_vectors_of_the_reference(i):
+    cs, qz, o, p = _run_case(i)
+    for (layer, role), sc in qz.scales.items():
+        ref = GOLD[p + "scale_" + role]
+        assert np.allclose(sc.numpy(), ref, rtol=1e-12, atol=0), (cs, role)
+    codes = np.stack([c.to(torch.int8).numpy() for c in qz.trace])
+    assert np.array_equal(codes, GOLD[p + "codes"]), f"{cs}: stored INT8 state codes differ"
+    ref_o = GOLD[p + "o"]
+    assert np.abs(o.numpy() - ref_o).max() <= 1e-9 * np.abs(ref_o).max(), cs
+
+
+def test_golden_cover_every_cell_and_policy():
+    seen = set()
+    for i in range(N_CASES):
+        cs = ast.literal_eval(str(GOLD[f"c{i:02d}_meta"]))
+        seen.add((cs["cell"], cs["policy"]))
+    assert {(c, p) for c in CELLS for p in ("kernel_static", "kernel_pt", "kernel_ptk")} <= seen
+
+
+def test_state_pass_known_answer():
+    """fp32-carry pass: the carry is never quantized, only the read copy (sc=0.5, gamma=0.9, local=0.3 x4)."""
+    qz = Z.ZooQuantizer("none", 8, ["ALL"], state_bits=8)
+    qz.scales[(0, "state")] = torch.full((1, 1), 0.5, dtype=torch.float64)
+    S, carry, ref = torch.zeros(1, 1, 1, 1, dtype=torch.float64), None, 0.0
+    for step, lc in enumerate((0.3, 0.3, 0.3, 0.3)):
+        S, carry = Z._carry_update(S, carry, torch.full((1, 1, 1, 1), 0.9, dtype=torch.float64),
+                                   torch.full((1, 1, 1, 1), lc, dtype=torch.float64), qz)
+        ref = 0.9 * ref + lc
+        assert abs(carry.item() - ref) < 1e-12 and abs(S.item() - round(ref / 0.5) * 0.5) < 1e-12
+        assert np.allclose([S.item(), carry.item()], GOLD["kat_state_pass"][step], atol=1e-15)
+
+
+def test_hadamard_sign_streams_and_orthogonality():
+    for name in GOLD.files:
+        if name.startswith("hadamard_"):
+            _, n, seed = name.split("_")
+            R = Z.signed_hadamard(int(n), int(seed))
+            assert np.array_equal(np.sign(R.numpy()[0]), GOLD[name])
+            assert torch.allclose(R @ R.T, torch.eye(int(n), dtype=R.dtype), atol=1e-12)
+
+
+# ----------------------------------------------------------------------------- brute force (no quantization)
+def _token_recurrence(q, k, v, g, beta, family, decay, scale):
+    """S_t = Diag(exp g_t) S_{t-1} + k_t v_t^T (linear) or the (gated) delta rule; o_t = (q_t scale) S_t."""
+    q, k, v = q.double(), k.double(), v.double()
+    Bn, Tn, Hn, Kn = q.shape
+    S = torch.zeros(Bn, Hn, Kn, v.shape[-1], dtype=torch.float64)
+    out = torch.zeros(Bn, Tn, Hn, v.shape[-1], dtype=torch.float64)
+    for t in range(Tn):
+        if g is not None:
+            gt = g[:, t].double().exp()
+            S = S * (gt[..., None, None] if decay == "scalar" else gt[..., None])
+        kt, vt = k[:, t], v[:, t]
+        if family == "delta":
+            bt = beta[:, t].double()[..., None]
+            vt = bt * (vt - torch.einsum("bhk,bhkv->bhv", kt, S))
+        S = S + kt[..., None] * vt[..., None, :]
+        out[:, t] = torch.einsum("bhk,bhkv->bhv", q[:, t] * scale, S)
+    return out
+
+
+@pytest.mark.parametrize("cell", list(CELLS))
+def test_unquantized_matches_token_recurrence(cell):
+    fam, dec = CELLS[cell]
+    q, k, v, g, beta = make_inputs(cell, seed=5)
+    ref = _token_recurrence(q, k, v, g, beta, fam, dec, K ** -0.5)
+    noq = Z.ZooQuantizer("none")
+    for kw in (dict(), dict(eta=0.5), dict(rho=0.5, tau=0.5), dict(read_post=True), dict(C=32)):
+        if dec == "none" and "eta" in kw:
+            continue
+        o = Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=noq, out_dtype=torch.float64, **kw)
+        assert (o - ref).abs().max() / ref.abs().max() < 1e-9, (cell, kw)
+
+
+@pytest.mark.parametrize("cell", list(CELLS))
+def test_rotation_and_storage_invariances(cell):
+    fam, dec = CELLS[cell]
+    q, k, v, g, beta = make_inputs(cell, seed=6)
+    noq = Z.ZooQuantizer("none")
+    run = lambda **kw: Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=noq,  # noqa: E731
+                                       out_dtype=torch.float64, **kw)
+    base = run()
+    Rq, Rv = Z.signed_hadamard(K, 0), Z.signed_hadamard(V, 1)
+    for kw in (dict(rot_qk=Rq), dict(rot_v=Rv), dict(rot_v=Rv, storage="canonical"), dict(rot_qk=Rq, rot_v=Rv)):
+        assert (run(**kw) - base).abs().max() / base.abs().max() < 1e-9, (cell, list(kw))
+
+
+def test_diagonal_key_scaling_invariance():
+    for cell in ("mamba2", "gla"):
+        fam, dec = CELLS[cell]
+        q, k, v, g, beta = make_inputs(cell, seed=7)
+        noq = Z.ZooQuantizer("none")
+        D = torch.rand(H, K, generator=torch.Generator().manual_seed(2)).double() + 0.5
+        base = Z.chunk_forward(q.double(), k.double(), v.double(), g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=noq)
+        out = Z.chunk_forward(q.double() * D, k.double() / D, v.double(), g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=noq)
+        assert (out - base).abs().max() / base.abs().max() < 1e-9
+
+
+def test_kernel_profile_is_close_to_exact_and_policies_differ():
+    """INT8 emulation stays within a few percent of the unquantized result; per-tensor scales are coarser."""
+    q, k, v, g, beta = make_inputs("gated_deltanet", seed=8)
+    exact = _token_recurrence(q, k, v, g, beta, "delta", "scalar", K ** -0.5)
+    errs = {}
+    for policy in ("kernel_static", "kernel_pt"):
+        qz = Z.ZooQuantizer.kernel_profile(policy)
+        kw = dict(family="delta", decay="scalar", scale=K ** -0.5, qz=qz, eta=1.0, read_post=True, C=C, out_dtype=torch.float64)
+        qz.calibrating = True
+        Z.chunk_forward(q, k, v, g, beta, **kw)
+        qz.finalize()
+        o = Z.chunk_forward(q, k, v, g, beta, **kw)
+        errs[policy] = ((o - exact).abs().max() / exact.abs().max()).item()
+        sc = qz.kernel_scales(0, H, K, V, delta=True)
+        assert sc["q"].shape == (H,) and sc["kw"].shape == (H, K) and sc["state"].shape == (H, V) and sc["ew"].shape == (H, V)
+        assert all(t.dtype == torch.float32 for t in sc.values())
+    assert errs["kernel_static"] < 0.05 and errs["kernel_pt"] < 0.1
