@@ -199,6 +199,119 @@ typedef struct {
 } lq_kron_hadamard_args;
 int lq_kron_hadamard(const lq_kron_hadamard_args* args, hipStream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Zoo chunk kernels: linear attention (no / scalar decay), GLA, DeltaNet / Gated DeltaNet, KDA.
+ * q,k (B,T,H,K) and v (B,T,H,V) fp16 contiguous, T a multiple of the chunk size, K in {64,128},
+ * V a multiple of 64.  g holds the chunk-local cumulative log decay (lq_zoo_cumsum).  Scales are
+ * fp32: q,k,w (H,), kw (H,K), vw,vl,el,ew,state (H,V).  h_i8 is the per-chunk INT8 stored state in
+ * V-major layout (B,NT,H,V,K): an internal buffer shared by the state and output kernels.
+ * qmax is 127 (INT8) or 31 (INT6 codes in INT8 containers); the stored state always uses 127.
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces the torch prep of the zoo wrappers: chunk-local fp32 cumsum of g and the log envelope
+ * (linquant/kernels/zoo/simple_gla.py:191, gla.py:249-251, gated_delta_rule.py:174, kda.py:168-170) */
+typedef struct {
+  const float* g;            /* (B,T,H) or (B,T,H,K) fp32 contiguous */
+  float* gc;                 /* same shape */
+  float* logenv;             /* (B,T,H) max_k(gc_last[k] - gc[t,k]); diagonal decay only, else NULL */
+  int32_t batch, seqlen, nheads, kdim; /* kdim = 0: scalar decay */
+  int32_t chunk_size;
+} lq_zoo_cumsum_args;
+int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
+
+#define LQ_FAMILY_LINEAR 0
+#define LQ_FAMILY_DELTA 1
+#define LQ_DECAY_NONE 0
+#define LQ_DECAY_SCALAR 1
+#define LQ_DECAY_DIAGONAL 2
+
+/* replaces _state_kernel (linquant/kernels/zoo/simple_gla.py:23-95), _gla_state_kernel (gla.py:102-167),
+ * _delta_state_kernel (gated_delta_rule.py:50-136) and _kda_state_kernel (kda.py:68-151): sequential chunk
+ * loop with an fp32 carry, INT8 stored copy per chunk, INT8 write product (and, delta family, the INT8 state
+ * read W.S and the pseudo-values E = (U - W.S) * fw, stored fp16 for the output kernel). */
+typedef struct {
+  const void* k;             /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16 */
+  const void* v;             /* value operand: v (linear) or U (delta), (B,T,H,V) fp16 */
+  const void* w;             /* delta: W (B,T,H,K) fp16; linear: NULL */
+  const float* fw;           /* delta: (B,T,H) fp32 value-side share of the outer beta factor */
+  const float* g;            /* cumulative log decay (B,T,H) / (B,T,H,K), or NULL for no decay */
+  const float* logenv;       /* diagonal decay: (B,T,H) */
+  int8_t* h_i8;              /* (B,NT,H,V,K) int8 */
+  void* e_out;               /* delta: (B,T,H,V) fp16 */
+  float* ht;                 /* (B,H,K,V) fp32 final carry, or NULL */
+  const float* skw;          /* (H,K) key write scale */
+  const float* svw;          /* (H,V) value write scale: vw (linear) or ew (delta) */
+  const float* sw;           /* (H,) W scale (delta) */
+  const float* ss;           /* (H,V) state scale */
+  const void* unrot;         /* (V,V) fp16 R_V^T for canonical storage, or NULL */
+  float eta;
+  int32_t qmax;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
+  int32_t family, decay;
+} lq_zoo_state_args;
+int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
+
+/* replaces _output_kernel (linquant/kernels/zoo/simple_gla.py:98-172) and _gla_output_kernel
+ * (gla.py:170-232): o = dequant(q8(q).h_i8) [* exp(g)] + (fp16(A) . fp16(q8(v))) * svl, with A computed
+ * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay). */
+typedef struct {
+  const void* q;             /* (B,T,H,K) fp16 */
+  const void* k;             /* no / scalar decay: k or Hw (B,T,H,K) fp16; diagonal: NULL */
+  const void* v;             /* local value operand: v or e_out (B,T,H,V) fp16 */
+  const int8_t* h_i8;        /* (B,NT,H,V,K) */
+  const float* g;            /* cumulative log decay or NULL */
+  const float* A;            /* diagonal decay: (B,T,H,C) fp32 lower-triangular intra-chunk product */
+  void* o;                   /* (B,T,H,V) fp16, or fp32 when o_is_f32 */
+  int32_t o_is_f32;
+  const float* sq;           /* (H,) */
+  const float* sk;           /* (H,) (no / scalar decay) */
+  const float* svl;          /* (H,V) */
+  const float* ss;           /* (H,V) */
+  const void* unrot;         /* (V,V) fp16 or NULL */
+  float scale;
+  int32_t qmax;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
+  int32_t decay;
+} lq_zoo_output_args;
+int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
+
+/* replaces _gla_A_inter + _gla_A_intra (linquant/kernels/zoo/gla.py:27-99): intra-chunk product under
+ * per-channel decay, 16-token sub-blocks: INT8 dots on anchor-rescaled operands off the diagonal, fp32
+ * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows, zeros above
+ * the diagonal. */
+typedef struct {
+  const void* q;             /* (B,T,H,K) fp16 */
+  const void* k;             /* (B,T,H,K) fp16: k (GLA) or Hw (KDA) */
+  const float* g;            /* (B,T,H,K) cumulative log decay */
+  float* A;                  /* (B,T,H,C) fp32 */
+  const void* rot;           /* (K,K) fp16 local R_QK, or NULL */
+  const float* sq;
+  const float* sk;
+  float scale;
+  int32_t qmax;
+  int32_t batch, seqlen, nheads, kdim, chunk_size;
+} lq_zoo_gla_A_args;
+int lq_zoo_gla_A(const lq_zoo_gla_A_args* args, hipStream_t stream);
+
+/* replaces the WY / UT prep of the delta family (linquant/kernels/zoo/gated_delta_rule.py:20-47 and
+ * kda.py:22-53; the reference's default sigma=tau=1 route through fla-core's prep kernels is replaced by
+ * the same native prep): fp32 Gram with decay, unit-lower-triangular inverse, W = T.(L*exp(g)),
+ * U = T.(beta^sigma v), Hw = beta^((1-sigma)tau) k, fw = beta^((1-sigma)(1-tau)). */
+typedef struct {
+  const void* k;             /* (B,T,H,K) fp16 */
+  const void* v;             /* (B,T,H,V) fp16 */
+  const float* beta;         /* (B,T,H) fp32 */
+  const float* g;            /* cumulative log decay (B,T,H) / (B,T,H,K) or NULL */
+  void* Hw;                  /* (B,T,H,K) fp16 */
+  void* W;                   /* (B,T,H,K) fp16 */
+  void* U;                   /* (B,T,H,V) fp16 */
+  float* fw;                 /* (B,T,H) fp32 */
+  float sigma, tau;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
+  int32_t decay;
+} lq_zoo_wy_prep_args;
+int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 1; }
+extern "C" int lq_abi_version(void) { return 2; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)
@@ -19,5 +19,10 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_chunk_scan_args);
   LQ_SIZE_OF(lq_split_rotate_quant_xBC_args);
   LQ_SIZE_OF(lq_kron_hadamard_args);
+  LQ_SIZE_OF(lq_zoo_cumsum_args);
+  LQ_SIZE_OF(lq_zoo_state_args);
+  LQ_SIZE_OF(lq_zoo_output_args);
+  LQ_SIZE_OF(lq_zoo_gla_A_args);
+  LQ_SIZE_OF(lq_zoo_wy_prep_args);
   return LQ_ERR_SHAPE;
 }

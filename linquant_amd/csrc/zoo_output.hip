@@ -1,0 +1,263 @@
+// Zoo output kernels: o = state read + intra-chunk local product, fully parallel over chunks.
+// Replaces _output_body (linquant/kernels/zoo/simple_gla.py:98-153) and _gla_output_body (gla.py:170-213).
+//
+//   no / scalar decay:  qq = q8(q*scale, 1/sq), kq = q8(k, 1/sk)
+//                       of = float(qq . h_i8) * sq * ss[v] [* exp(g_i)]
+//                       Af = float(qq . kq^T) * (sq*sk) [* exp(g_i - g_j)], zero above the diagonal
+//   diagonal decay:     qq = q8(q*exp(g)*scale, 1/sq);  of = float(qq . h_i8) * sq * ss[v];  Af = A (fp32 input)
+//   both:               o  = of + (fp16(Af) . fp16(q8(v, 1/svl))) * svl[v]
+//
+// One 4-wave workgroup per (64-column V tile, chunk, batch*head); wave w owns rows 16w..16w+15 of the chunk.
+// q / k codes are produced once per workgroup into LDS (K-contiguous rows: plain 16-byte INT8 MFMA operands);
+// the stored state is V-major in HBM, so its operand is a plain 16-byte global load.  The local value
+// operand goes to LDS as token-pair interleaved fp16 (dword = two consecutive tokens of one channel), the
+// same layout trick as the Mamba-2 chunk scan: four 16-byte reads give the operands of the four MFMA calls
+// that cover channels {4*(lane&15)+j}, and every lane ends up with 4 adjacent output channels.
+#include "zoo_common.h"
+#include "../../include/linquant_hip.h"
+
+namespace {
+
+constexpr int BV = 64;
+constexpr int kAS = 72;  // halves per row of the fp16 A tile in LDS
+constexpr int kVW = 68;  // dwords per token-pair row of the value tile
+
+struct OutParams {
+  const _Float16* q;
+  const _Float16* k;
+  const _Float16* v;
+  const int8_t* h_i8;
+  const float* g;
+  const float* A;
+  void* o;
+  int o_is_f32;
+  const float* sq;
+  const float* sk;
+  const float* svl;
+  const float* ss;
+  float scale;
+  int qmax;
+  int B, T, H, V, NT;
+};
+
+template <bool GLA, bool USE_G, int K>
+__global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
+  constexpr int QS = K + 16;  // byte stride of a code row
+  __shared__ __align__(16) unsigned char qc[64 * QS];
+  __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
+  __shared__ __align__(16) _Float16 Afl[GLA ? 8 : 64 * kAS];
+  __shared__ __align__(16) uint32_t vP[32 * kVW];
+  __shared__ float g_s[64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
+  const int v0 = blockIdx.x * BV;
+  const int ct = blockIdx.y;
+  const int b = blockIdx.z / p.H, h = blockIdx.z % p.H;
+  const int H = p.H, V = p.V;
+  const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
+  const float sq = p.sq[h];
+  const float inv_sq = 1.0f / sq;
+  const float sk = GLA ? 1.0f : p.sk[h];
+  const float inv_sk = 1.0f / sk;
+  const int qmax = p.qmax;
+
+  // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
+  for (int it = tid; it < 64 * (K / 8); it += 256) {
+    const int t = it / (K / 8), c8 = it % (K / 8);
+    const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
+    const lq_v8h qv = *(const lq_v8h*)(p.q + off);
+    int cq[8];
+    if (GLA) {
+      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float x = (float)qv[e] * lq_expf(e < 4 ? g0[e & 3] : g1[e & 3]);
+        x = x * p.scale;
+        cq[e] = zoo_q8(x, inv_sq, qmax);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8((float)qv[e] * p.scale, inv_sq, qmax);
+    }
+    lq_v2i o;
+    o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
+    o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
+    *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
+    if (!GLA) {
+      const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+      int ck[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8((float)kv[e], inv_sk, qmax);
+      o[0] = (int)zoo_pack_codes(ck[0], ck[1], ck[2], ck[3]);
+      o[1] = (int)zoo_pack_codes(ck[4], ck[5], ck[6], ck[7]);
+      *(lq_v2i*)(kc + t * QS + 8 * c8) = o;
+    }
+  }
+  {
+    const int tp = tid >> 3, c8 = tid & 7;  // 32 token pairs x 8 groups of 8 channels
+    const int64_t off = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8;
+    const lq_v8h va = *(const lq_v8h*)(p.v + off);
+    const lq_v8h vb = *(const lq_v8h*)(p.v + off + (int64_t)H * V);
+    lq_v4i o0, o1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float inv = 1.0f / p.svl[h * V + v0 + 8 * c8 + e];
+      const float ca = (float)zoo_q8((float)va[e], inv, qmax);
+      const float cb = (float)zoo_q8((float)vb[e], inv, qmax);
+      const int w = (int)zoo_pack_h2(ca, cb);
+      if (e < 4) o0[e] = w; else o1[e - 4] = w;
+    }
+    *(lq_v4i*)(vP + tp * kVW + 8 * c8) = o0;
+    *(lq_v4i*)(vP + tp * kVW + 8 * c8 + 4) = o1;
+  }
+  if (USE_G && !GLA && tid < 64) g_s[tid] = p.g[(t0 + tid) * H + h];
+  __syncthreads();
+
+  // ---- phase 2: INT8 contractions of this wave's 16 rows
+  lq_v4i o32[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) o32[jj] = lq_v4i{0, 0, 0, 0};
+  lq_v4i a32[4];
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
+  const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
+#pragma unroll
+  for (int ks = 0; ks < K / 64; ++ks) {
+    const lq_v4i qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const lq_v4i hop = *(const lq_v4i*)(hp + (4 * rl + jj) * K + 64 * ks + 16 * kg);
+      o32[jj] = lq_mfma_i8(qop, hop, o32[jj]);
+    }
+    if (!GLA) {
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt) {
+        if (jt > wave) continue;  // strictly above the diagonal (wave-uniform)
+        const lq_v4i kop = *(const lq_v4i*)(kc + (16 * jt + rl) * QS + 64 * ks + 16 * kg);
+        a32[jt] = lq_mfma_i8(qop, kop, a32[jt]);
+      }
+    }
+  }
+
+  // ---- phase 3: dequantize; A -> fp16 in operand layout
+  float of[4][4];  // [jj][r]: rows 16w + 4kg + r, channels v0 + 4rl + jj
+  {
+    float ssv[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) ssv[jj] = p.ss[h * V + v0 + 4 * rl + jj];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float eg = (USE_G && !GLA) ? __expf(g_s[16 * wave + 4 * kg + r]) : 1.0f;
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        float x = (float)o32[jj][r] * sq;
+        x = x * ssv[jj];
+        of[jj][r] = (USE_G && !GLA) ? x * eg : x;
+      }
+    }
+  }
+  if (!GLA) {
+    const float sqk = sq * sk;
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) {
+      if (jt > wave + 1) continue;
+      const int j = 16 * jt + rl;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * wave + 4 * kg + r;
+        float x = 0.0f;
+        if (jt <= wave && j <= i) {
+          x = (float)a32[jt][r] * sqk;
+          if (USE_G) x = x * __expf(g_s[i] - g_s[j]);
+        }
+        Afl[i * kAS + j] = (_Float16)x;
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- phase 4: local product on the fp16 MFMA and store
+  lq_v4f loc[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) loc[jj] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+  const int nslab = (16 * wave + 15) / 32 + 1;
+  for (int js = 0; js < nslab; ++js) {
+    lq_v8h aop;
+    if (GLA) {
+      const float* ap = p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg;
+      const lq_v4f x0 = *(const lq_v4f*)ap, x1 = *(const lq_v4f*)(ap + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        aop[e] = (_Float16)x0[e];
+        aop[4 + e] = (_Float16)x1[e];
+      }
+    } else {
+      aop = *(const lq_v8h*)(Afl + (16 * wave + rl) * kAS + 32 * js + 8 * kg);
+    }
+    lq_v4i xop[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const lq_v4i vv = *(const lq_v4i*)(vP + (16 * js + 4 * kg + d) * kVW + 4 * rl);
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) xop[jj][d] = vv[jj];
+    }
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) loc[jj] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[jj]), loc[jj]);
+  }
+  float svl[4];
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) svl[jj] = p.svl[h * V + v0 + 4 * rl + jj];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + 4 * rl;
+    float res[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) res[jj] = of[jj][r] + loc[jj][r] * svl[jj];
+    if (p.o_is_f32) {
+      *(lq_v4f*)((float*)p.o + off) = lq_v4f{res[0], res[1], res[2], res[3]};
+    } else {
+      lq_v2i w;
+      w[0] = (int)zoo_pack_h2(res[0], res[1]);
+      w[1] = (int)zoo_pack_h2(res[2], res[3]);
+      *(lq_v2i*)((_Float16*)p.o + off) = w;
+    }
+  }
+}
+
+template <bool GLA, bool USE_G>
+int launch(const OutParams& p, int K, dim3 grid, hipStream_t stream) {
+  if (K == 128)
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, 128>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, 64>), grid, dim3(256), 0, stream, p);
+  return lq_check_launch();
+}
+
+}  // namespace
+
+extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
+  if (!a || !a->q || !a->v || !a->h_i8 || !a->o || !a->sq || !a->svl || !a->ss) return LQ_ERR_NULL;
+  const bool gla = a->decay == LQ_DECAY_DIAGONAL;
+  if (gla && (!a->A || !a->g)) return LQ_ERR_NULL;
+  if (!gla && (!a->k || !a->sk)) return LQ_ERR_NULL;
+  if (a->decay == LQ_DECAY_SCALAR && !a->g) return LQ_ERR_NULL;
+  if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
+  if (a->unrot) return LQ_ERR_SHAPE;  // canonical storage (in-kernel un-rotation) is not built yet
+  if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
+  if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
+  if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
+  if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
+  if (!zoo_al(a->q, 16) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16))
+    return LQ_ERR_SHAPE;
+  if ((int64_t)a->batch * a->nheads > 65535 || a->seqlen / 64 > 65535) return LQ_ERR_SHAPE;
+  OutParams p = {};
+  p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.v = (const _Float16*)a->v;
+  p.h_i8 = a->h_i8, p.g = a->g, p.A = a->A, p.o = a->o, p.o_is_f32 = a->o_is_f32;
+  p.sq = a->sq, p.sk = a->sk, p.svl = a->svl, p.ss = a->ss, p.scale = a->scale, p.qmax = a->qmax;
+  p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
+  dim3 grid(a->vdim / BV, p.NT, a->batch * a->nheads);
+  if (gla) return launch<true, true>(p, a->kdim, grid, stream);
+  if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, grid, stream);
+  return launch<false, false>(p, a->kdim, grid, stream);
+}
