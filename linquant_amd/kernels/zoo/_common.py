@@ -1,0 +1,95 @@
+"""Shared launch helpers of the zoo wrappers (thin ctypes calls into liblinquant_hip.so)."""
+
+from __future__ import annotations
+
+import torch
+
+from linquant_amd import _lib
+
+FAMILY_LINEAR, FAMILY_DELTA = 0, 1
+DECAY_NONE, DECAY_SCALAR, DECAY_DIAGONAL = 0, 1, 2
+CHUNK = 64
+
+
+def check_shapes(q, k, v, chunk_size):
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    assert T % chunk_size == 0, f"T={T} must be a multiple of the chunk size {chunk_size}"
+    assert K <= 128, f"K={K}: the state kernels hold the whole key axis (K <= 128)"
+    assert chunk_size == CHUNK, f"chunk_size={chunk_size}: the HIP kernels are built for 64-token chunks"
+    assert K in (64, 128), f"K={K}: built for key dims 64 and 128"
+    assert V % 64 == 0, f"V={V}: value dim must be a multiple of 64"
+    assert q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16, "fp16 activations"
+    assert k.shape == q.shape and v.shape[:3] == q.shape[:3]
+    return B, T, H, K, V
+
+
+def f32(t):
+    return t if (t.dtype == torch.float32 and t.is_contiguous()) else t.float().contiguous()
+
+
+def no_rotation(**named):
+    for name, val in named.items():
+        if val is not None:
+            raise NotImplementedError(
+                f"{name}: in-kernel rotation / canonical storage is not built in the HIP zoo kernels yet; "
+                "rotate the operands outside and use rotated storage (out_dtype=torch.float32 + exit un-rotation)")
+
+
+def cumsum(g, B, T, H, kdim):
+    """Chunk-local cumulative log decay (fp32) and, for per-channel decay, the log envelope."""
+    g = f32(g)
+    gc = torch.empty_like(g)
+    logenv = torch.empty(B, T, H, dtype=torch.float32, device=g.device) if kdim else None
+    _lib.call("lq_zoo_cumsum", g.device, g=_lib.ptr(g), gc=_lib.ptr(gc), logenv=_lib.ptr(logenv), batch=B, seqlen=T,
+              nheads=H, kdim=kdim, chunk_size=CHUNK)
+    return gc, logenv
+
+
+def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
+              sw=None):
+    B, T, H, K, V = dims
+    _lib.call("lq_zoo_state", key.device, k=_lib.ptr(key), v=_lib.ptr(value), w=_lib.ptr(w), fw=_lib.ptr(fw), g=_lib.ptr(g),
+              logenv=_lib.ptr(logenv), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
+              svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=None, eta=float(eta), qmax=int(qmax), batch=B,
+              seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, family=family, decay=decay)
+
+
+def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay):
+    B, T, H, K, V = dims
+    _lib.call("lq_zoo_output", q.device, q=_lib.ptr(q), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
+              g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
+              sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=None, scale=float(scale), qmax=int(qmax),
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay)
+
+
+def run_gla_A(q, key, gc, A, sq, sk, scale, qmax, dims):
+    B, T, H, K, _ = dims
+    _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), rot=None,
+              sq=_lib.ptr(sq), sk=_lib.ptr(sk), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K,
+              chunk_size=CHUNK)
+
+
+def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay):
+    """Returns (Hw, W, U, fw): fp16 operands of the delta state kernel and the value-side share of beta."""
+    B, T, H, K, V = dims
+    Hw, W = torch.empty_like(k), torch.empty_like(k)
+    U = torch.empty_like(v)
+    fw = torch.empty(B, T, H, dtype=torch.float32, device=k.device)
+    _lib.call("lq_zoo_wy_prep", k.device, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
+              Hw=_lib.ptr(Hw), W=_lib.ptr(W), U=_lib.ptr(U), fw=_lib.ptr(fw), sigma=float(sigma), tau=float(tau),
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay)
+    return Hw, W, U, fw
+
+
+def out_buffer(v, out_dtype):
+    dt = out_dtype or v.dtype
+    assert dt in (torch.float16, torch.float32), f"output dtype {dt}: fp16 or fp32"
+    return torch.empty(v.shape, dtype=dt, device=v.device)
+
+
+def export_debug(debug, h_i8, **extra):
+    """Optional hook for tests: the stored INT8 state in the reference's (B,NT,H,K,V) orientation."""
+    if debug is not None:
+        debug["h_i8"] = h_i8.transpose(-1, -2)
+        debug.update(extra)

@@ -1,0 +1,42 @@
+"""INT8 chunk_gated_delta_rule / chunk_delta_rule (delta family, no or scalar decay) on HIP.
+
+Call surface of linquant/kernels/zoo/gated_delta_rule.py:159-203: WY prep (Gram, triangular inverse,
+W = T.(beta^sigma k * exp(g)), U = T.(beta^sigma v)) -> state kernel with E = (U - W.S) * fw formed inside the
+chunk loop -> the simple_gla output kernel on (q, Hw, E).  The prep is always the native fp32 HIP kernel
+(``fla_prep`` is accepted for compatibility and ignored)."""
+
+from __future__ import annotations
+
+import torch
+
+from . import _common as C
+
+
+def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, scale=None, chunk_size=64,
+                     output_final_state=False, unrot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
+    """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None (DeltaNet), beta [B,T,H].
+    scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
+    q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
+    dims = C.check_shapes(q, k, v, chunk_size)
+    B, T, H, K, V = dims
+    assert beta.shape == (B, T, H)
+    C.no_rotation(unrot=unrot)
+    scale = K ** -0.5 if scale is None else scale
+    qmax = 2 ** (bits - 1) - 1
+    decay = C.DECAY_NONE if g is None else C.DECAY_SCALAR
+    gg = None
+    if g is not None:
+        assert g.shape == (B, T, H)
+        gg, _ = C.cumsum(g, B, T, H, 0)
+    Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay)
+    sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
+    NT = T // chunk_size
+    h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
+    e_out = torch.empty_like(v)
+    ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+    o = C.out_buffer(v, out_dtype)
+    C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
+                w=W, fw=fw, e_out=e_out, sw=sc["w"])
+    C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay)
+    C.export_debug(_debug, h_i8, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
+    return o, ht

@@ -1,0 +1,39 @@
+"""INT8 chunk_gla (linear attention with diagonal, per-channel decay) on HIP.
+
+Call surface of linquant/kernels/zoo/gla.py:235-279: intra-chunk product A over 16-token sub-blocks (INT8 dots
+on anchor-rescaled operands off the diagonal, fp32 reduction on the diagonal blocks), state kernel with
+per-channel write gates under the scalar eta envelope, output o = q8(q*exp(g)*scale).h + A.q8(v)."""
+
+from __future__ import annotations
+
+import torch
+
+from . import _common as C
+
+BC = 16  # secondary chunk
+
+
+def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, output_final_state=False, unrot=None,
+                   rot=None, bits=8, out_dtype=None, _debug=None):
+    """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
+    Returns (o, final fp32 state or None)."""
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    dims = C.check_shapes(q, k, v, chunk_size)
+    B, T, H, K, V = dims
+    assert chunk_size % BC == 0 and g.shape == (B, T, H, K)
+    C.no_rotation(unrot=unrot, rot=rot)
+    scale = K ** -0.5 if scale is None else scale
+    qmax = 2 ** (bits - 1) - 1
+    gc, logenv = C.cumsum(g, B, T, H, K)
+    sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
+    A = torch.empty(B, T, H, chunk_size, dtype=torch.float32, device=q.device)
+    C.run_gla_A(q, k, gc, A, sc["q"], sc["k"], scale, qmax, dims)
+    NT = T // chunk_size
+    h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
+    ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+    o = C.out_buffer(v, out_dtype)
+    C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
+                C.DECAY_DIAGONAL)
+    C.run_output(q, None, v, h_i8, gc, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL)
+    C.export_debug(_debug, h_i8, A=A, g=gc, logenv=logenv)
+    return o, ht

@@ -1,0 +1,40 @@
+"""INT8 chunk_kda (delta rule with diagonal, per-channel decay) on HIP.
+
+Call surface of linquant/kernels/zoo/kda.py:154-203: fp32 WY prep with per-channel gates, the GLA A kernel on
+(q, Hw), a state kernel with E = (U - W.S) * fw formed in-loop and per-channel write gates under the scalar
+eta envelope, and the GLA output kernel on (q, E, A).  ``fla_prep`` is accepted and ignored."""
+
+from __future__ import annotations
+
+import torch
+
+from . import _common as C
+from .gla import BC
+
+
+def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, scale=None, chunk_size=64,
+                   output_final_state=False, unrot=None, rot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
+    """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay, beta [B,T,H].
+    scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
+    q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
+    dims = C.check_shapes(q, k, v, chunk_size)
+    B, T, H, K, V = dims
+    assert chunk_size % BC == 0 and g.shape == (B, T, H, K) and beta.shape == (B, T, H)
+    C.no_rotation(unrot=unrot, rot=rot)
+    scale = K ** -0.5 if scale is None else scale
+    qmax = 2 ** (bits - 1) - 1
+    gc, logenv = C.cumsum(g, B, T, H, K)
+    Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL)
+    sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
+    A = torch.empty(B, T, H, chunk_size, dtype=torch.float32, device=q.device)
+    C.run_gla_A(q, Hw, gc, A, sc["q"], sc["k"], scale, qmax, dims)
+    NT = T // chunk_size
+    h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
+    e_out = torch.empty_like(v)
+    ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
+    o = C.out_buffer(v, out_dtype)
+    C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
+                C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"])
+    C.run_output(q, None, e_out, h_i8, gc, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL)
+    C.export_debug(_debug, h_i8, A=A, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
+    return o, ht
