@@ -41,9 +41,199 @@ def stage_bytes(s, keyside):
     }
 
 
+ZOO_WORKLOADS = {
+    # name: (cell, B, T, H, K, V, description) -- shapes of BASELINE.json configs[0..3]
+    "c1": ("mamba2", 1, 2048, 8, 64, 64, "configs[0]: Mamba-2 cell (linear family, scalar decay) B=1 T=2048 H=8 K=V=64 chunk 64"),
+    "c2_la": ("linear_none", 4, 4096, 16, 128, 128, "configs[1]: linear attention B=4 T=4096 H=16 K=V=128 chunk 64, q,k pre-rotated"),
+    "c2_gla": ("gla", 4, 4096, 16, 128, 128, "configs[1]: GLA B=4 T=4096 H=16 K=V=128 chunk 64, local R_QK in the A kernel"),
+    "c3_deltanet": ("deltanet", 4, 4096, 16, 128, 128, "configs[2]: DeltaNet B=4 T=4096 H=16 K=V=128 chunk 64, sigma=0.5"),
+    "c3_gdn": ("gated_deltanet", 4, 4096, 16, 128, 128, "configs[2]: Gated DeltaNet B=4 T=4096 H=16 K=V=128 chunk 64, sigma=0.5"),
+    "c4_kda": ("kda", 2, 8192, 32, 128, 128, "configs[3]: KDA B=2 T=8192 H=32 K=V=128 chunk 64, local R_QK in the A kernel"),
+}
+ZOO_CELLS = {"linear_none": ("linear", "none"), "mamba2": ("linear", "scalar"), "gla": ("linear", "diagonal"),
+             "deltanet": ("delta", "none"), "gated_deltanet": ("delta", "scalar"), "kda": ("delta", "diagonal")}
+
+
+def zoo_stage_bytes(fam, dec, B, T, H, K, V):
+    """Algorithmic HBM bytes per zoo stage: every tensor the stage must read or write, counted once."""
+    qk, vv, tok = B * T * H * K * 2, B * T * H * V * 2, B * T * H * 4
+    g = 0 if dec == "none" else (tok if dec == "scalar" else B * T * H * K * 4)
+    h8 = B * (T // 64) * H * K * V
+    A = B * T * H * 64 * 4
+    out = {}
+    if dec != "none":
+        out["cumsum"] = 2 * g + (tok if dec == "diagonal" else 0)
+    if fam == "delta":
+        out["wy_prep"] = qk + vv + tok + g + 2 * qk + vv + tok
+    if dec == "diagonal":
+        out["gla_A"] = 2 * qk + g + A
+    out["state"] = qk + vv + g + h8 + (qk + tok + vv if fam == "delta" else 0) + (tok if dec == "diagonal" else 0)
+    out["output"] = qk + (qk if dec != "diagonal" else A) + vv + h8 + g + vv
+    return out
+
+
+def hadamard_signed(n, seed, device):
+    import torch
+
+    Hm = torch.ones(1, 1, dtype=torch.float64)
+    while Hm.shape[0] < n:
+        Hm = torch.cat([torch.cat([Hm, Hm], 1), torch.cat([Hm, -Hm], 1)], 0)
+    signs = torch.randint(0, 2, (n,), generator=torch.Generator().manual_seed(seed)).double() * 2 - 1
+    return (Hm / n ** 0.5 * signs).to(device)
+
+
+def bench_zoo(args):
+    """One step = one chunk-forward call (cumsum, WY prep, A, state, output kernels) over inputs resident in HBM."""
+    import torch
+
+    from linquant_amd import _lib
+    from linquant_amd.kernels import zoo
+    from linquant_amd.kernels.zoo import _common as C
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    cell, B, T, H, K, V, desc = ZOO_WORKLOADS[args.workload]
+    fam, dec = ZOO_CELLS[cell]
+    gen = torch.Generator().manual_seed(0)
+    rn = lambda *shape: torch.randn(*shape, generator=gen)  # noqa: E731
+    q = rn(B, T, H, K)
+    k = rn(B, T, H, K)
+    if fam == "delta":
+        k = torch.nn.functional.normalize(k, dim=-1)
+    v = rn(B, T, H, V)
+    beta = torch.sigmoid(rn(B, T, H)).to(dev) if fam == "delta" else None
+    g = None
+    if cell == "gla":
+        g = torch.nn.functional.logsigmoid(rn(B, T, H, K)) / 16
+    elif cell == "kda":
+        g = torch.nn.functional.logsigmoid(rn(B, T, H, K) + 1.0)
+    elif cell == "gated_deltanet":
+        g = torch.nn.functional.logsigmoid(rn(B, T, H) + 2.0)
+    elif cell == "mamba2":
+        g = -torch.nn.functional.softplus(rn(B, T, H) * 0.5 - 2.0) * torch.exp(torch.rand(H, generator=gen) * 2.77)
+    R = hadamard_signed(K, 1, dev)
+    rot = R if dec == "diagonal" else None
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    if dec != "diagonal" and args.workload != "c1":  # persistent R_QK: folded into the projections in deployment
+        q, k = (q.double() @ R).float(), (k.double() @ R).float()
+    q, k, v = q.half(), k.half(), v.half()
+    g = g.float().to(dev) if g is not None else None
+    scale = 1.0 if args.workload == "c1" else K ** -0.5
+    sigma = 0.5 if args.workload.startswith("c3") else 1.0
+    eta = 0.0 if dec == "diagonal" else 1.0
+
+    def call(sc, **kw):
+        if fam == "linear" and dec == "diagonal":
+            return zoo.chunk_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, rot=rot, **kw)
+        if fam == "linear":
+            return zoo.chunk_simple_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, **kw)
+        if dec == "diagonal":
+            return zoo.chunk_kda_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, rot=rot, **kw)
+        return zoo.chunk_delta_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, **kw)
+
+    # static scales: operand roles from the inputs' absmax (decay factors are <= 1), state / pseudo-value roles from a
+    # pilot run of the kernels themselves with a coarse state grid
+    ph = lambda t: (t.float().abs().amax(dim=(0, 1, 3)) / 127).clamp_min(1e-6)  # noqa: E731
+    pc = lambda t: (t.float().abs().amax(dim=(0, 1)) / 127).clamp_min(1e-6)  # noqa: E731
+    sc = {"q": ph(q) * scale, "k": ph(k), "w": ph(k) * 2, "kw": pc(k), "vw": pc(v), "vl": pc(v),
+          "el": pc(v) * 2, "ew": pc(v) * 2, "state": torch.full((H, V), 1.0, device=dev)}
+    sc = {n: t.contiguous() for n, t in sc.items()}
+    dbg = {}
+    _, ht = call(sc, output_final_state=True, _debug=dbg)
+    sc["state"] = (ht.abs().amax(dim=(0, 2)) / 127 * 1.5).clamp_min(1e-6).contiguous()
+    if fam == "delta":
+        sc["el"] = sc["ew"] = (dbg["e_out"].float().abs().amax(dim=(0, 1)) / 127).clamp_min(1e-6).contiguous()
+        sc["w"] = ph(dbg["W"]).contiguous()
+    del dbg, ht
+    torch.cuda.synchronize()
+
+    for _ in range(args.warmup):
+        call(sc)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        call(sc)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    tokens = B * T
+
+    records = {}
+    names = {"cumsum": "cumsum", "run_wy_prep": "wy_prep", "run_gla_A": "gla_A", "run_state": "state", "run_output": "output"}
+    saved = {n: getattr(C, n) for n in names}
+
+    def timed(fn, label):
+        def wrapper(*a, **kw):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **kw)
+            e1.record()
+            records.setdefault(label, []).append((e0, e1))
+            return r
+        return wrapper
+
+    try:
+        for n, label in names.items():
+            setattr(C, n, timed(saved[n], label))
+        for _ in range(max(10, args.steps)):
+            call(sc)
+        torch.cuda.synchronize()
+    finally:
+        for n, f in saved.items():
+            setattr(C, n, f)
+    nbytes = zoo_stage_bytes(fam, dec, B, T, H, K, V)
+    stages = {}
+    for label, evs in records.items():
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        med = statistics.median(ts)
+        stages[label] = {"ms": round(med, 4), "p25": round(ts[len(ts) // 4], 4), "p75": round(ts[(3 * len(ts)) // 4], 4),
+                         "MB": round(nbytes[label] / 1e6, 1), "GBps": round(nbytes[label] / 1e6 / med, 1),
+                         "hbm_frac": round(nbytes[label] / 1e6 / med / HBM_PEAK_GBS, 4)}
+    dom = max(stages, key=lambda n: stages[n]["ms"])
+    avg_dom = statistics.mean(a.elapsed_time(b) for a, b in records[dom])
+    achieved = nbytes[dom] / 1e6 / avg_dom
+    roofline = {"kernel": "zoo_" + dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "avg_ms": round(avg_dom, 4),
+                "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import zoo_reference as Z
+
+        threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+        torch.set_num_threads(threads)
+        hs, ts_ = min(2, H), min(T, 2048)
+        cut = lambda t: None if t is None else t[:1, :ts_, :hs].cpu()  # noqa: E731
+        qz = Z.ZooQuantizer.kernel_profile("kernel_static", 8)
+        run = lambda: Z.chunk_forward(cut(q), cut(k), cut(v), cut(g), cut(beta), family=fam, decay=dec, scale=scale, qz=qz,  # noqa: E731
+                                      eta=eta, rho=sigma, tau=1.0, read_post=True, C=64,
+                                      rot_qk=None if rot is None else rot.cpu())
+        qz.calibrating = True
+        run()
+        qz.finalize()
+        t0 = time.perf_counter()
+        run()
+        t_cpu = time.perf_counter() - t0
+        frac = (hs * ts_) / (B * H * T)
+        cpu = {"value": round(tokens * frac / t_cpu, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+               "sample": f"float64 torch oracle on batch 1 x {hs} of {H} heads x {ts_} tokens ({frac:.5f} of the job) in "
+                         f"{t_cpu:.2f} s; value = job-equivalent tokens/s", "host_cpus": os.cpu_count(),
+               "torch_threads": torch.get_num_threads()}
+    line = {
+        "metric": f"prefill tokens/s per layer at T={T}", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": f"{args.workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
+                   "tokens_per_step": tokens},
+        "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
+    }
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--workload", default="c5", choices=["c5"] + list(ZOO_WORKLOADS),
+                    help="c5 (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on; others: zoo kernels")
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--value-side", action="store_true", help="value-side absorption instead of key-side")
@@ -54,6 +244,15 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards over batch x head "
               "with no communication); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload != "c5":
+        from linquant_amd import _lib as _l
+
+        if not _l.LIB_PATH.exists():
+            from linquant_amd.build import build
+
+            build()
+        return bench_zoo(args)
 
     import torch
 

@@ -11,6 +11,8 @@
 // operands are K-contiguous, so each lane builds its own 16-slot INT8 MFMA operand from plain global loads
 // (no LDS).  The diagonal block stages INT8 codes and the decay rows of its 16 tokens in LDS and lets lane
 // (i = lane & 15, j-group = lane >> 4) accumulate four (i, j) pairs.
+// With a local R_QK (rot, (K,K) fp16, x -> x.R) the anchored off-diagonal operands are rounded to fp16 and rotated
+// on the fp16 MFMA before quantization (gla.py:53-57); the diagonal blocks are not rotated.
 #include "zoo_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -23,16 +25,45 @@ struct AParams {
   float* A;
   const float* sq;
   const float* sk;
+  const _Float16* rot;
   float scale;
   int qmax;
   int B, T, H;
 };
 
+// diagonal block of wave's sub-block: lane (i = rl, j = 4kg + jj) reduces over the staged codes in fp32
 template <int K>
+LQ_DEV void diag_block(const AParams& p, const float (*g_s)[K + 1], const int8_t (*qd_s)[K + 4], const int8_t (*kd_s)[K + 4],
+                       float sq, float sk, int rl, int kg, int64_t row0, int h, int i0) {
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < K; ++n) {
+    const float qi = (float)qd_s[rl][n] * sq;
+    const float gi = g_s[rl][n];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int j = 4 * kg + jj;
+      const float kj = (float)kd_s[j][n] * sk;
+      const float w = (j <= rl) ? lq_expf(gi - g_s[j][n]) : 0.0f;
+      s[jj] = s[jj] + (qi * kj) * w;
+    }
+  }
+  lq_v4f o;
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) o[jj] = (4 * kg + jj <= rl) ? s[jj] : 0.0f;
+  *(lq_v4f*)(p.A + ((row0 + rl) * p.H + h) * 64 + i0 + 4 * kg) = o;
+}
+
+template <int K, bool ROT>
 __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
-  __shared__ float g_s[4][16][K + 1];
-  __shared__ int8_t qd_s[4][16][K + 4];
-  __shared__ int8_t kd_s[4][16][K + 4];
+  constexpr int GS = 4 * 16 * (K + 1) * 4;  // bytes of the decay rows
+  constexpr int QS = 4 * 16 * (K + 4);      // bytes of one code tile
+  constexpr int RS = K + 8;                 // halves per row of the transposed rotation
+  static_assert(K * RS * 2 <= GS + 2 * QS, "the rotation tile reuses the diagonal-block staging space");
+  __shared__ __align__(16) unsigned char smem[GS + 2 * QS];
+  float (*g_s)[16][K + 1] = reinterpret_cast<float (*)[16][K + 1]>(smem);
+  int8_t (*qd_s)[16][K + 4] = reinterpret_cast<int8_t (*)[16][K + 4]>(smem + GS);
+  int8_t (*kd_s)[16][K + 4] = reinterpret_cast<int8_t (*)[16][K + 4]>(smem + GS + QS);
+  _Float16* RT = reinterpret_cast<_Float16*>(smem);  // ROT: RT[m][n] = R[n][m], after the diagonal blocks are done
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -60,67 +91,161 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
     }
   }
 
-  // ---- off-diagonal blocks J < wave (INT8 MFMA on anchored operands)
   lq_v4i acc[3];
 #pragma unroll
   for (int J = 0; J < 3; ++J) acc[J] = lq_v4i{0, 0, 0, 0};
-  if (wave > 0) {
+
+  if constexpr (!ROT) {
+    // ---- off-diagonal blocks J < wave: INT8 MFMA on anchored operands built from plain global loads
+    if (wave > 0) {
 #pragma unroll
-    for (int ks = 0; ks < K / 64; ++ks) {
-      const int kk = 64 * ks + 16 * kg;
-      float an[16];
-      {
+      for (int ks = 0; ks < K / 64; ++ks) {
+        const int kk = 64 * ks + 16 * kg;
+        float an[16];
+        {
+          const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const lq_v4f a4 = *(const lq_v4f*)(ap + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) an[4 * e4 + e] = a4[e];
+          }
+        }
+        lq_v4i qop;
+        {
+          const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
+          const lq_v8h q0 = *(const lq_v8h*)(p.q + off), q1 = *(const lq_v8h*)(p.q + off + 8);
+          int cd[16];
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int n = 4 * e4 + e;
+              const float qf = n < 8 ? (float)q0[n & 7] : (float)q1[n & 7];
+              float x = qf * lq_expf(g4[e] - an[n]);
+              x = x * p.scale;
+              cd[n] = zoo_q8(x, inv_sq, qmax);
+            }
+          }
+#pragma unroll
+          for (int d = 0; d < 4; ++d) qop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
+        }
+#pragma unroll
+        for (int J = 0; J < 3; ++J) {
+          if (J >= wave) continue;
+          const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
+          const lq_v8h k0 = *(const lq_v8h*)(p.k + off), k1 = *(const lq_v8h*)(p.k + off + 8);
+          int cd[16];
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int n = 4 * e4 + e;
+              const float kf = n < 8 ? (float)k0[n & 7] : (float)k1[n & 7];
+              cd[n] = zoo_q8(kf * lq_expf(an[n] - g4[e]), inv_sk, qmax);
+            }
+          }
+          lq_v4i kop;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) kop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
+          acc[J] = lq_mfma_i8(qop, kop, acc[J]);
+        }
+      }
+    }
+    __syncthreads();  // staged diagonal rows visible (each wave only reads its own block)
+    diag_block<K>(p, g_s[wave], qd_s[wave], kd_s[wave], sq, sk, rl, kg, t0 + i0, h, i0);
+  } else {
+    // ---- local R_QK: the anchored operands are rotated (fp16 MFMA, fp32 accumulate) before quantization.
+    // Transposed product R^T . X^T: lane (rl, kg) receives, for token rl, channels 16mt + 4kg + r, which it packs
+    // as dword mt of its INT8 operand; q and k operands share that channel -> slot map, so the INT8 dot is exact.
+    constexpr int KS = K / 32, MT = K / 16;
+    __syncthreads();
+    diag_block<K>(p, g_s[wave], qd_s[wave], kd_s[wave], sq, sk, rl, kg, t0 + i0, h, i0);
+    __syncthreads();  // every wave is done with the staged rows: reuse the space for R^T
+    for (int it = tid; it < K * (K / 8); it += 256) {
+      const int n = it / (K / 8), m8 = it % (K / 8);
+      const lq_v8h rv = *(const lq_v8h*)(p.rot + (int64_t)n * K + 8 * m8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) RT[(8 * m8 + e) * RS + n] = rv[e];
+    }
+    // anchored fp16 operands: tensor 0 = q rows of this sub-block, tensor 1 + J = k rows of sub-block J < wave
+    lq_v8h xop[4][KS];
+    if (wave > 0) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int kk = 32 * ks + 8 * kg;
         const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
+        const lq_v4f a0 = *(const lq_v4f*)ap, a1 = *(const lq_v4f*)(ap + 4);
+        {
+          const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
+          const lq_v8h qv = *(const lq_v8h*)(p.q + off);
+          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-        for (int e4 = 0; e4 < 4; ++e4) {
-          const lq_v4f a4 = *(const lq_v4f*)(ap + 4 * e4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) an[4 * e4 + e] = a4[e];
-        }
-      }
-      lq_v4i qop;
-      {
-        const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
-        const lq_v8h q0 = *(const lq_v8h*)(p.q + off), q1 = *(const lq_v8h*)(p.q + off + 8);
-        int cd[16];
-#pragma unroll
-        for (int e4 = 0; e4 < 4; ++e4) {
-          const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int n = 4 * e4 + e;
-            const float qf = n < 8 ? (float)q0[n & 7] : (float)q1[n & 7];
-            float x = qf * lq_expf(g4[e] - an[n]);
+          for (int e = 0; e < 8; ++e) {
+            const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
+            float x = (float)qv[e] * lq_expf(gg - an);
             x = x * p.scale;
-            cd[n] = zoo_q8(x, inv_sq, qmax);
+            xop[0][ks][e] = (_Float16)x;
           }
         }
 #pragma unroll
-        for (int d = 0; d < 4; ++d) qop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
+        for (int J = 0; J < 3; ++J) {
+          if (J >= wave) continue;
+          const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
+          const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
+            xop[1 + J][ks][e] = (_Float16)((float)kv[e] * lq_expf(an - gg));
+          }
+        }
+      }
+    }
+    __syncthreads();  // R^T staged
+    if (wave > 0) {
+      uint32_t cd[4][MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        lq_v4f ra[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) ra[t] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const lq_v8h rop = *(const lq_v8h*)(RT + (16 * mt + rl) * RS + 32 * ks + 8 * kg);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            if (t > wave) continue;
+            ra[t] = lq_mfma_f16(rop, xop[t][ks], ra[t]);
+          }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          if (t > wave) continue;
+          const float inv = t == 0 ? inv_sq : inv_sk;
+          cd[t][mt] = zoo_pack_codes(zoo_q8(ra[t][0], inv, qmax), zoo_q8(ra[t][1], inv, qmax), zoo_q8(ra[t][2], inv, qmax),
+                                     zoo_q8(ra[t][3], inv, qmax));
+        }
       }
 #pragma unroll
-      for (int J = 0; J < 3; ++J) {
-        if (J >= wave) continue;
-        const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
-        const lq_v8h k0 = *(const lq_v8h*)(p.k + off), k1 = *(const lq_v8h*)(p.k + off + 8);
-        int cd[16];
+      for (int s = 0; s < K / 64; ++s) {
+        lq_v4i qop;
 #pragma unroll
-        for (int e4 = 0; e4 < 4; ++e4) {
-          const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
+        for (int d = 0; d < 4; ++d) qop[d] = (int)cd[0][4 * s + d];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int n = 4 * e4 + e;
-            const float kf = n < 8 ? (float)k0[n & 7] : (float)k1[n & 7];
-            cd[n] = zoo_q8(kf * lq_expf(an[n] - g4[e]), inv_sk, qmax);
-          }
+        for (int J = 0; J < 3; ++J) {
+          if (J >= wave) continue;
+          lq_v4i kop;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) kop[d] = (int)cd[1 + J][4 * s + d];
+          acc[J] = lq_mfma_i8(qop, kop, acc[J]);
         }
-        lq_v4i kop;
-#pragma unroll
-        for (int d = 0; d < 4; ++d) kop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
-        acc[J] = lq_mfma_i8(qop, kop, acc[J]);
       }
     }
   }
+
   const float sqk = sq * sk;
 #pragma unroll
   for (int J = 0; J < 3; ++J) {
@@ -133,49 +258,34 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
   for (int J = wave + 1; J < 4; ++J)
 #pragma unroll
     for (int r = 0; r < 4; ++r) p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = 0.0f;
-
-  __syncthreads();  // staged diagonal rows visible (each wave only reads its own block)
-
-  // ---- diagonal block: lane (i = rl, j = 4kg + jj)
-  {
-    float s[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int n = 0; n < K; ++n) {
-      const float qi = (float)qd_s[wave][rl][n] * sq;
-      const float gi = g_s[wave][rl][n];
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int j = 4 * kg + jj;
-        const float kj = (float)kd_s[wave][j][n] * sk;
-        const float w = (j <= rl) ? lq_expf(gi - g_s[wave][j][n]) : 0.0f;
-        s[jj] = s[jj] + (qi * kj) * w;
-      }
-    }
-    lq_v4f o;
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) o[jj] = (4 * kg + jj <= rl) ? s[jj] : 0.0f;
-    *(lq_v4f*)(p.A + ((t0 + i0 + rl) * H + h) * 64 + i0 + 4 * kg) = o;
-  }
 }
 
 }  // namespace
 
 extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   if (!a || !a->q || !a->k || !a->g || !a->A || !a->sq || !a->sk) return LQ_ERR_NULL;
-  if (a->rot) return LQ_ERR_SHAPE;  // local R_QK rotation of the anchored operands is not built yet
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if (a->kdim != 64 && a->kdim != 128) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (!zoo_al(a->q, 16) || !zoo_al(a->k, 16) || !zoo_al(a->g, 16) || !zoo_al(a->A, 16)) return LQ_ERR_SHAPE;
+  if (a->rot && !zoo_al(a->rot, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   AParams p = {};
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.g = a->g, p.A = a->A;
-  p.sq = a->sq, p.sk = a->sk, p.scale = a->scale, p.qmax = a->qmax;
+  p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);
-  if (a->kdim == 128)
-    hipLaunchKernelGGL(zoo_gla_A_kernel<128>, grid, dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL(zoo_gla_A_kernel<64>, grid, dim3(256), 0, stream, p);
+  if (a->kdim == 128) {
+    if (a->rot)
+      hipLaunchKernelGGL((zoo_gla_A_kernel<128, true>), grid, dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL((zoo_gla_A_kernel<128, false>), grid, dim3(256), 0, stream, p);
+  } else {
+    if (a->rot)
+      hipLaunchKernelGGL((zoo_gla_A_kernel<64, true>), grid, dim3(256), 0, stream, p);
+    else
+      hipLaunchKernelGGL((zoo_gla_A_kernel<64, false>), grid, dim3(256), 0, stream, p);
+  }
   return lq_check_launch();
 }

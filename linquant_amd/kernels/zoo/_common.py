@@ -63,9 +63,10 @@ def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims,
               batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay)
 
 
-def run_gla_A(q, key, gc, A, sq, sk, scale, qmax, dims):
+def run_gla_A(q, key, gc, A, sq, sk, scale, qmax, dims, rot=None):
     B, T, H, K, _ = dims
-    _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), rot=None,
+    assert rot is None or tuple(rot.shape) == (K, K), "rot: (K, K) R_QK"
+    _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), rot=_lib.ptr(rot),
               sq=_lib.ptr(sq), sk=_lib.ptr(sk), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K,
               chunk_size=CHUNK)
 

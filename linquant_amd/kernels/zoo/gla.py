@@ -21,13 +21,14 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
     assert chunk_size % BC == 0 and g.shape == (B, T, H, K)
-    C.no_rotation(unrot=unrot, rot=rot)
+    C.no_rotation(unrot=unrot)
+    R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     gc, logenv = C.cumsum(g, B, T, H, K)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
     A = torch.empty(B, T, H, chunk_size, dtype=torch.float32, device=q.device)
-    C.run_gla_A(q, k, gc, A, sc["q"], sc["k"], scale, qmax, dims)
+    C.run_gla_A(q, k, gc, A, sc["q"], sc["k"], scale, qmax, dims, rot=R)
     NT = T // chunk_size
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None

@@ -20,14 +20,15 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
     assert chunk_size % BC == 0 and g.shape == (B, T, H, K) and beta.shape == (B, T, H)
-    C.no_rotation(unrot=unrot, rot=rot)
+    C.no_rotation(unrot=unrot)
+    R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     gc, logenv = C.cumsum(g, B, T, H, K)
     Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
     A = torch.empty(B, T, H, chunk_size, dtype=torch.float32, device=q.device)
-    C.run_gla_A(q, Hw, gc, A, sc["q"], sc["k"], scale, qmax, dims)
+    C.run_gla_A(q, Hw, gc, A, sc["q"], sc["k"], scale, qmax, dims, rot=R)
     NT = T // chunk_size
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)

@@ -15,9 +15,11 @@ pytestmark = pytest.mark.gpu
 DEFAULT_ETA = {"linear_none": 1.0, "mamba2": 1.0, "gla": 0.0, "deltanet": 1.0, "gated_deltanet": 1.0, "kda": 0.0}
 
 
-def _go(cell, tensors, *, policy="kernel_static", bits=8, eta=None, rho=1.0, tau=1.0, label=None, **kw):
+def _go(cell, tensors, *, policy="kernel_static", bits=8, eta=None, rho=1.0, tau=1.0, label=None, rot=None, **kw):
     eta = DEFAULT_ETA[cell] if eta is None else eta
-    qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau)
+    qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau, rot_qk=rot)
+    if rot is not None:
+        kw["rot"] = rot
     B, T, H, K = tensors[0].shape
     V = tensors[2].shape[-1]
     scales = qz.kernel_scales(0, H, K, V, delta=zc.CELLS[cell][0] == "delta")
@@ -75,6 +77,19 @@ def test_strong_decay_stays_finite(cuda, cell, eta):
     tensors = zc.inputs(cell, gscale=40.0)
     out, _, qz, run = _go(cell, tensors, eta=eta)
     zc.check(out, run, qz, f"{cell} strong decay eta={eta}")
+
+
+@pytest.mark.parametrize("cell", ["gla", "kda"])
+@pytest.mark.parametrize("n,K", [(128, 64), (512, 64), (256, 128)])
+def test_local_rqk_rotation(cuda, cell, n, K):
+    """R_QK on a diagonal-decay cell is local: only the anchored operands of the off-diagonal sub-blocks are rotated
+    (/root/reference tests/test_kernel_gla.py:47-60)."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell, K=K, H=2 if K == 128 else 4), n)
+    R = signed_hadamard(K, 3)
+    out, _, qz, run = _go(cell, tensors, rot=R)
+    zc.check(out, run, qz, f"{cell} local R_QK T={n} K={K}")
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))
