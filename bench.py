@@ -67,7 +67,10 @@ def zoo_stage_bytes(fam, dec, B, T, H, K, V):
         out["wy_prep"] = qk + vv + tok + g + 2 * qk + vv + tok
     if dec == "diagonal":
         out["gla_A"] = 2 * qk + g + A
-    out["state"] = qk + vv + g + h8 + (qk + tok + vv if fam == "delta" else 0) + (tok if dec == "diagonal" else 0)
+    # the state stage of the reference reads the fp16 operands; the split pipeline adds the INT8 code round trip
+    out["write_codes"] = qk + g + (qk if fam == "delta" else vv) + (tok if dec == "diagonal" else 0) + qk // 2 + \
+        (qk // 2 if fam == "delta" else vv // 2)
+    out["state"] = qk // 2 + h8 + ((qk // 2 + 2 * tok + 2 * vv) if fam == "delta" else vv // 2)
     out["output"] = qk + (qk if dec != "diagonal" else A) + vv + h8 + g + vv
     return out
 
@@ -158,7 +161,8 @@ def bench_zoo(args):
     tokens = B * T
 
     records = {}
-    names = {"cumsum": "cumsum", "run_wy_prep": "wy_prep", "run_gla_A": "gla_A", "run_state": "state", "run_output": "output"}
+    names = {"cumsum": "cumsum", "run_wy_prep": "wy_prep", "run_gla_A": "gla_A", "write_codes": "write_codes",
+             "state_kernel": "state", "run_output": "output"}
     saved = {n: getattr(C, n) for n in names}
 
     def timed(fn, label):

@@ -225,29 +225,56 @@ int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
 #define LQ_DECAY_SCALAR 1
 #define LQ_DECAY_DIAGONAL 2
 
-/* replaces _state_kernel (linquant/kernels/zoo/simple_gla.py:23-95), _gla_state_kernel (gla.py:102-167),
- * _delta_state_kernel (gated_delta_rule.py:50-136) and _kda_state_kernel (kda.py:68-151): sequential chunk
- * loop with an fp32 carry, INT8 stored copy per chunk, INT8 write product (and, delta family, the INT8 state
- * read W.S and the pseudo-values E = (U - W.S) * fw, stored fp16 for the output kernel). */
+/* replaces the operand preparation inside the reference's state kernels (linquant/kernels/zoo/simple_gla.py:55-66,
+ * gla.py:124-141, gated_delta_rule.py:85-105, kda.py:100-124): every write operand that does not depend on the
+ * carried state is quantized once, in parallel over chunks, into the layout lq_zoo_state consumes.
+ * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers. */
 typedef struct {
-  const void* k;             /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16 */
-  const void* v;             /* value operand: v (linear) or U (delta), (B,T,H,V) fp16 */
-  const void* w;             /* delta: W (B,T,H,K) fp16; linear: NULL */
-  const float* fw;           /* delta: (B,T,H) fp32 value-side share of the outer beta factor */
+  const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16 */
+  const void* val;           /* linear family: v (B,T,H,V) fp16; delta family: NULL */
+  const void* w;             /* delta family: W (B,T,H,K) fp16; linear family: NULL */
   const float* g;            /* cumulative log decay (B,T,H) / (B,T,H,K), or NULL for no decay */
   const float* logenv;       /* diagonal decay: (B,T,H) */
+  int8_t* kqT;               /* (B,NT,H,K,64) int8 key write codes */
+  int8_t* vqT;               /* (B,NT,H,V,64) int8 value write codes (linear family) */
+  int8_t* wq;                /* (B,T,H,K) int8 state-read codes of W (delta family) */
+  float* ev;                 /* (B,T,H) fp32 value-side decay factor of each token */
+  float* gam;                /* (B,NT,H,K) fp32 chunk decay of each state row */
+  const float* skw;          /* (H,K) key write scale */
+  const float* svw;          /* (H,V) value write scale (linear family) */
+  const float* sw;           /* (H,) W scale (delta family) */
+  float eta;
+  int32_t qmax;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
+  int32_t decay;
+} lq_zoo_write_codes_args;
+int lq_zoo_write_codes(const lq_zoo_write_codes_args* args, hipStream_t stream);
+
+/* replaces the chunk loops of _state_kernel (linquant/kernels/zoo/simple_gla.py:23-95), _gla_state_kernel
+ * (gla.py:102-167), _delta_state_kernel (gated_delta_rule.py:50-136) and _kda_state_kernel (kda.py:68-151):
+ * sequential chunk loop with an fp32 carry, INT8 stored copy per chunk, INT8 write product (and, delta family,
+ * the INT8 state read W.S and the pseudo-values E = (U - W.S) * fw, stored fp16 for the output kernel).
+ * Consumes the buffers written by lq_zoo_write_codes. */
+typedef struct {
+  const int8_t* kqT;         /* (B,NT,H,K,64) */
+  const int8_t* vqT;         /* linear family: (B,NT,H,V,64) */
+  const int8_t* wq;          /* delta family: (B,T,H,K) */
+  const void* u;             /* delta family: U (B,T,H,V) fp16 */
+  const float* fw;           /* delta family: (B,T,H) fp32 value-side share of the outer beta factor */
+  const float* ev;           /* delta family: (B,T,H) */
+  const float* gam;          /* (B,NT,H,K) */
   int8_t* h_i8;              /* (B,NT,H,V,K) int8 */
-  void* e_out;               /* delta: (B,T,H,V) fp16 */
+  void* e_out;               /* delta family: (B,T,H,V) fp16 */
   float* ht;                 /* (B,H,K,V) fp32 final carry, or NULL */
   const float* skw;          /* (H,K) key write scale */
   const float* svw;          /* (H,V) value write scale: vw (linear) or ew (delta) */
   const float* sw;           /* (H,) W scale (delta) */
   const float* ss;           /* (H,V) state scale */
   const void* unrot;         /* (V,V) fp16 R_V^T for canonical storage, or NULL */
-  float eta;
   int32_t qmax;
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
-  int32_t family, decay;
+  int32_t family;
+  int32_t vtile;             /* value columns per workgroup: 16, 32, 64, or 0 = chosen from the grid size */
 } lq_zoo_state_args;
 int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
 

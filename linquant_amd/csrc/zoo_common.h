@@ -37,3 +37,7 @@ LQ_DEV uint32_t zoo_pack_h2(float a, float b) {
 }
 
 static inline bool zoo_al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
+
+// exp on the hardware exp2 unit (x * log2(e), then v_exp_f32): the arithmetic tl.exp lowers to in the reference's
+// Triton kernels.  Large negative arguments give 0, never NaN.
+LQ_DEV float zoo_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }

@@ -46,13 +46,40 @@ def cumsum(g, B, T, H, kdim):
     return gc, logenv
 
 
-def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
-              sw=None):
+def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay):
+    """Write-operand pre-pass: INT8 codes (and decay factors) of everything that does not depend on the carry."""
     B, T, H, K, V = dims
-    _lib.call("lq_zoo_state", key.device, k=_lib.ptr(key), v=_lib.ptr(value), w=_lib.ptr(w), fw=_lib.ptr(fw), g=_lib.ptr(g),
-              logenv=_lib.ptr(logenv), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
-              svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=None, eta=float(eta), qmax=int(qmax), batch=B,
-              seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, family=family, decay=decay)
+    dev, NT = key.device, T // CHUNK
+    delta = family == FAMILY_DELTA
+    c = {"kqT": torch.empty(B, NT, H, K, CHUNK, dtype=torch.int8, device=dev),
+         "vqT": None if delta else torch.empty(B, NT, H, V, CHUNK, dtype=torch.int8, device=dev),
+         "wq": torch.empty(B, T, H, K, dtype=torch.int8, device=dev) if delta else None,
+         "ev": torch.empty(B, T, H, dtype=torch.float32, device=dev),
+         "gam": torch.empty(B, NT, H, K, dtype=torch.float32, device=dev)}
+    _lib.call("lq_zoo_write_codes", dev, key=_lib.ptr(key), val=None if delta else _lib.ptr(value), w=_lib.ptr(w),
+              g=_lib.ptr(g), logenv=_lib.ptr(logenv), kqT=_lib.ptr(c["kqT"]), vqT=_lib.ptr(c["vqT"]), wq=_lib.ptr(c["wq"]),
+              ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]), skw=_lib.ptr(skw), svw=None if delta else _lib.ptr(svw),
+              sw=_lib.ptr(sw), eta=float(eta), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K, vdim=V,
+              chunk_size=CHUNK, decay=decay)
+    return c
+
+
+def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile=0):
+    """Sequential chunk recurrence over the pre-quantized operands ``c`` (see write_codes)."""
+    B, T, H, K, V = dims
+    delta = family == FAMILY_DELTA
+    _lib.call("lq_zoo_state", h_i8.device, kqT=_lib.ptr(c["kqT"]), vqT=_lib.ptr(c["vqT"]), wq=_lib.ptr(c["wq"]),
+              u=_lib.ptr(value) if delta else None, fw=_lib.ptr(fw), ev=_lib.ptr(c["ev"]) if delta else None,
+              gam=_lib.ptr(c["gam"]), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
+              svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=None, qmax=int(qmax), batch=B, seqlen=T, nheads=H,
+              kdim=K, vdim=V, chunk_size=CHUNK, family=family, vtile=int(vtile))
+
+
+def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
+              sw=None, vtile=0):
+    """``value`` is v (linear family) or U (delta family)."""
+    c = write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay)
+    state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile)
 
 
 def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay):
