@@ -9,8 +9,9 @@
 //
 // One 4-wave workgroup per (chunk, batch*head); wave w owns the 16 rows of sub-block w.  Off-diagonal
 // operands are K-contiguous, so each lane builds its own 16-slot INT8 MFMA operand from plain global loads
-// (no LDS).  The diagonal block stages INT8 codes and the decay rows of its 16 tokens in LDS and lets lane
-// (i = lane & 15, j-group = lane >> 4) accumulate four (i, j) pairs.
+// (no LDS).  The diagonal block factorizes the decay weight around the block's first row whenever the decay spread
+// inside the block allows it and then runs as an fp32 MFMA product; otherwise lane (i = lane & 15, j-group =
+// lane >> 4) accumulates four (i, j) pairs with one exponential per (i, j, channel).
 // With a local R_QK (rot, (K,K) fp16, x -> x.R) the anchored off-diagonal operands are rounded to fp16 and rotated
 // on the fp16 MFMA before quantization (gla.py:53-57); the diagonal blocks are not rotated.
 #include "zoo_common.h"
@@ -31,39 +32,95 @@ struct AParams {
   int B, T, H;
 };
 
-// diagonal block of wave's sub-block: lane (i = rl, j = 4kg + jj) reduces over the staged codes in fp32
+LQ_DEV float wave_max(float m) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  return m;
+}
+
+// Diagonal 16x16 block of one wave (rows row0 .. row0+15), written to A[row][i0 + j].
+//   A[i][j] = sum_n qh[i][n] kh[j][n] exp(g[i][n] - g[j][n]),  j <= i,  qh / kh the dequantized codes.
+// When the decay spread inside the block is small (every |g[r][n] - g[first][n]| <= 40) the weight factorizes
+// safely around the first row: the operands qh*exp(g_i - a) and kh*exp(a - g_j) stay normal fp32 numbers and
+// the sum is an fp32 16x16xK matrix product (lane (rl, kg) owns K/4 contiguous channels of token rl).
+// Otherwise every (i, j, n) weight is evaluated on its own, masked before use, as the reference does.
 template <int K>
-LQ_DEV void diag_block(const AParams& p, const float (*g_s)[K + 1], const int8_t (*qd_s)[K + 4], const int8_t (*kd_s)[K + 4],
-                       float sq, float sk, int rl, int kg, int64_t row0, int h, int i0) {
+LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float inv_sk, int rl, int kg, int64_t row0, int h,
+                       int i0) {
+  constexpr int NCH = K / 4;
+  const int H = p.H, qmax = p.qmax;
+  const int c0 = NCH * kg;
+  const int64_t off = ((row0 + rl) * H + h) * K + c0;
+  const int64_t aoff = (row0 * H + h) * K + c0;
+  float gv[NCH], av[NCH];
+  float spread = 0.0f;
+#pragma unroll
+  for (int e4 = 0; e4 < NCH / 4; ++e4) {
+    const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4), a4 = *(const lq_v4f*)(p.g + aoff + 4 * e4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      gv[4 * e4 + e] = g4[e];
+      av[4 * e4 + e] = a4[e];
+      spread = fmaxf(spread, __builtin_fabsf(g4[e] - a4[e]));
+    }
+  }
+  spread = wave_max(spread);
+  if (spread <= 40.0f) {
+    float qa[NCH], ka[NCH];
+#pragma unroll
+    for (int e8 = 0; e8 < NCH / 8; ++e8) {
+      const lq_v8h qv = *(const lq_v8h*)(p.q + off + 8 * e8), kv = *(const lq_v8h*)(p.k + off + 8 * e8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int n = 8 * e8 + e;
+        const float d = gv[n] - av[n];
+        const float qh = (float)zoo_q8((float)qv[e] * p.scale, inv_sq, qmax) * sq;
+        const float kh = (float)zoo_q8((float)kv[e], inv_sk, qmax) * sk;
+        qa[n] = qh * zoo_exp(d);
+        ka[n] = kh * zoo_exp(-d);
+      }
+    }
+    lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int n = 0; n < NCH; ++n) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[n], ka[n], acc, 0, 0, 0);
+    // lane holds column j = rl, rows i = 4kg + r
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      p.A[((row0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (rl <= 4 * kg + r) ? acc[r] : 0.0f;
+    return;
+  }
+  // exact path: lane (i = rl, j = 4kg + jj), 8 channels per step
   float s[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int n = 0; n < K; ++n) {
-    const float qi = (float)qd_s[rl][n] * sq;
-    const float gi = g_s[rl][n];
+  const int64_t irow = ((row0 + rl) * H + h) * K;
+  for (int n8 = 0; n8 < K; n8 += 8) {
+    const lq_v8h qv = *(const lq_v8h*)(p.q + irow + n8);
+    const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int j = 4 * kg + jj;
-      const float kj = (float)kd_s[j][n] * sk;
-      const float w = (j <= rl) ? lq_expf(gi - g_s[j][n]) : 0.0f;
-      s[jj] = s[jj] + (qi * kj) * w;
+      const int64_t jrow = ((row0 + j) * H + h) * K;
+      const lq_v8h kv = *(const lq_v8h*)(p.k + jrow + n8);
+      const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float qh = (float)zoo_q8((float)qv[e] * p.scale, inv_sq, qmax) * sq;
+        const float kh = (float)zoo_q8((float)kv[e], inv_sk, qmax) * sk;
+        const float gi = e < 4 ? gi0[e & 3] : gi1[e & 3], gj = e < 4 ? gj0[e & 3] : gj1[e & 3];
+        const float w = (j <= rl) ? zoo_exp(gi - gj) : 0.0f;
+        s[jj] = s[jj] + (qh * kh) * w;
+      }
     }
   }
   lq_v4f o;
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) o[jj] = (4 * kg + jj <= rl) ? s[jj] : 0.0f;
-  *(lq_v4f*)(p.A + ((row0 + rl) * p.H + h) * 64 + i0 + 4 * kg) = o;
+  *(lq_v4f*)(p.A + ((row0 + rl) * H + h) * 64 + i0 + 4 * kg) = o;
 }
 
 template <int K, bool ROT>
 __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
-  constexpr int GS = 4 * 16 * (K + 1) * 4;  // bytes of the decay rows
-  constexpr int QS = 4 * 16 * (K + 4);      // bytes of one code tile
-  constexpr int RS = K + 8;                 // halves per row of the transposed rotation
-  static_assert(K * RS * 2 <= GS + 2 * QS, "the rotation tile reuses the diagonal-block staging space");
-  __shared__ __align__(16) unsigned char smem[GS + 2 * QS];
-  float (*g_s)[16][K + 1] = reinterpret_cast<float (*)[16][K + 1]>(smem);
-  int8_t (*qd_s)[16][K + 4] = reinterpret_cast<int8_t (*)[16][K + 4]>(smem + GS);
-  int8_t (*kd_s)[16][K + 4] = reinterpret_cast<int8_t (*)[16][K + 4]>(smem + GS + QS);
-  _Float16* RT = reinterpret_cast<_Float16*>(smem);  // ROT: RT[m][n] = R[n][m], after the diagonal blocks are done
+  constexpr int RS = K + 8;  // halves per row of the transposed rotation
+  __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -76,20 +133,18 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
   const int qmax = p.qmax;
   const int i0 = 16 * wave;
 
-  // ---- stage the diagonal block: codes of q*scale and k, decay rows
-  for (int it = lane; it < 16 * (K / 8); it += 64) {
-    const int r = it / (K / 8), c8 = it % (K / 8);
-    const int64_t off = ((t0 + i0 + r) * H + h) * K + 8 * c8;
-    const lq_v8h qv = *(const lq_v8h*)(p.q + off);
-    const lq_v8h kv = *(const lq_v8h*)(p.k + off);
-    const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+  if constexpr (ROT) {
+    // lanes walk m (coalesced rows of R), each thread gathers 8 consecutive n and writes one 16-byte piece of a row
+    for (int it = tid; it < K * (K / 8); it += 256) {
+      const int m = it % K, n8 = it / K;
+      lq_v8h rv;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      qd_s[wave][r][8 * c8 + e] = (int8_t)zoo_q8((float)qv[e] * p.scale, inv_sq, qmax);
-      kd_s[wave][r][8 * c8 + e] = (int8_t)zoo_q8((float)kv[e], inv_sk, qmax);
-      g_s[wave][r][8 * c8 + e] = e < 4 ? g0[e & 3] : g1[e & 3];
+      for (int e = 0; e < 8; ++e) rv[e] = p.rot[(int64_t)(8 * n8 + e) * K + m];
+      *(lq_v8h*)(RT + m * RS + 8 * n8) = rv;
     }
   }
+
+  diag_block<K>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
 
   lq_v4i acc[3];
 #pragma unroll
@@ -123,7 +178,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
             for (int e = 0; e < 4; ++e) {
               const int n = 4 * e4 + e;
               const float qf = n < 8 ? (float)q0[n & 7] : (float)q1[n & 7];
-              float x = qf * lq_expf(g4[e] - an[n]);
+              float x = qf * zoo_exp(g4[e] - an[n]);
               x = x * p.scale;
               cd[n] = zoo_q8(x, inv_sq, qmax);
             }
@@ -144,7 +199,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
             for (int e = 0; e < 4; ++e) {
               const int n = 4 * e4 + e;
               const float kf = n < 8 ? (float)k0[n & 7] : (float)k1[n & 7];
-              cd[n] = zoo_q8(kf * lq_expf(an[n] - g4[e]), inv_sk, qmax);
+              cd[n] = zoo_q8(kf * zoo_exp(an[n] - g4[e]), inv_sk, qmax);
             }
           }
           lq_v4i kop;
@@ -154,22 +209,11 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
         }
       }
     }
-    __syncthreads();  // staged diagonal rows visible (each wave only reads its own block)
-    diag_block<K>(p, g_s[wave], qd_s[wave], kd_s[wave], sq, sk, rl, kg, t0 + i0, h, i0);
   } else {
     // ---- local R_QK: the anchored operands are rotated (fp16 MFMA, fp32 accumulate) before quantization.
     // Transposed product R^T . X^T: lane (rl, kg) receives, for token rl, channels 16mt + 4kg + r, which it packs
     // as dword mt of its INT8 operand; q and k operands share that channel -> slot map, so the INT8 dot is exact.
     constexpr int KS = K / 32, MT = K / 16;
-    __syncthreads();
-    diag_block<K>(p, g_s[wave], qd_s[wave], kd_s[wave], sq, sk, rl, kg, t0 + i0, h, i0);
-    __syncthreads();  // every wave is done with the staged rows: reuse the space for R^T
-    for (int it = tid; it < K * (K / 8); it += 256) {
-      const int n = it / (K / 8), m8 = it % (K / 8);
-      const lq_v8h rv = *(const lq_v8h*)(p.rot + (int64_t)n * K + 8 * m8);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) RT[(8 * m8 + e) * RS + n] = rv[e];
-    }
     // anchored fp16 operands: tensor 0 = q rows of this sub-block, tensor 1 + J = k rows of sub-block J < wave
     lq_v8h xop[4][KS];
     if (wave > 0) {
@@ -185,7 +229,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            float x = (float)qv[e] * lq_expf(gg - an);
+            float x = (float)qv[e] * zoo_exp(gg - an);
             x = x * p.scale;
             xop[0][ks][e] = (_Float16)x;
           }
@@ -199,7 +243,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            xop[1 + J][ks][e] = (_Float16)((float)kv[e] * lq_expf(an - gg));
+            xop[1 + J][ks][e] = (_Float16)((float)kv[e] * zoo_exp(an - gg));
           }
         }
       }

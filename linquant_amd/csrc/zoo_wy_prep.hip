@@ -6,12 +6,16 @@
 //   G[i][j] = sum_n L[i][n] Hg[j][n] * decay(i,j,n)  for i > j, decay = 1 | exp(g_i - g_j) | exp(g_in - g_jn)
 //   T = (I + G)^-1  (unit lower triangular, forward substitution)
 //   W = T (L * exp(g)),  U = T (beta^sigma v),  Hw = beta^((1-sigma) tau) k,  fw = beta^((1-sigma)(1-tau))
-// Every decay exponent is <= 0 (i > j and g is non-increasing inside a chunk), so the per-channel Gram needs
-// no anchoring when evaluated element by element.
 //
-// One 4-wave workgroup per (chunk, batch*head).  Tiles live in LDS as fp32; the Gram and the two products
-// are register-tiled 4x4 per thread; the triangular inverse is done by one wavefront, lane c carrying
-// column c of T in registers and reading G rows as LDS broadcasts.
+// One 4-wave workgroup per (chunk, batch*head); every product runs on the fp32 MFMA (16x16x4).
+//   Gram: wave w owns row block w; operands come straight from global memory (lane (rl, kg) supplies 16 contiguous
+//     channels of token rl per 64-channel pass).  Per-channel decay is factorized around the first row of the row
+//     block (off-diagonal blocks: both factors <= 1; diagonal block: only when the decay spread inside the block is
+//     small, otherwise one exponential per (i, j, channel)).
+//   Inverse: the four 16x16 diagonal blocks by forward substitution (lane per column), then block rows 1..3:
+//     T_IJ = -T_II . sum_{J <= M < I} G_IM . T_MJ.
+//   W, U: T . X with X staged in LDS as fp32; each wave takes row block w for the first half of the column tiles
+//     and row block 3 - w for the second half (equal work), and stores four adjacent channels per lane.
 #include "zoo_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -36,28 +40,50 @@ LQ_DEV float powb(float b, float e) {
   return __builtin_amdgcn_exp2f(e * __builtin_amdgcn_logf(b));
 }
 
+LQ_DEV lq_v4f mfma_f32(float a, float b, lq_v4f c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+
+LQ_DEV float wy_wave_max(float m) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  return m;
+}
+
+constexpr int kGS = 68;  // floats per row of the G / T tiles: 4*row + slot hits 64 distinct banks
+
+// D^T tile of T . X for row block I and 16 columns starting at col: lane (rl = token, kg) gets columns col + 4kg + r
+template <int LS>
+LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl, int kg) {
+  lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
+  for (int J = 0; J <= I; ++J)
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int m = 16 * J + 4 * s + kg;
+      acc = mfma_f32(X_s[m * LS + col + rl], T_s[(16 * I + rl) * kGS + m], acc);
+    }
+  return acc;
+}
+
 template <int DECAY, int K>
 __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
-  constexpr int LS = K + 1;
-  extern __shared__ __align__(16) float lds[];
-  float* L_s = lds;                    // [64][LS]   L, later L * exp(g)
-  float* H_s = L_s + 64 * LS;          // [64][LS]   Hg, later the value tile (64 columns at a time)
-  float* G_s = H_s + 64 * LS;          // [64][65]   G, then T in place
-  float* gd_s = G_s + 64 * 65;         // [64][LS]   per-channel cumulative decay (diagonal only)
-  float* gs_s = (DECAY == LQ_DECAY_DIAGONAL) ? gd_s + 64 * LS : gd_s;  // [64] scalar cumulative decay
-  float* bs_s = gs_s + 64;             // [64] beta^sigma
+  constexpr int LS = K + 16;  // floats per row of X: rows 4s + kg land in disjoint bank groups
+  __shared__ __align__(16) float G_s[64 * kGS];
+  __shared__ __align__(16) float T_s[64 * kGS];
+  __shared__ __align__(16) float X_s[64 * LS];
+  __shared__ float gs_s[64], bs_s[64], bh_s[64];
 
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
   const int ct = blockIdx.x;
   const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
   const float sigma = p.sigma, tau = p.tau;
 
-  // ---- load: L, Hg, decay rows; Hw and fw are written straight out
+  // ---- per-token factors; Hw and fw are written straight out; X = beta^sigma k exp(g) staged for the W product
   if (tid < 64) {
     const float bt = p.beta[(t0 + tid) * H + h];
     bs_s[tid] = powb(bt, sigma);
+    bh_s[tid] = powb(bt, 1.0f - sigma);
     p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
     if (DECAY == LQ_DECAY_SCALAR) gs_s[tid] = p.g[(t0 + tid) * H + h];
   }
@@ -66,164 +92,221 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
     const int64_t off = ((t0 + r) * H + h) * K + 8 * c8;
     const lq_v8h kv = *(const lq_v8h*)(p.k + off);
     const float bt = p.beta[(t0 + r) * H + h];
-    const float bl = powb(bt, sigma), bh = powb(bt, 1.0f - sigma), bw = powb(bt, (1.0f - sigma) * tau);
-    lq_v8h hw;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float kf = (float)kv[e];
-      L_s[r * LS + 8 * c8 + e] = bl * kf;
-      H_s[r * LS + 8 * c8 + e] = bh * kf;
-      hw[e] = (_Float16)(bw * kf);
-    }
-    *(lq_v8h*)(p.Hw + off) = hw;
+    const float bw = powb(bt, (1.0f - sigma) * tau);
+    float bl = powb(bt, sigma);
+    if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(p.g[(t0 + r) * H + h]);
+    float ge[8];
     if (DECAY == LQ_DECAY_DIAGONAL) {
       const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) gd_s[r * LS + 8 * c8 + e] = e < 4 ? g0[e & 3] : g1[e & 3];
+      for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
     }
+    lq_v8h hw;
+    lq_v4f x0, x1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float kf = (float)kv[e];
+      float x = bl * kf;
+      if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
+      if (e < 4) x0[e] = x; else x1[e - 4] = x;
+      hw[e] = (_Float16)(bw * kf);
+    }
+    *(lq_v8h*)(p.Hw + off) = hw;
+    *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
+    *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
   }
   __syncthreads();
 
-  // ---- Gram, strictly lower part: thread (ti, tj) owns rows 4ti..4ti+3, cols 4tj..4tj+3
+  // ---- Gram, row block I = wave: G[i][j] for i > j
   {
-    const int ti = tid >> 4, tj = tid & 15;
-    float a[4][4];
+    const int I = wave;
+    const int64_t irow = ((t0 + 16 * I + rl) * H + h) * K;
+    const int64_t arow = ((t0 + 16 * I) * H + h) * K;
+    const float bs_i = bs_s[16 * I + rl];
+    lq_v4f acc[4];
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+    for (int J = 0; J < 4; ++J) acc[J] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+    bool exact_diag = false;
+    if (DECAY == LQ_DECAY_DIAGONAL) {
+      float spread = 0.0f;
+      for (int c = 16 * kg; c < K; c += 64)
 #pragma unroll
-      for (int y = 0; y < 4; ++y) a[x][y] = 0.0f;
-    if (tj <= ti) {
-      for (int n = 0; n < K; ++n) {
-        float lv[4], hv[4], gi[4], gj[4];
+        for (int e4 = 0; e4 < 4; ++e4) {
+          const lq_v4f g4 = *(const lq_v4f*)(p.g + irow + c + 4 * e4), a4 = *(const lq_v4f*)(p.g + arow + c + 4 * e4);
 #pragma unroll
-        for (int x = 0; x < 4; ++x) {
-          lv[x] = L_s[(4 * ti + x) * LS + n];
-          hv[x] = H_s[(4 * tj + x) * LS + n];
-          if (DECAY == LQ_DECAY_DIAGONAL) {
-            gi[x] = gd_s[(4 * ti + x) * LS + n];
-            gj[x] = gd_s[(4 * tj + x) * LS + n];
-          }
+          for (int e = 0; e < 4; ++e) spread = fmaxf(spread, __builtin_fabsf(g4[e] - a4[e]));
         }
+      exact_diag = wy_wave_max(spread) > 40.0f;
+    }
 #pragma unroll
-        for (int x = 0; x < 4; ++x)
+    for (int ps = 0; ps < K / 64; ++ps) {
+      const int c0 = 64 * ps + 16 * kg;
+      float Lr[16], gi[16], an[16];
+      {
+        const lq_v8h k0 = *(const lq_v8h*)(p.k + irow + c0), k1 = *(const lq_v8h*)(p.k + irow + c0 + 8);
 #pragma unroll
-          for (int y = 0; y < 4; ++y) {
-            if (DECAY == LQ_DECAY_DIAGONAL) {
-              const float w = (4 * ti + x > 4 * tj + y) ? __expf(gi[x] - gj[y]) : 0.0f;
-              a[x][y] = fmaf(lv[x] * hv[y], w, a[x][y]);
-            } else {
-              a[x][y] = fmaf(lv[x], hv[y], a[x][y]);
+        for (int e = 0; e < 16; ++e) Lr[e] = bs_i * (float)(e < 8 ? k0[e & 7] : k1[e & 7]);
+        if (DECAY == LQ_DECAY_DIAGONAL) {
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const lq_v4f g4 = *(const lq_v4f*)(p.g + irow + c0 + 4 * e4), a4 = *(const lq_v4f*)(p.g + arow + c0 + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              gi[4 * e4 + e] = g4[e];
+              an[4 * e4 + e] = a4[e];
             }
           }
+#pragma unroll
+          for (int e = 0; e < 16; ++e) Lr[e] = Lr[e] * zoo_exp(gi[e] - an[e]);
+        }
+      }
+#pragma unroll
+      for (int J = 0; J < 4; ++J) {
+        if (J > I) continue;
+        if (DECAY == LQ_DECAY_DIAGONAL && J == I && exact_diag) continue;
+        const int64_t jrow = ((t0 + 16 * J + rl) * H + h) * K;
+        const float bh_j = bh_s[16 * J + rl];
+        const lq_v8h k0 = *(const lq_v8h*)(p.k + jrow + c0), k1 = *(const lq_v8h*)(p.k + jrow + c0 + 8);
+        float Hr[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) Hr[e] = bh_j * (float)(e < 8 ? k0[e & 7] : k1[e & 7]);
+        if (DECAY == LQ_DECAY_DIAGONAL) {
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const lq_v4f g4 = *(const lq_v4f*)(p.g + jrow + c0 + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Hr[4 * e4 + e] = Hr[4 * e4 + e] * zoo_exp(an[4 * e4 + e] - g4[e]);
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[J] = mfma_f32(Lr[e], Hr[e], acc[J]);
       }
     }
+    // lane holds column j = rl of block J, rows i = 4kg + r of block I
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+    for (int J = 0; J < 4; ++J) {
+      if (J > I) continue;
+      if (DECAY == LQ_DECAY_DIAGONAL && J == I && exact_diag) continue;
 #pragma unroll
-      for (int y = 0; y < 4; ++y) {
-        const int i = 4 * ti + x, j = 4 * tj + y;
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * I + 4 * kg + r, j = 16 * J + rl;
         float v = 0.0f;
         if (i > j) {
-          v = a[x][y];
-          if (DECAY == LQ_DECAY_SCALAR) v = v * __expf(gs_s[i] - gs_s[j]);
+          v = acc[J][r];
+          if (DECAY == LQ_DECAY_SCALAR) v = v * zoo_exp(gs_s[i] - gs_s[j]);
         }
-        G_s[i * 65 + j] = v;
+        G_s[i * kGS + j] = v;
       }
+    }
+    if (DECAY == LQ_DECAY_DIAGONAL && exact_diag) {
+      // lane (i = rl, j = 4kg + jj) of the diagonal block, one exponential per (i, j, channel)
+      float sacc[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int n8 = 0; n8 < K; n8 += 8) {
+        const lq_v8h ki = *(const lq_v8h*)(p.k + irow + n8);
+        const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int j = 4 * kg + jj;
+          const int64_t jrow = ((t0 + 16 * I + j) * H + h) * K;
+          const lq_v8h kj = *(const lq_v8h*)(p.k + jrow + n8);
+          const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
+          const float bh_j = bh_s[16 * I + j];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float gi_ = e < 4 ? gi0[e & 3] : gi1[e & 3], gj_ = e < 4 ? gj0[e & 3] : gj1[e & 3];
+            const float w = (rl > j) ? zoo_exp(gi_ - gj_) : 0.0f;
+            sacc[jj] = fmaf((bs_i * (float)ki[e]) * (bh_j * (float)kj[e]), w, sacc[jj]);
+          }
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) G_s[(16 * I + rl) * kGS + 16 * I + 4 * kg + jj] = (rl > 4 * kg + jj) ? sacc[jj] : 0.0f;
+    }
   }
   __syncthreads();
 
-  // ---- T = (I + G)^-1 by forward substitution (wave 0; lane c holds column c), stored over G
-  if (tid < 64) {
-    float tc[64];
+  // ---- T = (I + G)^-1: diagonal blocks by forward substitution (wave w, lane c < 16 holds column c of block w)
+  if (lane < 16) {
+    const int o = 16 * wave;
+    float tc[16];
 #pragma unroll
-    for (int i = 0; i < 64; ++i) {
-      float acc = (i == tid) ? 1.0f : 0.0f;
+    for (int i = 0; i < 16; ++i) {
+      float a = (i == lane) ? 1.0f : 0.0f;
 #pragma unroll
-      for (int j = 0; j < i; ++j) acc = fmaf(-G_s[i * 65 + j], tc[j], acc);
-      tc[i] = acc;
+      for (int j = 0; j < i; ++j) a = fmaf(-G_s[(o + i) * kGS + o + j], tc[j], a);
+      tc[i] = a;
     }
 #pragma unroll
-    for (int i = 0; i < 64; ++i) G_s[i * 65 + tid] = tc[i];
-  }
-  // meanwhile: L <- L * exp(g) (read-side decay of W's right-hand side)
-  if (DECAY != LQ_DECAY_NONE && tid >= 64) {
-    for (int it = tid - 64; it < 64 * K; it += 192) {
-      const int r = it / K, n = it % K;
-      const float gg = (DECAY == LQ_DECAY_SCALAR) ? gs_s[r] : gd_s[r * LS + n];
-      L_s[r * LS + n] = L_s[r * LS + n] * __expf(gg);
-    }
+    for (int i = 0; i < 16; ++i) T_s[(o + i) * kGS + o + lane] = tc[i];
   }
   __syncthreads();
-
-  // ---- W = T . L'  (64 x K): thread owns rows 4ti..+3, cols {tj + 16c}
-  {
-    const int ti = tid >> 4, tj = tid & 15;
-    constexpr int NC = K / 16;
-    float a[4][NC];
+  // block rows 1..3: wave J < I computes T_IJ = -T_II . sum_{J <= M < I} G_IM . T_MJ
+  for (int I = 1; I < 4; ++I) {
+    if (wave < I) {
+      const int J = wave;
+      lq_v4f sacc = {0.f, 0.f, 0.f, 0.f};
+      for (int M = J; M < I; ++M)
 #pragma unroll
-    for (int x = 0; x < 4; ++x)
+        for (int s = 0; s < 4; ++s) {
+          const int m = 16 * M + 4 * s + kg;
+          sacc = mfma_f32(G_s[(16 * I + rl) * kGS + m], T_s[m * kGS + 16 * J + rl], sacc);
+        }
+      // sacc: lane (rl = column, kg) holds rows 4kg + r, which is contraction index 4kg + s of the next product
+      lq_v4f tacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < NC; ++c) a[x][c] = 0.0f;
-    for (int j = 0; j < 4 * ti + 4; ++j) {
-      float tv[4];
+      for (int s = 0; s < 4; ++s) tacc = mfma_f32(T_s[(16 * I + rl) * kGS + 16 * I + 4 * kg + s], sacc[s], tacc);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) tv[x] = G_s[(4 * ti + x) * 65 + j];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const float r = L_s[j * LS + tj + 16 * c];
-#pragma unroll
-        for (int x = 0; x < 4; ++x) a[x][c] = fmaf(tv[x], r, a[x][c]);
-      }
+      for (int r = 0; r < 4; ++r) T_s[(16 * I + 4 * kg + r) * kGS + 16 * J + rl] = -tacc[r];
     }
-#pragma unroll
-    for (int x = 0; x < 4; ++x)
-#pragma unroll
-      for (int c = 0; c < NC; ++c) p.W[((t0 + 4 * ti + x) * H + h) * K + tj + 16 * c] = (_Float16)a[x][c];
-  }
-
-  // ---- U = T . (beta^sigma v), 64 value columns at a time through the Hg buffer
-  for (int vc = 0; vc < V; vc += 64) {
     __syncthreads();
-    for (int it = tid; it < 64 * 8; it += 256) {
-      const int r = it >> 3, c8 = it & 7;
+  }
+
+  // ---- W = T . X
+  {
+    constexpr int NTL = K / 16;
+    for (int nt = 0; nt < NTL; ++nt) {
+      const int I = nt < NTL / 2 ? wave : 3 - wave;
+      const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
+      lq_v2i o;
+      o[0] = (int)zoo_pack_h2(a[0], a[1]);
+      o[1] = (int)zoo_pack_h2(a[2], a[3]);
+      *(lq_v2i*)(p.W + ((t0 + 16 * I + rl) * H + h) * K + 16 * nt + 4 * kg) = o;
+    }
+  }
+
+  // ---- U = T . (beta^sigma v), up to K value columns per pass through the X buffer
+  for (int vc = 0; vc < V; vc += K) {
+    const int pw = (V - vc) < K ? (V - vc) : K;  // 64 or K columns
+    __syncthreads();
+    for (int it = tid; it < 64 * (pw / 8); it += 256) {
+      const int r = it / (pw / 8), c8 = it % (pw / 8);
       const lq_v8h vv = *(const lq_v8h*)(p.v + ((t0 + r) * H + h) * V + vc + 8 * c8);
       const float bsr = bs_s[r];
+      lq_v4f x0, x1;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) H_s[r * LS + 8 * c8 + e] = bsr * (float)vv[e];
+      for (int e = 0; e < 4; ++e) {
+        x0[e] = bsr * (float)vv[e];
+        x1[e] = bsr * (float)vv[4 + e];
+      }
+      *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
+      *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
     }
     __syncthreads();
-    const int ti = tid >> 4, tj = tid & 15;
-    float a[4][4];
-#pragma unroll
-    for (int x = 0; x < 4; ++x)
-#pragma unroll
-      for (int c = 0; c < 4; ++c) a[x][c] = 0.0f;
-    for (int j = 0; j < 4 * ti + 4; ++j) {
-      float tv[4];
-#pragma unroll
-      for (int x = 0; x < 4; ++x) tv[x] = G_s[(4 * ti + x) * 65 + j];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const float r = H_s[j * LS + tj + 16 * c];
-#pragma unroll
-        for (int x = 0; x < 4; ++x) a[x][c] = fmaf(tv[x], r, a[x][c]);
-      }
+    const int ntl = pw / 16;
+    for (int nt = 0; nt < ntl; ++nt) {
+      const int I = nt < ntl / 2 ? wave : 3 - wave;
+      const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
+      lq_v2i o;
+      o[0] = (int)zoo_pack_h2(a[0], a[1]);
+      o[1] = (int)zoo_pack_h2(a[2], a[3]);
+      *(lq_v2i*)(p.U + ((t0 + 16 * I + rl) * H + h) * V + vc + 16 * nt + 4 * kg) = o;
     }
-#pragma unroll
-    for (int x = 0; x < 4; ++x)
-#pragma unroll
-      for (int c = 0; c < 4; ++c) p.U[((t0 + 4 * ti + x) * H + h) * V + vc + tj + 16 * c] = (_Float16)a[x][c];
   }
 }
 
 template <int DECAY, int K>
 int launch(const WyParams& p, dim3 grid, hipStream_t stream) {
-  constexpr int LS = K + 1;
-  const size_t lds = sizeof(float) * (2 * 64 * LS + 64 * 65 + (DECAY == LQ_DECAY_DIAGONAL ? 64 * LS : 0) + 128);
-  if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&zoo_wy_prep_kernel<DECAY, K>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-    return LQ_ERR_LAUNCH;
-  hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K>), grid, dim3(256), lds, stream, p);
+  hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K>), grid, dim3(256), 0, stream, p);
   return lq_check_launch();
 }
 
