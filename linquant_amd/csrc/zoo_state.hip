@@ -279,8 +279,13 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   // narrower V tiles when batch*head alone cannot fill the 256 compute units
   int BV = a->vtile;
   if (BV == 0) {
+    // measured on 256 compute units: the delta family (two barriers and two dependent products per chunk) is fastest
+    // with 32 columns, the linear family with 16, until the grid alone fills the chip
     const int64_t wg64 = (int64_t)a->batch * a->nheads * (a->vdim / 64);
-    BV = wg64 >= 512 ? 64 : (wg64 >= 192 ? 32 : 16);
+    if (delta)
+      BV = wg64 >= 512 ? 64 : 32;
+    else
+      BV = wg64 >= 1024 ? 64 : (wg64 >= 512 ? 32 : 16);
   }
   if (delta) return a->kdim == 128 ? launch_bv<true, 128>(p, BV, a->batch, stream) : launch_bv<true, 64>(p, BV, a->batch, stream);
   return a->kdim == 128 ? launch_bv<false, 128>(p, BV, a->batch, stream) : launch_bv<false, 64>(p, BV, a->batch, stream);
