@@ -13,7 +13,7 @@
 // operand goes to LDS as token-pair interleaved fp16 (dword = two consecutive tokens of one channel), the
 // same layout trick as the Mamba-2 chunk scan: four 16-byte reads give the operands of the four MFMA calls
 // that cover channels {4*(lane&15)+j}, and every lane ends up with 4 adjacent output channels.
-#include "zoo_common.h"
+#include "zoo_params.h"
 #include "../../include/linquant_hip.h"
 
 namespace {
@@ -22,23 +22,7 @@ constexpr int BV = 64;
 constexpr int kAS = 72;  // halves per row of the fp16 A tile in LDS
 constexpr int kVW = 68;  // dwords per token-pair row of the value tile
 
-struct OutParams {
-  const _Float16* q;
-  const _Float16* k;
-  const _Float16* v;
-  const int8_t* h_i8;
-  const float* g;
-  const float* A;
-  void* o;
-  int o_is_f32;
-  const float* sq;
-  const float* sk;
-  const float* svl;
-  const float* ss;
-  float scale;
-  int qmax;
-  int B, T, H, V, NT;
-};
+using OutParams = ZooOutParams;
 
 template <bool GLA, bool USE_G, int K>
 __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
@@ -243,7 +227,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if (!gla && (!a->k || !a->sk)) return LQ_ERR_NULL;
   if (a->decay == LQ_DECAY_SCALAR && !a->g) return LQ_ERR_NULL;
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
-  if (a->unrot) return LQ_ERR_SHAPE;  // canonical storage (in-kernel un-rotation) is not built yet
+  if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
@@ -256,6 +240,8 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.h_i8 = a->h_i8, p.g = a->g, p.A = a->A, p.o = a->o, p.o_is_f32 = a->o_is_f32;
   p.sq = a->sq, p.sk = a->sk, p.svl = a->svl, p.ss = a->ss, p.scale = a->scale, p.qmax = a->qmax;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
+  p.unrot = (const _Float16*)a->unrot;
+  if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
   dim3 grid(a->vdim / BV, p.NT, a->batch * a->nheads);
   if (gla) return launch<true, true>(p, a->kdim, grid, stream);
   if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, grid, stream);

@@ -1,0 +1,48 @@
+// Kernel parameter blocks of the zoo state / output kernels, shared by the rotated-storage kernels and the
+// canonical-storage (in-kernel un-rotation) variants.
+#pragma once
+
+#include "zoo_common.h"
+
+struct ZooStateParams {
+  const int8_t* kqT;
+  const int8_t* vqT;
+  const int8_t* wq;
+  const _Float16* u;
+  const float* fw;
+  const float* ev;
+  const float* gam;
+  int8_t* h_i8;
+  _Float16* e_out;
+  float* ht;
+  const float* skw;
+  const float* svw;
+  const float* sw;
+  const float* ss;
+  const _Float16* unrot;
+  int qmax;
+  int T, H, V, NT;
+};
+
+struct ZooOutParams {
+  const _Float16* q;
+  const _Float16* k;
+  const _Float16* v;
+  const int8_t* h_i8;
+  const float* g;
+  const float* A;
+  void* o;
+  int o_is_f32;
+  const float* sq;
+  const float* sk;
+  const float* svl;
+  const float* ss;
+  const _Float16* unrot;
+  float scale;
+  int qmax;
+  int B, T, H, V, NT;
+};
+
+// canonical storage: one workgroup spans all V value channels (V = 64 or 128); defined in zoo_unrot.hip
+int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, hipStream_t stream);
+int zoo_output_unrot_launch(const ZooOutParams& p, int decay, int K, hipStream_t stream);

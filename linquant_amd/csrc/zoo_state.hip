@@ -16,29 +16,12 @@
 // LDS V-major so that it is copied out coalesced and read back as the K-contiguous operand of the state read;
 // the pseudo-value codes go through LDS channel-major so that they are the token-contiguous operand of the
 // write product.  All global operands of chunk c+1 are fetched into registers while chunk c is computed.
-#include "zoo_common.h"
+#include "zoo_params.h"
 #include "../../include/linquant_hip.h"
 
 namespace {
 
-struct StateParams {
-  const int8_t* kqT;
-  const int8_t* vqT;
-  const int8_t* wq;
-  const _Float16* u;
-  const float* fw;
-  const float* ev;
-  const float* gam;
-  int8_t* h_i8;
-  _Float16* e_out;
-  float* ht;
-  const float* skw;
-  const float* svw;
-  const float* sw;
-  const float* ss;
-  int qmax;
-  int T, H, V, NT;
-};
+using StateParams = ZooStateParams;
 
 template <bool DELTA, int K, int BV>
 struct StepOps {
@@ -261,7 +244,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (a->family != LQ_FAMILY_LINEAR && !delta) return LQ_ERR_SHAPE;
   if (delta && (!a->wq || !a->u || !a->fw || !a->ev || !a->e_out || !a->sw)) return LQ_ERR_NULL;
   if (!delta && !a->vqT) return LQ_ERR_NULL;
-  if (a->unrot) return LQ_ERR_SHAPE;  // canonical storage (in-kernel un-rotation) is not built yet
+  if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
@@ -275,7 +258,9 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   p.kqT = a->kqT, p.vqT = a->vqT, p.wq = a->wq, p.u = (const _Float16*)a->u, p.fw = a->fw, p.ev = a->ev, p.gam = a->gam;
   p.h_i8 = a->h_i8, p.e_out = (_Float16*)a->e_out, p.ht = a->ht;
   p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.ss = a->ss, p.qmax = a->qmax;
+  p.unrot = (const _Float16*)a->unrot;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
+  if (a->unrot) return zoo_state_unrot_launch(p, delta, a->kdim, a->batch, stream);
   // narrower V tiles when batch*head alone cannot fill the 256 compute units
   int BV = a->vtile;
   if (BV == 0) {

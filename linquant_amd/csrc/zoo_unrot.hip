@@ -1,0 +1,454 @@
+// Canonical-storage variants of the zoo state and output kernels (value rotation R_V with in-kernel un-rotation).
+// Replaces _state_kernel_unrot / _output_kernel_unrot (linquant/kernels/zoo/simple_gla.py:86-95, 165-172 with
+// USE_UNROT in _state_body :67-70 and _output_body :147-150), _gla_state_kernel_unrot / _gla_output_kernel_unrot
+// (gla.py), _delta_state_kernel_unrot (gated_delta_rule.py:60-63, 93-95, 107-109) and _kda_state_kernel_unrot (kda.py):
+// v (or U) arrives in the rotated value basis, the carried and stored state stay canonical.
+//   state:  h += fp16(dequantized write product) . Ru                 Ru = R_V^T, (V,V) fp16
+//           delta family: the dequantized state read is rotated first, ws = fp16(ws) . Ru^T, so E stays rotated
+//   output: o = state read (canonical) + fp16(local product * svl) . Ru
+// One workgroup spans all V value channels (V = 64 or 128).  Every product is computed transposed (value channel
+// on the accumulator rows): a lane then holds, for one token or one key channel, the value channels
+// 16*vt + 4*(lane >> 4) + r, which is exactly a B operand of the fp16 rotation product when the rotation matrix
+// rows are read with the matching channel -> slot map.  Nothing is transposed through LDS except the INT8 codes.
+#include "zoo_params.h"
+#include "../../include/linquant_hip.h"
+
+namespace {
+
+// out[v'][c] = sum_v Rs[v'][v] * x[v][c] for one 16-column tile c: x arrives as accumulator fragments
+// d[vt][r] (rows v = 16vt + 4kg + r); slot e of step sg is channel 16*(2sg + (e >> 2)) + 4kg + (e & 3).
+template <int V>
+LQ_DEV void rotate_tile(const _Float16* Rs, const float (&d)[V / 16][4], lq_v4f (&out)[V / 16], int rl, int kg) {
+  constexpr int RS = V + 8;
+  lq_v8h bop[V / 32];
+#pragma unroll
+  for (int sg = 0; sg < V / 32; ++sg)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) bop[sg][e] = (_Float16)d[2 * sg + (e >> 2)][e & 3];
+#pragma unroll
+  for (int vt = 0; vt < V / 16; ++vt) {
+    lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sg = 0; sg < V / 32; ++sg) {
+      const lq_v4h a0 = *(const lq_v4h*)(Rs + (16 * vt + rl) * RS + 32 * sg + 4 * kg);
+      const lq_v4h a1 = *(const lq_v4h*)(Rs + (16 * vt + rl) * RS + 32 * sg + 16 + 4 * kg);
+      lq_v8h aop;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        aop[e] = a0[e];
+        aop[4 + e] = a1[e];
+      }
+      acc = lq_mfma_f16(aop, bop[sg], acc);
+    }
+    out[vt] = acc;
+  }
+}
+
+// Rs[m][n] = R[n][m] (transposed copy, lanes walk m) or Rs[m][n] = R[m][n]
+template <int V, bool TRANSPOSE>
+LQ_DEV void stage_rotation(_Float16* Rs, const _Float16* R, int tid) {
+  constexpr int RS = V + 8;
+  for (int it = tid; it < V * (V / 8); it += 256) {
+    if (TRANSPOSE) {
+      const int m = it % V, n8 = it / V;
+      lq_v8h rv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) rv[e] = R[(8 * n8 + e) * V + m];
+      *(lq_v8h*)(Rs + m * RS + 8 * n8) = rv;
+    } else {
+      const int m = it / (V / 8), n8 = it % (V / 8);
+      *(lq_v8h*)(Rs + m * RS + 8 * n8) = *(const lq_v8h*)(R + m * V + 8 * n8);
+    }
+  }
+}
+
+template <bool DELTA, int K, int V>
+struct UStepOps {
+  lq_v4i kop[K / 64];
+  float gam[K / 64];
+  lq_v4i vop[DELTA ? 1 : V / 16];
+  lq_v4i wop[DELTA ? K / 64 : 1];
+  lq_v2i u[DELTA ? V / 16 : 1];
+  float fw, ev;
+};
+
+template <bool DELTA, int K, int V>
+__global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) {
+  constexpr int KR = K / 4, KT = KR / 16, VT = V / 16;
+  constexpr int HS = K + 16, ES = 64 + 16, RS = V + 8;
+  __shared__ __align__(16) unsigned char hT[V * HS];
+  __shared__ __align__(16) unsigned char eT[DELTA ? V * ES : 16];
+  __shared__ __align__(16) _Float16 RuT_s[V * RS];          // RuT_s[v'][v] = Ru[v][v']: x . Ru
+  __shared__ __align__(16) _Float16 Ru_s[DELTA ? V * RS : 8];  // Ru_s[v'][v] = Ru[v'][v]: x . Ru^T
+  __shared__ __align__(16) float ss_s[V], inv_ss_s[V], svw_s[V], inv_svw_s[V];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
+  const int b = blockIdx.x / p.H, h = blockIdx.x % p.H;
+  const int H = p.H, T = p.T, NT = p.NT;
+  const int qmax = p.qmax;
+
+  stage_rotation<V, true>(RuT_s, p.unrot, tid);
+  if (DELTA) stage_rotation<V, false>(Ru_s, p.unrot, tid);
+  if (tid < V) {
+    const float s = p.ss[h * V + tid], w = p.svw[h * V + tid];
+    ss_s[tid] = s, inv_ss_s[tid] = 1.0f / s, svw_s[tid] = w, inv_svw_s[tid] = 1.0f / w;
+  }
+  float skw_c[KT];
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt) skw_c[kt] = p.skw[h * K + KR * wave + 16 * kt + rl];
+  const float sw = DELTA ? p.sw[h] : 0.0f;
+
+  auto load_step = [&](int ct, UStepOps<DELTA, K, V>& o) {
+    const int64_t cb = ((int64_t)b * NT + ct) * H + h;
+    const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + KR * wave + 16 * kt + rl) * 64 + 16 * kg);
+      o.gam[kt] = p.gam[cb * K + KR * wave + 16 * kt + rl];
+    }
+    if constexpr (!DELTA) {
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) o.vop[vt] = *(const lq_v4i*)(p.vqT + (cb * V + 16 * vt + rl) * 64 + 16 * kg);
+    } else {
+      const int64_t tr = (t0 + 16 * wave + rl) * H + h;
+#pragma unroll
+      for (int ks = 0; ks < K / 64; ++ks) o.wop[ks] = *(const lq_v4i*)(p.wq + tr * K + 64 * ks + 16 * kg);
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) o.u[vt] = *(const lq_v2i*)(p.u + tr * V + 16 * vt + 4 * kg);
+      o.fw = p.fw[tr];
+      o.ev = p.ev[tr];
+    }
+  };
+
+  // carry, transposed: rows v = 16vt + 4kg + r, column k = KR*wave + 16kt + rl
+  float hc[VT][KT][4];
+#pragma unroll
+  for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) hc[vt][kt][r] = 0.0f;
+
+  UStepOps<DELTA, K, V> cur, nxt;
+  load_step(0, cur);
+  nxt = cur;
+  __syncthreads();
+
+  for (int ct = 0; ct < NT; ++ct) {
+    const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
+    // ---- stored copy of the incoming state -> LDS (V-major), one byte per (v, k)
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) {
+      const lq_v4f is4 = *(const lq_v4f*)(inv_ss_s + 16 * vt + 4 * kg);
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          hT[(16 * vt + 4 * kg + r) * HS + KR * wave + 16 * kt + rl] = (unsigned char)zoo_q8(hc[vt][kt][r], is4[r], 127);
+    }
+    if (ct + 1 < NT) load_step(ct + 1, nxt);
+    __syncthreads();
+    {
+      int8_t* dst = p.h_i8 + (((int64_t)b * NT + ct) * H + h) * V * K;
+      constexpr int SEG = K / 16;
+      for (int it = tid; it < V * SEG; it += 256) {
+        const int vr = it / SEG, sg = it % SEG;
+        *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hT + vr * HS + sg * 16);
+      }
+    }
+
+    if constexpr (DELTA) {
+      // ---- state read (transposed: rows v, columns = the wave's 16 tokens), rotated into the value basis of U
+      float ws[VT][4];
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        lq_v4i acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < K / 64; ++ks)
+          acc = lq_mfma_i8(*(const lq_v4i*)(hT + (16 * vt + rl) * HS + 64 * ks + 16 * kg), cur.wop[ks], acc);
+        const lq_v4f s4 = *(const lq_v4f*)(ss_s + 16 * vt + 4 * kg);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float x = (float)acc[r] * sw;
+          ws[vt][r] = x * s4[r];
+        }
+      }
+      lq_v4f wsr[VT];
+      rotate_tile<V>(Ru_s, ws, wsr, rl, kg);
+      const int64_t eoff = ((t0 + 16 * wave + rl) * H + h) * V;
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        const lq_v4f iw4 = *(const lq_v4f*)(inv_svw_s + 16 * vt + 4 * kg);
+        float ef[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float u = (float)zoo_half_of((uint32_t)cur.u[vt][r >> 1], r & 1);
+          ef[r] = (u - wsr[vt][r]) * cur.fw;
+          eT[(16 * vt + 4 * kg + r) * ES + 16 * wave + rl] = (unsigned char)zoo_q8(ef[r] * cur.ev, iw4[r], qmax);
+        }
+        lq_v2i eo;
+        eo[0] = (int)zoo_pack_h2(ef[0], ef[1]);
+        eo[1] = (int)zoo_pack_h2(ef[2], ef[3]);
+        *(lq_v2i*)(p.e_out + eoff + 16 * vt + 4 * kg) = eo;
+      }
+      __syncthreads();
+    }
+
+    // ---- write product (transposed), dequantized, un-rotated, added to the canonical carry
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      float d[VT][4];
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        lq_v4i aop;
+        if constexpr (DELTA)
+          aop = *(const lq_v4i*)(eT + (16 * vt + rl) * ES + 16 * kg);
+        else
+          aop = cur.vop[vt];
+        const lq_v4i a = lq_mfma_i8(aop, cur.kop[kt], lq_v4i{0, 0, 0, 0});
+        const lq_v4f w4 = *(const lq_v4f*)(svw_s + 16 * vt + 4 * kg);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float x = (float)a[r] * skw_c[kt];
+          d[vt][r] = x * w4[r];
+        }
+      }
+      lq_v4f rot[VT];
+      rotate_tile<V>(RuT_s, d, rot, rl, kg);
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) hc[vt][kt][r] = hc[vt][kt][r] * cur.gam[kt] + rot[vt][r];
+    }
+    cur = nxt;
+  }
+
+  if (p.ht) {
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+        *(lq_v4f*)(p.ht + (((int64_t)b * H + h) * K + KR * wave + 16 * kt + rl) * V + 16 * vt + 4 * kg) =
+            lq_v4f{hc[vt][kt][0], hc[vt][kt][1], hc[vt][kt][2], hc[vt][kt][3]};
+  }
+}
+
+constexpr int kAS = 72;  // halves per row of the fp16 A tile in LDS
+
+template <bool GLA, bool USE_G, int K, int V>
+__global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
+  constexpr int QS = K + 16, VT = V / 16, RS = V + 8, VW = V + 4;
+  __shared__ __align__(16) unsigned char qc[64 * QS];
+  __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
+  __shared__ __align__(16) _Float16 Afl[GLA ? 8 : 64 * kAS];
+  __shared__ __align__(16) uint32_t vP[32 * VW];
+  __shared__ __align__(16) _Float16 RuT_s[V * RS];
+  __shared__ __align__(16) float g_s[64], ss_s[V], svl_s[V];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
+  const int ct = blockIdx.x;
+  const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+  const int H = p.H;
+  const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
+  const float sq = p.sq[h];
+  const float inv_sq = 1.0f / sq;
+  const float sk = GLA ? 1.0f : p.sk[h];
+  const float inv_sk = 1.0f / sk;
+  const int qmax = p.qmax;
+
+  // ---- phase 1: codes and tables -> LDS
+  stage_rotation<V, true>(RuT_s, p.unrot, tid);
+  if (tid < V) ss_s[tid] = p.ss[h * V + tid], svl_s[tid] = p.svl[h * V + tid];
+  for (int it = tid; it < 64 * (K / 8); it += 256) {
+    const int t = it / (K / 8), c8 = it % (K / 8);
+    const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
+    const lq_v8h qv = *(const lq_v8h*)(p.q + off);
+    int cq[8];
+    if (GLA) {
+      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float x = (float)qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+        x = x * p.scale;
+        cq[e] = zoo_q8(x, inv_sq, qmax);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8((float)qv[e] * p.scale, inv_sq, qmax);
+    }
+    lq_v2i o;
+    o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
+    o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
+    *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
+    if (!GLA) {
+      const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+      int ck[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8((float)kv[e], inv_sk, qmax);
+      o[0] = (int)zoo_pack_codes(ck[0], ck[1], ck[2], ck[3]);
+      o[1] = (int)zoo_pack_codes(ck[4], ck[5], ck[6], ck[7]);
+      *(lq_v2i*)(kc + t * QS + 8 * c8) = o;
+    }
+  }
+  for (int it = tid; it < 32 * (V / 8); it += 256) {
+    const int tp = it / (V / 8), c8 = it % (V / 8);  // token pair, group of 8 value channels
+    const int64_t off = ((t0 + 2 * tp) * H + h) * V + 8 * c8;
+    const lq_v8h va = *(const lq_v8h*)(p.v + off);
+    const lq_v8h vb = *(const lq_v8h*)(p.v + off + (int64_t)H * V);
+    lq_v4i o0, o1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float inv = 1.0f / p.svl[h * V + 8 * c8 + e];
+      const int w = (int)zoo_pack_h2((float)zoo_q8((float)va[e], inv, qmax), (float)zoo_q8((float)vb[e], inv, qmax));
+      if (e < 4) o0[e] = w; else o1[e - 4] = w;
+    }
+    *(lq_v4i*)(vP + tp * VW + 8 * c8) = o0;
+    *(lq_v4i*)(vP + tp * VW + 8 * c8 + 4) = o1;
+  }
+  if (USE_G && !GLA && tid < 64) g_s[tid] = p.g[(t0 + tid) * H + h];
+  __syncthreads();
+
+  // ---- phase 2: INT8 contractions of this wave's 16 tokens (state read transposed: rows v, columns tokens)
+  lq_v4i o32[VT];
+#pragma unroll
+  for (int vt = 0; vt < VT; ++vt) o32[vt] = lq_v4i{0, 0, 0, 0};
+  lq_v4i a32[4];
+#pragma unroll
+  for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
+  const int8_t* hp = p.h_i8 + (((int64_t)b * p.NT + ct) * H + h) * V * K;
+#pragma unroll
+  for (int ks = 0; ks < K / 64; ++ks) {
+    const lq_v4i qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt)
+      o32[vt] = lq_mfma_i8(*(const lq_v4i*)(hp + (16 * vt + rl) * K + 64 * ks + 16 * kg), qop, o32[vt]);
+    if (!GLA) {
+#pragma unroll
+      for (int jt = 0; jt < 4; ++jt) {
+        if (jt > wave) continue;
+        const lq_v4i kop = *(const lq_v4i*)(kc + (16 * jt + rl) * QS + 64 * ks + 16 * kg);
+        a32[jt] = lq_mfma_i8(qop, kop, a32[jt]);
+      }
+    }
+  }
+
+  // ---- phase 3: A -> fp16 in operand layout
+  if (!GLA) {
+    const float sqk = sq * sk;
+#pragma unroll
+    for (int jt = 0; jt < 4; ++jt) {
+      if (jt > wave + 1) continue;
+      const int j = 16 * jt + rl;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * wave + 4 * kg + r;
+        float x = 0.0f;
+        if (jt <= wave && j <= i) {
+          x = (float)a32[jt][r] * sqk;
+          if (USE_G) x = x * zoo_exp(g_s[i] - g_s[j]);
+        }
+        Afl[i * kAS + j] = (_Float16)x;
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- phase 4: local product (transposed), scaled, un-rotated; output = state read + rotated local product
+  float d[VT][4];
+  {
+    lq_v4f loc[VT];
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) loc[vt] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+    const int nslab = (16 * wave + 15) / 32 + 1;
+    for (int js = 0; js < nslab; ++js) {
+      lq_v8h aop;
+      if (GLA) {
+        const float* ap = p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg;
+        const lq_v4f x0 = *(const lq_v4f*)ap, x1 = *(const lq_v4f*)(ap + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          aop[e] = (_Float16)x0[e];
+          aop[4 + e] = (_Float16)x1[e];
+        }
+      } else {
+        aop = *(const lq_v8h*)(Afl + (16 * wave + rl) * kAS + 32 * js + 8 * kg);
+      }
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) {
+        lq_v4i vv;
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) vv[dd] = (int)vP[(16 * js + 4 * kg + dd) * VW + 16 * vt + rl];
+        loc[vt] = lq_mfma_f16(__builtin_bit_cast(lq_v8h, vv), aop, loc[vt]);
+      }
+    }
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) {
+      const lq_v4f s4 = *(const lq_v4f*)(svl_s + 16 * vt + 4 * kg);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) d[vt][r] = loc[vt][r] * s4[r];
+    }
+  }
+  lq_v4f rot[VT];
+  rotate_tile<V>(RuT_s, d, rot, rl, kg);
+  const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + rl]) : 1.0f;
+  const int64_t ooff = ((t0 + 16 * wave + rl) * H + h) * V;
+#pragma unroll
+  for (int vt = 0; vt < VT; ++vt) {
+    const lq_v4f s4 = *(const lq_v4f*)(ss_s + 16 * vt + 4 * kg);
+    float res[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = (float)o32[vt][r] * sq;
+      x = x * s4[r];
+      if (USE_G && !GLA) x = x * eg;
+      res[r] = x + rot[vt][r];
+    }
+    if (p.o_is_f32) {
+      *(lq_v4f*)((float*)p.o + ooff + 16 * vt + 4 * kg) = lq_v4f{res[0], res[1], res[2], res[3]};
+    } else {
+      lq_v2i w;
+      w[0] = (int)zoo_pack_h2(res[0], res[1]);
+      w[1] = (int)zoo_pack_h2(res[2], res[3]);
+      *(lq_v2i*)((_Float16*)p.o + ooff + 16 * vt + 4 * kg) = w;
+    }
+  }
+}
+
+template <bool DELTA, int K>
+int launch_state(const ZooStateParams& p, int batch, hipStream_t stream) {
+  dim3 grid(batch * p.H);
+  if (p.V == 128)
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64>), grid, dim3(256), 0, stream, p);
+  return lq_check_launch();
+}
+
+template <bool GLA, bool USE_G, int K>
+int launch_output(const ZooOutParams& p, hipStream_t stream) {
+  dim3 grid(p.NT, p.B * p.H);
+  if (p.V == 128)
+    hipLaunchKernelGGL((zoo_output_unrot_kernel<GLA, USE_G, K, 128>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_output_unrot_kernel<GLA, USE_G, K, 64>), grid, dim3(256), 0, stream, p);
+  return lq_check_launch();
+}
+
+}  // namespace
+
+int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, hipStream_t stream) {
+  if (p.V != 64 && p.V != 128) return LQ_ERR_SHAPE;
+  if (delta) return K == 128 ? launch_state<true, 128>(p, batch, stream) : launch_state<true, 64>(p, batch, stream);
+  return K == 128 ? launch_state<false, 128>(p, batch, stream) : launch_state<false, 64>(p, batch, stream);
+}
+
+int zoo_output_unrot_launch(const ZooOutParams& p, int decay, int K, hipStream_t stream) {
+  if (p.V != 64 && p.V != 128) return LQ_ERR_SHAPE;
+  if (decay == LQ_DECAY_DIAGONAL)
+    return K == 128 ? launch_output<true, true, 128>(p, stream) : launch_output<true, true, 64>(p, stream);
+  if (decay == LQ_DECAY_SCALAR)
+    return K == 128 ? launch_output<false, true, 128>(p, stream) : launch_output<false, true, 64>(p, stream);
+  return K == 128 ? launch_output<false, false, 128>(p, stream) : launch_output<false, false, 64>(p, stream);
+}

@@ -28,12 +28,13 @@ def f32(t):
     return t if (t.dtype == torch.float32 and t.is_contiguous()) else t.float().contiguous()
 
 
-def no_rotation(**named):
-    for name, val in named.items():
-        if val is not None:
-            raise NotImplementedError(
-                f"{name}: in-kernel rotation / canonical storage is not built in the HIP zoo kernels yet; "
-                "rotate the operands outside and use rotated storage (out_dtype=torch.float32 + exit un-rotation)")
+def unrot_matrix(unrot, V):
+    """(V,V) fp16 R_V^T of canonical storage (v arrives rotated, the state and the output come out canonical)."""
+    if unrot is None:
+        return None
+    assert V in (64, 128), "canonical storage needs one V-tile spanning all value channels"
+    assert tuple(unrot.shape) == (V, V)
+    return unrot.to(torch.float16).contiguous()
 
 
 def cumsum(g, B, T, H, kdim):
@@ -64,29 +65,29 @@ def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family,
     return c
 
 
-def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile=0):
+def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile=0, unrot=None):
     """Sequential chunk recurrence over the pre-quantized operands ``c`` (see write_codes)."""
     B, T, H, K, V = dims
     delta = family == FAMILY_DELTA
     _lib.call("lq_zoo_state", h_i8.device, kqT=_lib.ptr(c["kqT"]), vqT=_lib.ptr(c["vqT"]), wq=_lib.ptr(c["wq"]),
               u=_lib.ptr(value) if delta else None, fw=_lib.ptr(fw), ev=_lib.ptr(c["ev"]) if delta else None,
               gam=_lib.ptr(c["gam"]), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
-              svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=None, qmax=int(qmax), batch=B, seqlen=T, nheads=H,
+              svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), qmax=int(qmax), batch=B, seqlen=T, nheads=H,
               kdim=K, vdim=V, chunk_size=CHUNK, family=family, vtile=int(vtile))
 
 
 def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
-              sw=None, vtile=0):
+              sw=None, vtile=0, unrot=None):
     """``value`` is v (linear family) or U (delta family)."""
     c = write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay)
-    state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile)
+    state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile, unrot)
 
 
-def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay):
+def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None):
     B, T, H, K, V = dims
     _lib.call("lq_zoo_output", q.device, q=_lib.ptr(q), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
               g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
-              sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=None, scale=float(scale), qmax=int(qmax),
+              sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),
               batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay)
 
 

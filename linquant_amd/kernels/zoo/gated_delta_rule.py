@@ -20,7 +20,7 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
     assert beta.shape == (B, T, H)
-    C.no_rotation(unrot=unrot)
+    Ru = C.unrot_matrix(unrot, V)
     scale = K ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     decay = C.DECAY_NONE if g is None else C.DECAY_SCALAR
@@ -36,7 +36,7 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
     C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
-                w=W, fw=fw, e_out=e_out, sw=sc["w"])
-    C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay)
+                w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru)
+    C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
     C.export_debug(_debug, h_i8, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return o, ht

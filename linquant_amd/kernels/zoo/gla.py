@@ -21,7 +21,7 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
     assert chunk_size % BC == 0 and g.shape == (B, T, H, K)
-    C.no_rotation(unrot=unrot)
+    Ru = C.unrot_matrix(unrot, V)
     R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
@@ -34,7 +34,7 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
     C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
-                C.DECAY_DIAGONAL)
-    C.run_output(q, None, v, h_i8, gc, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL)
+                C.DECAY_DIAGONAL, unrot=Ru)
+    C.run_output(q, None, v, h_i8, gc, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL, unrot=Ru)
     C.export_debug(_debug, h_i8, A=A, g=gc, logenv=logenv)
     return o, ht

@@ -20,7 +20,7 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
     assert chunk_size % BC == 0 and g.shape == (B, T, H, K) and beta.shape == (B, T, H)
-    C.no_rotation(unrot=unrot)
+    Ru = C.unrot_matrix(unrot, V)
     R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
@@ -35,7 +35,7 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
     C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
-                C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"])
-    C.run_output(q, None, e_out, h_i8, gc, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL)
+                C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru)
+    C.run_output(q, None, e_out, h_i8, gc, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL, unrot=Ru)
     C.export_debug(_debug, h_i8, A=A, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return o, ht

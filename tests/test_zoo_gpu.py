@@ -17,9 +17,13 @@ pytestmark = pytest.mark.gpu
 DEFAULT_ETA = {"linear_none": 1.0, "mamba2": 1.0, "gla": 0.0, "deltanet": 1.0, "gated_deltanet": 1.0, "kda": 0.0}
 
 
-def _go(cell, tensors, *, policy="kernel_static", bits=8, eta=None, rho=1.0, tau=1.0, label=None, rot=None, **kw):
+def _go(cell, tensors, *, policy="kernel_static", bits=8, eta=None, rho=1.0, tau=1.0, label=None, rot=None, rot_v=None, **kw):
     eta = DEFAULT_ETA[cell] if eta is None else eta
-    qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau, rot_qk=rot)
+    qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau, rot_qk=rot, rot_v=rot_v)
+    if rot_v is not None:  # the kernel receives the rotated value operand, materialized in the activation dtype
+        q_, k_, v_, g_, b_ = tensors
+        tensors = (q_, k_, (v_.double() @ rot_v).half(), g_, b_)
+        kw["unrot"] = rot_v.T.contiguous()
     if rot is not None:
         kw["rot"] = rot
     B, T, H, K = tensors[0].shape
@@ -96,6 +100,18 @@ def test_local_rqk_rotation(cuda, cell, n, K):
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))
+@pytest.mark.parametrize("n,K,V", [(128, 64, 128), (512, 64, 128), (256, 128, 64)])
+def test_canonical_storage_rv(cuda, cell, n, K, V):
+    """R_V with canonical storage: v rotated outside, every product un-rotated in-kernel before it joins the fp32
+    carry / the output (/root/reference tests/test_kernel_simple_gla.py:84-104, test_kernel_gla.py:63-75)."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell, K=K, V=V, H=2 if K == 128 else 4), n)
+    out, _, qz, run = _go(cell, tensors, eta=1.0, rot_v=signed_hadamard(V, 7))
+    zc.check(out, run, qz, f"{cell} canonical R_V T={n} K={K} V={V}")
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
 def test_stored_state_codes_and_final_state(cuda, cell):
     tensors = zc.cut(zc.inputs(cell, seed=4), 256)
     dbg = {}
@@ -131,5 +147,5 @@ def test_rejections(cuda):
     sc = {n: s.cuda() for n, s in sc.items()}
     with pytest.raises(AssertionError):
         zoo.chunk_simple_gla_int8(q[:, :100], k[:, :100], v[:, :100], g[:, :100], sc)
-    with pytest.raises(NotImplementedError):
-        zoo.chunk_simple_gla_int8(q, k, v, g, sc, unrot=torch.eye(128, device="cuda", dtype=torch.float16))
+    with pytest.raises(AssertionError):
+        zoo.chunk_simple_gla_int8(q, k, v, g, sc, unrot=torch.eye(64, device="cuda", dtype=torch.float16))

@@ -28,7 +28,7 @@ def cut(tensors, n):
     return [t[:, :n].contiguous() if t is not None else None for t in tensors]
 
 
-def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None):
+def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None):
     """Returns (qz, run): the oracle's quantizer with scales calibrated on these inputs, and a closure that
     evaluates the oracle (float32 result) under the quantizer's current arithmetic mode."""
     fam, dec = CELLS[cell]
@@ -38,7 +38,8 @@ def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.
 
     def run():
         return Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=qz, eta=eta, rho=rho,
-                               tau=tau, read_post=True, C=64, out_dtype=torch.float32, rot_qk=rot_qk)
+                               tau=tau, read_post=True, C=64, out_dtype=torch.float32, rot_qk=rot_qk, rot_v=rot_v,
+                               storage="canonical" if rot_v is not None else "rotated")
 
     qz.calibrating = True
     run()
@@ -47,7 +48,7 @@ def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.
 
 
 def run_kernel(cell, tensors, scales, *, eta=1.0, rho=1.0, tau=1.0, bits=8, out_dtype=None, final_state=False,
-               debug=None, device="cuda", rot=None):
+               debug=None, device="cuda", rot=None, unrot=None):
     from linquant_amd.kernels import zoo
 
     fam, dec = CELLS[cell]
@@ -58,6 +59,8 @@ def run_kernel(cell, tensors, scales, *, eta=1.0, rho=1.0, tau=1.0, bits=8, out_
               _debug=debug)
     if rot is not None:
         kw["rot"] = rot.to(device)
+    if unrot is not None:
+        kw["unrot"] = unrot.to(device)
     if fam == "linear":
         fn = zoo.chunk_gla_int8 if dec == "diagonal" else zoo.chunk_simple_gla_int8
         return fn(q, k, v, g, sc, **kw)
