@@ -36,6 +36,7 @@ typedef struct ihipStream_t* hipStream_t;
 #define LQ_DT_F16 0
 #define LQ_DT_F32 1
 #define LQ_DT_I8 2
+#define LQ_DT_BF16 3
 
 /* ABI version; bumped whenever a struct layout changes. */
 int lq_abi_version(void);
@@ -201,7 +202,7 @@ int lq_kron_hadamard(const lq_kron_hadamard_args* args, hipStream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Zoo chunk kernels: linear attention (no / scalar decay), GLA, DeltaNet / Gated DeltaNet, KDA.
- * q,k (B,T,H,K) and v (B,T,H,V) fp16 contiguous, T a multiple of the chunk size, K in {64,128},
+ * q,k (B,T,H,K) and v (B,T,H,V) fp16/bf16 contiguous, T a multiple of the chunk size, K in {64,128},
  * V a multiple of 64.  g holds the chunk-local cumulative log decay (lq_zoo_cumsum).  Scales are
  * fp32: q,k,w (H,), kw (H,K), vw,vl,el,ew,state (H,V).  h_i8 is the per-chunk INT8 stored state in
  * V-major layout (B,NT,H,V,K): an internal buffer shared by the state and output kernels.
@@ -230,9 +231,9 @@ int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
  * carried state is quantized once, in parallel over chunks, into the layout lq_zoo_state consumes.
  * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers. */
 typedef struct {
-  const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16 */
-  const void* val;           /* linear family: v (B,T,H,V) fp16; delta family: NULL */
-  const void* w;             /* delta family: W (B,T,H,K) fp16; linear family: NULL */
+  const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16/bf16 */
+  const void* val;           /* linear family: v (B,T,H,V) fp16/bf16; delta family: NULL */
+  const void* w;             /* delta family: W (B,T,H,K) fp16/bf16; linear family: NULL */
   const float* g;            /* cumulative log decay (B,T,H) / (B,T,H,K), or NULL for no decay */
   const float* logenv;       /* diagonal decay: (B,T,H) */
   int8_t* kqT;               /* (B,NT,H,K,64) int8 key write codes */
@@ -247,6 +248,7 @@ typedef struct {
   int32_t qmax;
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
   int32_t decay;
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
 } lq_zoo_write_codes_args;
 int lq_zoo_write_codes(const lq_zoo_write_codes_args* args, hipStream_t stream);
 
@@ -259,12 +261,12 @@ typedef struct {
   const int8_t* kqT;         /* (B,NT,H,K,64) */
   const int8_t* vqT;         /* linear family: (B,NT,H,V,64) */
   const int8_t* wq;          /* delta family: (B,T,H,K) */
-  const void* u;             /* delta family: U (B,T,H,V) fp16 */
+  const void* u;             /* delta family: U (B,T,H,V) fp16/bf16 */
   const float* fw;           /* delta family: (B,T,H) fp32 value-side share of the outer beta factor */
   const float* ev;           /* delta family: (B,T,H) */
   const float* gam;          /* (B,NT,H,K) */
   int8_t* h_i8;              /* (B,NT,H,V,K) int8 */
-  void* e_out;               /* delta family: (B,T,H,V) fp16 */
+  void* e_out;               /* delta family: (B,T,H,V) fp16/bf16 */
   float* ht;                 /* (B,H,K,V) fp32 final carry, or NULL */
   const float* skw;          /* (H,K) key write scale */
   const float* svw;          /* (H,V) value write scale: vw (linear) or ew (delta) */
@@ -275,6 +277,7 @@ typedef struct {
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
   int32_t family;
   int32_t vtile;             /* value columns per workgroup: 16, 32, 64, or 0 = chosen from the grid size */
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
 } lq_zoo_state_args;
 int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
 
@@ -282,13 +285,13 @@ int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
  * (gla.py:170-232): o = dequant(q8(q).h_i8) [* exp(g)] + (fp16(A) . fp16(q8(v))) * svl, with A computed
  * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay). */
 typedef struct {
-  const void* q;             /* (B,T,H,K) fp16 */
-  const void* k;             /* no / scalar decay: k or Hw (B,T,H,K) fp16; diagonal: NULL */
-  const void* v;             /* local value operand: v or e_out (B,T,H,V) fp16 */
+  const void* q;             /* (B,T,H,K) fp16/bf16 */
+  const void* k;             /* no / scalar decay: k or Hw (B,T,H,K) fp16/bf16; diagonal: NULL */
+  const void* v;             /* local value operand: v or e_out (B,T,H,V) fp16/bf16 */
   const int8_t* h_i8;        /* (B,NT,H,V,K) */
   const float* g;            /* cumulative log decay or NULL */
   const float* A;            /* diagonal decay: (B,T,H,C) fp32 lower-triangular intra-chunk product */
-  void* o;                   /* (B,T,H,V) fp16, or fp32 when o_is_f32 */
+  void* o;                   /* (B,T,H,V) fp16/bf16, or fp32 when o_is_f32 */
   int32_t o_is_f32;
   const float* sq;           /* (H,) */
   const float* sk;           /* (H,) (no / scalar decay) */
@@ -299,6 +302,7 @@ typedef struct {
   int32_t qmax;
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
   int32_t decay;
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
 } lq_zoo_output_args;
 int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
 
@@ -307,8 +311,8 @@ int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
  * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows, zeros above
  * the diagonal. */
 typedef struct {
-  const void* q;             /* (B,T,H,K) fp16 */
-  const void* k;             /* (B,T,H,K) fp16: k (GLA) or Hw (KDA) */
+  const void* q;             /* (B,T,H,K) fp16/bf16 */
+  const void* k;             /* (B,T,H,K) fp16/bf16: k (GLA) or Hw (KDA) */
   const float* g;            /* (B,T,H,K) cumulative log decay */
   float* A;                  /* (B,T,H,C) fp32 */
   const void* rot;           /* (K,K) fp16 local R_QK, or NULL */
@@ -317,6 +321,7 @@ typedef struct {
   float scale;
   int32_t qmax;
   int32_t batch, seqlen, nheads, kdim, chunk_size;
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
 } lq_zoo_gla_A_args;
 int lq_zoo_gla_A(const lq_zoo_gla_A_args* args, hipStream_t stream);
 
@@ -325,17 +330,18 @@ int lq_zoo_gla_A(const lq_zoo_gla_A_args* args, hipStream_t stream);
  * the same native prep): fp32 Gram with decay, unit-lower-triangular inverse, W = T.(L*exp(g)),
  * U = T.(beta^sigma v), Hw = beta^((1-sigma)tau) k, fw = beta^((1-sigma)(1-tau)). */
 typedef struct {
-  const void* k;             /* (B,T,H,K) fp16 */
-  const void* v;             /* (B,T,H,V) fp16 */
+  const void* k;             /* (B,T,H,K) fp16/bf16 */
+  const void* v;             /* (B,T,H,V) fp16/bf16 */
   const float* beta;         /* (B,T,H) fp32 */
   const float* g;            /* cumulative log decay (B,T,H) / (B,T,H,K) or NULL */
-  void* Hw;                  /* (B,T,H,K) fp16 */
-  void* W;                   /* (B,T,H,K) fp16 */
-  void* U;                   /* (B,T,H,V) fp16 */
+  void* Hw;                  /* (B,T,H,K) fp16/bf16 */
+  void* W;                   /* (B,T,H,K) fp16/bf16 */
+  void* U;                   /* (B,T,H,V) fp16/bf16 */
   float* fw;                 /* (B,T,H) fp32 */
   float sigma, tau;
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
   int32_t decay;
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
 } lq_zoo_wy_prep_args;
 int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
 

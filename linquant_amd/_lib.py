@@ -13,9 +13,9 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 HEADER = ROOT.parent / "include" / "linquant_hip.h"
 LIB_PATH = ROOT / "csrc" / "liblinquant_hip.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
-LQ_DT_F16, LQ_DT_F32, LQ_DT_I8 = 0, 1, 2
+LQ_DT_F16, LQ_DT_F32, LQ_DT_I8, LQ_DT_BF16 = 0, 1, 2, 3
 
 _CTYPES = {"int64_t": ctypes.c_int64, "int32_t": ctypes.c_int32, "float": ctypes.c_float, "int": ctypes.c_int}
 _ERRORS = {-14: "a required pointer is missing (LQ_E_NULL)",

@@ -41,3 +41,40 @@ static inline bool zoo_al(const void* q, int n) { return ((uintptr_t)q % n) == 0
 // exp on the hardware exp2 unit (x * log2(e), then v_exp_f32): the arithmetic tl.exp lowers to in the reference's
 // Triton kernels.  Large negative arguments give 0, never NaN.
 LQ_DEV float zoo_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
+// ---- activation dtype: q, k, v (and the prepared Hw, W, U, E) are fp16 or bf16; `bf` is uniform per launch.
+// Pointers are typed _Float16* for their 2-byte element stride only.
+LQ_DEV void zoo_dec2(uint32_t w, bool bf, float& lo, float& hi) {
+  if (bf) {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+  } else {
+    const lq_v2h h = __builtin_bit_cast(lq_v2h, w);
+    lo = (float)h[0];
+    hi = (float)h[1];
+  }
+}
+LQ_DEV float zoo_dec1(uint32_t bits16, bool bf) {
+  return bf ? __uint_as_float(bits16 << 16) : (float)__builtin_bit_cast(_Float16, (uint16_t)bits16);
+}
+LQ_DEV void zoo_ld8(const _Float16* p, bool bf, float (&o)[8]) {
+  const lq_v4i raw = *(const lq_v4i*)p;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) zoo_dec2((uint32_t)raw[d], bf, o[2 * d], o[2 * d + 1]);
+}
+LQ_DEV void zoo_ld4(const _Float16* p, bool bf, float (&o)[4]) {
+  const lq_v2i raw = *(const lq_v2i*)p;
+#pragma unroll
+  for (int d = 0; d < 2; ++d) zoo_dec2((uint32_t)raw[d], bf, o[2 * d], o[2 * d + 1]);
+}
+// round-to-nearest-even bf16 bits of a finite fp32 value
+LQ_DEV uint32_t zoo_bf16_bits(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+LQ_DEV uint32_t zoo_enc2(float a, float b, bool bf) {
+  return bf ? (zoo_bf16_bits(a) | (zoo_bf16_bits(b) << 16)) : zoo_pack_h2(a, b);
+}
+LQ_DEV uint16_t zoo_enc1(float a, bool bf) {
+  return bf ? (uint16_t)zoo_bf16_bits(a) : __builtin_bit_cast(uint16_t, (_Float16)a);
+}

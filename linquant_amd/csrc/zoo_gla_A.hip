@@ -29,6 +29,7 @@ struct AParams {
   const _Float16* rot;
   float scale;
   int qmax;
+  int bf;
   int B, T, H;
 };
 
@@ -49,6 +50,7 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
                        int i0) {
   constexpr int NCH = K / 4;
   const int H = p.H, qmax = p.qmax;
+  const bool bf = p.bf != 0;
   const int c0 = NCH * kg;
   const int64_t off = ((row0 + rl) * H + h) * K + c0;
   const int64_t aoff = (row0 * H + h) * K + c0;
@@ -69,13 +71,16 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
     float qa[NCH], ka[NCH];
 #pragma unroll
     for (int e8 = 0; e8 < NCH / 8; ++e8) {
-      const lq_v8h qv = *(const lq_v8h*)(p.q + off + 8 * e8), kv = *(const lq_v8h*)(p.k + off + 8 * e8);
+      float qv[8];
+      zoo_ld8(p.q + off + 8 * e8, bf, qv);
+      float kv[8];
+      zoo_ld8(p.k + off + 8 * e8, bf, kv);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int n = 8 * e8 + e;
         const float d = gv[n] - av[n];
-        const float qh = (float)zoo_q8((float)qv[e] * p.scale, inv_sq, qmax) * sq;
-        const float kh = (float)zoo_q8((float)kv[e], inv_sk, qmax) * sk;
+        const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
+        const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
         qa[n] = qh * zoo_exp(d);
         ka[n] = kh * zoo_exp(-d);
       }
@@ -93,18 +98,20 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
   float s[4] = {0.f, 0.f, 0.f, 0.f};
   const int64_t irow = ((row0 + rl) * H + h) * K;
   for (int n8 = 0; n8 < K; n8 += 8) {
-    const lq_v8h qv = *(const lq_v8h*)(p.q + irow + n8);
+    float qv[8];
+    zoo_ld8(p.q + irow + n8, bf, qv);
     const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const int j = 4 * kg + jj;
       const int64_t jrow = ((row0 + j) * H + h) * K;
-      const lq_v8h kv = *(const lq_v8h*)(p.k + jrow + n8);
+      float kv[8];
+      zoo_ld8(p.k + jrow + n8, bf, kv);
       const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float qh = (float)zoo_q8((float)qv[e] * p.scale, inv_sq, qmax) * sq;
-        const float kh = (float)zoo_q8((float)kv[e], inv_sk, qmax) * sk;
+        const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
+        const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
         const float gi = e < 4 ? gi0[e & 3] : gi1[e & 3], gj = e < 4 ? gj0[e & 3] : gj1[e & 3];
         const float w = (j <= rl) ? zoo_exp(gi - gj) : 0.0f;
         s[jj] = s[jj] + (qh * kh) * w;
@@ -131,6 +138,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
   const float sq = p.sq[h], sk = p.sk[h];
   const float inv_sq = 1.0f / sq, inv_sk = 1.0f / sk;
   const int qmax = p.qmax;
+  const bool bf = p.bf != 0;
   const int i0 = 16 * wave;
 
   if constexpr (ROT) {
@@ -169,7 +177,10 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
         lq_v4i qop;
         {
           const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
-          const lq_v8h q0 = *(const lq_v8h*)(p.q + off), q1 = *(const lq_v8h*)(p.q + off + 8);
+          float q0[8];
+          zoo_ld8(p.q + off, bf, q0);
+          float q1[8];
+          zoo_ld8(p.q + off + 8, bf, q1);
           int cd[16];
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
@@ -177,7 +188,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int n = 4 * e4 + e;
-              const float qf = n < 8 ? (float)q0[n & 7] : (float)q1[n & 7];
+              const float qf = n < 8 ? q0[n & 7] : q1[n & 7];
               float x = qf * zoo_exp(g4[e] - an[n]);
               x = x * p.scale;
               cd[n] = zoo_q8(x, inv_sq, qmax);
@@ -190,7 +201,10 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
         for (int J = 0; J < 3; ++J) {
           if (J >= wave) continue;
           const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
-          const lq_v8h k0 = *(const lq_v8h*)(p.k + off), k1 = *(const lq_v8h*)(p.k + off + 8);
+          float k0[8];
+          zoo_ld8(p.k + off, bf, k0);
+          float k1[8];
+          zoo_ld8(p.k + off + 8, bf, k1);
           int cd[16];
 #pragma unroll
           for (int e4 = 0; e4 < 4; ++e4) {
@@ -198,7 +212,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int n = 4 * e4 + e;
-              const float kf = n < 8 ? (float)k0[n & 7] : (float)k1[n & 7];
+              const float kf = n < 8 ? k0[n & 7] : k1[n & 7];
               cd[n] = zoo_q8(kf * zoo_exp(an[n] - g4[e]), inv_sk, qmax);
             }
           }
@@ -224,12 +238,13 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
         const lq_v4f a0 = *(const lq_v4f*)ap, a1 = *(const lq_v4f*)(ap + 4);
         {
           const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
-          const lq_v8h qv = *(const lq_v8h*)(p.q + off);
+          float qv[8];
+          zoo_ld8(p.q + off, bf, qv);
           const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            float x = (float)qv[e] * zoo_exp(gg - an);
+            float x = qv[e] * zoo_exp(gg - an);
             x = x * p.scale;
             xop[0][ks][e] = (_Float16)x;
           }
@@ -238,12 +253,13 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
         for (int J = 0; J < 3; ++J) {
           if (J >= wave) continue;
           const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
-          const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+          float kv[8];
+          zoo_ld8(p.k + off, bf, kv);
           const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            xop[1 + J][ks][e] = (_Float16)((float)kv[e] * zoo_exp(an - gg));
+            xop[1 + J][ks][e] = (_Float16)(kv[e] * zoo_exp(an - gg));
           }
         }
       }
@@ -312,12 +328,13 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if (a->kdim != 64 && a->kdim != 128) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
+  if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (!zoo_al(a->q, 16) || !zoo_al(a->k, 16) || !zoo_al(a->g, 16) || !zoo_al(a->A, 16)) return LQ_ERR_SHAPE;
   if (a->rot && !zoo_al(a->rot, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   AParams p = {};
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.g = a->g, p.A = a->A;
-  p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax;
+  p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);
   if (a->kdim == 128) {

@@ -45,34 +45,37 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   const float sk = GLA ? 1.0f : p.sk[h];
   const float inv_sk = 1.0f / sk;
   const int qmax = p.qmax;
+  const bool bf = p.bf != 0;
 
   // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
   for (int it = tid; it < 64 * (K / 8); it += 256) {
     const int t = it / (K / 8), c8 = it % (K / 8);
     const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
-    const lq_v8h qv = *(const lq_v8h*)(p.q + off);
+    float qv[8];
+    zoo_ld8(p.q + off, bf, qv);
     int cq[8];
     if (GLA) {
       const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float x = (float)qv[e] * lq_expf(e < 4 ? g0[e & 3] : g1[e & 3]);
+        float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
         x = x * p.scale;
         cq[e] = zoo_q8(x, inv_sq, qmax);
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8((float)qv[e] * p.scale, inv_sq, qmax);
+      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
     }
     lq_v2i o;
     o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
     o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
     *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
     if (!GLA) {
-      const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+      float kv[8];
+      zoo_ld8(p.k + off, bf, kv);
       int ck[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8((float)kv[e], inv_sk, qmax);
+      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8(kv[e], inv_sk, qmax);
       o[0] = (int)zoo_pack_codes(ck[0], ck[1], ck[2], ck[3]);
       o[1] = (int)zoo_pack_codes(ck[4], ck[5], ck[6], ck[7]);
       *(lq_v2i*)(kc + t * QS + 8 * c8) = o;
@@ -81,14 +84,16 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   {
     const int tp = tid >> 3, c8 = tid & 7;  // 32 token pairs x 8 groups of 8 channels
     const int64_t off = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8;
-    const lq_v8h va = *(const lq_v8h*)(p.v + off);
-    const lq_v8h vb = *(const lq_v8h*)(p.v + off + (int64_t)H * V);
+    float va[8];
+    zoo_ld8(p.v + off, bf, va);
+    float vb[8];
+    zoo_ld8(p.v + off + (int64_t)H * V, bf, vb);
     lq_v4i o0, o1;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float inv = 1.0f / p.svl[h * V + v0 + 8 * c8 + e];
-      const float ca = (float)zoo_q8((float)va[e], inv, qmax);
-      const float cb = (float)zoo_q8((float)vb[e], inv, qmax);
+      const float ca = (float)zoo_q8(va[e], inv, qmax);
+      const float cb = (float)zoo_q8(vb[e], inv, qmax);
       const int w = (int)zoo_pack_h2(ca, cb);
       if (e < 4) o0[e] = w; else o1[e - 4] = w;
     }
@@ -132,7 +137,7 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
     for (int jj = 0; jj < 4; ++jj) ssv[jj] = p.ss[h * V + v0 + 4 * rl + jj];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float eg = (USE_G && !GLA) ? __expf(g_s[16 * wave + 4 * kg + r]) : 1.0f;
+      const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + 4 * kg + r]) : 1.0f;
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         float x = (float)o32[jj][r] * sq;
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
         float x = 0.0f;
         if (jt <= wave && j <= i) {
           x = (float)a32[jt][r] * sqk;
-          if (USE_G) x = x * __expf(g_s[i] - g_s[j]);
+          if (USE_G) x = x * zoo_exp(g_s[i] - g_s[j]);
         }
         Afl[i * kAS + j] = (_Float16)x;
       }
@@ -202,8 +207,8 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
       *(lq_v4f*)((float*)p.o + off) = lq_v4f{res[0], res[1], res[2], res[3]};
     } else {
       lq_v2i w;
-      w[0] = (int)zoo_pack_h2(res[0], res[1]);
-      w[1] = (int)zoo_pack_h2(res[2], res[3]);
+      w[0] = (int)zoo_enc2(res[0], res[1], bf);
+      w[1] = (int)zoo_enc2(res[2], res[3], bf);
       *(lq_v2i*)((_Float16*)p.o + off) = w;
     }
   }
@@ -232,13 +237,14 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
+  if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (!zoo_al(a->q, 16) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16))
     return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535 || a->seqlen / 64 > 65535) return LQ_ERR_SHAPE;
   OutParams p = {};
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.v = (const _Float16*)a->v;
   p.h_i8 = a->h_i8, p.g = a->g, p.A = a->A, p.o = a->o, p.o_is_f32 = a->o_is_f32;
-  p.sq = a->sq, p.sk = a->sk, p.svl = a->svl, p.ss = a->ss, p.scale = a->scale, p.qmax = a->qmax;
+  p.sq = a->sq, p.sk = a->sk, p.svl = a->svl, p.ss = a->ss, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   p.unrot = (const _Float16*)a->unrot;
   if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);

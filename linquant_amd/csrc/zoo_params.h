@@ -21,6 +21,7 @@ struct ZooStateParams {
   const float* ss;
   const _Float16* unrot;
   int qmax;
+  int bf;  // activations are bf16
   int T, H, V, NT;
 };
 
@@ -40,6 +41,7 @@ struct ZooOutParams {
   const _Float16* unrot;
   float scale;
   int qmax;
+  int bf;  // activations (and a 16-bit output) are bf16
   int B, T, H, V, NT;
 };
 

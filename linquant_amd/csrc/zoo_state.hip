@@ -52,6 +52,7 @@ __global__ __launch_bounds__(256) void zoo_state_kernel(StateParams p) {
   const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
   const int H = p.H, V = p.V, T = p.T, NT = p.NT;
   const int qmax = p.qmax;
+  const bool bf = p.bf != 0;
 
   // per-lane scales of the carry tile: rows k = KR*wave + 16kt + 4kg + r, cols v = v0 + 16vt + rl
   float skw_r[KT][4], svw_c[VT], inv_ss_c[VT];
@@ -169,19 +170,19 @@ __global__ __launch_bounds__(256) void zoo_state_kernel(StateParams p) {
         for (int jj = 0; jj < NJ; ++jj) {
           float ws = (float)aw[jj][r] * sw;
           ws = ws * ss_d[jj];
-          const float u = (float)zoo_half_of(cur.u[r][jj >> 1], jj & 1);
+          const float u = zoo_dec1((cur.u[r][jj >> 1] >> (16 * (jj & 1))) & 0xffffu, bf);
           ef[jj] = (u - ws) * cur.fw[r];
           ecode[jj][r] = (uint32_t)zoo_q8(ef[jj] * cur.ev[r], inv_ew_d[jj], qmax);
         }
         if constexpr (NJ == 4) {
           lq_v2i eo;
-          eo[0] = (int)zoo_pack_h2(ef[0], ef[1]);
-          eo[1] = (int)zoo_pack_h2(ef[2], ef[3]);
+          eo[0] = (int)zoo_enc2(ef[0], ef[1], bf);
+          eo[1] = (int)zoo_enc2(ef[2], ef[3], bf);
           *(lq_v2i*)(p.e_out + off) = eo;
         } else if constexpr (NJ == 2) {
-          *(uint32_t*)(p.e_out + off) = zoo_pack_h2(ef[0], ef[1]);
+          *(uint32_t*)(p.e_out + off) = zoo_enc2(ef[0], ef[1], bf);
         } else {
-          p.e_out[off] = (_Float16)ef[0];
+          *(uint16_t*)(p.e_out + off) = zoo_enc1(ef[0], bf);
         }
       }
 #pragma unroll
@@ -249,6 +250,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
+  if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (a->vtile != 0 && a->vtile != 16 && a->vtile != 32 && a->vtile != 64) return LQ_ERR_SHAPE;
   if (!zoo_al(a->kqT, 16) || !zoo_al(a->gam, 16) || !zoo_al(a->h_i8, 16) || (!delta && !zoo_al(a->vqT, 16)) ||
       (delta && (!zoo_al(a->wq, 16) || !zoo_al(a->u, 8) || !zoo_al(a->e_out, 8))))
@@ -257,7 +259,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   StateParams p = {};
   p.kqT = a->kqT, p.vqT = a->vqT, p.wq = a->wq, p.u = (const _Float16*)a->u, p.fw = a->fw, p.ev = a->ev, p.gam = a->gam;
   p.h_i8 = a->h_i8, p.e_out = (_Float16*)a->e_out, p.ht = a->ht;
-  p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.ss = a->ss, p.qmax = a->qmax;
+  p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.ss = a->ss, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.unrot = (const _Float16*)a->unrot;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   if (a->unrot) return zoo_state_unrot_launch(p, delta, a->kdim, a->batch, stream);

@@ -87,6 +87,7 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
   const int b = blockIdx.x / p.H, h = blockIdx.x % p.H;
   const int H = p.H, T = p.T, NT = p.NT;
   const int qmax = p.qmax;
+  const bool bf = p.bf != 0;
 
   stage_rotation<V, true>(RuT_s, p.unrot, tid);
   if (DELTA) stage_rotation<V, false>(Ru_s, p.unrot, tid);
@@ -183,13 +184,13 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
         float ef[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float u = (float)zoo_half_of((uint32_t)cur.u[vt][r >> 1], r & 1);
+          const float u = zoo_dec1(((uint32_t)cur.u[vt][r >> 1] >> (16 * (r & 1))) & 0xffffu, bf);
           ef[r] = (u - wsr[vt][r]) * cur.fw;
           eT[(16 * vt + 4 * kg + r) * ES + 16 * wave + rl] = (unsigned char)zoo_q8(ef[r] * cur.ev, iw4[r], qmax);
         }
         lq_v2i eo;
-        eo[0] = (int)zoo_pack_h2(ef[0], ef[1]);
-        eo[1] = (int)zoo_pack_h2(ef[2], ef[3]);
+        eo[0] = (int)zoo_enc2(ef[0], ef[1], bf);
+        eo[1] = (int)zoo_enc2(ef[2], ef[3], bf);
         *(lq_v2i*)(p.e_out + eoff + 16 * vt + 4 * kg) = eo;
       }
       __syncthreads();
@@ -257,6 +258,7 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
   const float sk = GLA ? 1.0f : p.sk[h];
   const float inv_sk = 1.0f / sk;
   const int qmax = p.qmax;
+  const bool bf = p.bf != 0;
 
   // ---- phase 1: codes and tables -> LDS
   stage_rotation<V, true>(RuT_s, p.unrot, tid);
@@ -264,29 +266,31 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
   for (int it = tid; it < 64 * (K / 8); it += 256) {
     const int t = it / (K / 8), c8 = it % (K / 8);
     const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
-    const lq_v8h qv = *(const lq_v8h*)(p.q + off);
+    float qv[8];
+    zoo_ld8(p.q + off, bf, qv);
     int cq[8];
     if (GLA) {
       const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float x = (float)qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+        float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
         x = x * p.scale;
         cq[e] = zoo_q8(x, inv_sq, qmax);
       }
     } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8((float)qv[e] * p.scale, inv_sq, qmax);
+      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
     }
     lq_v2i o;
     o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
     o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
     *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
     if (!GLA) {
-      const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+      float kv[8];
+      zoo_ld8(p.k + off, bf, kv);
       int ck[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8((float)kv[e], inv_sk, qmax);
+      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8(kv[e], inv_sk, qmax);
       o[0] = (int)zoo_pack_codes(ck[0], ck[1], ck[2], ck[3]);
       o[1] = (int)zoo_pack_codes(ck[4], ck[5], ck[6], ck[7]);
       *(lq_v2i*)(kc + t * QS + 8 * c8) = o;
@@ -295,13 +299,15 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
   for (int it = tid; it < 32 * (V / 8); it += 256) {
     const int tp = it / (V / 8), c8 = it % (V / 8);  // token pair, group of 8 value channels
     const int64_t off = ((t0 + 2 * tp) * H + h) * V + 8 * c8;
-    const lq_v8h va = *(const lq_v8h*)(p.v + off);
-    const lq_v8h vb = *(const lq_v8h*)(p.v + off + (int64_t)H * V);
+    float va[8];
+    zoo_ld8(p.v + off, bf, va);
+    float vb[8];
+    zoo_ld8(p.v + off + (int64_t)H * V, bf, vb);
     lq_v4i o0, o1;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float inv = 1.0f / p.svl[h * V + 8 * c8 + e];
-      const int w = (int)zoo_pack_h2((float)zoo_q8((float)va[e], inv, qmax), (float)zoo_q8((float)vb[e], inv, qmax));
+      const int w = (int)zoo_pack_h2((float)zoo_q8(va[e], inv, qmax), (float)zoo_q8(vb[e], inv, qmax));
       if (e < 4) o0[e] = w; else o1[e - 4] = w;
     }
     *(lq_v4i*)(vP + tp * VW + 8 * c8) = o0;
@@ -409,8 +415,8 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
       *(lq_v4f*)((float*)p.o + ooff + 16 * vt + 4 * kg) = lq_v4f{res[0], res[1], res[2], res[3]};
     } else {
       lq_v2i w;
-      w[0] = (int)zoo_pack_h2(res[0], res[1]);
-      w[1] = (int)zoo_pack_h2(res[2], res[3]);
+      w[0] = (int)zoo_enc2(res[0], res[1], bf);
+      w[1] = (int)zoo_enc2(res[2], res[3], bf);
       *(lq_v2i*)((_Float16*)p.o + ooff + 16 * vt + 4 * kg) = w;
     }
   }

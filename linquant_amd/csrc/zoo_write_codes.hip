@@ -31,6 +31,7 @@ struct CodesParams {
   const float* sw;
   float eta;
   int qmax;
+  int bf;
   int T, H, V, NT;
 };
 
@@ -49,6 +50,7 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   const int64_t cb = ((int64_t)b * p.NT + ct) * H + h;  // (batch, chunk, head) index
   const float eta = p.eta;
   const int qmax = p.qmax;
+  const bool bf = p.bf != 0;
 
   if (tid < 64) {
     float ekv = 1.0f, evv = 1.0f;
@@ -86,15 +88,10 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
       const int tl = 4 * tq + t;
       const int64_t off = ((t0 + tl) * H + h) * K + CK * cg;
       float kv[CK];
-      if constexpr (CK == 8) {
-        const lq_v8h v8 = *(const lq_v8h*)(p.key + off);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) kv[e] = (float)v8[e];
-      } else {
-        const lq_v4h v4 = *(const lq_v4h*)(p.key + off);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) kv[e] = (float)v4[e];
-      }
+      if constexpr (CK == 8)
+        zoo_ld8(p.key + off, bf, kv);
+      else
+        zoo_ld4(p.key + off, bf, kv);
       if (DECAY == LQ_DECAY_SCALAR) {
         const float f = ek_s[tl];
 #pragma unroll
@@ -110,18 +107,19 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
       for (int e = 0; e < CK; ++e) kcode[e][t] = (uint32_t)zoo_q8(kv[e], inv_skw[e], qmax);
       if (p.w) {
         int wc[CK];
+        float wv[CK];
         if constexpr (CK == 8) {
-          const lq_v8h v8 = *(const lq_v8h*)(p.w + off);
+          zoo_ld8(p.w + off, bf, wv);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) wc[e] = zoo_q8((float)v8[e], inv_sw, qmax);
+          for (int e = 0; e < 8; ++e) wc[e] = zoo_q8(wv[e], inv_sw, qmax);
           lq_v2i o;
           o[0] = (int)zoo_pack_codes(wc[0], wc[1], wc[2], wc[3]);
           o[1] = (int)zoo_pack_codes(wc[4], wc[5], wc[6], wc[7]);
           *(lq_v2i*)(p.wq + off) = o;
         } else {
-          const lq_v4h v4 = *(const lq_v4h*)(p.w + off);
+          zoo_ld4(p.w + off, bf, wv);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) wc[e] = zoo_q8((float)v4[e], inv_sw, qmax);
+          for (int e = 0; e < 4; ++e) wc[e] = zoo_q8(wv[e], inv_sw, qmax);
           *(uint32_t*)(p.wq + off) = zoo_pack_codes(wc[0], wc[1], wc[2], wc[3]);
         }
       }
@@ -146,11 +144,12 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
       uint32_t vcode[4][4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const lq_v4h v4 = *(const lq_v4h*)(p.val + ((t0 + 4 * tq + t) * H + h) * V + vc + 4 * cg);
+        float v4[4];
+        zoo_ld4(p.val + ((t0 + 4 * tq + t) * H + h) * V + vc + 4 * cg, bf, v4);
         const float f = ev_s[4 * tq + t];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float x = (DECAY == LQ_DECAY_NONE) ? (float)v4[e] : (float)v4[e] * f;
+          const float x = (DECAY == LQ_DECAY_NONE) ? v4[e] : v4[e] * f;
           vcode[e][t] = (uint32_t)zoo_q8(x, inv_svw[e], qmax);
         }
       }
@@ -189,6 +188,7 @@ extern "C" int lq_zoo_write_codes(const lq_zoo_write_codes_args* a, hipStream_t 
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
+  if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (!zoo_al(a->key, 16) || !zoo_al(a->kqT, 16) || (a->val && (!zoo_al(a->val, 8) || !zoo_al(a->vqT, 16))) ||
       (a->w && (!zoo_al(a->w, 16) || !zoo_al(a->wq, 8))) || (a->g && !zoo_al(a->g, 16)))
     return LQ_ERR_SHAPE;
@@ -196,7 +196,7 @@ extern "C" int lq_zoo_write_codes(const lq_zoo_write_codes_args* a, hipStream_t 
   CodesParams p = {};
   p.key = (const _Float16*)a->key, p.val = (const _Float16*)a->val, p.w = (const _Float16*)a->w;
   p.g = a->g, p.logenv = a->logenv, p.kqT = a->kqT, p.vqT = a->vqT, p.wq = a->wq, p.ev = a->ev, p.gam = a->gam;
-  p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.eta = a->eta, p.qmax = a->qmax;
+  p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.eta = a->eta, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   dim3 grid(p.NT, a->batch * a->nheads);
   return a->kdim == 128 ? launch<128>(p, a->decay, grid, stream) : launch<64>(p, a->decay, grid, stream);

@@ -31,6 +31,7 @@ struct WyParams {
   _Float16* U;
   float* fw;
   float sigma, tau;
+  int bf;
   int B, T, H, V;
 };
 
@@ -78,6 +79,7 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
   const float sigma = p.sigma, tau = p.tau;
+  const bool bf = p.bf != 0;
 
   // ---- per-token factors; Hw and fw are written straight out; X = beta^sigma k exp(g) staged for the W product
   if (tid < 64) {
@@ -90,7 +92,8 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
   for (int it = tid; it < 64 * (K / 8); it += 256) {
     const int r = it / (K / 8), c8 = it % (K / 8);
     const int64_t off = ((t0 + r) * H + h) * K + 8 * c8;
-    const lq_v8h kv = *(const lq_v8h*)(p.k + off);
+    float kv[8];
+    zoo_ld8(p.k + off, bf, kv);
     const float bt = p.beta[(t0 + r) * H + h];
     const float bw = powb(bt, (1.0f - sigma) * tau);
     float bl = powb(bt, sigma);
@@ -101,17 +104,22 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
     }
-    lq_v8h hw;
+    float hw[8];
     lq_v4f x0, x1;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float kf = (float)kv[e];
+      const float kf = kv[e];
       float x = bl * kf;
       if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
       if (e < 4) x0[e] = x; else x1[e - 4] = x;
-      hw[e] = (_Float16)(bw * kf);
+      hw[e] = bw * kf;
     }
-    *(lq_v8h*)(p.Hw + off) = hw;
+    {
+      lq_v4i o;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+      *(lq_v4i*)(p.Hw + off) = o;
+    }
     *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
     *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
   }
@@ -143,7 +151,10 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
       const int c0 = 64 * ps + 16 * kg;
       float Lr[16], gi[16], an[16];
       {
-        const lq_v8h k0 = *(const lq_v8h*)(p.k + irow + c0), k1 = *(const lq_v8h*)(p.k + irow + c0 + 8);
+        float k0[8];
+        zoo_ld8(p.k + irow + c0, bf, k0);
+        float k1[8];
+        zoo_ld8(p.k + irow + c0 + 8, bf, k1);
 #pragma unroll
         for (int e = 0; e < 16; ++e) Lr[e] = bs_i * (float)(e < 8 ? k0[e & 7] : k1[e & 7]);
         if (DECAY == LQ_DECAY_DIAGONAL) {
@@ -166,7 +177,10 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
         if (DECAY == LQ_DECAY_DIAGONAL && J == I && exact_diag) continue;
         const int64_t jrow = ((t0 + 16 * J + rl) * H + h) * K;
         const float bh_j = bh_s[16 * J + rl];
-        const lq_v8h k0 = *(const lq_v8h*)(p.k + jrow + c0), k1 = *(const lq_v8h*)(p.k + jrow + c0 + 8);
+        float k0[8];
+        zoo_ld8(p.k + jrow + c0, bf, k0);
+        float k1[8];
+        zoo_ld8(p.k + jrow + c0 + 8, bf, k1);
         float Hr[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) Hr[e] = bh_j * (float)(e < 8 ? k0[e & 7] : k1[e & 7]);
@@ -202,20 +216,22 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
       // lane (i = rl, j = 4kg + jj) of the diagonal block, one exponential per (i, j, channel)
       float sacc[4] = {0.f, 0.f, 0.f, 0.f};
       for (int n8 = 0; n8 < K; n8 += 8) {
-        const lq_v8h ki = *(const lq_v8h*)(p.k + irow + n8);
+        float ki[8];
+        zoo_ld8(p.k + irow + n8, bf, ki);
         const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
           const int j = 4 * kg + jj;
           const int64_t jrow = ((t0 + 16 * I + j) * H + h) * K;
-          const lq_v8h kj = *(const lq_v8h*)(p.k + jrow + n8);
+          float kj[8];
+          zoo_ld8(p.k + jrow + n8, bf, kj);
           const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
           const float bh_j = bh_s[16 * I + j];
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float gi_ = e < 4 ? gi0[e & 3] : gi1[e & 3], gj_ = e < 4 ? gj0[e & 3] : gj1[e & 3];
             const float w = (rl > j) ? zoo_exp(gi_ - gj_) : 0.0f;
-            sacc[jj] = fmaf((bs_i * (float)ki[e]) * (bh_j * (float)kj[e]), w, sacc[jj]);
+            sacc[jj] = fmaf((bs_i * ki[e]) * (bh_j * kj[e]), w, sacc[jj]);
           }
         }
       }
@@ -268,8 +284,8 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
       const int I = nt < NTL / 2 ? wave : 3 - wave;
       const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
       lq_v2i o;
-      o[0] = (int)zoo_pack_h2(a[0], a[1]);
-      o[1] = (int)zoo_pack_h2(a[2], a[3]);
+      o[0] = (int)zoo_enc2(a[0], a[1], bf);
+      o[1] = (int)zoo_enc2(a[2], a[3], bf);
       *(lq_v2i*)(p.W + ((t0 + 16 * I + rl) * H + h) * K + 16 * nt + 4 * kg) = o;
     }
   }
@@ -280,13 +296,14 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
     __syncthreads();
     for (int it = tid; it < 64 * (pw / 8); it += 256) {
       const int r = it / (pw / 8), c8 = it % (pw / 8);
-      const lq_v8h vv = *(const lq_v8h*)(p.v + ((t0 + r) * H + h) * V + vc + 8 * c8);
+      float vv[8];
+      zoo_ld8(p.v + ((t0 + r) * H + h) * V + vc + 8 * c8, bf, vv);
       const float bsr = bs_s[r];
       lq_v4f x0, x1;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        x0[e] = bsr * (float)vv[e];
-        x1[e] = bsr * (float)vv[4 + e];
+        x0[e] = bsr * vv[e];
+        x1[e] = bsr * vv[4 + e];
       }
       *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
       *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
@@ -297,8 +314,8 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
       const int I = nt < ntl / 2 ? wave : 3 - wave;
       const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
       lq_v2i o;
-      o[0] = (int)zoo_pack_h2(a[0], a[1]);
-      o[1] = (int)zoo_pack_h2(a[2], a[3]);
+      o[0] = (int)zoo_enc2(a[0], a[1], bf);
+      o[1] = (int)zoo_enc2(a[2], a[3], bf);
       *(lq_v2i*)(p.U + ((t0 + 16 * I + rl) * H + h) * V + vc + 16 * nt + 4 * kg) = o;
     }
   }
@@ -328,12 +345,13 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
+  if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (!zoo_al(a->k, 16) || !zoo_al(a->v, 16) || !zoo_al(a->Hw, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   WyParams p = {};
   p.k = (const _Float16*)a->k, p.v = (const _Float16*)a->v, p.beta = a->beta, p.g = a->g;
   p.Hw = (_Float16*)a->Hw, p.W = (_Float16*)a->W, p.U = (_Float16*)a->U, p.fw = a->fw;
-  p.sigma = a->sigma, p.tau = a->tau;
+  p.sigma = a->sigma, p.tau = a->tau, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);
   return a->kdim == 128 ? launch_decay<128>(p, a->decay, grid, stream) : launch_decay<64>(p, a->decay, grid, stream);

@@ -19,9 +19,14 @@ def check_shapes(q, k, v, chunk_size):
     assert chunk_size == CHUNK, f"chunk_size={chunk_size}: the HIP kernels are built for 64-token chunks"
     assert K in (64, 128), f"K={K}: built for key dims 64 and 128"
     assert V % 64 == 0, f"V={V}: value dim must be a multiple of 64"
-    assert q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16, "fp16 activations"
+    assert q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype, \
+        "q, k, v: one 16-bit activation dtype (fp16 or bf16)"
     assert k.shape == q.shape and v.shape[:3] == q.shape[:3]
     return B, T, H, K, V
+
+
+def act_code(t):
+    return _lib.LQ_DT_BF16 if t.dtype == torch.bfloat16 else _lib.LQ_DT_F16
 
 
 def f32(t):
@@ -61,7 +66,7 @@ def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family,
               g=_lib.ptr(g), logenv=_lib.ptr(logenv), kqT=_lib.ptr(c["kqT"]), vqT=_lib.ptr(c["vqT"]), wq=_lib.ptr(c["wq"]),
               ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]), skw=_lib.ptr(skw), svw=None if delta else _lib.ptr(svw),
               sw=_lib.ptr(sw), eta=float(eta), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K, vdim=V,
-              chunk_size=CHUNK, decay=decay)
+              chunk_size=CHUNK, decay=decay, act_dtype=act_code(key))
     return c
 
 
@@ -73,7 +78,8 @@ def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, fa
               u=_lib.ptr(value) if delta else None, fw=_lib.ptr(fw), ev=_lib.ptr(c["ev"]) if delta else None,
               gam=_lib.ptr(c["gam"]), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
               svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), qmax=int(qmax), batch=B, seqlen=T, nheads=H,
-              kdim=K, vdim=V, chunk_size=CHUNK, family=family, vtile=int(vtile))
+              kdim=K, vdim=V, chunk_size=CHUNK, family=family, vtile=int(vtile),
+              act_dtype=act_code(value))
 
 
 def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
@@ -88,7 +94,7 @@ def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims,
     _lib.call("lq_zoo_output", q.device, q=_lib.ptr(q), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
               g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
               sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay)
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(q))
 
 
 def run_gla_A(q, key, gc, A, sq, sk, scale, qmax, dims, rot=None):
@@ -96,7 +102,7 @@ def run_gla_A(q, key, gc, A, sq, sk, scale, qmax, dims, rot=None):
     assert rot is None or tuple(rot.shape) == (K, K), "rot: (K, K) R_QK"
     _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), rot=_lib.ptr(rot),
               sq=_lib.ptr(sq), sk=_lib.ptr(sk), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K,
-              chunk_size=CHUNK)
+              chunk_size=CHUNK, act_dtype=act_code(q))
 
 
 def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay):
@@ -107,13 +113,13 @@ def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay):
     fw = torch.empty(B, T, H, dtype=torch.float32, device=k.device)
     _lib.call("lq_zoo_wy_prep", k.device, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
               Hw=_lib.ptr(Hw), W=_lib.ptr(W), U=_lib.ptr(U), fw=_lib.ptr(fw), sigma=float(sigma), tau=float(tau),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay)
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(k))
     return Hw, W, U, fw
 
 
 def out_buffer(v, out_dtype):
     dt = out_dtype or v.dtype
-    assert dt in (torch.float16, torch.float32), f"output dtype {dt}: fp16 or fp32"
+    assert dt in (v.dtype, torch.float32), f"output dtype {dt}: the activation dtype {v.dtype} or fp32"
     return torch.empty(v.shape, dtype=dt, device=v.device)
 
 

@@ -19,10 +19,11 @@ DEFAULT_ETA = {"linear_none": 1.0, "mamba2": 1.0, "gla": 0.0, "deltanet": 1.0, "
 
 def _go(cell, tensors, *, policy="kernel_static", bits=8, eta=None, rho=1.0, tau=1.0, label=None, rot=None, rot_v=None, **kw):
     eta = DEFAULT_ETA[cell] if eta is None else eta
-    qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau, rot_qk=rot, rot_v=rot_v)
+    qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau, rot_qk=rot, rot_v=rot_v,
+                            out_dtype=kw.get("out_dtype"))
     if rot_v is not None:  # the kernel receives the rotated value operand, materialized in the activation dtype
         q_, k_, v_, g_, b_ = tensors
-        tensors = (q_, k_, (v_.double() @ rot_v).half(), g_, b_)
+        tensors = (q_, k_, (v_.double() @ rot_v).to(v_.dtype), g_, b_)
         kw["unrot"] = rot_v.T.contiguous()
     if rot is not None:
         kw["rot"] = rot
@@ -109,6 +110,24 @@ def test_canonical_storage_rv(cuda, cell, n, K, V):
     tensors = zc.cut(zc.inputs(cell, K=K, V=V, H=2 if K == 128 else 4), n)
     out, _, qz, run = _go(cell, tensors, eta=1.0, rot_v=signed_hadamard(V, 7))
     zc.check(out, run, qz, f"{cell} canonical R_V T={n} K={K} V={V}")
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+@pytest.mark.parametrize("variant", ["plain", "rotated"])
+def test_bf16_activations(cuda, cell, variant):
+    """bf16 q, k, v (the dtype of the reference's timing script, /root/reference bench/zoo_kernels.py:60-63): prepared
+    operands and the output are materialized in bf16, the local product stays fp16."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell, seed=6, dtype=torch.bfloat16), 256)
+    kw = {}
+    if variant == "rotated":
+        kw["rot_v"] = signed_hadamard(128, 7)
+        if zc.CELLS[cell][1] == "diagonal":
+            kw["rot"] = signed_hadamard(64, 3)
+    out, _, qz, run = _go(cell, tensors, **kw)
+    assert out.dtype == torch.bfloat16
+    zc.check(out, run, qz, f"{cell} bf16 {variant}")
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))

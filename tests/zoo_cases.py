@@ -9,12 +9,12 @@ from oracle import zoo_reference as Z
 CELLS = Z.CELLS
 
 
-def inputs(cell, B=2, T=512, H=4, K=64, V=128, seed=0, gscale=1.0):
+def inputs(cell, B=2, T=512, H=4, K=64, V=128, seed=0, gscale=1.0, dtype=torch.float16):
     fam, dec = CELLS[cell]
     gen = torch.Generator().manual_seed(seed)
-    q = torch.nn.functional.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).half()
-    k = torch.nn.functional.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).half()
-    v = torch.randn(B, T, H, V, generator=gen).half()
+    q = torch.nn.functional.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).to(dtype)
+    k = torch.nn.functional.normalize(torch.randn(B, T, H, K, generator=gen), dim=-1).to(dtype)
+    v = torch.randn(B, T, H, V, generator=gen).to(dtype)
     g = None
     if dec == "scalar":
         g = (torch.nn.functional.logsigmoid(torch.randn(B, T, H, generator=gen) * 3) / 4).float() * gscale
@@ -28,9 +28,10 @@ def cut(tensors, n):
     return [t[:, :n].contiguous() if t is not None else None for t in tensors]
 
 
-def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None):
+def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None, out_dtype=None):
     """Returns (qz, run): the oracle's quantizer with scales calibrated on these inputs, and a closure that
-    evaluates the oracle (float32 result) under the quantizer's current arithmetic mode."""
+    evaluates the oracle under the quantizer's current arithmetic mode; like the kernels, the oracle materializes its
+    output in the activation dtype unless ``out_dtype`` says otherwise."""
     fam, dec = CELLS[cell]
     q, k, v, g, beta = tensors
     K = q.shape[-1]
@@ -38,7 +39,7 @@ def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.
 
     def run():
         return Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=qz, eta=eta, rho=rho,
-                               tau=tau, read_post=True, C=64, out_dtype=torch.float32, rot_qk=rot_qk, rot_v=rot_v,
+                               tau=tau, read_post=True, C=64, out_dtype=out_dtype, rot_qk=rot_qk, rot_v=rot_v,
                                storage="canonical" if rot_v is not None else "rotated")
 
     qz.calibrating = True
