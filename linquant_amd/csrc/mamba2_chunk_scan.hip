@@ -4,7 +4,8 @@
 //   acc += sum_{k<=m} fp16(CB_i8[m,k] * S_cb * exp(dA_m - dA_k) * dt_k) * fp16(x[k,p])    (fp32 accumulate)
 //   acc += float(x[m,p]) * (D_scale * float(D_i8[h]))
 //
-// One workgroup per (64-col P tile, batch*chunk, head), one wavefront per 32 rows of the chunk.
+// One workgroup per (64-col P tile, batch*chunk, head), one wavefront per two 16-row tiles of the chunk: tile w
+// and tile 2*WAVES-1-w, an early and a late one, so every wave carries the same causal work.
 //
 // LDS holds two copies of the chunk's x tile, both "token-pair interleaved" (dword (kp, p) = {x[2kp][p],
 // x[2kp+1][p]}) so that an fp16 MFMA operand (8 tokens of one channel) is four 16-byte LDS reads covering the
@@ -13,10 +14,10 @@
 //   xS : x[k] * exp(dA_e(k) - dA_k) * S_cb * dt_k, where e(k) is the last token of k's 32-token slab.
 // For 32-token slabs strictly before a wave's rows the causal weight factors as
 //   exp(dA_m - dA_k) = exp(dA_m - dA_E) * exp(dA_E - dA_e) * exp(dA_e - dA_k),   all exponents <= 0,
-// (E = last token before the wave's rows), so those slabs need no per-element exponential: the B operand is
+// (E = last token before the tile's own 32-token slab), so those slabs need no per-element exponential: the B operand is
 // xS, the A operand is the CB code times the per-slab scalar exp(dA_E - dA_e), produced by the same packed
 // fp16 instruction that finishes the int8 -> fp16 conversion, and the row factor exp(dA_m - dA_E) is applied
-// once to the slab accumulator.  Only the wave's own 32-token slab evaluates exp(dA_m - dA_k) per element
+// once to the slab accumulator.  Only the tile's own 32-token slab evaluates exp(dA_m - dA_k) per element
 // (masked to k <= m).
 // State path: both INT8 operands are N-contiguous (16-byte global loads, INT8 MFMA).
 #include "lq_common.h"
@@ -103,14 +104,18 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     if (2 * kp < limit) r0[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp) * p.sx_l + c8 * 8);
     if (2 * kp + 1 < limit) r1[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp + 1) * p.sx_l + c8 * 8);
   }
-  const int mbase = wave * 32;
+  // Row tiles of this wave: 16w.. and 16(2*WAVES-1-w)..: an early and a late tile, so that every wave has the same
+  // number of causal slabs to process.
+  int rb[2];
+  rb[0] = 16 * wave;
+  rb[1] = 16 * (2 * WAVES - 1 - wave);
   // ---- state path (INT8 MFMA), issued before the staging barrier so its global loads overlap the x tile's
   lq_v4i ai[2][4];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) ai[i][j] = lq_v4i{0, 0, 0, 0};
-  if (mbase < limit) {
+  if (rb[0] < limit) {
     const int8_t* Cp = p.C + (int64_t)b * p.sC_b + (int64_t)c * Q * p.sC_l + (int64_t)g * p.sC_g;
     const int8_t* Sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P) * p.N;
     for (int n0 = 0; n0 < p.N; n0 += 64) {
@@ -118,7 +123,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       lq_v4i cop[2], sop[4];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
-        const int m = min(mbase + 16 * i + rl, limit - 1);
+        const int m = min(rb[i] + rl, limit - 1);
         cop[i] = *(const lq_v4i*)(Cp + (int64_t)m * p.sC_l + nn);
       }
 #pragma unroll
@@ -152,10 +157,10 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   }
   __syncthreads();
 
-  if (mbase >= limit) return;
+  if (rb[0] >= limit) return;  // the early tile is past the sequence end, so is the late one
 
   // ---- state read dequantized and gated: float(acc) * (sC * ss[p]) * exp(dA_m)
-  lq_v4f acc[2][4];  // [16-row tile][channel call j]
+  lq_v4f acc[2][4];  // [row tile][channel call j]
   {
     const float gscale = p.C_scale[g];
     float ssv[4];
@@ -165,97 +170,80 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float rg = fexp2(dA2_s[mbase + 16 * i + 4 * kg + r]);
+        const float rg = fexp2(dA2_s[rb[i] + 4 * kg + r]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j][r] = (float)ai[i][j][r] * (ssv[j] * rg);
       }
   }
 
   const int8_t* cbp = p.cb + ((((int64_t)b * p.nchunks + c) * p.G + g) * Q) * Q;
-  const int nslab = mbase >> 5;  // 32-token slabs strictly before this wave's rows
 
-  // ---- slabs before the wave's rows: (scaled CB codes) x (anchor-scaled x), row factor applied once
-  if (nslab > 0) {
-    lq_v4f off[2][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 2; ++i) {
+    if (rb[i] >= limit) continue;
+    const int nslab = rb[i] >> 5;      // 32-token slabs strictly before the slab that holds this tile
+    const int sbase = 32 * nslab;      // first token of the tile's own slab
+    const int8_t* crow = cbp + (int64_t)(rb[i] + rl) * Q;
+    // ---- slabs before the tile's own slab: (scaled CB codes) x (anchor-scaled x), row factor applied once
+    if (nslab > 0) {
+      lq_v4f off[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) off[i][j] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-    const float aE = dA2_s[mbase - 1];
-    lq_v2i cw[2], cwn[2];
+      for (int j = 0; j < 4; ++j) off[j] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+      const float aE = dA2_s[sbase - 1];
+      lq_v2i cw = *(const lq_v2i*)(crow + 8 * kg), cwn = cw;
+      for (int J = 0; J < nslab; ++J) {
+        if (J + 1 < nslab) cwn = *(const lq_v2i*)(crow + 32 * (J + 1) + 8 * kg);
+        const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
+        const lq_v2h s2 = {sh, sh};
+        const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
+        const int kp0 = 16 * J + 4 * kg;  // token pair index of this lane's first slot
+        lq_v4i xop[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) cw[i] = *(const lq_v2i*)(cbp + (int64_t)(mbase + 16 * i + rl) * Q + 8 * kg);
-    for (int J = 0; J < nslab; ++J) {
-      if (J + 1 < nslab) {
+        for (int d = 0; d < 4; ++d) {
+          const lq_v4i v = *(const lq_v4i*)(xS + (kp0 + d) * kRow + 4 * rl);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) cwn[i] = *(const lq_v2i*)(cbp + (int64_t)(mbase + 16 * i + rl) * Q + 32 * (J + 1) + 8 * kg);
-      }
-      const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
-      const lq_v2h s2 = {sh, sh};
-      const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
-      const int kp0 = 16 * J + 4 * kg;  // token pair index of this lane's first slot
-      lq_v4i xop[4];
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const lq_v4i v = *(const lq_v4i*)(xS + (kp0 + d) * kRow + 4 * rl);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
+          for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
+        }
         lq_v4i aw;
         uint32_t lo, hi;
-        i8x4_to_f16x4((uint32_t)cw[i][0], s2, o2, lo, hi);
+        i8x4_to_f16x4((uint32_t)cw[0], s2, o2, lo, hi);
         aw[0] = (int)lo, aw[1] = (int)hi;
-        i8x4_to_f16x4((uint32_t)cw[i][1], s2, o2, lo, hi);
+        i8x4_to_f16x4((uint32_t)cw[1], s2, o2, lo, hi);
         aw[2] = (int)lo, aw[3] = (int)hi;
         const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) off[i][j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[i][j]);
+        for (int j = 0; j < 4; ++j) off[j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[j]);
+        cw = cwn;
       }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) cw[i] = cwn[i];
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float rf = fexp2(dA2_s[mbase + 16 * i + 4 * kg + r] - aE);
+        const float rf = fexp2(dA2_s[rb[i] + 4 * kg + r] - aE);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j][r] = fmaf(off[i][j][r], rf, acc[i][j][r]);
+        for (int j = 0; j < 4; ++j) acc[i][j][r] = fmaf(off[j][r], rf, acc[i][j][r]);
       }
-  }
+    }
 
-  // ---- the wave's own 32-token slab: per-element weights exp2(dA2_m - (dA2_k - log2(S_cb dt_k))), k <= m
-  {
-    float dAm[2];
+    // ---- the tile's own 32-token slab: per-element weights exp2(dA2_m - (dA2_k - log2(S_cb dt_k))), k <= m
+    {
+      const int m = rb[i] + rl;
+      const float dAm = dA2_s[m];
+      const int kb = sbase + 8 * kg;
+      lq_v4i xop[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) dAm[i] = dA2_s[mbase + 16 * i + rl];
-    const int kb = mbase + 8 * kg;
-    lq_v4i xop[4];
+      for (int d = 0; d < 4; ++d) {
+        const lq_v4i v = *(const lq_v4i*)(xP + (kb / 2 + d) * kRow + 4 * rl);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const lq_v4i v = *(const lq_v4i*)(xP + (kb / 2 + d) * kRow + 4 * rl);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
-    }
-    const lq_v4f a0 = *(const lq_v4f*)(dA2_s + kb), a1 = *(const lq_v4f*)(dA2_s + kb + 4);
-    const lq_v4f w0 = *(const lq_v4f*)(w_s + kb), w1 = *(const lq_v4f*)(w_s + kb + 4);
-    float akw[8];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      akw[t] = a0[t] - __builtin_amdgcn_logf(w0[t]);
-      akw[4 + t] = a1[t] - __builtin_amdgcn_logf(w1[t]);
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int m = mbase + 16 * i + rl;
-      const lq_v2i cw = *(const lq_v2i*)(cbp + (int64_t)m * Q + kb);
+        for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
+      }
+      const lq_v4f a0 = *(const lq_v4f*)(dA2_s + kb), a1 = *(const lq_v4f*)(dA2_s + kb + 4);
+      const lq_v4f w0 = *(const lq_v4f*)(w_s + kb), w1 = *(const lq_v4f*)(w_s + kb + 4);
+      const lq_v2i cw = *(const lq_v2i*)(crow + kb);
       float v[8];
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
+        const float akw = (t < 4 ? a0[t & 3] : a1[t & 3]) - __builtin_amdgcn_logf(t < 4 ? w0[t & 3] : w1[t & 3]);
         const float cf = (float)lq_sbyte((uint32_t)cw[t >> 2], t & 3);
-        v[t] = cf * fexp2(dAm[i] - akw[t]);
+        v[t] = cf * fexp2(dAm - akw);
         if (kb + t > m) v[t] = 0.0f;
       }
       lq_v4i aw;
@@ -280,7 +268,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int m = mbase + 16 * i + 4 * kg + r;
+      const int m = rb[i] + 4 * kg + r;
       if (m >= limit) continue;
       const lq_v4i xv = *(const lq_v4i*)(xP + (m >> 1) * kRow + 4 * rl);
       lq_v4h o;
