@@ -19,6 +19,10 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch at the default workload (key-side), from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by what the
+# same counters read for a plain 256 MiB copy (x2.0 / x1.0); summary in profiles/mamba2_ssd_c5_keyside_hbm_traffic.md
+C5_KEYSIDE_TRAFFIC_MB = {"chunk_scan": 860.2, "chunk_state": 509.1, "state_passing": 173.2, "chunk_cumsum": 63.1,
+                         "bmm_chunk": 42.2, "prologue": 25.2, "rotate_b_fp": 16.8}
 
 
 def stage_bytes(s, keyside):
@@ -242,6 +246,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--value-side", action="store_true", help="value-side absorption instead of key-side")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain device copy of 256 MiB (reference point for HBM byte counters)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="heads of the CPU-oracle sample (batch 1)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -297,6 +303,13 @@ def main():
             static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], **kw)
         return out
 
+    if args.copy_probe:
+        probe = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        probe.zero_()
+        probe_dst = torch.empty_like(probe)
+        probe_dst.copy_(probe)
+        torch.cuda.synchronize()
+        del probe, probe_dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -362,8 +375,9 @@ def main():
     avg_dom = statistics.mean(a.elapsed_time(b) for a, b in records[dom])
     achieved = nbytes[dom] / 1e6 / avg_dom
     roofline = {"kernel": dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "avg_ms": round(avg_dom, 4),
-                "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": int(C5_KEYSIDE_TRAFFIC_MB[dom] * 1e6) if keyside and dom in C5_KEYSIDE_TRAFFIC_MB else None,
+                "avg_ms": round(avg_dom, 4), "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
 
     # ---- CPU baseline: the CPU oracle on a bounded sample (batch 1 x a few heads x full length), same seeds
     cpu = None
