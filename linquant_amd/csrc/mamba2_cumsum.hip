@@ -1,8 +1,9 @@
 // Mamba-2 SSD stage 1: dt pipeline + chunk-local cumulative sum of dt*A.
 // Replaces the reference stage linquant/kernels/mamba2/chunk_cumsum.py:27-74 (launcher :77-100).
 //
-// One wavefront per (head, chunk, batch).  Lane l owns the E = Q/64 consecutive positions
-// l*E .. l*E+E-1 of the chunk.  The prefix sum is: sequential inside the lane, Hillis-Steele
+// One 8-wave workgroup per (16 heads, chunk, batch): the (token, head) tile of raw dt is staged through LDS with
+// head-contiguous reads (dt is laid out (B, L, H): a head's tokens are H elements apart), then each wavefront
+// scans two heads.  Lane l owns the E = Q/64 consecutive positions l*E .. l*E+E-1 of the chunk.  The prefix sum is: sequential inside the lane, Hillis-Steele
 // inclusive scan of the lane totals over the wave (offsets 1,2,4,...,32, "t = t + up"), then
 // exclusive lane prefix + local prefix.  The CPU checker restates exactly this order.
 #include "lq_common.h"
@@ -18,53 +19,72 @@ LQ_DEV float load_dt(const void* p, int64_t off, int dtype) {
   return (float)((const int8_t*)p)[off];
 }
 
-__global__ __launch_bounds__(64) void chunk_cumsum_kernel(
+constexpr int kHG = 16;   // heads per workgroup: one token row of the tile is 16 adjacent heads (32 bytes of fp16 dt)
+constexpr int kWaves = 8;  // two heads per wave
+
+__global__ __launch_bounds__(kWaves * 64) void chunk_cumsum_kernel(
     const void* __restrict__ dt_in, int dt_dtype, int64_t sdt_b, int64_t sdt_l, int64_t sdt_h,
     const float* __restrict__ dt_scale_p, const int8_t* __restrict__ a_log, int64_t sa_h,
     const float* __restrict__ a_log_scale_p, const float* __restrict__ dt_bias, int64_t sbias_h,
     float* __restrict__ dt_out, float* __restrict__ dA_cs, int seqlen, int nheads, int nchunks, int Q,
     int softplus, float dt_min, float dt_max) {
-  const int h = blockIdx.x, c = blockIdx.y, b = blockIdx.z;
-  const int lane = threadIdx.x;
+  extern __shared__ float tile[];  // [Q][kHG + 1] raw dt as float
+  const int h0 = blockIdx.x * kHG, c = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int E = Q >> 6;
   const int limit = min(Q, seqlen - c * Q);
+  // ---- stage the (token, head) tile: consecutive lanes read consecutive heads of one token
+  for (int it = tid; it < Q * kHG; it += kWaves * 64) {
+    const int pos = it / kHG, hh = it % kHG;
+    float v = 0.0f;
+    if (pos < limit && h0 + hh < nheads)
+      v = load_dt(dt_in, (int64_t)b * sdt_b + (int64_t)(c * Q + pos) * sdt_l + (int64_t)(h0 + hh) * sdt_h, dt_dtype);
+    tile[pos * (kHG + 1) + hh] = v;
+  }
+  __syncthreads();
   const float dt_scale = *dt_scale_p;
-  const float A = -lq_expf((*a_log_scale_p) * (float)a_log[(int64_t)h * sa_h]);
-  const float bias = dt_bias ? dt_bias[(int64_t)h * sbias_h] : 0.0f;
-
-  float dtv[kMaxE], pre[kMaxE];
-  float run = 0.0f;
+  const float a_scale = *a_log_scale_p;
 #pragma unroll
-  for (int i = 0; i < kMaxE; ++i) {
-    if (i < E) {
-      const int pos = lane * E + i;
-      float v = 0.0f;
-      if (pos < limit) {
-        v = dt_scale * load_dt(dt_in, (int64_t)b * sdt_b + (int64_t)(c * Q + pos) * sdt_l + (int64_t)h * sdt_h, dt_dtype);
-        if (dt_bias) v = v + bias;
-        if (softplus) v = (v > 20.0f) ? v : lq_logf(1.0f + lq_expf(v));
-        v = fminf(fmaxf(v, dt_min), dt_max);
+  for (int hw = 0; hw < kHG / kWaves; ++hw) {
+    const int hh = wave * (kHG / kWaves) + hw;
+    const int h = h0 + hh;
+    if (h >= nheads) continue;
+    const float A = -lq_expf(a_scale * (float)a_log[(int64_t)h * sa_h]);
+    const float bias = dt_bias ? dt_bias[(int64_t)h * sbias_h] : 0.0f;
+    float dtv[kMaxE], pre[kMaxE];
+    float run = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kMaxE; ++i) {
+      if (i < E) {
+        const int pos = lane * E + i;
+        float v = 0.0f;
+        if (pos < limit) {
+          v = dt_scale * tile[pos * (kHG + 1) + hh];
+          if (dt_bias) v = v + bias;
+          if (softplus) v = (v > 20.0f) ? v : lq_logf(1.0f + lq_expf(v));
+          v = fminf(fmaxf(v, dt_min), dt_max);
+        }
+        dtv[i] = v;
+        const float dA = v * A;
+        run = (i == 0) ? dA : run + dA;
+        pre[i] = run;
       }
-      dtv[i] = v;
-      const float dA = v * A;
-      run = (i == 0) ? dA : run + dA;
-      pre[i] = run;
     }
-  }
-  float t = run;
+    float t = run;
 #pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const float up = __shfl_up(t, off, 64);
-    if (lane >= off) t = t + up;
-  }
-  float ex = __shfl_up(t, 1, 64);
-  if (lane == 0) ex = 0.0f;
-  const int64_t base = (((int64_t)b * nheads + h) * nchunks + c) * Q + lane * E;
+    for (int off = 1; off < 64; off <<= 1) {
+      const float up = __shfl_up(t, off, 64);
+      if (lane >= off) t = t + up;
+    }
+    float ex = __shfl_up(t, 1, 64);
+    if (lane == 0) ex = 0.0f;
+    const int64_t base = (((int64_t)b * nheads + h) * nchunks + c) * Q + lane * E;
 #pragma unroll
-  for (int i = 0; i < kMaxE; ++i) {
-    if (i < E) {
-      dt_out[base + i] = dtv[i];
-      dA_cs[base + i] = ex + pre[i];
+    for (int i = 0; i < kMaxE; ++i) {
+      if (i < E) {
+        dt_out[base + i] = dtv[i];
+        dA_cs[base + i] = ex + pre[i];
+      }
     }
   }
 }
@@ -79,8 +99,12 @@ extern "C" int lq_chunk_cumsum(const lq_chunk_cumsum_args* a, hipStream_t stream
   if (a->dt_dtype != LQ_DT_F16 && a->dt_dtype != LQ_DT_F32 && a->dt_dtype != LQ_DT_I8) return LQ_ERR_SHAPE;
   const int nchunks = (a->seqlen + Q - 1) / Q;
   if (nchunks > 65535) return LQ_ERR_SHAPE;
-  dim3 grid(a->nheads, nchunks, a->batch);
-  hipLaunchKernelGGL(chunk_cumsum_kernel, grid, dim3(64), 0, stream, a->dt, a->dt_dtype, a->dt_stride_b,
+  dim3 grid((a->nheads + kHG - 1) / kHG, nchunks, a->batch);
+  const size_t lds = (size_t)Q * (kHG + 1) * sizeof(float);
+  if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&chunk_cumsum_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return LQ_ERR_LAUNCH;
+  hipLaunchKernelGGL(chunk_cumsum_kernel, grid, dim3(kWaves * 64), lds, stream, a->dt, a->dt_dtype, a->dt_stride_b,
                      a->dt_stride_l, a->dt_stride_h, a->dt_scale, a->A_log, a->A_log_stride_h, a->A_log_scale,
                      a->dt_bias, a->dt_bias_stride_h, a->dt_out, a->dA_cumsum, a->seqlen, a->nheads, nchunks, Q,
                      a->dt_softplus, a->dt_min, a->dt_max);
