@@ -104,6 +104,20 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     if (2 * kp < limit) r0[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp) * p.sx_l + c8 * 8);
     if (2 * kp + 1 < limit) r1[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp + 1) * p.sx_l + c8 * 8);
   }
+  // Small per-head operands of the epilogues are fetched now: issued where they are used, each would expose a full
+  // memory round trip behind the barriers.
+  float ssv[4], Dv[4] = {0.f, 0.f, 0.f, 0.f};
+  {
+    const float gscale = p.C_scale[g];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ssv[j] = gscale * p.ss[(int64_t)h * p.sss_h + (int64_t)(p0 + 4 * rl + j) * p.sss_p];
+    if (p.D) {
+      const float dsc = *p.D_scale;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        Dv[j] = dsc * (float)p.D[(int64_t)h * p.sD_h + (p.D_has_hdim ? p0 + 4 * rl + j : 0)];
+    }
+  }
   // Row tiles of this wave: 16w.. and 16(2*WAVES-1-w)..: an early and a late tile, so that every wave has the same
   // number of causal slabs to process.
   int rb[2];
@@ -162,10 +176,6 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   // ---- state read dequantized and gated: float(acc) * (sC * ss[p]) * exp(dA_m)
   lq_v4f acc[2][4];  // [row tile][channel call j]
   {
-    const float gscale = p.C_scale[g];
-    float ssv[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ssv[j] = gscale * p.ss[(int64_t)h * p.sss_h + (int64_t)(p0 + 4 * rl + j) * p.sss_p];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -256,13 +266,6 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   }
 
   // ---- D residual + store
-  float Dv[4] = {0.f, 0.f, 0.f, 0.f};
-  if (p.D) {
-    const float dsc = *p.D_scale;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      Dv[j] = dsc * (float)p.D[(int64_t)h * p.sD_h + (p.D_has_hdim ? p0 + 4 * rl + j : 0)];
-  }
   _Float16* op = p.out + (((int64_t)b * p.seqlen + (int64_t)c * Q) * p.nheads + h) * p.P + p0 + 4 * rl;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
