@@ -24,30 +24,56 @@ __global__ __launch_bounds__(256) void cumsum_scalar_kernel(const float* __restr
   }
 }
 
-// one workgroup per (batch, chunk, head); K threads; LDS tile [C][K+1] for the envelope reduction
+// one workgroup per (batch, chunk, head); 4*K threads: thread (k, q) scans tokens q*C/4 .. of channel k (all of its
+// loads are independent and issued up front), the four partial totals are combined through LDS; LDS tile [C][K+1]
+// for the envelope reduction
 __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restrict__ gc, float* __restrict__ logenv,
                                    int T, int H, int K, int C) {
-  extern __shared__ float tile[];
-  const int k = threadIdx.x;
+  extern __shared__ float tile[];           // [C][K + 1]
+  double* part = (double*)(tile + C * (K + 1));  // [4][K] segment totals
+  const int k = threadIdx.x % K, q = threadIdx.x / K;
+  const int SEG = C / 4;                    // tokens per thread (C is a multiple of 16)
   const int h = blockIdx.x % H;
   const int64_t bc = blockIdx.x / H;
   const int64_t row0 = bc * C;  // global token row of the chunk start (b * T + chunk * C)
-  const int64_t base = (row0 * H + h) * K + k;
+  const int64_t base = ((row0 + q * SEG) * H + h) * K + k;
   const int64_t tstride = (int64_t)H * K;
-  double run = 0.0;
-  for (int t = 0; t < C; ++t) {
-    run += (double)g[base + t * tstride];
-    const float v = (float)run;
-    gc[base + t * tstride] = v;
-    tile[t * (K + 1) + k] = v;
+  float v[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) v[t] = t < SEG ? g[base + t * tstride] : 0.0f;
+  double run = 0.0, pre[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    run += (double)v[t];
+    pre[t] = run;
   }
-  const float last = (float)run;
-  for (int t = 0; t < C; ++t) tile[t * (K + 1) + k] = last - tile[t * (K + 1) + k];
+  part[q * K + k] = run;
   __syncthreads();
-  for (int t = threadIdx.x; t < C; t += blockDim.x) {
-    float m = tile[t * (K + 1)];
-    for (int j = 1; j < K; ++j) m = fmaxf(m, tile[t * (K + 1) + j]);
-    logenv[(row0 + t) * H + h] = m;
+  double off = 0.0, total = 0.0;
+#pragma unroll
+  for (int qq = 0; qq < 4; ++qq) {
+    const double pt = part[qq * K + k];
+    if (qq < q) off += pt;
+    total += pt;
+  }
+  const float last = (float)total;
+#pragma unroll
+  for (int t = 0; t < 16; ++t)
+    if (t < SEG) {
+      const float c = (float)(off + pre[t]);
+      gc[base + t * tstride] = c;
+      tile[(q * SEG + t) * (K + 1) + k] = last - c;
+    }
+  __syncthreads();
+  // envelope: 8 lanes per token, each over a contiguous K/8 slice, then a max over the 8 lanes
+  const int sub = threadIdx.x & 7, KS = K / 8;
+  for (int t = threadIdx.x >> 3; t < C; t += blockDim.x >> 3) {
+    const float* row = tile + t * (K + 1) + sub * KS;
+    float m = row[0];
+    for (int j = 1; j < KS; ++j) m = fmaxf(m, row[j]);
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
+    if (sub == 0) logenv[(row0 + t) * H + h] = m;
   }
 }
 
@@ -64,10 +90,10 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
                        a->seqlen, a->nheads, a->chunk_size, total);
   } else {
     if (!a->logenv) return LQ_ERR_NULL;
-    if (a->kdim > 1024) return LQ_ERR_SHAPE;
-    const size_t lds = (size_t)a->chunk_size * (a->kdim + 1) * sizeof(float);
+    if (a->kdim > 256 || a->kdim % 16 != 0 || a->chunk_size % 16 != 0 || a->chunk_size > 64) return LQ_ERR_SHAPE;
+    const size_t lds = (size_t)a->chunk_size * (a->kdim + 1) * sizeof(float) + 4 * (size_t)a->kdim * sizeof(double);
     if (lds > 64 * 1024) return LQ_ERR_SHAPE;
-    hipLaunchKernelGGL(cumsum_diag_kernel, dim3((unsigned)((int64_t)a->batch * NT * a->nheads)), dim3(a->kdim), lds,
+    hipLaunchKernelGGL(cumsum_diag_kernel, dim3((unsigned)((int64_t)a->batch * NT * a->nheads)), dim3(4 * a->kdim), lds,
                        stream, a->g, a->gc, a->logenv, a->seqlen, a->nheads, a->kdim, a->chunk_size);
   }
   return lq_check_launch();

@@ -45,12 +45,12 @@ LQ_DEV float wave_max(float m) {
 // safely around the first row: the operands qh*exp(g_i - a) and kh*exp(a - g_j) stay normal fp32 numbers and
 // the sum is an fp32 16x16xK matrix product (lane (rl, kg) owns K/4 contiguous channels of token rl).
 // Otherwise every (i, j, n) weight is evaluated on its own, masked before use, as the reference does.
-template <int K>
+template <int K, bool BF>
 LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float inv_sk, int rl, int kg, int64_t row0, int h,
                        int i0) {
   constexpr int NCH = K / 4;
   const int H = p.H, qmax = p.qmax;
-  const bool bf = p.bf != 0;
+  constexpr bool bf = BF;
   const int c0 = NCH * kg;
   const int64_t off = ((row0 + rl) * H + h) * K + c0;
   const int64_t aoff = (row0 * H + h) * K + c0;
@@ -124,7 +124,7 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
   *(lq_v4f*)(p.A + ((row0 + rl) * H + h) * 64 + i0 + 4 * kg) = o;
 }
 
-template <int K, bool ROT>
+template <int K, bool ROT, bool BF>
 __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
   constexpr int RS = K + 8;  // halves per row of the transposed rotation
   __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
   const float sq = p.sq[h], sk = p.sk[h];
   const float inv_sq = 1.0f / sq, inv_sk = 1.0f / sk;
   const int qmax = p.qmax;
-  const bool bf = p.bf != 0;
+  constexpr bool bf = BF;
   const int i0 = 16 * wave;
 
   if constexpr (ROT) {
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
     }
   }
 
-  diag_block<K>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
+  diag_block<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
 
   lq_v4i acc[3];
 #pragma unroll
@@ -337,16 +337,24 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);
+#define LQ_A_LAUNCH(KV, ROTV)                                                                              \
+  do {                                                                                                     \
+    if (p.bf)                                                                                              \
+      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, true>), grid, dim3(256), 0, stream, p);               \
+    else                                                                                                   \
+      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, false>), grid, dim3(256), 0, stream, p);              \
+  } while (0)
   if (a->kdim == 128) {
     if (a->rot)
-      hipLaunchKernelGGL((zoo_gla_A_kernel<128, true>), grid, dim3(256), 0, stream, p);
+      LQ_A_LAUNCH(128, true);
     else
-      hipLaunchKernelGGL((zoo_gla_A_kernel<128, false>), grid, dim3(256), 0, stream, p);
+      LQ_A_LAUNCH(128, false);
   } else {
     if (a->rot)
-      hipLaunchKernelGGL((zoo_gla_A_kernel<64, true>), grid, dim3(256), 0, stream, p);
+      LQ_A_LAUNCH(64, true);
     else
-      hipLaunchKernelGGL((zoo_gla_A_kernel<64, false>), grid, dim3(256), 0, stream, p);
+      LQ_A_LAUNCH(64, false);
   }
+#undef LQ_A_LAUNCH
   return lq_check_launch();
 }

@@ -24,7 +24,7 @@ constexpr int kVW = 68;  // dwords per token-pair row of the value tile
 
 using OutParams = ZooOutParams;
 
-template <bool GLA, bool USE_G, int K>
+template <bool GLA, bool USE_G, int K, bool BF>
 __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   constexpr int QS = K + 16;  // byte stride of a code row
   __shared__ __align__(16) unsigned char qc[64 * QS];
@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   const float sk = GLA ? 1.0f : p.sk[h];
   const float inv_sk = 1.0f / sk;
   const int qmax = p.qmax;
-  const bool bf = p.bf != 0;
+  constexpr bool bf = BF;
 
   // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
   for (int it = tid; it < 64 * (K / 8); it += 256) {
@@ -214,12 +214,20 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   }
 }
 
+template <bool GLA, bool USE_G, int K>
+void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
+  if (p.bf)
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false>), grid, dim3(256), 0, stream, p);
+}
+
 template <bool GLA, bool USE_G>
 int launch(const OutParams& p, int K, dim3 grid, hipStream_t stream) {
   if (K == 128)
-    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, 128>), grid, dim3(256), 0, stream, p);
+    launch_bf<GLA, USE_G, 128>(p, grid, stream);
   else
-    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, 64>), grid, dim3(256), 0, stream, p);
+    launch_bf<GLA, USE_G, 64>(p, grid, stream);
   return lq_check_launch();
 }
 

@@ -35,7 +35,7 @@ struct CodesParams {
   int T, H, V, NT;
 };
 
-template <int DECAY, int K>
+template <int DECAY, int K, bool BF>
 __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   constexpr int CK = K / 16;  // key channels per thread
   constexpr int TS = 20;      // dwords per channel row of the transposed tile (16 token quads + pad)
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   const int64_t cb = ((int64_t)b * p.NT + ct) * H + h;  // (batch, chunk, head) index
   const float eta = p.eta;
   const int qmax = p.qmax;
-  const bool bf = p.bf != 0;
+  constexpr bool bf = BF;
 
   if (tid < 64) {
     float ekv = 1.0f, evv = 1.0f;
@@ -165,12 +165,20 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   }
 }
 
+template <int DECAY, int K>
+void launch_bf(const CodesParams& p, dim3 grid, hipStream_t stream) {
+  if (p.bf)
+    hipLaunchKernelGGL((zoo_write_codes_kernel<DECAY, K, true>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_write_codes_kernel<DECAY, K, false>), grid, dim3(256), 0, stream, p);
+}
+
 template <int K>
 int launch(const CodesParams& p, int decay, dim3 grid, hipStream_t stream) {
   switch (decay) {
-    case LQ_DECAY_NONE: hipLaunchKernelGGL((zoo_write_codes_kernel<LQ_DECAY_NONE, K>), grid, dim3(256), 0, stream, p); break;
-    case LQ_DECAY_SCALAR: hipLaunchKernelGGL((zoo_write_codes_kernel<LQ_DECAY_SCALAR, K>), grid, dim3(256), 0, stream, p); break;
-    case LQ_DECAY_DIAGONAL: hipLaunchKernelGGL((zoo_write_codes_kernel<LQ_DECAY_DIAGONAL, K>), grid, dim3(256), 0, stream, p); break;
+    case LQ_DECAY_NONE: launch_bf<LQ_DECAY_NONE, K>(p, grid, stream); break;
+    case LQ_DECAY_SCALAR: launch_bf<LQ_DECAY_SCALAR, K>(p, grid, stream); break;
+    case LQ_DECAY_DIAGONAL: launch_bf<LQ_DECAY_DIAGONAL, K>(p, grid, stream); break;
     default: return LQ_ERR_SHAPE;
   }
   return lq_check_launch();

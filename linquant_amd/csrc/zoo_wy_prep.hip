@@ -64,7 +64,7 @@ LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl
   return acc;
 }
 
-template <int DECAY, int K>
+template <int DECAY, int K, bool BF>
 __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
   constexpr int LS = K + 16;  // floats per row of X: rows 4s + kg land in disjoint bank groups
   __shared__ __align__(16) float G_s[64 * kGS];
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
   const float sigma = p.sigma, tau = p.tau;
-  const bool bf = p.bf != 0;
+  constexpr bool bf = BF;
 
   // ---- per-token factors; Hw and fw are written straight out; X = beta^sigma k exp(g) staged for the W product
   if (tid < 64) {
@@ -323,7 +323,10 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
 
 template <int DECAY, int K>
 int launch(const WyParams& p, dim3 grid, hipStream_t stream) {
-  hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K>), grid, dim3(256), 0, stream, p);
+  if (p.bf)
+    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, true>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, false>), grid, dim3(256), 0, stream, p);
   return lq_check_launch();
 }
 
