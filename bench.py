@@ -209,7 +209,7 @@ def bench_zoo(args):
 
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
         torch.set_num_threads(threads)
-        hs, ts_ = min(2, H), min(T, 2048)
+        hs, ts_ = H, T
         cut = lambda t: None if t is None else t[:1, :ts_, :hs].cpu()  # noqa: E731
         qz = Z.ZooQuantizer.kernel_profile("kernel_static", 8)
         run = lambda: Z.chunk_forward(cut(q), cut(k), cut(v), cut(g), cut(beta), family=fam, decay=dec, scale=scale, qz=qz,  # noqa: E731
@@ -248,7 +248,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of 256 MiB (reference point for HBM byte counters)")
-    ap.add_argument("--cpu-heads", type=int, default=8, help="heads of the CPU-oracle sample (batch 1)")
+    ap.add_argument("--cpu-heads", type=int, default=8, help="heads per slice of the CPU-oracle sample")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="stop the CPU-oracle sample after about this long")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards over batch x head "
@@ -390,23 +391,35 @@ def main():
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
         torch.set_num_threads(threads)
         npy = lambda t: t.detach().cpu().numpy()  # noqa: E731
-        xs = npy(xBC[:1, :, :nh * s.headdim]).reshape(1, s.seqlen, nh, s.headdim)
-        xBC_s = np.concatenate([xs.reshape(1, s.seqlen, -1), npy(xBC[:1, :, s.d_ssm:])], axis=-1)
-        t0 = time.perf_counter()
-        x_o, qB_o, qC_o = O.split_rotate_quant_xBC(xBC_s, npy(p["r_signs"]), nh, s.ngroups, s.dstate, s.headdim,
-                                                   npy(sc["B_inv_scale"]), npy(sc["C_inv_scale"]))
-        bfp_o = O.kron_hadamard(xBC_s[..., nh * s.headdim:nh * s.headdim + gn].reshape(1, s.seqlen, s.ngroups, s.dstate),
-                                npy(p["r_signs"])) if keyside else None
-        O.ssd_combined(x_o, npy(dt_raw[:1, :, :nh]), 1.0, npy(p["A_log"][:nh]), float(p["A_log_scale"]), qB_o,
-                       npy(sc["B_scale"]), qC_o, npy(sc["C_scale"]), s.chunk, npy(p["D"][:nh]), float(p["D_scale"]),
-                       dt_bias=npy(p["dt_bias"][:nh]), dt_softplus=True,
-                       static_state_scale=npy(sc["static_state_scale"][:nh]), static_cb_scale=npy(sc["static_cb_scale"]),
-                       alpha_hp=npy(sc["alpha_hp"][:nh]), bscale_g=npy(sc["bscale_g"]), keyside=keyside,
-                       x_scale_hp=npy(sc["x_scale_hp"][:nh]), b_fp=bfp_o, b_gate_scale=npy(sc["b_gate_scale"][:, :, :nh]))
+
+        def cpu_slice(bi, h0):
+            """The whole hot path of the oracle on batch row bi, heads h0 .. h0+nh-1."""
+            hs = slice(h0, h0 + nh)
+            xs = npy(xBC[bi:bi + 1, :, h0 * s.headdim:(h0 + nh) * s.headdim])
+            xBC_s = np.concatenate([xs, npy(xBC[bi:bi + 1, :, s.d_ssm:])], axis=-1)
+            x_o, qB_o, qC_o = O.split_rotate_quant_xBC(xBC_s, npy(p["r_signs"]), nh, s.ngroups, s.dstate, s.headdim,
+                                                       npy(sc["B_inv_scale"]), npy(sc["C_inv_scale"]))
+            bfp_o = O.kron_hadamard(xBC_s[..., nh * s.headdim:nh * s.headdim + gn].reshape(1, s.seqlen, s.ngroups, s.dstate),
+                                    npy(p["r_signs"])) if keyside else None
+            O.ssd_combined(x_o, npy(dt_raw[bi:bi + 1, :, hs]), 1.0, npy(p["A_log"][hs]), float(p["A_log_scale"]), qB_o,
+                           npy(sc["B_scale"]), qC_o, npy(sc["C_scale"]), s.chunk, npy(p["D"][hs]), float(p["D_scale"]),
+                           dt_bias=npy(p["dt_bias"][hs]), dt_softplus=True,
+                           static_state_scale=npy(sc["static_state_scale"][hs]), static_cb_scale=npy(sc["static_cb_scale"]),
+                           alpha_hp=npy(sc["alpha_hp"][hs]), bscale_g=npy(sc["bscale_g"]), keyside=keyside,
+                           x_scale_hp=npy(sc["x_scale_hp"][hs]), b_fp=bfp_o, b_gate_scale=npy(sc["b_gate_scale"][:, :, hs]))
+
+        # bounded sample: (batch row, head group) slices until about args.cpu_seconds of CPU work are done
+        slices = [(bi, h0) for bi in range(s.batch) for h0 in range(0, s.nheads - nh + 1, nh)]
+        done, t0 = 0, time.perf_counter()
+        for bi, h0 in slices:
+            cpu_slice(bi, h0)
+            done += 1
+            if time.perf_counter() - t0 >= args.cpu_seconds:
+                break
         t_cpu = time.perf_counter() - t0
-        frac = nh / (s.batch * s.nheads)
+        frac = done * nh / (s.batch * s.nheads)
         cpu = {"value": round(tokens * frac / t_cpu, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
-               "sample": f"numpy/BLAS oracle on batch 1 x {nh} of {s.nheads} heads x {s.seqlen} tokens "
+               "sample": f"numpy/BLAS oracle on {done} slices of 1 batch row x {nh} of {s.nheads} heads x {s.seqlen} tokens "
                          f"({frac:.4f} of the layer) in {t_cpu:.2f} s; value = layer-equivalent tokens/s",
                "host_cpus": os.cpu_count(), "torch_threads": torch.get_num_threads()}
 
