@@ -168,3 +168,83 @@ def test_rejections(cuda):
         zoo.chunk_simple_gla_int8(q[:, :100], k[:, :100], v[:, :100], g[:, :100], sc)
     with pytest.raises(AssertionError):
         zoo.chunk_simple_gla_int8(q, k, v, g, sc, unrot=torch.eye(64, device="cuda", dtype=torch.float16))
+
+
+def _wy_reference(k, v, beta, gc, decay, sigma, tau):
+    """float64 WY / UT transform per 64-token chunk (/root/reference linquant/kernels/zoo/gated_delta_rule.py:20-47,
+    kda.py:22-53): returns Hw, W, U, fw."""
+    B, T, H, K = k.shape
+    nc = T // 64
+    ch = lambda t: t.double().reshape(B, nc, 64, H, -1).permute(0, 3, 1, 2, 4)  # noqa: E731  [B,H,nc,64,D]
+    kc, vc, bt = ch(k), ch(v), ch(beta)
+    L, Hg = bt ** sigma * kc, bt ** (1 - sigma) * kc
+    tril = torch.ones(64, 64, dtype=torch.bool).tril(-1)
+    if decay == "none":
+        G, pq = L @ Hg.transpose(-1, -2), torch.ones_like(kc[..., :1])
+    elif decay == "scalar":
+        g = ch(gc)[..., 0]
+        G = (L @ Hg.transpose(-1, -2)) * (g[..., :, None] - g[..., None, :]).masked_fill(~tril, float("-inf")).exp()
+        pq = g.exp()[..., None]
+    else:
+        g = ch(gc)
+        w = (g[..., :, None, :] - g[..., None, :, :]).masked_fill(~tril[..., None], float("-inf")).exp()
+        G = torch.einsum("...in,...jn,...ijn->...ij", L, Hg, w)
+        pq = g.exp()
+    G = G.masked_fill(~tril, 0.0)
+    eye = torch.eye(64, dtype=torch.float64)
+    Tm = torch.linalg.solve_triangular(eye + G, eye.expand(G.shape).clone(), upper=False, unitriangular=True)
+    back = lambda t: t.permute(0, 2, 3, 1, 4).reshape(B, T, H, -1)  # noqa: E731
+    return (back(bt ** ((1 - sigma) * tau) * kc), back(Tm @ (L * pq)), back(Tm @ (bt ** sigma * vc)),
+            back(bt ** ((1 - sigma) * (1 - tau)))[..., 0])
+
+
+@pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet", "kda"])
+@pytest.mark.parametrize("sigma,tau", [(1.0, 1.0), (0.5, 0.5), (0.0, 1.0)])
+@pytest.mark.parametrize("K,gscale", [(64, 1.0), (128, 1.0), (64, 40.0)])
+def test_wy_prep_kernel(cuda, cell, sigma, tau, K, gscale):
+    """The fp32-MFMA WY prep (Gram, blocked triangular inverse, T.X) against the float64 transform, including the
+    strongly decaying regime that takes the per-element path of the diagonal Gram blocks."""
+    from linquant_amd.kernels.zoo import _common as C
+
+    decay = zc.CELLS[cell][1]
+    if decay == "none" and gscale != 1.0:
+        pytest.skip("no decay")
+    q, k, v, g, beta = zc.cut(zc.inputs(cell, B=1, H=2, K=K, V=64, seed=8, gscale=gscale), 128)
+    B, T, H, V = 1, 128, 2, 64
+    gc = None
+    if g is not None:
+        gc = g.double().reshape(B, T // 64, 64, H, -1).cumsum(2).reshape(g.shape).float()
+    code = {"none": C.DECAY_NONE, "scalar": C.DECAY_SCALAR, "diagonal": C.DECAY_DIAGONAL}[decay]
+    Hw, W, U, fw = C.run_wy_prep(k.cuda(), v.cuda(), beta.cuda(), None if gc is None else gc.cuda(), sigma, tau,
+                                 (B, T, H, K, V), code)
+    torch.cuda.synchronize()
+    rHw, rW, rU, rfw = _wy_reference(k, v, beta, gc, decay, sigma, tau)
+    for name, got, ref in (("Hw", Hw, rHw), ("W", W, rW), ("U", U, rU), ("fw", fw, rfw)):
+        err = (got.double().cpu() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
+        assert err <= 1e-3, f"{cell} {name}: rel max {err:.2e}"  # half-precision storage: 2^-11 per element
+
+
+def test_reference_mamba2_cell_config(cuda):
+    """BASELINE configs[0]: the Mamba-2 cell through chunk_simple_gla (q = C, k = B broadcast to heads, v = x*dt,
+    g = dt*A, scale = 1), B1 T2048 H8 K = V = 64, per-head / per-channel static scales."""
+    from linquant_amd.kernels import zoo
+    from oracle import zoo_reference as Z
+
+    gen = torch.Generator().manual_seed(0)
+    Bn, T, H, P, N = 1, 2048, 8, 64, 64
+    x = torch.randn(Bn, T, H, P, generator=gen)
+    Bm = torch.randn(Bn, T, 1, N, generator=gen).expand(Bn, T, H, N)
+    Cm = torch.randn(Bn, T, 1, N, generator=gen).expand(Bn, T, H, N)
+    dt = torch.nn.functional.softplus(torch.randn(Bn, T, H, generator=gen) * 0.5 - 2.0)
+    A = -torch.exp(torch.rand(H, generator=gen) * 2.7726)
+    q, k, v, g = Cm.half().contiguous(), Bm.half().contiguous(), (x * dt[..., None]).half(), (dt * A).float()
+    qz = Z.ZooQuantizer.kernel_profile("kernel_static", 8)
+    run = lambda: Z.chunk_forward(q, k, v, g, None, family="linear", decay="scalar", scale=1.0, qz=qz, eta=1.0,  # noqa: E731
+                                  read_post=True, C=64)
+    qz.calibrating = True
+    run()
+    qz.finalize()
+    sc = {n: s.cuda() for n, s in qz.kernel_scales(0, H, N, P).items()}
+    out, _ = zoo.chunk_simple_gla_int8(q.cuda(), k.cuda(), v.cuda(), g.cuda(), sc, eta=1.0, scale=1.0, chunk_size=64)
+    torch.cuda.synchronize()
+    zc.check(out, run, qz, "Mamba-2 cell at the c1 shape")
