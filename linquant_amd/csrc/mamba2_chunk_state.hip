@@ -59,6 +59,18 @@ LQ_DEV uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
   return lo | hi;
 }
 
+// float(half of the packed fp16 pair w) * f in one instruction: the mixed-precision fma converts the selected half
+// exactly and rounds the product once, so the result equals the separate convert-then-multiply bit for bit.
+template <int HI>
+LQ_DEV float mul_half(uint32_t w, float f) {
+  float r;
+  if (HI)
+    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(w), "v"(f));
+  else
+    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(w), "v"(f));
+  return r;
+}
+
 template <bool KEYSIDE, int NT>
 __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -164,8 +176,7 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const uint32_t w = (uint32_t)xr[t][e >> 1];
-          const _Float16 hv = __builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
-          float y = (float)hv * xinv[e];
+          float y = (e & 1) ? mul_half<1>(w, xinv[e]) : mul_half<0>(w, xinv[e]);
           if (KEYSIDE) {
             cd[t] = rint_code(y);
           } else {
@@ -189,8 +200,7 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const uint32_t w = (uint32_t)br[t][e >> 1];
-            const _Float16 hv = __builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu)));
-            float y = (float)hv * gt[t];
+            float y = (e & 1) ? mul_half<1>(w, gt[t]) : mul_half<0>(w, gt[t]);
             y = y * binv[e];
             cd[t] = rint_code(y);
           }
