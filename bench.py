@@ -70,12 +70,12 @@ def zoo_stage_bytes(fam, dec, B, T, H, K, V):
     if fam == "delta":
         out["wy_prep"] = qk + vv + tok + g + 2 * qk + vv + tok
     if dec == "diagonal":
-        out["gla_A"] = 2 * qk + g + A
+        out["gla_A"] = 2 * qk + g + A // 2 + qk // 2  # A in fp16, INT8 codes of the decayed query
     # the state stage of the reference reads the fp16 operands; the split pipeline adds the INT8 code round trip
     out["write_codes"] = qk + g + (qk if fam == "delta" else vv) + (tok if dec == "diagonal" else 0) + qk // 2 + \
         (qk // 2 if fam == "delta" else vv // 2)
     out["state"] = qk // 2 + h8 + ((qk // 2 + 2 * tok + 2 * vv) if fam == "delta" else vv // 2)
-    out["output"] = qk + (qk if dec != "diagonal" else A) + vv + h8 + g + vv
+    out["output"] = (2 * qk + g if dec != "diagonal" else qk // 2 + A // 2) + vv + h8 + vv
     return out
 
 

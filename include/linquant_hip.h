@@ -285,12 +285,13 @@ int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
  * (gla.py:170-232): o = dequant(q8(q).h_i8) [* exp(g)] + (fp16(A) . fp16(q8(v))) * svl, with A computed
  * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay). */
 typedef struct {
-  const void* q;             /* (B,T,H,K) fp16/bf16 */
+  const void* q;             /* no / scalar decay: (B,T,H,K) fp16/bf16; diagonal decay: NULL */
+  const int8_t* qg;          /* diagonal decay: (B,T,H,K) int8 codes of q*exp(g)*scale written by lq_zoo_gla_A */
   const void* k;             /* no / scalar decay: k or Hw (B,T,H,K) fp16/bf16; diagonal: NULL */
   const void* v;             /* local value operand: v or e_out (B,T,H,V) fp16/bf16 */
   const int8_t* h_i8;        /* (B,NT,H,V,K) */
   const float* g;            /* cumulative log decay or NULL */
-  const float* A;            /* diagonal decay: (B,T,H,C) fp32 lower-triangular intra-chunk product */
+  const void* A;             /* diagonal decay: (B,T,H,C) fp16 lower-triangular intra-chunk product */
   void* o;                   /* (B,T,H,V) fp16/bf16, or fp32 when o_is_f32 */
   int32_t o_is_f32;
   const float* sq;           /* (H,) */
@@ -309,12 +310,13 @@ int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
 /* replaces _gla_A_inter + _gla_A_intra (linquant/kernels/zoo/gla.py:27-99): intra-chunk product under
  * per-channel decay, 16-token sub-blocks: INT8 dots on anchor-rescaled operands off the diagonal, fp32
  * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows, zeros above
- * the diagonal. */
+ * the diagonal, and the INT8 codes of the decayed query (gla.py:188-190 computes them in the output kernel). */
 typedef struct {
   const void* q;             /* (B,T,H,K) fp16/bf16 */
   const void* k;             /* (B,T,H,K) fp16/bf16: k (GLA) or Hw (KDA) */
   const float* g;            /* (B,T,H,K) cumulative log decay */
-  float* A;                  /* (B,T,H,C) fp32 */
+  void* A;                   /* (B,T,H,C) fp16: the fp32 product rounded once, as the local product consumes it */
+  int8_t* qg;                /* (B,T,H,K) int8 codes q8(q*exp(g)*scale, 1/sq): the state-read operand of the output kernel */
   const void* rot;           /* (K,K) fp16 local R_QK, or NULL */
   const float* sq;
   const float* sk;

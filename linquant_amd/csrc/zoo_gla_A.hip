@@ -23,7 +23,8 @@ struct AParams {
   const _Float16* q;
   const _Float16* k;
   const float* g;
-  float* A;
+  _Float16* A;
+  int8_t* qg;
   const float* sq;
   const float* sk;
   const _Float16* rot;
@@ -91,7 +92,7 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
     // lane holds column j = rl, rows i = 4kg + r
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      p.A[((row0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (rl <= 4 * kg + r) ? acc[r] : 0.0f;
+      p.A[((row0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((rl <= 4 * kg + r) ? acc[r] : 0.0f);
     return;
   }
   // exact path: lane (i = rl, j = 4kg + jj), 8 channels per step
@@ -121,7 +122,12 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
   lq_v4f o;
 #pragma unroll
   for (int jj = 0; jj < 4; ++jj) o[jj] = (4 * kg + jj <= rl) ? s[jj] : 0.0f;
-  *(lq_v4f*)(p.A + ((row0 + rl) * H + h) * 64 + i0 + 4 * kg) = o;
+  {
+    lq_v2i oh;
+    oh[0] = (int)zoo_pack_h2(o[0], o[1]);
+    oh[1] = (int)zoo_pack_h2(o[2], o[3]);
+    *(lq_v2i*)(p.A + ((row0 + rl) * H + h) * 64 + i0 + 4 * kg) = oh;
+  }
 }
 
 template <int K, bool ROT, bool BF>
@@ -149,6 +155,28 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) rv[e] = p.rot[(int64_t)(8 * n8 + e) * K + m];
       *(lq_v8h*)(RT + m * RS + 8 * n8) = rv;
+    }
+  }
+
+  // ---- state-read operand of the output kernel: codes of q * exp(g) * scale
+  if (p.qg) {
+    for (int it = tid; it < 64 * (K / 8); it += 256) {
+      const int t = it / (K / 8), c8 = it % (K / 8);
+      const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
+      float qv[8];
+      zoo_ld8(p.q + off, bf, qv);
+      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+      int cq[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+        x = x * p.scale;
+        cq[e] = zoo_q8(x, inv_sq, qmax);
+      }
+      lq_v2i o;
+      o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
+      o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
+      *(lq_v2i*)(p.qg + off) = o;
     }
   }
 
@@ -312,12 +340,12 @@ __global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
     if (J >= wave) continue;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (float)acc[J][r] * sqk;
+      p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)((float)acc[J][r] * sqk);
   }
   // zero blocks above the diagonal
   for (int J = wave + 1; J < 4; ++J)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = 0.0f;
+    for (int r = 0; r < 4; ++r) p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)0.0f;
 }
 
 }  // namespace
@@ -329,11 +357,12 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   if (a->kdim != 64 && a->kdim != 128) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
-  if (!zoo_al(a->q, 16) || !zoo_al(a->k, 16) || !zoo_al(a->g, 16) || !zoo_al(a->A, 16)) return LQ_ERR_SHAPE;
+  if (!zoo_al(a->q, 16) || !zoo_al(a->k, 16) || !zoo_al(a->g, 16) || !zoo_al(a->A, 16) || (a->qg && !zoo_al(a->qg, 8)))
+    return LQ_ERR_SHAPE;
   if (a->rot && !zoo_al(a->rot, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   AParams p = {};
-  p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.g = a->g, p.A = a->A;
+  p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.g = a->g, p.A = (_Float16*)a->A, p.qg = a->qg;
   p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);

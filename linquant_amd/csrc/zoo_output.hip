@@ -27,7 +27,7 @@ using OutParams = ZooOutParams;
 template <bool GLA, bool USE_G, int K, bool BF>
 __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   constexpr int QS = K + 16;  // byte stride of a code row
-  __shared__ __align__(16) unsigned char qc[64 * QS];
+  __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) _Float16 Afl[GLA ? 8 : 64 * kAS];
   __shared__ __align__(16) uint32_t vP[32 * kVW];
@@ -48,29 +48,20 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   constexpr bool bf = BF;
 
   // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
+  if (!GLA)
   for (int it = tid; it < 64 * (K / 8); it += 256) {
     const int t = it / (K / 8), c8 = it % (K / 8);
     const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
     float qv[8];
     zoo_ld8(p.q + off, bf, qv);
     int cq[8];
-    if (GLA) {
-      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-        x = x * p.scale;
-        cq[e] = zoo_q8(x, inv_sq, qmax);
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
-    }
+    for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
     lq_v2i o;
     o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
     o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
     *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
-    if (!GLA) {
+    {
       float kv[8];
       zoo_ld8(p.k + off, bf, kv);
       int ck[8];
@@ -113,7 +104,8 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
-    const lq_v4i qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+    const lq_v4i qop = GLA ? *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg)
+                           : *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
       const lq_v4i hop = *(const lq_v4i*)(hp + (4 * rl + jj) * K + 64 * ks + 16 * kg);
@@ -174,13 +166,7 @@ __global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
   for (int js = 0; js < nslab; ++js) {
     lq_v8h aop;
     if (GLA) {
-      const float* ap = p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg;
-      const lq_v4f x0 = *(const lq_v4f*)ap, x1 = *(const lq_v4f*)(ap + 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        aop[e] = (_Float16)x0[e];
-        aop[4 + e] = (_Float16)x1[e];
-      }
+      aop = *(const lq_v8h*)(p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg);
     } else {
       aop = *(const lq_v8h*)(Afl + (16 * wave + rl) * kAS + 32 * js + 8 * kg);
     }
@@ -234,10 +220,10 @@ int launch(const OutParams& p, int K, dim3 grid, hipStream_t stream) {
 }  // namespace
 
 extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
-  if (!a || !a->q || !a->v || !a->h_i8 || !a->o || !a->sq || !a->svl || !a->ss) return LQ_ERR_NULL;
+  if (!a || !a->v || !a->h_i8 || !a->o || !a->sq || !a->svl || !a->ss) return LQ_ERR_NULL;
   const bool gla = a->decay == LQ_DECAY_DIAGONAL;
-  if (gla && (!a->A || !a->g)) return LQ_ERR_NULL;
-  if (!gla && (!a->k || !a->sk)) return LQ_ERR_NULL;
+  if (gla && (!a->A || !a->qg)) return LQ_ERR_NULL;
+  if (!gla && (!a->q || !a->k || !a->sk)) return LQ_ERR_NULL;
   if (a->decay == LQ_DECAY_SCALAR && !a->g) return LQ_ERR_NULL;
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
@@ -246,12 +232,12 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
-  if (!zoo_al(a->q, 16) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16))
+  if ((a->q && !zoo_al(a->q, 16)) || (a->qg && !zoo_al(a->qg, 16)) || (a->A && !zoo_al(a->A, 16)) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16))
     return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535 || a->seqlen / 64 > 65535) return LQ_ERR_SHAPE;
   OutParams p = {};
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.v = (const _Float16*)a->v;
-  p.h_i8 = a->h_i8, p.g = a->g, p.A = a->A, p.o = a->o, p.o_is_f32 = a->o_is_f32;
+  p.h_i8 = a->h_i8, p.g = a->g, p.A = (const _Float16*)a->A, p.qg = a->qg, p.o = a->o, p.o_is_f32 = a->o_is_f32;
   p.sq = a->sq, p.sk = a->sk, p.svl = a->svl, p.ss = a->ss, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   p.unrot = (const _Float16*)a->unrot;

@@ -31,7 +31,8 @@ struct ZooOutParams {
   const _Float16* v;
   const int8_t* h_i8;
   const float* g;
-  const float* A;
+  const _Float16* A;
+  const int8_t* qg;
   void* o;
   int o_is_f32;
   const float* sq;

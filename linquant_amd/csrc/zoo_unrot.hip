@@ -240,7 +240,7 @@ constexpr int kAS = 72;  // halves per row of the fp16 A tile in LDS
 template <bool GLA, bool USE_G, int K, int V>
 __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
   constexpr int QS = K + 16, VT = V / 16, RS = V + 8, VW = V + 4;
-  __shared__ __align__(16) unsigned char qc[64 * QS];
+  __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) _Float16 Afl[GLA ? 8 : 64 * kAS];
   __shared__ __align__(16) uint32_t vP[32 * VW];
@@ -263,29 +263,20 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
   // ---- phase 1: codes and tables -> LDS
   stage_rotation<V, true>(RuT_s, p.unrot, tid);
   if (tid < V) ss_s[tid] = p.ss[h * V + tid], svl_s[tid] = p.svl[h * V + tid];
+  if (!GLA)
   for (int it = tid; it < 64 * (K / 8); it += 256) {
     const int t = it / (K / 8), c8 = it % (K / 8);
     const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
     float qv[8];
     zoo_ld8(p.q + off, bf, qv);
     int cq[8];
-    if (GLA) {
-      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-        x = x * p.scale;
-        cq[e] = zoo_q8(x, inv_sq, qmax);
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
-    }
+    for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
     lq_v2i o;
     o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
     o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
     *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
-    if (!GLA) {
+    {
       float kv[8];
       zoo_ld8(p.k + off, bf, kv);
       int ck[8];
@@ -326,7 +317,8 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
   const int8_t* hp = p.h_i8 + (((int64_t)b * p.NT + ct) * H + h) * V * K;
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
-    const lq_v4i qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+    const lq_v4i qop = GLA ? *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg)
+                           : *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt)
       o32[vt] = lq_mfma_i8(*(const lq_v4i*)(hp + (16 * vt + rl) * K + 64 * ks + 16 * kg), qop, o32[vt]);
@@ -371,13 +363,7 @@ __global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
     for (int js = 0; js < nslab; ++js) {
       lq_v8h aop;
       if (GLA) {
-        const float* ap = p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg;
-        const lq_v4f x0 = *(const lq_v4f*)ap, x1 = *(const lq_v4f*)(ap + 4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          aop[e] = (_Float16)x0[e];
-          aop[4 + e] = (_Float16)x1[e];
-        }
+        aop = *(const lq_v8h*)(p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg);
       } else {
         aop = *(const lq_v8h*)(Afl + (16 * wave + rl) * kAS + 32 * js + 8 * kg);
       }

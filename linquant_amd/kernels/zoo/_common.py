@@ -89,20 +89,26 @@ def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, fa
     state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile, unrot)
 
 
-def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None):
+def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None, qg=None):
+    """``A`` (fp16) and ``qg`` (INT8 codes of the decayed query) come from run_gla_A under per-channel decay; q and key
+    are only read under no / scalar decay."""
     B, T, H, K, V = dims
-    _lib.call("lq_zoo_output", q.device, q=_lib.ptr(q), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
+    _lib.call("lq_zoo_output", value.device, q=_lib.ptr(q), qg=_lib.ptr(qg), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
               g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
               sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(q))
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(value))
 
 
-def run_gla_A(q, key, gc, A, sq, sk, scale, qmax, dims, rot=None):
+def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None):
+    """Returns (A fp16 (B,T,H,64), qg int8 (B,T,H,K)): the intra-chunk product and the codes of q*exp(g)*scale."""
     B, T, H, K, _ = dims
+    A = torch.empty(B, T, H, CHUNK, dtype=torch.float16, device=q.device)
+    qg = torch.empty(B, T, H, K, dtype=torch.int8, device=q.device)
     assert rot is None or tuple(rot.shape) == (K, K), "rot: (K, K) R_QK"
-    _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), rot=_lib.ptr(rot),
+    _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), qg=_lib.ptr(qg), rot=_lib.ptr(rot),
               sq=_lib.ptr(sq), sk=_lib.ptr(sk), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K,
               chunk_size=CHUNK, act_dtype=act_code(q))
+    return A, qg
 
 
 def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay):

@@ -27,8 +27,7 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     gc, logenv = C.cumsum(g, B, T, H, K)
     Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
-    A = torch.empty(B, T, H, chunk_size, dtype=torch.float32, device=q.device)
-    C.run_gla_A(q, Hw, gc, A, sc["q"], sc["k"], scale, qmax, dims, rot=R)
+    A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R)
     NT = T // chunk_size
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
@@ -36,6 +35,7 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     o = C.out_buffer(v, out_dtype)
     C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
                 C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru)
-    C.run_output(q, None, e_out, h_i8, gc, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL, unrot=Ru)
+    C.run_output(None, None, e_out, h_i8, None, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
+                 unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, A=A, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return o, ht
