@@ -66,10 +66,11 @@ LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl
 
 template <int DECAY, int K, bool BF>
 __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
-  constexpr int LS = K + 16;  // floats per row of X: rows 4s + kg land in disjoint bank groups
-  __shared__ __align__(16) float G_s[64 * kGS];
+  constexpr int LS = K + 8;  // floats per row of X
+  static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
   __shared__ __align__(16) float T_s[64 * kGS];
-  __shared__ __align__(16) float X_s[64 * LS];
+  __shared__ __align__(16) float X_s[64 * LS];  // 52 KB of LDS in all at K = 128: three workgroups per compute unit
+  float* G_s = X_s;
   __shared__ float gs_s[64], bs_s[64], bh_s[64];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -81,47 +82,13 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
   const float sigma = p.sigma, tau = p.tau;
   constexpr bool bf = BF;
 
-  // ---- per-token factors; Hw and fw are written straight out; X = beta^sigma k exp(g) staged for the W product
+  // ---- per-token factors; fw is written straight out
   if (tid < 64) {
     const float bt = p.beta[(t0 + tid) * H + h];
     bs_s[tid] = powb(bt, sigma);
     bh_s[tid] = powb(bt, 1.0f - sigma);
     p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
     if (DECAY == LQ_DECAY_SCALAR) gs_s[tid] = p.g[(t0 + tid) * H + h];
-  }
-  for (int it = tid; it < 64 * (K / 8); it += 256) {
-    const int r = it / (K / 8), c8 = it % (K / 8);
-    const int64_t off = ((t0 + r) * H + h) * K + 8 * c8;
-    float kv[8];
-    zoo_ld8(p.k + off, bf, kv);
-    const float bt = p.beta[(t0 + r) * H + h];
-    const float bw = powb(bt, (1.0f - sigma) * tau);
-    float bl = powb(bt, sigma);
-    if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(p.g[(t0 + r) * H + h]);
-    float ge[8];
-    if (DECAY == LQ_DECAY_DIAGONAL) {
-      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-    }
-    float hw[8];
-    lq_v4f x0, x1;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float kf = kv[e];
-      float x = bl * kf;
-      if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
-      if (e < 4) x0[e] = x; else x1[e - 4] = x;
-      hw[e] = bw * kf;
-    }
-    {
-      lq_v4i o;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
-      *(lq_v4i*)(p.Hw + off) = o;
-    }
-    *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
-    *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
   }
   __syncthreads();
 
@@ -276,6 +243,43 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
     }
     __syncthreads();
   }
+
+  // ---- Hw is written straight out; X = beta^sigma k exp(g) is staged for the W product (over the dead Gram tile)
+  for (int it = tid; it < 64 * (K / 8); it += 256) {
+    const int r = it / (K / 8), c8 = it % (K / 8);
+    const int64_t off = ((t0 + r) * H + h) * K + 8 * c8;
+    float kv[8];
+    zoo_ld8(p.k + off, bf, kv);
+    const float bt = p.beta[(t0 + r) * H + h];
+    const float bw = powb(bt, (1.0f - sigma) * tau);
+    float bl = powb(bt, sigma);
+    if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(p.g[(t0 + r) * H + h]);
+    float ge[8];
+    if (DECAY == LQ_DECAY_DIAGONAL) {
+      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+    }
+    float hw[8];
+    lq_v4f x0, x1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float kf = kv[e];
+      float x = bl * kf;
+      if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
+      if (e < 4) x0[e] = x; else x1[e - 4] = x;
+      hw[e] = bw * kf;
+    }
+    {
+      lq_v4i o;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+      *(lq_v4i*)(p.Hw + off) = o;
+    }
+    *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
+    *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
+  }
+  __syncthreads();
 
   // ---- W = T . X
   {
