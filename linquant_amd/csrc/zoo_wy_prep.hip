@@ -66,10 +66,10 @@ LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl
 
 template <int DECAY, int K, bool BF>
 __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
-  constexpr int LS = K + 8;  // floats per row of X
+  constexpr int LS = 64 + 8;  // floats per row of X: the T . X products run over 64 columns at a time
   static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
   __shared__ __align__(16) float T_s[64 * kGS];
-  __shared__ __align__(16) float X_s[64 * LS];  // 52 KB of LDS in all at K = 128: three workgroups per compute unit
+  __shared__ __align__(16) float X_s[64 * LS];  // 36 KB of LDS in all: four workgroups per compute unit
   float* G_s = X_s;
   __shared__ float gs_s[64], bs_s[64], bh_s[64];
 
@@ -244,59 +244,58 @@ __global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
     __syncthreads();
   }
 
-  // ---- Hw is written straight out; X = beta^sigma k exp(g) is staged for the W product (over the dead Gram tile)
-  for (int it = tid; it < 64 * (K / 8); it += 256) {
-    const int r = it / (K / 8), c8 = it % (K / 8);
-    const int64_t off = ((t0 + r) * H + h) * K + 8 * c8;
-    float kv[8];
-    zoo_ld8(p.k + off, bf, kv);
-    const float bt = p.beta[(t0 + r) * H + h];
-    const float bw = powb(bt, (1.0f - sigma) * tau);
-    float bl = powb(bt, sigma);
-    if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(p.g[(t0 + r) * H + h]);
-    float ge[8];
-    if (DECAY == LQ_DECAY_DIAGONAL) {
-      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+  // ---- Hw is written straight out; X = beta^sigma k exp(g) is staged 64 columns at a time (over the dead Gram tile)
+  for (int kc = 0; kc < K; kc += 64) {
+    if (kc > 0) __syncthreads();
+    for (int it = tid; it < 64 * 8; it += 256) {
+      const int r = it >> 3, c8 = it & 7;
+      const int64_t off = ((t0 + r) * H + h) * K + kc + 8 * c8;
+      float kv[8];
+      zoo_ld8(p.k + off, bf, kv);
+      const float bt = p.beta[(t0 + r) * H + h];
+      const float bw = powb(bt, (1.0f - sigma) * tau);
+      float bl = powb(bt, sigma);
+      if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(p.g[(t0 + r) * H + h]);
+      float ge[8];
+      if (DECAY == LQ_DECAY_DIAGONAL) {
+        const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-    }
-    float hw[8];
-    lq_v4f x0, x1;
+        for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+      }
+      float hw[8];
+      lq_v4f x0, x1;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float kf = kv[e];
-      float x = bl * kf;
-      if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
-      if (e < 4) x0[e] = x; else x1[e - 4] = x;
-      hw[e] = bw * kf;
-    }
-    {
-      lq_v4i o;
+      for (int e = 0; e < 8; ++e) {
+        const float kf = kv[e];
+        float x = bl * kf;
+        if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
+        if (e < 4) x0[e] = x; else x1[e - 4] = x;
+        hw[e] = bw * kf;
+      }
+      {
+        lq_v4i o;
 #pragma unroll
-      for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
-      *(lq_v4i*)(p.Hw + off) = o;
+        for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+        *(lq_v4i*)(p.Hw + off) = o;
+      }
+      *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
+      *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
     }
-    *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
-    *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
-  }
-  __syncthreads();
-
-  // ---- W = T . X
-  {
-    constexpr int NTL = K / 16;
-    for (int nt = 0; nt < NTL; ++nt) {
-      const int I = nt < NTL / 2 ? wave : 3 - wave;
+    __syncthreads();
+    // W = T . X for these 64 columns
+    for (int nt = 0; nt < 4; ++nt) {
+      const int I = nt < 2 ? wave : 3 - wave;
       const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
       lq_v2i o;
       o[0] = (int)zoo_enc2(a[0], a[1], bf);
       o[1] = (int)zoo_enc2(a[2], a[3], bf);
-      *(lq_v2i*)(p.W + ((t0 + 16 * I + rl) * H + h) * K + 16 * nt + 4 * kg) = o;
+      *(lq_v2i*)(p.W + ((t0 + 16 * I + rl) * H + h) * K + kc + 16 * nt + 4 * kg) = o;
     }
   }
 
-  // ---- U = T . (beta^sigma v), up to K value columns per pass through the X buffer
-  for (int vc = 0; vc < V; vc += K) {
-    const int pw = (V - vc) < K ? (V - vc) : K;  // 64 or K columns
+  // ---- U = T . (beta^sigma v), 64 value columns per pass through the X buffer
+  for (int vc = 0; vc < V; vc += 64) {
+    constexpr int pw = 64;
     __syncthreads();
     for (int it = tid; it < 64 * (pw / 8); it += 256) {
       const int r = it / (pw / 8), c8 = it % (pw / 8);
