@@ -237,10 +237,85 @@ def bench_zoo(args):
     print(json.dumps(line), flush=True)
 
 
+def bench_front(args):
+    """The two element-wise stages in front of the SSD prologue at the Mamba-2 2.7B shape: activation quantizer of
+    in_proj ([B*L, 2560] fp16 -> int8) and causal conv1d + SiLU on xBC ([B, L, 5376], a slice of the in_proj output)."""
+    import torch
+
+    from linquant_amd import _lib
+    from linquant_amd.kernels.mamba2.causal_conv1d import causal_conv1d_fn
+    from linquant_amd.w4a8_linear import _fused_fp16_to_int8
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    B, L, d_model, d_ssm, conv_dim, H = 4, 8192, 2560, 5120, 5376, 80
+    gen = torch.Generator().manual_seed(0)
+    hidden = torch.randn(B * L, d_model, generator=gen).half().to(dev)
+    proj = torch.randn(B, L, d_ssm + conv_dim + H, generator=gen).half().to(dev)
+    xBC = proj[..., d_ssm:d_ssm + conv_dim]
+    w = (torch.randn(conv_dim, 4, generator=gen) * 0.5).half().to(dev)
+    bias = (torch.randn(conv_dim, generator=gen) * 0.1).half().to(dev)
+    scale = torch.tensor(4.0 / 127, device=dev)
+    stages = {"fp16_to_int8": (lambda: _fused_fp16_to_int8(hidden, scale, clamp_min=-128.0, reciprocal=False), B * L * d_model * 3),
+              "causal_conv1d_silu": (lambda: causal_conv1d_fn(xBC.transpose(1, 2), w, bias, activation="silu"), B * L * conv_dim * 4)}
+
+    def step():
+        for fn, _ in stages.values():
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    out = {}
+    for name, (fn, nbytes) in stages.items():
+        ts = []
+        for _ in range(max(10, args.steps)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        med = statistics.median(ts)
+        out[name] = {"ms": round(med, 4), "MB": round(nbytes / 1e6, 1), "GBps": round(nbytes / 1e6 / med, 1),
+                     "hbm_frac": round(nbytes / 1e6 / med / HBM_PEAK_GBS, 4), "avg_ms": round(statistics.mean(ts), 4)}
+    dom = max(out, key=lambda n: out[n]["ms"])
+    nb = stages[dom][1]
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": round(nb / 1e6 / out[dom]["avg_ms"], 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(nb / 1e6 / out[dom]["avg_ms"] / HBM_PEAK_GBS, 4), "traffic": None,
+                "avg_ms": out[dom]["avg_ms"], "algorithmic_MB": round(nb / 1e6, 1)}
+    cpu = None
+    if not args.no_cpu_baseline:
+        import numpy as np
+
+        from oracle import mamba2_front as O
+
+        rows = 2048
+        hx, xs = hidden[:rows].cpu().numpy(), xBC[:1, :rows].cpu().numpy()
+        t0 = time.perf_counter()
+        O.fp16_to_int8(hx, np.float32(scale.item()), -128.0, False)
+        O.causal_conv1d_silu(xs, w.cpu().numpy(), bias.cpu().numpy())
+        t_cpu = time.perf_counter() - t0
+        cpu = {"value": round(rows / t_cpu, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
+               "sample": f"numpy oracle on {rows} of {B * L} tokens in {t_cpu:.2f} s", "host_cpus": os.cpu_count()}
+    print(json.dumps({
+        "metric": "prefill tokens/s per layer at T=8192", "value": round(B * L / ms_per_step * 1e3, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16->int8", "data": "synthetic",
+        "config": {"workload": "c5_front: in_proj activation quantizer + causal conv1d/SiLU at the Mamba-2 2.7B shape "
+                               "(B=4 L=8192 d_model=2560 conv_dim=5376 width 4)", "tokens_per_step": B * L},
+        "roofline": roofline, "cpu_baseline": cpu, "stages": out}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="c5", choices=["c5"] + list(ZOO_WORKLOADS),
+    ap.add_argument("--workload", default="c5", choices=["c5", "c5_front"] + list(ZOO_WORKLOADS),
                     help="c5 (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on; others: zoo kernels")
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
@@ -263,7 +338,7 @@ def main():
             from linquant_amd.build import build
 
             build()
-        return bench_zoo(args)
+        return bench_front(args) if args.workload == "c5_front" else bench_zoo(args)
 
     import torch
 

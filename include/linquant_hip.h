@@ -347,6 +347,36 @@ typedef struct {
 } lq_zoo_wy_prep_args;
 int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Element-wise stages in front of the Mamba-2 SSD prologue.
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces _fused_fp16_to_int8 (linquant/w4a8_linear.py:36-98): q = clamp(rint(x * (1/s)) or rint(x / s), clamp_min, 127) */
+typedef struct {
+  const void* x;             /* (M,N) fp16, unit column stride */
+  int64_t x_stride;          /* row stride in elements */
+  int8_t* out;               /* (M,N) int8 contiguous */
+  const void* scale;         /* device scalar */
+  int32_t scale_dtype;       /* LQ_DT_F16 / LQ_DT_F32 */
+  int32_t rows, cols;        /* cols a multiple of 8 */
+  float clamp_min;           /* -127 (default) or -128 */
+  int32_t reciprocal;        /* 1: x * (1/s);  0: IEEE x / s */
+} lq_fp16_to_int8_args;
+int lq_fp16_to_int8(const lq_fp16_to_int8_args* args, hipStream_t stream);
+
+/* replaces causal_conv1d_fn(x, weight, bias, activation="silu") of causal-conv1d==1.5.3.post1 as called at
+ * linquant/quantized_mamba2.py:262-268 (channel-last layout, no initial state) */
+typedef struct {
+  const void* x;             /* (B,L,D) fp16, unit D stride */
+  int64_t x_stride_b, x_stride_l;
+  const void* weight;        /* (D,W) fp16 contiguous */
+  const void* bias;          /* (D,) fp16 or NULL */
+  void* out;                 /* (B,L,D) fp16 contiguous */
+  int32_t batch, seqlen, dim, width; /* dim a multiple of 8, width 2..4 */
+  int32_t silu;              /* 1: SiLU activation, 0: none */
+} lq_causal_conv1d_args;
+int lq_causal_conv1d(const lq_causal_conv1d_args* args, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

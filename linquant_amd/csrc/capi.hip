@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 5; }
+extern "C" int lq_abi_version(void) { return 6; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)
@@ -19,6 +19,8 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_chunk_scan_args);
   LQ_SIZE_OF(lq_split_rotate_quant_xBC_args);
   LQ_SIZE_OF(lq_kron_hadamard_args);
+  LQ_SIZE_OF(lq_fp16_to_int8_args);
+  LQ_SIZE_OF(lq_causal_conv1d_args);
   LQ_SIZE_OF(lq_zoo_cumsum_args);
   LQ_SIZE_OF(lq_zoo_write_codes_args);
   LQ_SIZE_OF(lq_zoo_state_args);

@@ -35,7 +35,7 @@ def test_struct_layouts_match_the_library():
 def test_every_declaration_cites_the_reference():
     header = (ROOT / "include" / "linquant_hip.h").read_text()
     for m in re.finditer(r"/\*((?:(?!\*/).)*?)\*/\s*typedef struct", header, flags=re.S):
-        assert re.search(r"linquant/kernels/[\w/]+\.py:\d+", m.group(1)), m.group(1)[:80]
+        assert re.search(r"linquant/[\w/]+\.py:\d+", m.group(1)), m.group(1)[:80]
 
 
 def test_null_and_shape_errors_without_launch():

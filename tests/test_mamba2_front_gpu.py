@@ -1,0 +1,51 @@
+"""GPU parity (through the C ABI) of the fp16 -> int8 quantizer (bit-exact against the numpy restatement) and the
+causal conv1d + SiLU (bit-exact without the activation; with SiLU the hardware exp2 / reciprocal leave at most one
+fp16 unit in the last place at rounding boundaries)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import mamba2_front as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("reciprocal", [True, False])
+@pytest.mark.parametrize("clamp_min", [-127.0, -128.0])
+@pytest.mark.parametrize("scale_dtype", [torch.float32, torch.float16])
+def test_fused_fp16_to_int8(cuda, reciprocal, clamp_min, scale_dtype):
+    from linquant_amd.w4a8_linear import _fused_fp16_to_int8
+
+    gen = torch.Generator().manual_seed(0)
+    big = (torch.randn(300, 2560 + 64, generator=gen) * 4).half()
+    x = big[:, :2560]                                    # strided rows
+    scale = torch.tensor(0.0313, dtype=scale_dtype)
+    got = _fused_fp16_to_int8(x.cuda(), scale.cuda(), clamp_min=clamp_min, reciprocal=reciprocal)
+    torch.cuda.synchronize()
+    ref = O.fp16_to_int8(x.numpy(), np.float32(scale.float().item()), clamp_min, reciprocal)
+    assert got.dtype == torch.int8 and np.array_equal(got.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("width,bias,act", [(4, True, "silu"), (4, False, "silu"), (3, True, None), (2, True, "silu")])
+@pytest.mark.parametrize("L", [1, 37, 512])
+def test_causal_conv1d(cuda, width, bias, act, L):
+    from linquant_amd.kernels.mamba2.causal_conv1d import causal_conv1d_fn
+
+    gen = torch.Generator().manual_seed(1)
+    B, D = 2, 5376 // 4
+    proj = torch.randn(B, L, D + 40, generator=gen).half()           # xBC is a slice of the in_proj output
+    xBC = proj[..., 8:8 + D]
+    w = (torch.randn(D, width, generator=gen) * 0.5).half()
+    bs = (torch.randn(D, generator=gen) * 0.1).half() if bias else None
+    out = causal_conv1d_fn(xBC.cuda().transpose(1, 2), w.cuda(), None if bs is None else bs.cuda(), activation=act)
+    torch.cuda.synchronize()
+    assert out.shape == (B, D, L)
+    ref = O.causal_conv1d_silu(xBC.numpy(), w.numpy(), None if bs is None else bs.numpy(), silu=act is not None)
+    got = out.transpose(1, 2).cpu().numpy()
+    if act is None:
+        assert np.array_equal(got, ref)
+    else:
+        diff = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+        assert (diff <= np.spacing(np.abs(ref)).astype(np.float64)).all(), "more than one fp16 ulp apart"
+        assert (got != ref).mean() < 1e-2
