@@ -16,24 +16,39 @@ __global__ __launch_bounds__(256) void fp16_to_int8_kernel(const _Float16* __res
                                                            int scale_dtype, int rows, int cols, float clamp_min,
                                                            int reciprocal) {
   const float s = scale_dtype == LQ_DT_F16 ? (float)*(const _Float16*)scale : *(const float*)scale;
-  const float inv = 1.0f / s;
-  const int c8n = cols >> 3;  // 16-byte pieces per row
-  const int64_t total = (int64_t)rows * c8n;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    const int64_t r = i / c8n;
-    const int c = (int)(i % c8n) * 8;
-    const lq_v8h v = *(const lq_v8h*)(x + r * x_stride + c);
+  const float inv = 1.0f / s;  // correctly rounded
+  // x / s with a uniform divisor: q0 = RN(x * inv), r = x - q0 * s (exact in one fma), q = RN(q0 + r * inv) is the
+  // correctly rounded quotient whenever nothing under- or overflows (Markstein's final-quotient step). fp16 inputs span
+  // 2^-24 .. 2^16, so a scale within 2^-60 .. 2^60 keeps x, q0, r and r * inv in the normal range; outside it the plain
+  // IEEE divide runs.
+  const float as = __builtin_fabsf(s);
+  const bool fast_div = as > 0x1p-60f && as < 0x1p60f;
+  const uint32_t c8n = (uint32_t)cols >> 3;  // 16-byte pieces per row
+  const uint32_t total = (uint32_t)rows * c8n;  // the launcher rejects 2^32 pieces or more
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+    const uint32_t r = i / c8n;
+    const uint32_t c = (i - r * c8n) * 8u;
+    const lq_v8h v = *(const lq_v8h*)(x + (int64_t)r * x_stride + c);
     int code[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float xf = (float)v[e];
-      const float y = reciprocal ? xf * inv : xf / s;
+      float y = xf * inv;
+      if (!reciprocal) {
+        if (fast_div) {
+          const float rem = __builtin_fmaf(-y, s, xf);
+          const float y2 = __builtin_fmaf(rem, inv, y);
+          y = y2 == y2 ? y2 : y;  // an infinite x gives rem = NaN: keep the infinite first quotient
+        } else {
+          y = xf / s;
+        }
+      }
       code[e] = (int)fminf(fmaxf(__builtin_rintf(y), clamp_min), 127.0f);
     }
     lq_v2i o;
     o[0] = (int)lq_pack4(code[0], code[1], code[2], code[3]);
     o[1] = (int)lq_pack4(code[4], code[5], code[6], code[7]);
-    *(lq_v2i*)(out + r * cols + c) = o;
+    *(lq_v2i*)(out + (int64_t)r * cols + c) = o;
   }
 }
 
@@ -69,26 +84,32 @@ __global__ __launch_bounds__(256) void causal_conv1d_kernel(const _Float16* __re
     for (int e = 0; e < 8; ++e) win[j + 1][e] = (float)v[e];
   }
   _Float16* op = out + ((int64_t)b * L) * D + c;
+  // all rows of the block are requested before the first one is used (the clamped row index keeps a ragged last block
+  // inside the sequence; its surplus rows are computed and not stored)
+  lq_v8h rows[kTL];
+#pragma unroll
+  for (int i = 0; i < kTL; ++i) {
+    const int t = t0 + i < L ? t0 + i : L - 1;
+    rows[i] = *(const lq_v8h*)(xp + (int64_t)t * sx_l);
+  }
 #pragma unroll
   for (int i = 0; i < kTL; ++i) {
     const int t = t0 + i;
-    if (t >= L) break;
 #pragma unroll
     for (int j = 0; j < W - 1; ++j)
 #pragma unroll
       for (int e = 0; e < 8; ++e) win[j][e] = win[j + 1][e];
-    const lq_v8h v = *(const lq_v8h*)(xp + (int64_t)t * sx_l);
     lq_v8h o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      win[W - 1][e] = (float)v[e];
+      win[W - 1][e] = (float)rows[i][e];
       float a = bv[e];
 #pragma unroll
       for (int j = 0; j < W; ++j) a = a + w[j][e] * win[j][e];
       if (silu) a = a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a * -1.44269504088896340736f));
       o[e] = (_Float16)a;
     }
-    *(lq_v8h*)(op + (int64_t)t * D) = o;
+    if (t < L) *(lq_v8h*)(op + (int64_t)t * D) = o;
   }
 }
 
@@ -103,6 +124,7 @@ extern "C" int lq_fp16_to_int8(const lq_fp16_to_int8_args* a, hipStream_t stream
   if (!al(a->x, 16) || !al(a->out, 8)) return LQ_ERR_SHAPE;
   if (!(a->clamp_min >= -128.0f && a->clamp_min <= 0.0f)) return LQ_ERR_SHAPE;
   const int64_t total = (int64_t)a->rows * (a->cols / 8);
+  if (total >= ((int64_t)1 << 32) - 256 * 256 * 32) return LQ_ERR_SHAPE;  // the kernel indexes pieces in 32 bits
   const int64_t blocks = (total + 255) / 256;
   const unsigned grid = (unsigned)(blocks < 256 * 32 ? blocks : 256 * 32);
   hipLaunchKernelGGL(fp16_to_int8_kernel, dim3(grid), dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride, a->out,

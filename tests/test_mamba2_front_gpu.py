@@ -27,6 +27,27 @@ def test_fused_fp16_to_int8(cuda, reciprocal, clamp_min, scale_dtype):
     assert got.dtype == torch.int8 and np.array_equal(got.cpu().numpy(), ref)
 
 
+def test_fused_fp16_to_int8_every_fp16_value(cuda):
+    """The divide form must equal IEEE x / s for every finite or infinite fp16 input, at scales of every magnitude the
+    fast correctly-rounded quotient covers and at the extremes where the kernel falls back to the plain divide."""
+    from linquant_amd.w4a8_linear import _fused_fp16_to_int8
+
+    bits = np.arange(65536, dtype=np.uint16).view(np.float16)
+    vals = bits[~np.isnan(bits)]
+    vals = np.concatenate([vals, vals[: (-len(vals)) % 64]]).reshape(-1, 64)
+    x = torch.from_numpy(vals.copy()).cuda()
+    rng = np.random.default_rng(7)
+    scales = np.concatenate([np.exp2(rng.uniform(-12, 6, 48)), [1.0, 0.1, 1 / 3, 0.0313, 2.0 ** -70, 2.0 ** 70,
+                                                                 np.float32(1.9999999), np.float32(1.0000001)]]).astype(np.float32)
+    for sc in scales:
+        for clamp_min in (-127.0, -128.0):
+            got = _fused_fp16_to_int8(x, torch.tensor(sc, dtype=torch.float32).cuda(), clamp_min=clamp_min, reciprocal=False)
+            with np.errstate(over="ignore", invalid="ignore"):
+                ref = O.fp16_to_int8(vals, sc, clamp_min, False)
+            bad = got.cpu().numpy() != ref
+            assert not bad.any(), (float(sc), vals[bad][:4], got.cpu().numpy()[bad][:4], ref[bad][:4])
+
+
 @pytest.mark.parametrize("width,bias,act", [(4, True, "silu"), (4, False, "silu"), (3, True, None), (2, True, "silu")])
 @pytest.mark.parametrize("L", [1, 37, 512])
 def test_causal_conv1d(cuda, width, bias, act, L):

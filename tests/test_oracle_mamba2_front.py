@@ -54,3 +54,29 @@ def test_causal_conv1d_silu_against_float64():
     x2 = x.copy()
     x2[:, 20:] = 0
     assert np.array_equal(O.causal_conv1d_silu(x2, w, bias)[:, :20], O.causal_conv1d_silu(x, w, bias)[:, :20])
+
+
+def test_two_fma_quotient_equals_ieee_division():
+    """The HIP quantizer divides by a uniform scale as q0 = RN(x * RN(1/s)), r = fma(-q0, s, x), q = fma(r, RN(1/s), q0).
+    Restated here in float64 (every product of two fp32 values is exact there; the one inexact sum is checked for
+    fp32 ties) over every finite fp16 value and scales of many magnitudes: q must be the IEEE fp32 quotient."""
+    bits = np.arange(65536, dtype=np.uint16).view(np.float16)
+    x = bits[np.isfinite(bits)].astype(np.float32)
+    rng = np.random.default_rng(3)
+    scales = np.concatenate([np.exp2(rng.uniform(-59, 59, 64)), np.exp2(rng.uniform(-12, 6, 192)),
+                             [1.0, 0.1, 1 / 3, 0.0313, 1.9999999, 1.0000001]]).astype(np.float32)
+    for s in scales:
+        inv = np.float32(1.0) / s
+        q0 = (x * inv).astype(np.float32)
+        rem64 = x.astype(np.float64) - q0.astype(np.float64) * np.float64(s)
+        rem = rem64.astype(np.float32)    # float64 holds x - q0 * s exactly (at most 26 significant bits): one rounding, as the fma
+        sum64 = q0.astype(np.float64) + rem.astype(np.float64) * np.float64(inv)
+        q = sum64.astype(np.float32)
+        ref = x / s
+        differ = q != ref
+        if differ.any():
+            # a float64 sum that landed on an fp32 tie was rounded twice: decide those exactly
+            from fractions import Fraction
+            for i in np.nonzero(differ)[0]:
+                exact = Fraction(float(q0[i])) + Fraction(float(rem[i])) * Fraction(float(inv))
+                assert abs(exact - Fraction(float(ref[i]))) <= abs(exact - Fraction(float(q[i]))), (float(s), float(x[i]))
