@@ -377,6 +377,59 @@ typedef struct {
 } lq_causal_conv1d_args;
 int lq_causal_conv1d(const lq_causal_conv1d_args* args, hipStream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Stages behind the Mamba-2 SSD: gated RMSNorm and the Hadamard + INT8 quantizer of the out_proj input.
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces `self.norm(y, z)` at linquant/quantized_mamba2.py:354-358 (RMSNormGated with norm_before_gate = False and
+ * group_size = d_ssm / ngroups; the gate stays fp16):
+ *   v = x * (z * sigmoid(z));  out = fp16(v * rsqrt(mean_group(v^2) + eps) * weight), all in fp32 */
+typedef struct {
+  const void* x;             /* (rows, dim) fp16, unit column stride */
+  int64_t x_stride;          /* row stride in elements, a multiple of 8 */
+  const void* z;             /* gate, (rows, dim) fp16, or NULL for a plain RMSNorm */
+  int64_t z_stride;
+  const void* weight;        /* (dim,) */
+  int32_t weight_dtype;      /* LQ_DT_F16 / LQ_DT_F32 */
+  void* out;                 /* (rows, dim) fp16 contiguous */
+  int32_t rows, dim;         /* dim = 128 * g, g <= 64 */
+  int32_t group_size;        /* divides dim, a multiple of 8 */
+  float eps;
+} lq_rmsnorm_gated_args;
+int lq_rmsnorm_gated(const lq_rmsnorm_gated_args* args, hipStream_t stream);
+
+/* replaces qhad_transform (linquant/hadamard_utils.py:9-19), i.e. the fast_hadamard_transform_{12N,20N,28N,40N,pow2}
+ * kernels with INT8 output: q = clamp(round_half_away((H x) * scale), -127, 127) per row, H = had (x) H_128:
+ * the row is cut into g = dim / 128 contiguous chunks; chunk c' of H x is sum_c had[c'][c] * H_128 chunk_c with the
+ * Sylvester H_128.  For dim = m * 2^k, had = H_m (x) Sylvester H_(2^k / 128). */
+typedef struct {
+  const void* x;             /* (rows, dim) fp16, unit column stride */
+  int64_t x_stride;          /* row stride in elements, a multiple of 8 */
+  const int8_t* had;         /* (g, g) entries +1 / -1, row-major */
+  int8_t* out;               /* (rows, dim) int8 contiguous */
+  int32_t rows, dim;         /* dim = 128 * g, g <= 64 */
+  float scale;               /* had_scale / input_scale = 1 / (sqrt(dim) * input_scale) */
+} lq_qhad_transform_args;
+int lq_qhad_transform(const lq_qhad_transform_args* args, hipStream_t stream);
+
+/* the two stages above in one launch (linquant/quantized_mamba2.py:354-364 when d_mlp = 0): the normalized row is
+ * rounded to fp16 exactly as the separate stages would store it, but never leaves the compute unit */
+typedef struct {
+  const void* x;             /* as in lq_rmsnorm_gated_args */
+  int64_t x_stride;
+  const void* z;
+  int64_t z_stride;
+  const void* weight;
+  int32_t weight_dtype;
+  void* norm_out;            /* NULL, or (rows, dim) fp16 contiguous: the normalized rows are stored as well */
+  int32_t rows, dim, group_size;
+  float eps;
+  const int8_t* had;         /* as in lq_qhad_transform_args */
+  int8_t* out;
+  float scale;
+} lq_rmsnorm_gated_qhad_args;
+int lq_rmsnorm_gated_qhad(const lq_rmsnorm_gated_qhad_args* args, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 6; }
+extern "C" int lq_abi_version(void) { return 7; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)
@@ -21,6 +21,9 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_kron_hadamard_args);
   LQ_SIZE_OF(lq_fp16_to_int8_args);
   LQ_SIZE_OF(lq_causal_conv1d_args);
+  LQ_SIZE_OF(lq_rmsnorm_gated_args);
+  LQ_SIZE_OF(lq_qhad_transform_args);
+  LQ_SIZE_OF(lq_rmsnorm_gated_qhad_args);
   LQ_SIZE_OF(lq_zoo_cumsum_args);
   LQ_SIZE_OF(lq_zoo_write_codes_args);
   LQ_SIZE_OF(lq_zoo_state_args);

@@ -1,0 +1,372 @@
+// Stages behind the Mamba-2 SSD: gated RMSNorm and the Hadamard + INT8 quantizer of the out_proj input.
+//   lq_rmsnorm_gated       replaces `self.norm(y, z)` at linquant/quantized_mamba2.py:354-358 (RMSNormGated,
+//                          norm_before_gate = False, group_size = d_ssm / ngroups, fp16 gate)
+//   lq_qhad_transform      replaces qhad_transform (linquant/hadamard_utils.py:9-19): Hadamard of the row, scale,
+//                          round half away, saturate to +-127 (patches/ssdi8.patch:101-112)
+//   lq_rmsnorm_gated_qhad  both in one launch (linquant/quantized_mamba2.py:354-364 with d_mlp = 0)
+//
+// One wave per row, four rows per workgroup.  A row of dim = 128 g channels is a g x 128 matrix X (chunk c, position
+// i); the transform is had (g x g, any +-1 matrix) across chunks times the Sylvester H_128 inside a chunk:
+//   stage 0  16-byte loads; optional gate + group RMS statistics in fp32; the fp16 row goes to LDS as X[c][i]
+//   stage 1  D1[i, c'] = sum_c X[c, i] had[c', c]      fp16 MFMA 16x16x32, fp32 accumulate (+-1 times fp16 is exact)
+//   stage 2  D2 = H_16 . D1 over the low four bits of i  fp32 MFMA 16x16x4: the accumulator layout of stage 1 (column
+//            = lane & 15, rows 4 (lane >> 4) + r) is the B-operand layout of this product with contraction slot 4 kg + r
+//            in step r, so nothing moves between lanes
+//   stage 3  H_8 over the high three bits of i: the eight 16-row tiles of one lane, butterflies in registers
+//   stage 4  * scale, round half away, clamp, four adjacent positions per dword -> LDS -> 16-byte coalesced stores
+// HBM-bound: 2 (or 4 with the gate) bytes in and 1 byte out per channel.
+#include "lq_common.h"
+#include "../../include/linquant_hip.h"
+
+namespace {
+
+constexpr int kLS = 132;    // halves per chunk in LDS (66 dwords: the eight chunks of one operand read fall in distinct banks)
+constexpr int kOS = 144;    // bytes per chunk in the INT8 staging tile (36 dwords: the 64 lanes of one write hit 64 banks)
+constexpr int kMaxG = 64;
+
+struct EpiParams {
+  const _Float16* x;
+  int64_t x_stride;
+  const _Float16* z;
+  int64_t z_stride;
+  const void* weight;
+  int weight_f32;
+  _Float16* norm_out;
+  const int8_t* had;
+  int8_t* out;
+  int rows, dim, g, group_size;
+  float eps, scale;
+};
+
+LQ_DEV float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
+  return v;
+}
+
+// IT = 16-byte pieces per lane (g <= 4 IT); NT = 16-column tiles of had, KS = 32-chunk contraction steps that follow
+// NORM: gate + RMSNorm in front; QHAD: Hadamard + INT8 behind (false: the kernel ends after storing the normalized row)
+template <int IT, bool NORM, bool QHAD>
+__global__ __launch_bounds__(256) void epilogue_kernel(EpiParams p) {
+  constexpr int kIt = IT, NT = (IT + 3) / 4, KS = (IT + 7) / 8;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int g = p.g, g8 = (g + 7) & ~7;
+  const int wave_bytes = g8 * kLS * 2;  // >= g * kOS and >= 16 g * 4
+  _Float16* Xs = (_Float16*)(smem + (size_t)wave * wave_bytes);
+  float* Ps = (float*)Xs;               // per-piece sums of squares (before X is written)
+  unsigned char* Os = (unsigned char*)Xs;  // INT8 staging (after the last operand read)
+  const int row_raw = blockIdx.x * 4 + wave;
+  const bool live = row_raw < p.rows;
+  const int row = live ? row_raw : p.rows - 1;  // surplus waves redo the last row and store nothing
+  const int pieces = 16 * g;
+
+  lq_v8h xv[kIt];
+  if constexpr (!NORM) {
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) {
+      const int pc = it * 64 + lane;
+      xv[it] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
+      if (pc < pieces) xv[it] = *(const lq_v8h*)(p.x + (int64_t)row * p.x_stride + pc * 8);
+    }
+  }
+
+  if constexpr (NORM) {
+    float v[kIt][8];
+    float part[kIt];
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) {
+      const int pc = it * 64 + lane;
+      lq_v8h xin = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0}, zv = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
+      if (pc < pieces) xin = *(const lq_v8h*)(p.x + (int64_t)row * p.x_stride + pc * 8);
+      if (p.z && pc < pieces) zv = *(const lq_v8h*)(p.z + (int64_t)row * p.z_stride + pc * 8);
+      float s = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float a = (float)xin[e];
+        if (p.z) {
+          const float zf = (float)zv[e];
+          const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * -1.44269504088896340736f));
+          a = a * (zf * sg);
+        }
+        v[it][e] = a;
+        s = s + a * a;
+      }
+      part[it] = s;
+    }
+    const int ngroups = p.dim / p.group_size;
+    const int ppg = p.group_size >> 3;  // pieces per group
+    float rstd[kIt];
+    if (ngroups == 1) {
+      float s = 0.0f;
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) s = s + part[it];
+      s = wave_sum(s);
+      const float r = 1.0f / __builtin_sqrtf(s / (float)p.group_size + p.eps);
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) rstd[it] = r;
+    } else {
+      int grp[kIt];
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) {
+        const int pc = it * 64 + lane;
+        if (pc < pieces) Ps[pc] = part[it];
+        grp[it] = pc / ppg;
+        rstd[it] = 0.0f;
+      }
+      __syncthreads();
+      for (int gi = 0; gi < ngroups; ++gi) {
+        float s = 0.0f;
+        for (int t = lane; t < ppg; t += 64) s = s + Ps[gi * ppg + t];
+        s = wave_sum(s);
+        const float r = 1.0f / __builtin_sqrtf(s / (float)p.group_size + p.eps);
+#pragma unroll
+        for (int it = 0; it < kIt; ++it)
+          if (grp[it] == gi) rstd[it] = r;
+      }
+      __syncthreads();
+    }
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) {
+      const int pc = it * 64 + lane;
+      xv[it] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
+      if (pc < pieces) {
+        float w[8];
+        if (p.weight_f32) {
+          const lq_v4f w0 = *(const lq_v4f*)((const float*)p.weight + pc * 8);
+          const lq_v4f w1 = *(const lq_v4f*)((const float*)p.weight + pc * 8 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { w[e] = w0[e]; w[e + 4] = w1[e]; }
+        } else {
+          const lq_v8h wh = *(const lq_v8h*)((const _Float16*)p.weight + pc * 8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) w[e] = (float)wh[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float y = (v[it][e] * rstd[it]) * w[e];
+          asm volatile("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
+          xv[it][e] = (_Float16)y;
+        }
+        if (p.norm_out && live) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + pc * 8) = xv[it];
+      }
+    }
+  }
+
+  if constexpr (QHAD) {
+    // ---- stage 0: the fp16 row into LDS, chunk-major with a padded chunk stride; zero the chunks g .. g8-1 ----
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) {
+      const int pc = it * 64 + lane;
+      if (pc < pieces) {
+        const int c = pc >> 4, i0 = (pc & 15) * 8;
+        lq_v4h lo = {xv[it][0], xv[it][1], xv[it][2], xv[it][3]};
+        lq_v4h hi = {xv[it][4], xv[it][5], xv[it][6], xv[it][7]};
+        *(lq_v4h*)(Xs + c * kLS + i0) = lo;
+        *(lq_v4h*)(Xs + c * kLS + i0 + 4) = hi;
+      }
+    }
+    for (int t = lane; t < (g8 - g) * 32; t += 64) {
+      const int c = g + (t >> 5), i0 = (t & 31) * 4;
+      *(lq_v4h*)(Xs + c * kLS + i0) = lq_v4h{0, 0, 0, 0};
+    }
+
+    // operands that do not depend on the row: had^T as the B operand of stage 1, H_16 as the A operand of stage 2
+    const int n = lane & 15, kg = lane >> 4;
+    lq_v8h bop[NT][KS];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int cp = 16 * nt + n;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int c = 32 * ks + 8 * kg + j;
+          bop[nt][ks][j] = (cp < g && c < g) ? (_Float16)(float)p.had[cp * g + c] : (_Float16)0.0f;
+        }
+      }
+    float h16[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h16[r] = (__builtin_popcount(n & (4 * kg + r)) & 1) ? -1.0f : 1.0f;
+    // chunk base of this lane's contraction slots; lanes whose eight chunks lie past g8 feed zeros
+    int cbase[KS];
+    bool kvalid[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c0 = 32 * ks + 8 * kg;
+      kvalid[ks] = c0 < g8;
+      cbase[ks] = (kvalid[ks] ? c0 : 0) * kLS;
+    }
+    __syncthreads();
+
+    // ---- stage 1 ----
+    lq_v4f acc[8][NT];
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = lq_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        lq_v8h a;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) a[j] = Xs[cbase[ks] + j * kLS + 16 * mt + n];
+        if (!kvalid[ks]) a = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = lq_mfma_f16(a, bop[nt][ks], acc[mt][nt]);
+      }
+    }
+    __syncthreads();  // every operand read is done: the buffer becomes the INT8 staging tile
+
+    // ---- stage 2: H_16 over the 16 rows of each tile ----
+#pragma unroll
+    for (int mt = 0; mt < 8; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        lq_v4f d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int r = 0; r < 4; ++r) d = __builtin_amdgcn_mfma_f32_16x16x4f32(h16[r], acc[mt][nt][r], d, 0, 0, 0);
+        acc[mt][nt] = d;
+      }
+
+    // ---- stage 3: H_8 across the tiles (bits 4..6 of the position) ----
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+      for (int mt = 0; mt < 8; ++mt)
+        if ((mt & h) == 0)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const lq_v4f a = acc[mt][nt], b = acc[mt + h][nt];
+            acc[mt][nt] = a + b;
+            acc[mt + h][nt] = a - b;
+          }
+
+    // ---- stage 4 ----
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const int cp = 16 * nt + n;
+      if (cp < g) {
+#pragma unroll
+        for (int mt = 0; mt < 8; ++mt) {
+          int q[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            q[r] = (int)fminf(fmaxf(__builtin_roundf(acc[mt][nt][r] * p.scale), -127.0f), 127.0f);
+          *(uint32_t*)(Os + cp * kOS + 16 * mt + 4 * kg) = lq_pack4(q[0], q[1], q[2], q[3]);
+        }
+      }
+    }
+    __syncthreads();
+    if (live) {
+#pragma unroll
+      for (int it = 0; it < (kIt + 1) / 2; ++it) {
+        const int pc = it * 64 + lane;  // 16-byte pieces of the INT8 row: 8 per chunk
+        if (pc < 8 * g) {
+          const lq_v4i o = *(const lq_v4i*)(Os + (pc >> 3) * kOS + (pc & 7) * 16);
+          *(lq_v4i*)(p.out + (int64_t)row * p.dim + pc * 16) = o;
+        }
+      }
+    }
+  }
+}
+
+bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
+
+template <bool NORM, bool QHAD>
+int launch(const EpiParams& p, hipStream_t stream) {
+  const int g = p.g, g8 = (g + 7) & ~7;
+  const size_t lds = QHAD || (NORM && p.dim / p.group_size > 1) ? (size_t)4 * g8 * kLS * 2 : 0;
+  const dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
+#define LQ_EPI_LAUNCH(IT_)                                                                                      \
+  do {                                                                                                          \
+    if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&epilogue_kernel<IT_, NORM, QHAD>),    \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+      return LQ_ERR_LAUNCH;                                                                                     \
+    hipLaunchKernelGGL((epilogue_kernel<IT_, NORM, QHAD>), grid, block, lds, stream, p);                        \
+  } while (0)
+  const int it = (g + 3) / 4;  // pieces per lane; the instantiated sizes cover every g up to 64
+  if (it <= 1) LQ_EPI_LAUNCH(1);
+  else if (it <= 2) LQ_EPI_LAUNCH(2);
+  else if (it <= 3) LQ_EPI_LAUNCH(3);
+  else if (it <= 4) LQ_EPI_LAUNCH(4);
+  else if (it <= 5) LQ_EPI_LAUNCH(5);
+  else if (it <= 6) LQ_EPI_LAUNCH(6);
+  else if (it <= 7) LQ_EPI_LAUNCH(7);
+  else if (it <= 8) LQ_EPI_LAUNCH(8);
+  else if (it <= 10) LQ_EPI_LAUNCH(10);
+  else if (it <= 12) LQ_EPI_LAUNCH(12);
+  else if (it <= 14) LQ_EPI_LAUNCH(14);
+  else LQ_EPI_LAUNCH(16);
+#undef LQ_EPI_LAUNCH
+  return lq_check_launch();
+}
+
+int check_row_tensor(const void* x, int64_t stride, int dim) {
+  if (!x) return LQ_ERR_NULL;
+  if (stride < dim || stride % 8 != 0 || !al(x, 16)) return LQ_ERR_SHAPE;
+  return LQ_OK;
+}
+
+int check_dims(int rows, int dim) {
+  if (rows <= 0 || dim < 128 || dim % 128 != 0 || dim / 128 > kMaxG) return LQ_ERR_SHAPE;
+  return LQ_OK;
+}
+
+int check_norm(const void* weight, int weight_dtype, int dim, int group_size, float eps) {
+  if (!weight) return LQ_ERR_NULL;
+  if (weight_dtype != LQ_DT_F16 && weight_dtype != LQ_DT_F32) return LQ_ERR_SHAPE;
+  if (!al(weight, 16)) return LQ_ERR_SHAPE;
+  if (group_size <= 0 || group_size % 8 != 0 || dim % group_size != 0) return LQ_ERR_SHAPE;
+  if (!(eps >= 0.0f)) return LQ_ERR_SHAPE;
+  return LQ_OK;
+}
+
+}  // namespace
+
+extern "C" int lq_rmsnorm_gated(const lq_rmsnorm_gated_args* a, hipStream_t stream) {
+  if (!a || !a->out) return LQ_ERR_NULL;
+  int rc = check_dims(a->rows, a->dim);
+  if (rc) return rc;
+  if ((rc = check_row_tensor(a->x, a->x_stride, a->dim))) return rc;
+  if (a->z && (rc = check_row_tensor(a->z, a->z_stride, a->dim))) return rc;
+  if ((rc = check_norm(a->weight, a->weight_dtype, a->dim, a->group_size, a->eps))) return rc;
+  if (!al(a->out, 16)) return LQ_ERR_SHAPE;
+  EpiParams p{};
+  p.x = (const _Float16*)a->x; p.x_stride = a->x_stride;
+  p.z = (const _Float16*)a->z; p.z_stride = a->z_stride;
+  p.weight = a->weight; p.weight_f32 = a->weight_dtype == LQ_DT_F32;
+  p.norm_out = (_Float16*)a->out;
+  p.rows = a->rows; p.dim = a->dim; p.g = a->dim / 128; p.group_size = a->group_size; p.eps = a->eps;
+  return launch<true, false>(p, stream);
+}
+
+extern "C" int lq_qhad_transform(const lq_qhad_transform_args* a, hipStream_t stream) {
+  if (!a || !a->had || !a->out) return LQ_ERR_NULL;
+  int rc = check_dims(a->rows, a->dim);
+  if (rc) return rc;
+  if ((rc = check_row_tensor(a->x, a->x_stride, a->dim))) return rc;
+  if (!al(a->out, 16) || !(a->scale == a->scale)) return LQ_ERR_SHAPE;
+  EpiParams p{};
+  p.x = (const _Float16*)a->x; p.x_stride = a->x_stride;
+  p.had = a->had; p.out = a->out; p.scale = a->scale;
+  p.rows = a->rows; p.dim = a->dim; p.g = a->dim / 128; p.group_size = a->dim;
+  return launch<false, true>(p, stream);
+}
+
+extern "C" int lq_rmsnorm_gated_qhad(const lq_rmsnorm_gated_qhad_args* a, hipStream_t stream) {
+  if (!a || !a->had || !a->out) return LQ_ERR_NULL;
+  int rc = check_dims(a->rows, a->dim);
+  if (rc) return rc;
+  if ((rc = check_row_tensor(a->x, a->x_stride, a->dim))) return rc;
+  if (a->z && (rc = check_row_tensor(a->z, a->z_stride, a->dim))) return rc;
+  if ((rc = check_norm(a->weight, a->weight_dtype, a->dim, a->group_size, a->eps))) return rc;
+  if (!al(a->out, 16) || (a->norm_out && !al(a->norm_out, 16)) || !(a->scale == a->scale)) return LQ_ERR_SHAPE;
+  EpiParams p{};
+  p.x = (const _Float16*)a->x; p.x_stride = a->x_stride;
+  p.z = (const _Float16*)a->z; p.z_stride = a->z_stride;
+  p.weight = a->weight; p.weight_f32 = a->weight_dtype == LQ_DT_F32;
+  p.norm_out = (_Float16*)a->norm_out;
+  p.had = a->had; p.out = a->out; p.scale = a->scale;
+  p.rows = a->rows; p.dim = a->dim; p.g = a->dim / 128; p.group_size = a->group_size; p.eps = a->eps;
+  return launch<true, true>(p, stream);
+}
