@@ -259,9 +259,71 @@ def bench_front(args):
     stages = {"fp16_to_int8": (lambda: _fused_fp16_to_int8(hidden, scale, clamp_min=-128.0, reciprocal=False), B * L * d_model * 3),
               "causal_conv1d_silu": (lambda: causal_conv1d_fn(xBC.transpose(1, 2), w, bias, activation="silu"), B * L * conv_dim * 4)}
 
+    def cpu_sample():
+        import numpy as np
+
+        from oracle import mamba2_front as O
+
+        rows = 2048
+        hx, xs = hidden[:rows].cpu().numpy(), xBC[:1, :rows].cpu().numpy()
+        t0 = time.perf_counter()
+        O.fp16_to_int8(hx, np.float32(scale.item()), -128.0, False)
+        O.causal_conv1d_silu(xs, w.cpu().numpy(), bias.cpu().numpy())
+        return rows, time.perf_counter() - t0
+
+    _stage_bench(args, stages, list(stages), B * L, "fp16->int8", cpu_sample,
+                 "c5_front: in_proj activation quantizer + causal conv1d/SiLU at the Mamba-2 2.7B shape "
+                 "(B=4 L=8192 d_model=2560 conv_dim=5376 width 4)")
+
+
+def bench_epilogue(args):
+    """The stages behind the SSD at the Mamba-2 2.7B shape: gated RMSNorm of y [B, L, 5120] with the gate z (a slice
+    of the in_proj output) and the Hadamard (H_40 x H_128) + INT8 quantizer of the out_proj input.  The timed step is
+    the fused launch; the two separate launches are timed beside it."""
+    import torch
+
+    from linquant_amd import _lib
+    from linquant_amd import hadamard_utils as HU
+    from linquant_amd.norm import rmsnorm_gated, rmsnorm_gated_qhad
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    B, L, d_ssm, conv_dim, H = 4, 8192, 5120, 5376, 80
+    HU.register_hadamard(40, HU.hadamard_matrix(40))
+    gen = torch.Generator().manual_seed(0)
+    y = torch.randn(B, L, d_ssm, generator=gen).half().to(dev)
+    proj = torch.randn(B, L, d_ssm + conv_dim + H, generator=gen).half().to(dev)
+    z = proj[..., :d_ssm]
+    w = (1 + 0.1 * torch.randn(d_ssm, generator=gen)).half().to(dev)
+    input_scale = 4.0 / 127
+    normed = rmsnorm_gated(y, z, w, 1e-5, d_ssm)
+    n = B * L * d_ssm
+    stages = {"rmsnorm_gated_qhad": (lambda: rmsnorm_gated_qhad(y, z, w, input_scale, 1e-5, d_ssm), n * 5),
+              "rmsnorm_gated": (lambda: rmsnorm_gated(y, z, w, 1e-5, d_ssm), n * 6),
+              "qhad_transform": (lambda: HU.qhad_transform(normed, input_scale), n * 3)}
+
+    def cpu_sample():
+        from oracle import mamba2_epilogue as O
+
+        rows = 2048
+        yx, zx = y[0, :rows].cpu().numpy(), z[0, :rows].cpu().numpy()
+        G, wx = HU.chunk_matrix(d_ssm), w.cpu().numpy()
+        t0 = time.perf_counter()
+        O.qhad_transform(O.rmsnorm_gated(yx, zx, wx, 1e-5, d_ssm), G, (1.0 / d_ssm ** 0.5) / input_scale)
+        return rows, time.perf_counter() - t0
+
+    _stage_bench(args, stages, ["rmsnorm_gated_qhad"], B * L, "fp16->int8", cpu_sample,
+                 "c5_epilogue: gated RMSNorm + Hadamard(40 x 128) + INT8 of the out_proj input at the Mamba-2 2.7B "
+                 "shape (B=4 L=8192 d_ssm=5120, one norm group), fused launch; separate launches timed beside it")
+
+
+def _stage_bench(args, stages, step_names, tokens, dtype, cpu_sample, workload):
+    """Times `step_names` back to back as the step, every stage on its own with events, and prints the JSON line."""
+    import torch
+
     def step():
-        for fn, _ in stages.values():
-            fn()
+        for name in step_names:
+            stages[name][0]()
 
     for _ in range(args.warmup):
         step()
@@ -284,38 +346,28 @@ def bench_front(args):
         med = statistics.median(ts)
         out[name] = {"ms": round(med, 4), "MB": round(nbytes / 1e6, 1), "GBps": round(nbytes / 1e6 / med, 1),
                      "hbm_frac": round(nbytes / 1e6 / med / HBM_PEAK_GBS, 4), "avg_ms": round(statistics.mean(ts), 4)}
-    dom = max(out, key=lambda n: out[n]["ms"])
+    dom = max(step_names, key=lambda n: out[n]["ms"])
     nb = stages[dom][1]
     roofline = {"kernel": dom, "bound": "hbm", "achieved": round(nb / 1e6 / out[dom]["avg_ms"], 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(nb / 1e6 / out[dom]["avg_ms"] / HBM_PEAK_GBS, 4), "traffic": None,
                 "avg_ms": out[dom]["avg_ms"], "algorithmic_MB": round(nb / 1e6, 1)}
     cpu = None
     if not args.no_cpu_baseline:
-        import numpy as np
-
-        from oracle import mamba2_front as O
-
-        rows = 2048
-        hx, xs = hidden[:rows].cpu().numpy(), xBC[:1, :rows].cpu().numpy()
-        t0 = time.perf_counter()
-        O.fp16_to_int8(hx, np.float32(scale.item()), -128.0, False)
-        O.causal_conv1d_silu(xs, w.cpu().numpy(), bias.cpu().numpy())
-        t_cpu = time.perf_counter() - t0
+        rows, t_cpu = cpu_sample()
         cpu = {"value": round(rows / t_cpu, 1), "unit": "tokens/s", "cores": 1, "kind": "port",
-               "sample": f"numpy oracle on {rows} of {B * L} tokens in {t_cpu:.2f} s", "host_cpus": os.cpu_count()}
+               "sample": f"numpy oracle on {rows} of {tokens} tokens in {t_cpu:.2f} s", "host_cpus": os.cpu_count()}
     print(json.dumps({
-        "metric": "prefill tokens/s per layer at T=8192", "value": round(B * L / ms_per_step * 1e3, 1), "unit": "tokens/s",
+        "metric": "prefill tokens/s per layer at T=8192", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16->int8", "data": "synthetic",
-        "config": {"workload": "c5_front: in_proj activation quantizer + causal conv1d/SiLU at the Mamba-2 2.7B shape "
-                               "(B=4 L=8192 d_model=2560 conv_dim=5376 width 4)", "tokens_per_step": B * L},
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": workload, "tokens_per_step": tokens},
         "roofline": roofline, "cpu_baseline": cpu, "stages": out}), flush=True)
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c5_front"] + list(ZOO_WORKLOADS),
+    ap.add_argument("--workload", default="c5", choices=["c5", "c5_front", "c5_epilogue"] + list(ZOO_WORKLOADS),
                     help="c5 (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on; others: zoo kernels")
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
@@ -338,7 +390,7 @@ def main():
             from linquant_amd.build import build
 
             build()
-        return bench_front(args) if args.workload == "c5_front" else bench_zoo(args)
+        return {"c5_front": bench_front, "c5_epilogue": bench_epilogue}.get(args.workload, bench_zoo)(args)
 
     import torch
 

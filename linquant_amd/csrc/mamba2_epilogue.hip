@@ -5,9 +5,10 @@
 //                          round half away, saturate to +-127 (patches/ssdi8.patch:101-112)
 //   lq_rmsnorm_gated_qhad  both in one launch (linquant/quantized_mamba2.py:354-364 with d_mlp = 0)
 //
-// One wave per row, four rows per workgroup.  A row of dim = 128 g channels is a g x 128 matrix X (chunk c, position
+// One wave per row, one row per workgroup.  A row of dim = 128 g channels is a g x 128 matrix X (chunk c, position
 // i); the transform is had (g x g, any +-1 matrix) across chunks times the Sylvester H_128 inside a chunk:
-//   stage 0  16-byte loads; optional gate + group RMS statistics in fp32; the fp16 row goes to LDS as X[c][i]
+//   stage 0  16-byte loads; optional gate + group RMS statistics in fp32; the fp16 row goes to LDS with the values of two
+//            adjacent chunks at one position sharing a dword (v_permlane16_swap pairs them up in registers)
 //   stage 1  D1[i, c'] = sum_c X[c, i] had[c', c]      fp16 MFMA 16x16x32, fp32 accumulate (+-1 times fp16 is exact)
 //   stage 2  D2 = H_16 . D1 over the low four bits of i  fp32 MFMA 16x16x4: the accumulator layout of stage 1 (column
 //            = lane & 15, rows 4 (lane >> 4) + r) is the B-operand layout of this product with contraction slot 4 kg + r
@@ -20,9 +21,13 @@
 
 namespace {
 
-constexpr int kLS = 132;    // halves per chunk in LDS (66 dwords: the eight chunks of one operand read fall in distinct banks)
+typedef uint32_t lq_v2u __attribute__((ext_vector_type(2)));
+
+constexpr int kLS = 132;    // halves per chunk in LDS
+constexpr int kPS = 132;    // dwords per chunk pair in LDS (4 kPS = 16 mod 64: the four contraction groups read distinct banks)
 constexpr int kOS = 144;    // bytes per chunk in the INT8 staging tile (36 dwords: the 64 lanes of one write hit 64 banks)
 constexpr int kMaxG = 64;
+constexpr int kWaves = 1;  // rows (waves) per workgroup: single-wave workgroups keep the rows independent of each other
 
 struct EpiParams {
   const _Float16* x;
@@ -38,6 +43,11 @@ struct EpiParams {
   float eps, scale;
 };
 
+// roundf as one add: y + copysign(0.5 - 2^-25, y) lands on the next integer exactly when |y| has a fraction >= 0.5
+// (the sum of a tie k + 0.5 is k + 1 - 2^-25, which rounds to k + 1; anything below the tie stays below k + 1), and the
+// float -> int conversion truncates toward zero and saturates.
+LQ_DEV int round_half_away(float y) { return (int)(y + __builtin_copysignf(0x1.fffffep-2f, y)); }
+
 LQ_DEV float wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
@@ -47,7 +57,7 @@ LQ_DEV float wave_sum(float v) {
 // IT = 16-byte pieces per lane (g <= 4 IT); NT = 16-column tiles of had, KS = 32-chunk contraction steps that follow
 // NORM: gate + RMSNorm in front; QHAD: Hadamard + INT8 behind (false: the kernel ends after storing the normalized row)
 template <int IT, bool NORM, bool QHAD>
-__global__ __launch_bounds__(256) void epilogue_kernel(EpiParams p) {
+__global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
   constexpr int kIt = IT, NT = (IT + 3) / 4, KS = (IT + 7) / 8;
   extern __shared__ __align__(16) unsigned char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -56,7 +66,7 @@ __global__ __launch_bounds__(256) void epilogue_kernel(EpiParams p) {
   _Float16* Xs = (_Float16*)(smem + (size_t)wave * wave_bytes);
   float* Ps = (float*)Xs;               // per-piece sums of squares (before X is written)
   unsigned char* Os = (unsigned char*)Xs;  // INT8 staging (after the last operand read)
-  const int row_raw = blockIdx.x * 4 + wave;
+  const int row_raw = blockIdx.x * kWaves + wave;
   const bool live = row_raw < p.rows;
   const int row = live ? row_raw : p.rows - 1;  // surplus waves redo the last row and store nothing
   const int pieces = 16 * g;
@@ -154,48 +164,65 @@ __global__ __launch_bounds__(256) void epilogue_kernel(EpiParams p) {
   }
 
   if constexpr (QHAD) {
-    // ---- stage 0: the fp16 row into LDS, chunk-major with a padded chunk stride; zero the chunks g .. g8-1 ----
+    // ---- stage 0: the fp16 row into LDS as dwords (X[2 cp][i], X[2 cp + 1][i]) at [cp][i]: the lanes of an even and
+    // an odd 16-lane row hold the same eight positions of two adjacent chunks; two row swaps give each lane four
+    // positions of both chunks, which it interleaves and stores with one 16-byte write ----
+    uint32_t* Xp = (uint32_t*)Xs;
+    const int n = lane & 15, kg = lane >> 4;
 #pragma unroll
     for (int it = 0; it < kIt; ++it) {
-      const int pc = it * 64 + lane;
-      if (pc < pieces) {
-        const int c = pc >> 4, i0 = (pc & 15) * 8;
-        lq_v4h lo = {xv[it][0], xv[it][1], xv[it][2], xv[it][3]};
-        lq_v4h hi = {xv[it][4], xv[it][5], xv[it][6], xv[it][7]};
-        *(lq_v4h*)(Xs + c * kLS + i0) = lo;
-        *(lq_v4h*)(Xs + c * kLS + i0 + 4) = hi;
-      }
+      const lq_v4i d = __builtin_bit_cast(lq_v4i, xv[it]);  // zero for the pieces past the row
+      const lq_v2u s02 = __builtin_amdgcn_permlane16_swap((uint32_t)d[0], (uint32_t)d[2], false, false);
+      const lq_v2u s13 = __builtin_amdgcn_permlane16_swap((uint32_t)d[1], (uint32_t)d[3], false, false);
+      lq_v4i w;
+      w[0] = (int)__builtin_amdgcn_perm(s02[1], s02[0], 0x05040100u);
+      w[1] = (int)__builtin_amdgcn_perm(s02[1], s02[0], 0x07060302u);
+      w[2] = (int)__builtin_amdgcn_perm(s13[1], s13[0], 0x05040100u);
+      w[3] = (int)__builtin_amdgcn_perm(s13[1], s13[0], 0x07060302u);
+      const int cp = 2 * it + (lane >> 5);
+      if (2 * cp < g8) *(lq_v4i*)(Xp + cp * kPS + n * 8 + 4 * (kg & 1)) = w;
     }
-    for (int t = lane; t < (g8 - g) * 32; t += 64) {
-      const int c = g + (t >> 5), i0 = (t & 31) * 4;
-      *(lq_v4h*)(Xs + c * kLS + i0) = lq_v4h{0, 0, 0, 0};
-    }
+    for (int t = lane; t < (g8 / 2 - 2 * kIt) * 32; t += 64)  // chunk pairs past the last piece (g8 > 4 kIt)
+      *(lq_v4i*)(Xp + (2 * kIt + (t >> 5)) * kPS + (t & 31) * 4) = lq_v4i{0, 0, 0, 0};
 
     // operands that do not depend on the row: had^T as the B operand of stage 1, H_16 as the A operand of stage 2
-    const int n = lane & 15, kg = lane >> 4;
     lq_v8h bop[NT][KS];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const int cp = 16 * nt + n;
+        const int cp = 16 * nt + n, c0 = 32 * ks + 8 * kg;
+        if ((g & 3) == 0) {
+          // +-1 bytes -> fp16 bits: 0x3C00 with the byte's sign bit on top
+          lq_v4i hb;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int c = 32 * ks + 8 * kg + j;
-          bop[nt][ks][j] = (cp < g && c < g) ? (_Float16)(float)p.had[cp * g + c] : (_Float16)0.0f;
+          for (int hw = 0; hw < 2; ++hw) {
+            uint32_t wd = 0;
+            const bool ok = cp < g && c0 + 4 * hw < g;
+            if (ok) wd = *(const uint32_t*)(p.had + cp * g + c0 + 4 * hw);
+            const uint32_t lo = 0x3C003C00u | ((wd & 0x80u) << 8) | ((wd & 0x8000u) << 16);
+            const uint32_t hi = 0x3C003C00u | ((wd & 0x800000u) >> 8) | (wd & 0x80000000u);
+            hb[2 * hw] = ok ? (int)lo : 0;
+            hb[2 * hw + 1] = ok ? (int)hi : 0;
+          }
+          bop[nt][ks] = __builtin_bit_cast(lq_v8h, hb);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            bop[nt][ks][j] = (cp < g && c0 + j < g) ? (_Float16)(float)p.had[cp * g + c0 + j] : (_Float16)0.0f;
         }
       }
     float h16[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) h16[r] = (__builtin_popcount(n & (4 * kg + r)) & 1) ? -1.0f : 1.0f;
-    // chunk base of this lane's contraction slots; lanes whose eight chunks lie past g8 feed zeros
-    int cbase[KS];
+    // pair-row base of this lane's contraction slots; lanes whose eight chunks lie past g8 feed zeros
+    int pbase[KS];
     bool kvalid[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int c0 = 32 * ks + 8 * kg;
       kvalid[ks] = c0 < g8;
-      cbase[ks] = (kvalid[ks] ? c0 : 0) * kLS;
+      pbase[ks] = (kvalid[ks] ? c0 / 2 : 0) * kPS + n;
     }
     __syncthreads();
 
@@ -207,10 +234,11 @@ __global__ __launch_bounds__(256) void epilogue_kernel(EpiParams p) {
       for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = lq_v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        lq_v8h a;
+        lq_v4i ad;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) a[j] = Xs[cbase[ks] + j * kLS + 16 * mt + n];
-        if (!kvalid[ks]) a = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
+        for (int jp = 0; jp < 4; ++jp) ad[jp] = (int)Xp[pbase[ks] + jp * kPS + 16 * mt];
+        if (!kvalid[ks]) ad = lq_v4i{0, 0, 0, 0};
+        const lq_v8h a = __builtin_bit_cast(lq_v8h, ad);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = lq_mfma_f16(a, bop[nt][ks], acc[mt][nt]);
       }
@@ -250,8 +278,7 @@ __global__ __launch_bounds__(256) void epilogue_kernel(EpiParams p) {
         for (int mt = 0; mt < 8; ++mt) {
           int q[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            q[r] = (int)fminf(fmaxf(__builtin_roundf(acc[mt][nt][r] * p.scale), -127.0f), 127.0f);
+          for (int r = 0; r < 4; ++r) q[r] = lq_clampi(round_half_away(acc[mt][nt][r] * p.scale), -127, 127);
           *(uint32_t*)(Os + cp * kOS + 16 * mt + 4 * kg) = lq_pack4(q[0], q[1], q[2], q[3]);
         }
       }
@@ -275,8 +302,8 @@ bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
 template <bool NORM, bool QHAD>
 int launch(const EpiParams& p, hipStream_t stream) {
   const int g = p.g, g8 = (g + 7) & ~7;
-  const size_t lds = QHAD || (NORM && p.dim / p.group_size > 1) ? (size_t)4 * g8 * kLS * 2 : 0;
-  const dim3 grid((unsigned)((p.rows + 3) / 4)), block(256);
+  const size_t lds = QHAD || (NORM && p.dim / p.group_size > 1) ? (size_t)kWaves * g8 * kLS * 2 : 0;
+  const dim3 grid((unsigned)((p.rows + kWaves - 1) / kWaves)), block(64 * kWaves);
 #define LQ_EPI_LAUNCH(IT_)                                                                                      \
   do {                                                                                                          \
     if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&epilogue_kernel<IT_, NORM, QHAD>),    \
@@ -345,7 +372,7 @@ extern "C" int lq_qhad_transform(const lq_qhad_transform_args* a, hipStream_t st
   int rc = check_dims(a->rows, a->dim);
   if (rc) return rc;
   if ((rc = check_row_tensor(a->x, a->x_stride, a->dim))) return rc;
-  if (!al(a->out, 16) || !(a->scale == a->scale)) return LQ_ERR_SHAPE;
+  if (!al(a->out, 16) || !al(a->had, 4) || !(a->scale == a->scale)) return LQ_ERR_SHAPE;
   EpiParams p{};
   p.x = (const _Float16*)a->x; p.x_stride = a->x_stride;
   p.had = a->had; p.out = a->out; p.scale = a->scale;
@@ -360,7 +387,8 @@ extern "C" int lq_rmsnorm_gated_qhad(const lq_rmsnorm_gated_qhad_args* a, hipStr
   if ((rc = check_row_tensor(a->x, a->x_stride, a->dim))) return rc;
   if (a->z && (rc = check_row_tensor(a->z, a->z_stride, a->dim))) return rc;
   if ((rc = check_norm(a->weight, a->weight_dtype, a->dim, a->group_size, a->eps))) return rc;
-  if (!al(a->out, 16) || (a->norm_out && !al(a->norm_out, 16)) || !(a->scale == a->scale)) return LQ_ERR_SHAPE;
+  if (!al(a->out, 16) || !al(a->had, 4) || (a->norm_out && !al(a->norm_out, 16)) || !(a->scale == a->scale))
+    return LQ_ERR_SHAPE;
   EpiParams p{};
   p.x = (const _Float16*)a->x; p.x_stride = a->x_stride;
   p.z = (const _Float16*)a->z; p.z_stride = a->z_stride;
