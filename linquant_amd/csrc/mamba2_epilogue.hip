@@ -56,12 +56,13 @@ LQ_DEV float wave_sum(float v) {
 
 // IT = 16-byte pieces per lane (g <= 4 IT); NT = 16-column tiles of had, KS = 32-chunk contraction steps that follow
 // NORM: gate + RMSNorm in front; QHAD: Hadamard + INT8 behind (false: the kernel ends after storing the normalized row)
-template <int IT, bool NORM, bool QHAD>
-__global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
+// GATE: z is given; EXACT: g = 4 IT, every lane owns IT whole pieces and no access needs a guard
+template <int IT, bool NORM, bool QHAD, bool GATE, bool EXACT>
+__global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel(EpiParams p) {
   constexpr int kIt = IT, NT = (IT + 3) / 4, KS = (IT + 7) / 8;
   extern __shared__ __align__(16) unsigned char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int g = p.g, g8 = (g + 7) & ~7;
+  const int g = EXACT ? 4 * IT : p.g, g8 = (g + 7) & ~7;
   const int wave_bytes = g8 * kLS * 2;  // >= g * kOS and >= 16 g * 4
   _Float16* Xs = (_Float16*)(smem + (size_t)wave * wave_bytes);
   float* Ps = (float*)Xs;               // per-piece sums of squares (before X is written)
@@ -71,36 +72,45 @@ __global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
   const int row = live ? row_raw : p.rows - 1;  // surplus waves redo the last row and store nothing
   const int pieces = 16 * g;
 
-  lq_v8h xv[kIt];
-  if constexpr (!NORM) {
+  // every load is issued before the first use; a piece past the row re-reads the last one and is zeroed in registers
+  bool valid[kIt];
+  int pcc[kIt];
 #pragma unroll
-    for (int it = 0; it < kIt; ++it) {
-      const int pc = it * 64 + lane;
-      xv[it] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
-      if (pc < pieces) xv[it] = *(const lq_v8h*)(p.x + (int64_t)row * p.x_stride + pc * 8);
-    }
+  for (int it = 0; it < kIt; ++it) {
+    const int pc = it * 64 + lane;
+    valid[it] = EXACT || pc < pieces;
+    pcc[it] = EXACT ? pc : min(pc, pieces - 1);
+  }
+  lq_v8h xv[kIt];
+  {
+    const _Float16* xr = p.x + (int64_t)row * p.x_stride;
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) xv[it] = *(const lq_v8h*)(xr + pcc[it] * 8);
   }
 
   if constexpr (NORM) {
+    lq_v8h zv[GATE ? kIt : 1];
+    if constexpr (GATE) {
+      const _Float16* zr = p.z + (int64_t)row * p.z_stride;
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) zv[it] = *(const lq_v8h*)(zr + pcc[it] * 8);
+    }
     float v[kIt][8];
     float part[kIt];
 #pragma unroll
     for (int it = 0; it < kIt; ++it) {
-      const int pc = it * 64 + lane;
-      lq_v8h xin = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0}, zv = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
-      if (pc < pieces) xin = *(const lq_v8h*)(p.x + (int64_t)row * p.x_stride + pc * 8);
-      if (p.z && pc < pieces) zv = *(const lq_v8h*)(p.z + (int64_t)row * p.z_stride + pc * 8);
       float s = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float a = (float)xin[e];
-        if (p.z) {
-          const float zf = (float)zv[e];
+        float a = (float)xv[it][e];
+        if constexpr (GATE) {
+          const float zf = (float)zv[it][e];
           const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * -1.44269504088896340736f));
           a = a * (zf * sg);
         }
+        if (!valid[it]) a = 0.0f;
         v[it][e] = a;
-        s = s + a * a;
+        s = __builtin_fmaf(a, a, s);
       }
       part[it] = s;
     }
@@ -120,7 +130,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
 #pragma unroll
       for (int it = 0; it < kIt; ++it) {
         const int pc = it * 64 + lane;
-        if (pc < pieces) Ps[pc] = part[it];
+        if (valid[it]) Ps[pc] = part[it];
         grp[it] = pc / ppg;
         rstd[it] = 0.0f;
       }
@@ -138,29 +148,29 @@ __global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
     }
 #pragma unroll
     for (int it = 0; it < kIt; ++it) {
-      const int pc = it * 64 + lane;
-      xv[it] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
-      if (pc < pieces) {
-        float w[8];
-        if (p.weight_f32) {
-          const lq_v4f w0 = *(const lq_v4f*)((const float*)p.weight + pc * 8);
-          const lq_v4f w1 = *(const lq_v4f*)((const float*)p.weight + pc * 8 + 4);
+      float w[8];
+      if (p.weight_f32) {
+        const lq_v4f w0 = *(const lq_v4f*)((const float*)p.weight + pcc[it] * 8);
+        const lq_v4f w1 = *(const lq_v4f*)((const float*)p.weight + pcc[it] * 8 + 4);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) { w[e] = w0[e]; w[e + 4] = w1[e]; }
-        } else {
-          const lq_v8h wh = *(const lq_v8h*)((const _Float16*)p.weight + pc * 8);
+        for (int e = 0; e < 4; ++e) { w[e] = w0[e]; w[e + 4] = w1[e]; }
+      } else {
+        const lq_v8h wh = *(const lq_v8h*)((const _Float16*)p.weight + pcc[it] * 8);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) w[e] = (float)wh[e];
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float y = (v[it][e] * rstd[it]) * w[e];
-          asm volatile("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
-          xv[it][e] = (_Float16)y;
-        }
-        if (p.norm_out && live) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + pc * 8) = xv[it];
+        for (int e = 0; e < 8; ++e) w[e] = (float)wh[e];
       }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float y = (v[it][e] * rstd[it]) * w[e];
+        asm volatile("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
+        xv[it][e] = (_Float16)y;
+      }
+      if (p.norm_out && live && valid[it]) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + (it * 64 + lane) * 8) = xv[it];
     }
+  } else if constexpr (!EXACT) {
+#pragma unroll
+    for (int it = 0; it < kIt; ++it)
+      if (!valid[it]) xv[it] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
   }
 
   if constexpr (QHAD) {
@@ -237,7 +247,7 @@ __global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
         lq_v4i ad;
 #pragma unroll
         for (int jp = 0; jp < 4; ++jp) ad[jp] = (int)Xp[pbase[ks] + jp * kPS + 16 * mt];
-        if (!kvalid[ks]) ad = lq_v4i{0, 0, 0, 0};
+        if (!(EXACT && 32 * ks + 24 < ((4 * IT + 7) & ~7)) && !kvalid[ks]) ad = lq_v4i{0, 0, 0, 0};
         const lq_v8h a = __builtin_bit_cast(lq_v8h, ad);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = lq_mfma_f16(a, bop[nt][ks], acc[mt][nt]);
@@ -299,32 +309,32 @@ __global__ __launch_bounds__(64 * kWaves, 2) void epilogue_kernel(EpiParams p) {
 
 bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
 
-template <bool NORM, bool QHAD>
+template <bool NORM, bool QHAD, bool GATE>
 int launch(const EpiParams& p, hipStream_t stream) {
   const int g = p.g, g8 = (g + 7) & ~7;
   const size_t lds = QHAD || (NORM && p.dim / p.group_size > 1) ? (size_t)kWaves * g8 * kLS * 2 : 0;
   const dim3 grid((unsigned)((p.rows + kWaves - 1) / kWaves)), block(64 * kWaves);
-#define LQ_EPI_LAUNCH(IT_)                                                                                      \
-  do {                                                                                                          \
-    if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&epilogue_kernel<IT_, NORM, QHAD>),    \
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
-      return LQ_ERR_LAUNCH;                                                                                     \
-    hipLaunchKernelGGL((epilogue_kernel<IT_, NORM, QHAD>), grid, block, lds, stream, p);                        \
+#define LQ_EPI_LAUNCH_(IT_, EX_)                                                                                  \
+  do {                                                                                                            \
+    auto kern = &epilogue_kernel<IT_, NORM, QHAD, GATE, EX_>;                                                     \
+    if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                                   \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)   \
+      return LQ_ERR_LAUNCH;                                                                                       \
+    hipLaunchKernelGGL(kern, grid, block, lds, stream, p);                                                        \
   } while (0)
-  const int it = (g + 3) / 4;  // pieces per lane; the instantiated sizes cover every g up to 64
-  if (it <= 1) LQ_EPI_LAUNCH(1);
-  else if (it <= 2) LQ_EPI_LAUNCH(2);
-  else if (it <= 3) LQ_EPI_LAUNCH(3);
-  else if (it <= 4) LQ_EPI_LAUNCH(4);
-  else if (it <= 5) LQ_EPI_LAUNCH(5);
-  else if (it <= 6) LQ_EPI_LAUNCH(6);
-  else if (it <= 7) LQ_EPI_LAUNCH(7);
-  else if (it <= 8) LQ_EPI_LAUNCH(8);
-  else if (it <= 10) LQ_EPI_LAUNCH(10);
-  else if (it <= 12) LQ_EPI_LAUNCH(12);
-  else if (it <= 14) LQ_EPI_LAUNCH(14);
-  else LQ_EPI_LAUNCH(16);
-#undef LQ_EPI_LAUNCH
+  // sizes with g = 4 IT run the guard-free kernel; any other g runs the guarded kernel of the next multiple of 16
+#define LQ_EPI_EXACT(IT_) case IT_: LQ_EPI_LAUNCH_(IT_, true); break
+  if (g % 4 == 0 && (g / 4 <= 8 || g / 4 == 10 || g / 4 == 12 || g / 4 == 14 || g / 4 == 16)) {
+    switch (g / 4) {
+      LQ_EPI_EXACT(1); LQ_EPI_EXACT(2); LQ_EPI_EXACT(3); LQ_EPI_EXACT(4); LQ_EPI_EXACT(5); LQ_EPI_EXACT(6);
+      LQ_EPI_EXACT(7); LQ_EPI_EXACT(8); LQ_EPI_EXACT(10); LQ_EPI_EXACT(12); LQ_EPI_EXACT(14); LQ_EPI_EXACT(16);
+    }
+  } else if (g <= 16) LQ_EPI_LAUNCH_(4, false);
+  else if (g <= 32) LQ_EPI_LAUNCH_(8, false);
+  else if (g <= 48) LQ_EPI_LAUNCH_(12, false);
+  else LQ_EPI_LAUNCH_(16, false);
+#undef LQ_EPI_EXACT
+#undef LQ_EPI_LAUNCH_
   return lq_check_launch();
 }
 
@@ -364,7 +374,7 @@ extern "C" int lq_rmsnorm_gated(const lq_rmsnorm_gated_args* a, hipStream_t stre
   p.weight = a->weight; p.weight_f32 = a->weight_dtype == LQ_DT_F32;
   p.norm_out = (_Float16*)a->out;
   p.rows = a->rows; p.dim = a->dim; p.g = a->dim / 128; p.group_size = a->group_size; p.eps = a->eps;
-  return launch<true, false>(p, stream);
+  return a->z ? launch<true, false, true>(p, stream) : launch<true, false, false>(p, stream);
 }
 
 extern "C" int lq_qhad_transform(const lq_qhad_transform_args* a, hipStream_t stream) {
@@ -377,7 +387,7 @@ extern "C" int lq_qhad_transform(const lq_qhad_transform_args* a, hipStream_t st
   p.x = (const _Float16*)a->x; p.x_stride = a->x_stride;
   p.had = a->had; p.out = a->out; p.scale = a->scale;
   p.rows = a->rows; p.dim = a->dim; p.g = a->dim / 128; p.group_size = a->dim;
-  return launch<false, true>(p, stream);
+  return launch<false, true, false>(p, stream);
 }
 
 extern "C" int lq_rmsnorm_gated_qhad(const lq_rmsnorm_gated_qhad_args* a, hipStream_t stream) {
@@ -396,5 +406,5 @@ extern "C" int lq_rmsnorm_gated_qhad(const lq_rmsnorm_gated_qhad_args* a, hipStr
   p.norm_out = (_Float16*)a->norm_out;
   p.had = a->had; p.out = a->out; p.scale = a->scale;
   p.rows = a->rows; p.dim = a->dim; p.g = a->dim / 128; p.group_size = a->group_size; p.eps = a->eps;
-  return launch<true, true>(p, stream);
+  return a->z ? launch<true, true, true>(p, stream) : launch<true, true, false>(p, stream);
 }
