@@ -48,6 +48,10 @@ struct EpiParams {
 // float -> int conversion truncates toward zero and saturates.
 LQ_DEV int round_half_away(float y) { return (int)(y + __builtin_copysignf(0x1.fffffep-2f, y)); }
 
+// float(h) * f as an explicit fma with a +0 addend: the compiler selects the mixed-precision fma, which converts the
+// half exactly and rounds the product once, as a conversion followed by a multiply would (a -0 product comes out +0)
+LQ_DEV float mul_half(_Float16 h, float f) { return __builtin_fmaf((float)h, f, 0.0f); }
+
 LQ_DEV float wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
@@ -102,11 +106,12 @@ __global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel
       float s = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float a = (float)xv[it][e];
+        float a;
         if constexpr (GATE) {
-          const float zf = (float)zv[it][e];
-          const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(zf * -1.44269504088896340736f));
-          a = a * (zf * sg);
+          const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(mul_half(zv[it][e], -1.44269504088896340736f)));
+          a = mul_half(xv[it][e], mul_half(zv[it][e], sg));
+        } else {
+          a = (float)xv[it][e];
         }
         if (!valid[it]) a = 0.0f;
         v[it][e] = a;
@@ -148,22 +153,23 @@ __global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel
     }
 #pragma unroll
     for (int it = 0; it < kIt; ++it) {
-      float w[8];
       if (p.weight_f32) {
         const lq_v4f w0 = *(const lq_v4f*)((const float*)p.weight + pcc[it] * 8);
         const lq_v4f w1 = *(const lq_v4f*)((const float*)p.weight + pcc[it] * 8 + 4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { w[e] = w0[e]; w[e + 4] = w1[e]; }
+        for (int e = 0; e < 8; ++e) {
+          float y = (v[it][e] * rstd[it]) * (e < 4 ? w0[e & 3] : w1[e & 3]);
+          asm volatile("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
+          xv[it][e] = (_Float16)y;
+        }
       } else {
         const lq_v8h wh = *(const lq_v8h*)((const _Float16*)p.weight + pcc[it] * 8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) w[e] = (float)wh[e];
-      }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float y = (v[it][e] * rstd[it]) * w[e];
-        asm volatile("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
-        xv[it][e] = (_Float16)y;
+        for (int e = 0; e < 8; ++e) {
+          float y = mul_half(wh[e], v[it][e] * rstd[it]);
+          asm volatile("" : "+v"(y));  // as above
+          xv[it][e] = (_Float16)y;
+        }
       }
       if (p.norm_out && live && valid[it]) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + (it * 64 + lane) * 8) = xv[it];
     }
