@@ -63,12 +63,9 @@ LQ_DEV uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
 // exactly and rounds the product once, so the result equals the separate convert-then-multiply bit for bit.
 template <int HI>
 LQ_DEV float mul_half(uint32_t w, float f) {
-  float r;
-  if (HI)
-    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(w), "v"(f));
-  else
-    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(w), "v"(f));
-  return r;
+  // an explicit fma with a +0 addend selects v_fma_mix_f32 and leaves the hazard bookkeeping to the compiler
+  const lq_v2h h = __builtin_bit_cast(lq_v2h, w);
+  return __builtin_fmaf((float)h[HI], f, 0.0f);
 }
 
 template <bool KEYSIDE, int NT>
