@@ -88,3 +88,30 @@ def test_rmsnorm_gated_against_torch(gate, groups, wdt):
     ref = torch.nn.functional.rms_norm(xt.view(rows, groups, dim // groups), (dim // groups,), eps=1e-5).view(rows, dim)
     ref = (ref * torch.from_numpy(w).double()).numpy()
     assert (np.abs(got - ref) <= np.spacing(np.abs(ref).astype(np.float16)).astype(np.float64) * 0.51 + 1e-7).all()
+
+
+def test_one_add_rounding_is_round_half_away():
+    """The HIP quantizer rounds with trunc(y + copysign(0.5 - 2^-25, y)); it must equal round-half-away-from-zero on
+    every tie, on the neighbours of every tie and integer, and on random values (the restatement uses floor(|y| + 0.5))."""
+    F = np.float32
+    c = F(0.5) - F(2.0 ** -25)
+    assert c == F(float.fromhex("0x1.fffffep-2"))
+
+    def trick(y):
+        return np.trunc((y + np.copysign(c, y).astype(F)).astype(F))
+
+    def ref(y):
+        y64 = y.astype(np.float64)
+        return np.sign(y64) * np.floor(np.abs(y64) + 0.5)
+
+    k = np.arange(0, 1 << 16, dtype=np.float64)
+    cands = []
+    for base in (k + 0.5, k, k + 0.25):
+        b = base.astype(F)
+        cands += [b, np.nextafter(b, F(np.inf)), np.nextafter(b, F(-np.inf))]
+    y = np.concatenate(cands)
+    y = np.concatenate([y, -y])
+    assert np.array_equal(trick(y), ref(y))
+    rng = np.random.default_rng(0)
+    y = (rng.standard_normal(2_000_000) * np.exp(rng.uniform(-10, 12, 2_000_000))).astype(F)
+    assert np.array_equal(trick(y), ref(y))
