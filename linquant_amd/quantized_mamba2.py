@@ -1,0 +1,281 @@
+"""Mamba-2 mixer with every stage between the two projections on the HIP kernels of this package; the module-level
+interface of linquant/quantized_mamba2.py:36-378 (constructor keywords, calibrated buffers, forward arguments, the
+prefill-only restriction and its error messages).
+
+Pipeline of ``forward`` (linquant/quantized_mamba2.py:205-378):
+  1. activation quantizer -> in_proj -> split z0, x0, z, xBC, dt
+  2. causal conv1d + SiLU on xBC (mask applied before and after)
+  3. split + optional D_qk rescale + Kronecker-Hadamard rotation + INT8 of B, C (x stays an fp16 view); key side: fp B rotated
+  4. INT8 SSD (cumsum, chunk state, fixed-point state passing, C.B^T, chunk scan) -> fp16 y
+  5. gated RMSNorm(y, z) and 6. Hadamard + INT8 of the out_proj input -- one launch when the norm is this package's
+     RMSNormGated and d_mlp = 0 -- then out_proj and 7. the output compensation
+
+The two projections are not part of this package: ``Int8InputLinear`` stands in for the W4A8 Marlin linear with the
+same ``input_scale`` / ``forward_int8(x_i8, scale)`` surface and an fp16 GEMM from torch behind it, so the mixer runs
+end to end on a ROCm build and the stage names below can be re-bound for per-stage timing exactly like
+bench/mamba2_components.py:56-77 of the reference does.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from linquant_amd.hadamard_utils import qhad_transform
+from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+from linquant_amd.kernels.mamba2.causal_conv1d import causal_conv1d_fn
+from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC, prepare_dqk
+from linquant_amd.kernels.mamba2.ssd_combined import _quant_mamba_chunk_scan_combined_fwd
+from linquant_amd.norm import RMSNormGated, rmsnorm_gated_qhad
+from linquant_amd.w4a8_linear import _fused_fp16_to_int8
+
+
+def _apply_mask(hidden_states, attention_mask):
+    """Zero the padded positions (linquant/quantized_mamba2.py:28-33)."""
+    if attention_mask is not None and attention_mask.shape[1] > 1:
+        hidden_states = (hidden_states * attention_mask[:, :, None]).to(hidden_states.dtype)
+    return hidden_states
+
+
+class Int8InputLinear(nn.Module):
+    """Stand-in for W4A8B16O16Linear (linquant/w4a8_linear.py): INT8 activations on a per-tensor static scale, fp16
+    output.  The weight stays fp16 and the product is torch's fp16 GEMM of the dequantized activations."""
+
+    def __init__(self, weight: torch.Tensor, input_scale: torch.Tensor, bias: torch.Tensor | None = None):
+        super().__init__()
+        self.register_buffer("weight", weight.detach().to(torch.float16).contiguous())
+        self.register_buffer("input_scale", torch.as_tensor(input_scale, dtype=torch.float32).reshape(()).clone())
+        self.register_buffer("bias", None if bias is None else bias.detach().to(torch.float16))
+
+    @classmethod
+    def from_fp16(cls, linear: nn.Linear, input_scale):
+        return cls(linear.weight, input_scale, linear.bias)
+
+    def forward_int8(self, x_i8: torch.Tensor, scale) -> torch.Tensor:
+        s = scale.to(device=x_i8.device, dtype=torch.float32) if isinstance(scale, torch.Tensor) else float(scale)
+        return torch.nn.functional.linear((x_i8.to(torch.float32) * s).to(torch.float16), self.weight, self.bias)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        x2 = x.reshape(-1, x.shape[-1])
+        q = _fused_fp16_to_int8(x2, self.input_scale.to(x.device))
+        return self.forward_int8(q.view(x.shape), self.input_scale)
+
+
+class QuantizedMamba2(nn.Module):
+    """Calibrated buffers attached after construction, as in the reference: B_scale/B_inv_scale, C_scale/C_inv_scale
+    (G,), A_log_scale, D_scale (scalars), alpha_hp (H, P), bscale_g (G,), static_state_scale (H, P), static_cb_scale
+    (G,), r_signs (G, N) or None, comp_out (d_model) or absent, dqk_b/dqk_c (G*N) or absent; key side additionally
+    ``keyside = True``, x_quant_scale_hp (H, P) and b_gate_scale (1, 1, H, N)."""
+
+    def __init__(self, *, d_model, d_ssm, nheads, headdim, d_state, ngroups, d_conv, chunk_size, in_proj, out_proj,
+                 conv1d, norm, A_log, D, dt_bias, dt_limit=(0.0, float("inf")), layer_idx=None):
+        super().__init__()
+        self.d_model, self.d_ssm, self.nheads, self.headdim = d_model, d_ssm, nheads, headdim
+        self.d_state, self.ngroups, self.d_conv, self.chunk_size = d_state, ngroups, d_conv, chunk_size
+        self.dt_limit, self.layer_idx = tuple(dt_limit), layer_idx
+        self.conv_dim = d_ssm + 2 * ngroups * d_state
+        self.register_buffer("_one", torch.tensor(1.0, dtype=torch.float32))
+        self.in_proj, self.out_proj, self.conv1d, self.norm = in_proj, out_proj, conv1d, norm
+        self.register_buffer("A_log", A_log)   # INT8, dequantized in the cumsum kernel with A_log_scale
+        self.D = D                             # INT8, dequantized in the scan with D_scale
+        self.dt_bias = dt_bias
+
+    @classmethod
+    def from_fp16(cls, original_mixer, scales, r_signs):
+        """Same contract as linquant/quantized_mamba2.py:105-203: ``original_mixer`` is any module with the Mamba2
+        attributes (mamba-ssm or HF names), ``scales`` holds B/C/A_log/D scales and the two projection input scales."""
+
+        def pick(*names):
+            for n in names:
+                v = getattr(original_mixer, n, None)
+                if v is not None:
+                    return v
+            return None
+
+        nheads, headdim = pick("nheads", "num_heads"), pick("headdim", "head_dim")
+        dt_limit = pick("dt_limit", "time_step_limit") or (0.0, float("inf"))
+        q_A_log = torch.clamp(torch.round(original_mixer.A_log.float() * scales["A_log_inv_scale"]), -127, 127).to(torch.int8)
+        q_D = torch.clamp(torch.round(original_mixer.D.float() * scales["D_inv_scale"]), -127, 127).to(torch.int8)
+        module = cls(
+            d_model=pick("d_model", "hidden_size"), d_ssm=nheads * headdim, nheads=nheads, headdim=headdim,
+            d_state=pick("d_state", "ssm_state_size"), ngroups=pick("ngroups", "n_groups"),
+            d_conv=pick("d_conv", "conv_kernel_size"), chunk_size=original_mixer.chunk_size,
+            in_proj=Int8InputLinear.from_fp16(original_mixer.in_proj, scales["in_proj_input_scale"]),
+            out_proj=Int8InputLinear.from_fp16(original_mixer.out_proj, scales["out_proj_input_scale"]),
+            conv1d=original_mixer.conv1d, norm=original_mixer.norm, A_log=q_A_log, D=q_D,
+            dt_bias=original_mixer.dt_bias, dt_limit=tuple(dt_limit), layer_idx=getattr(original_mixer, "layer_idx", None))
+        module.register_buffer("r_signs", r_signs)
+        for name in ("B_scale", "B_inv_scale", "C_scale", "C_inv_scale", "A_log_scale", "D_scale"):
+            module.register_buffer(name, scales[name])
+        return module
+
+    @torch.no_grad()
+    def forward(self, hidden_states, attention_mask=None, past_key_values=None, use_cache=False,
+                output_attentions=False, **kwargs):
+        if past_key_values is not None or kwargs.get("inference_params") is not None:
+            raise NotImplementedError(
+                "QuantizedMamba2 is prefill-only: cached/stateful decoding (past_key_values, inference_params) is not "
+                "implemented; the conv history and the SSM state are not carried between calls")
+        debug = kwargs.get("_debug")
+        if hidden_states.dtype == torch.bfloat16:
+            hidden_states = hidden_states.to(torch.float16)
+
+        # 1. in_proj on INT8 activations (rint(x / s) clamped to [-128, 127])
+        if hasattr(self.in_proj, "forward_int8"):
+            s = self.in_proj.input_scale
+            h_i8 = _fused_fp16_to_int8(hidden_states.reshape(-1, hidden_states.shape[-1]), s, clamp_min=-128.0,
+                                       reciprocal=False).view(hidden_states.shape)
+            projected = self.in_proj.forward_int8(h_i8, s)
+        else:
+            h_i8 = None
+            projected = self.in_proj(hidden_states)
+        gn = self.ngroups * self.d_state
+        d_mlp = (projected.shape[-1] - 2 * self.d_ssm - 2 * gn - self.nheads) // 2
+        z0, x0, z, xBC, dt = projected.split([d_mlp, d_mlp, self.d_ssm, self.conv_dim, self.nheads], dim=-1)
+
+        # 2. causal conv1d + SiLU
+        xBC = _apply_mask(xBC, attention_mask)
+        xBC = causal_conv1d_fn(x=xBC.transpose(1, 2), weight=self.conv1d.weight.reshape(self.conv_dim, -1),
+                               bias=self.conv1d.bias, activation="silu").transpose(1, 2)
+        xBC = _apply_mask(xBC, attention_mask)
+
+        # 3. split, rotate and quantize B / C; x stays an fp16 view of xBC
+        dqk_b, dqk_c = getattr(self, "dqk_b", None), getattr(self, "dqk_c", None)
+        if dqk_b is not None:
+            if getattr(self, "_dqk_prepared", None) is None:
+                self._dqk_prepared = (prepare_dqk(dqk_b), prepare_dqk(dqk_c))
+            dqk_b, dqk_c = self._dqk_prepared
+        r_signs = getattr(self, "r_signs", None)
+        x_fp, q_B, q_C = fused_split_rotate_quant_xBC(xBC, r_signs, self.nheads, self.ngroups, self.d_state, self.headdim,
+                                                      self.B_inv_scale, self.C_inv_scale, dqk_b=dqk_b, dqk_c=dqk_c)
+        keyside = getattr(self, "keyside", False)
+        keyside_kwargs = {}
+        if keyside:  # the fp B of the key-side chunk state carries D_qk and the rotation q_B was quantized under
+            b_fp = xBC[..., self.d_ssm:self.d_ssm + gn]
+            if dqk_b is not None:
+                b_fp = b_fp * dqk_b.to(xBC.dtype)
+            b_fp = b_fp.reshape(xBC.shape[0], xBC.shape[1], self.ngroups, self.d_state).contiguous()
+            if r_signs is not None:
+                b_fp = kronecker_hadamard_fwd(b_fp, r_signs, self.ngroups)
+            keyside_kwargs = dict(keyside=True, x_scale_hp=self.x_quant_scale_hp, b_fp=b_fp, b_gate_scale=self.b_gate_scale)
+
+        # 4. INT8 SSD
+        missing = [n for n in ("alpha_hp", "bscale_g", "static_state_scale", "static_cb_scale") if not hasattr(self, n)]
+        if missing:
+            raise RuntimeError(f"QuantizedMamba2 is not calibrated: missing buffers {missing} "
+                               "(from_fp16 builds the module; the calibration step must attach these before inference)")
+        dt_limit_kwargs = {} if self.dt_limit == (0.0, float("inf")) else {"dt_limit": self.dt_limit}
+        y, _ = _quant_mamba_chunk_scan_combined_fwd(
+            x_fp=x_fp, q_dt=dt, dt_scale=self._one.to(device=dt.device), q_A_log=self.A_log, A_log_scale=self.A_log_scale,
+            q_B=q_B, B_scale=self.B_scale, q_C=q_C, C_scale=self.C_scale, chunk_size=self.chunk_size, q_D=self.D,
+            D_scale=self.D_scale, dt_bias=self.dt_bias, dt_softplus=True, alpha_hp=self.alpha_hp, bscale_g=self.bscale_g,
+            static_state_scale=self.static_state_scale, static_cb_scale=self.static_cb_scale, **keyside_kwargs,
+            **dt_limit_kwargs)
+        y = y.reshape(y.shape[0], y.shape[1], self.d_ssm)
+
+        # 5 + 6. gated RMSNorm, Hadamard + INT8 of the out_proj input
+        out_scale = self.out_proj.input_scale
+        if d_mlp == 0 and isinstance(self.norm, RMSNormGated):
+            y_i8, scale = rmsnorm_gated_qhad(y, z, self.norm.weight, out_scale, self.norm.eps, self.norm.group_size)
+            normed = None
+        else:
+            normed = self.norm(y, z)
+            if d_mlp > 0:
+                normed = torch.cat([torch.nn.functional.silu(z0) * x0, normed], dim=-1)
+            y_i8, scale = qhad_transform(normed, out_scale)
+        out = self.out_proj.forward_int8(y_i8, scale) if hasattr(self.out_proj, "forward_int8") else self.out_proj(y_i8)
+
+        # 7. output compensation
+        comp_out = getattr(self, "comp_out", None)
+        if comp_out is not None:
+            out = out + comp_out
+        if debug is not None:
+            debug.update(h_i8=h_i8, projected=projected, xBC=xBC, x_fp=x_fp, q_B=q_B, q_C=q_C, dt=dt, z=z, y=y,
+                         normed=normed, y_i8=y_i8, out=out, b_fp=keyside_kwargs.get("b_fp"))
+        return out
+
+
+def random_calibrated_mixer(*, d_model, nheads, headdim, d_state, ngroups, chunk_size, d_conv=4, batch=2, seqlen=512,
+                            keyside=False, rotate=True, seed=0, device="cuda"):
+    """A QuantizedMamba2 with random fp16 weights, calibrated on one synthetic batch (static absmax scales), for tests
+    and timing: there are no checkpoints here.  Returns (module, calibration hidden states)."""
+    import math
+    from types import SimpleNamespace
+
+    from linquant_amd import hadamard_utils as HU
+    from linquant_amd.calibration import Mamba2Shape, calibrate_mamba2, mamba2_params
+
+    g = torch.Generator().manual_seed(seed)
+    d_ssm, gn = nheads * headdim, ngroups * d_state
+    conv_dim = d_ssm + 2 * gn
+    d_in = 2 * d_ssm + 2 * gn + nheads
+    in_proj = nn.Linear(d_model, d_in, bias=False)
+    out_proj = nn.Linear(d_ssm, d_model, bias=False)
+    conv1d = nn.Conv1d(conv_dim, conv_dim, d_conv, groups=conv_dim, padding=d_conv - 1)
+    with torch.no_grad():
+        in_proj.weight.copy_(torch.randn(d_in, d_model, generator=g) / math.sqrt(d_model))
+        in_proj.weight[-nheads:] *= 0.5                                  # raw dt rows: N(-2, 0.5) after the shift below
+        out_proj.weight.copy_(torch.randn(d_model, d_ssm, generator=g) / math.sqrt(d_ssm))
+        conv1d.weight.copy_(torch.randn(conv_dim, 1, d_conv, generator=g) * 0.5)
+        conv1d.bias.copy_(torch.randn(conv_dim, generator=g) * 0.1)
+    shape = Mamba2Shape(batch=batch, seqlen=seqlen, nheads=nheads, headdim=headdim, dstate=d_state, ngroups=ngroups,
+                        chunk=chunk_size)
+    params = mamba2_params(shape, seed=seed + 42, device=device)
+    params["dt_bias"] = torch.full((nheads,), -2.0, dtype=torch.float32, device=device)
+    norm = RMSNormGated(d_ssm, eps=1e-5, group_size=d_ssm // ngroups, device=device)
+    with torch.no_grad():
+        norm.weight.copy_((1 + 0.1 * torch.randn(d_ssm, generator=g)).to(device))
+    hidden = torch.randn(batch, seqlen, d_model, generator=g).to(torch.float16).to(device)
+
+    # calibration pass in plain torch: projection, conv + SiLU, then the SSD observers
+    in_scale = hidden.float().abs().amax() / 127.0
+    w_in = in_proj.weight.to(device).half()
+    proj = torch.nn.functional.linear(hidden, w_in)
+    z, xBC_raw, dt_raw = proj.split([d_ssm, conv_dim, nheads], dim=-1)
+    xc = torch.nn.functional.conv1d(xBC_raw.float().transpose(1, 2), conv1d.weight.to(device).float(),
+                                    conv1d.bias.to(device).float(), padding=d_conv - 1, groups=conv_dim)[..., :seqlen]
+    xBC = torch.nn.functional.silu(xc).transpose(1, 2).half().contiguous()
+    if not rotate:
+        params["r_signs"] = torch.ones_like(params["r_signs"])
+    sc = calibrate_mamba2(shape, xBC, dt_raw, params)
+    scales = dict(B_scale=sc["B_scale"], B_inv_scale=sc["B_inv_scale"], C_scale=sc["C_scale"], C_inv_scale=sc["C_inv_scale"],
+                  A_log_scale=params["A_log_scale"], D_scale=params["D_scale"], A_log_inv_scale=1.0, D_inv_scale=1.0,
+                  in_proj_input_scale=in_scale, out_proj_input_scale=torch.tensor(1.0))
+    original = SimpleNamespace(nheads=nheads, headdim=headdim, d_model=d_model, d_state=d_state, ngroups=ngroups,
+                               d_conv=d_conv, chunk_size=chunk_size, in_proj=in_proj.to(device), out_proj=out_proj.to(device),
+                               conv1d=conv1d.to(device).half(), norm=norm, A_log=params["A_log"].float(), D=params["D"].float(),
+                               dt_bias=params["dt_bias"], layer_idx=0)
+    m = QuantizedMamba2.from_fp16(original, scales, params["r_signs"])
+    for name in ("alpha_hp", "bscale_g", "static_state_scale", "static_cb_scale"):
+        m.register_buffer(name, sc[name])
+    if keyside:
+        m.keyside = True
+        m.register_buffer("x_quant_scale_hp", sc["x_scale_hp"])
+        m.register_buffer("b_gate_scale", sc["b_gate_scale"])
+    m = m.to(device)
+    # out_proj input scale: absmax of the rotated normalized activations of the calibration batch
+    small = HU.small_order(d_ssm)
+    if small != 1 and small not in HU._SMALL:
+        HU.register_hadamard(small, HU.hadamard_matrix(small))
+    dbg = {}
+    plain = m.norm
+    m.norm = _Unfused(plain)
+    m(hidden, _debug=dbg)
+    m.norm = plain
+    G = torch.from_numpy(HU.chunk_matrix(d_ssm).astype("float32")).to(device)
+    rows = dbg["normed"].float().reshape(-1, d_ssm // 128, 128)
+    H128 = torch.from_numpy(HU.sylvester(128).astype("float32")).to(device)
+    rot = torch.einsum("pc,rci->rpi", G, rows) @ H128
+    m.out_proj.input_scale.copy_(rot.abs().amax() / math.sqrt(d_ssm) / 127.0)
+    return m, hidden
+
+
+class _Unfused(nn.Module):
+    """Wraps a norm so that the mixer takes the two-launch route (norm, then Hadamard + INT8)."""
+
+    def __init__(self, inner):
+        super().__init__()
+        self.inner = inner
+
+    def forward(self, x, z=None):
+        return self.inner(x, z)
