@@ -317,6 +317,101 @@ def bench_epilogue(args):
                  "shape (B=4 L=8192 d_ssm=5120, one norm group), fused launch; separate launches timed beside it")
 
 
+def bench_layer(args):
+    """One whole Mamba-2 mixer at the 2.7B shape (d_model 2560, 80 heads x 64, N 128, one group, chunk 256, B=4
+    L=8192, key side): quantizer, in_proj, conv1d + SiLU, prologue, the INT8 SSD, fused gated norm + Hadamard + INT8,
+    out_proj.  The two projections are fp16 GEMMs of torch (stand-ins for the W4A8 linears, which are outside this
+    package); every other stage is a kernel of this library.  Stages are timed with events through the re-bindable
+    stage names, the way bench/mamba2_components.py of the reference does."""
+    import torch
+
+    import linquant_amd.kernels.mamba2.ssd_combined as M
+    import linquant_amd.quantized_mamba2 as QM
+    from linquant_amd import _lib
+
+    _lib.load()
+    B, L = 4, 8192
+    layer, hidden = QM.random_calibrated_mixer(d_model=2560, nheads=80, headdim=64, d_state=128, ngroups=1, chunk_size=256,
+                                               batch=B, seqlen=L, keyside=True, seed=0)
+    torch.cuda.synchronize()
+
+    def step():
+        return layer(hidden)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    records = {}
+
+    def timed(fn, label):
+        def wrapper(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            records.setdefault(label, []).append((e0, e1))
+            return r
+        return wrapper
+
+    qm_names = {"_fused_fp16_to_int8": "act_quant", "causal_conv1d_fn": "conv1d_silu",
+                "fused_split_rotate_quant_xBC": "prologue", "kronecker_hadamard_fwd": "rotate_b_fp",
+                "rmsnorm_gated_qhad": "norm_hadamard_int8"}
+    ssd_names = {"_quant_chunk_cumsum_fwd": "chunk_cumsum", "_chunk_state_keyside_fwd": "chunk_state",
+                 "_fixedpoint_state_passing_fwd": "state_passing", "_quant_bmm_chunk_fwd": "bmm_chunk",
+                 "_chunk_scan_v2": "chunk_scan"}
+    saved_qm = {n: getattr(QM, n) for n in qm_names}
+    saved_ssd = {n: getattr(M, n) for n in ssd_names}
+    saved_lin = (layer.in_proj.forward_int8, layer.out_proj.forward_int8)
+    try:
+        for n, lab in qm_names.items():
+            setattr(QM, n, timed(saved_qm[n], lab))
+        for n, lab in ssd_names.items():
+            setattr(M, n, timed(saved_ssd[n], lab))
+        layer.in_proj.forward_int8 = timed(saved_lin[0], "in_proj_gemm_fp16_standin")
+        layer.out_proj.forward_int8 = timed(saved_lin[1], "out_proj_gemm_fp16_standin")
+        for _ in range(max(10, args.steps)):
+            step()
+        torch.cuda.synchronize()
+    finally:
+        for n, f in saved_qm.items():
+            setattr(QM, n, f)
+        for n, f in saved_ssd.items():
+            setattr(M, n, f)
+        layer.in_proj.forward_int8, layer.out_proj.forward_int8 = saved_lin
+    stages = {}
+    for label, evs in records.items():
+        ts = sorted(a.elapsed_time(b) for a, b in evs)
+        stages[label] = {"ms": round(statistics.median(ts), 4), "avg_ms": round(statistics.mean(ts), 4)}
+    native = sum(v["ms"] for k, v in stages.items() if "standin" not in k)
+    scan = stages["chunk_scan"]
+    nb = stage_bytes(Mamba2ShapeLike(B, L, 80, 64, 128, 1, 256), True)["chunk_scan"]
+    roofline = {"kernel": "chunk_scan", "bound": "hbm", "achieved": round(nb / 1e6 / scan["avg_ms"], 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(nb / 1e6 / scan["avg_ms"] / HBM_PEAK_GBS, 4), "traffic": None,
+                "avg_ms": scan["avg_ms"], "algorithmic_MB": round(nb / 1e6, 1)}
+    print(json.dumps({
+        "metric": "prefill tokens/s per layer at T=8192", "value": round(B * L / ms_per_step * 1e3, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "c5_layer: whole Mamba-2 2.7B-shape mixer (B=4 L=8192 d_model=2560 H=80 P=64 N=128 G=1 "
+                               "chunk=256, key side) with fp16 torch GEMMs standing in for the two W4A8 projections",
+                   "tokens_per_step": B * L},
+        "roofline": roofline, "cpu_baseline": None, "stages": stages,
+        "native_stages_ms": round(native, 4)}), flush=True)
+
+
+class Mamba2ShapeLike:
+    def __init__(self, batch, seqlen, nheads, headdim, dstate, ngroups, chunk):
+        self.batch, self.seqlen, self.nheads, self.headdim = batch, seqlen, nheads, headdim
+        self.dstate, self.ngroups, self.chunk = dstate, ngroups, chunk
+        self.d_ssm = nheads * headdim
+
+
 def _stage_bench(args, stages, step_names, tokens, dtype, cpu_sample, workload):
     """Times `step_names` back to back as the step, every stage on its own with events, and prints the JSON line."""
     import torch
@@ -367,7 +462,7 @@ def _stage_bench(args, stages, step_names, tokens, dtype, cpu_sample, workload):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c5_front", "c5_epilogue"] + list(ZOO_WORKLOADS),
+    ap.add_argument("--workload", default="c5", choices=["c5", "c5_front", "c5_epilogue", "c5_layer"] + list(ZOO_WORKLOADS),
                     help="c5 (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on; others: zoo kernels")
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
@@ -390,7 +485,7 @@ def main():
             from linquant_amd.build import build
 
             build()
-        return {"c5_front": bench_front, "c5_epilogue": bench_epilogue}.get(args.workload, bench_zoo)(args)
+        return {"c5_front": bench_front, "c5_epilogue": bench_epilogue, "c5_layer": bench_layer}.get(args.workload, bench_zoo)(args)
 
     import torch
 

@@ -12,7 +12,7 @@
 namespace {
 
 template <bool B_IS_FP>
-__global__ __launch_bounds__(64) void bmm_chunk_kernel(const int8_t* __restrict__ a, int64_t sa_b, int64_t sa_l,
+__global__ __launch_bounds__(64, 2) void bmm_chunk_kernel(const int8_t* __restrict__ a, int64_t sa_b, int64_t sa_l,
                                                        int64_t sa_g, const void* __restrict__ bv, int64_t sb_b,
                                                        int64_t sb_l, int64_t sb_g, const float* __restrict__ a_scale,
                                                        const float* __restrict__ b_scale,

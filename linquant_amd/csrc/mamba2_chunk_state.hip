@@ -69,7 +69,7 @@ LQ_DEV float mul_half(uint32_t w, float f) {
 }
 
 template <bool KEYSIDE, int NT>
-__global__ __launch_bounds__(256) void chunk_state_kernel(Params p) {
+__global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int Q = p.Q;
   float* gate_s = (float*)lds_raw;                    // [Q]

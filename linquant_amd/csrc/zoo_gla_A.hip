@@ -131,7 +131,7 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
 }
 
 template <int K, bool ROT, bool BF>
-__global__ __launch_bounds__(256) void zoo_gla_A_kernel(AParams p) {
+__global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
   constexpr int RS = K + 8;  // halves per row of the transposed rotation
   __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
 

@@ -25,7 +25,7 @@ constexpr int kVW = 68;  // dwords per token-pair row of the value tile
 using OutParams = ZooOutParams;
 
 template <bool GLA, bool USE_G, int K, bool BF>
-__global__ __launch_bounds__(256) void zoo_output_kernel(OutParams p) {
+__global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   constexpr int QS = K + 16;  // byte stride of a code row
   __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];

@@ -34,7 +34,7 @@ struct StepOps {
 };
 
 template <bool DELTA, int K, int BV>
-__global__ __launch_bounds__(256) void zoo_state_kernel(StateParams p) {
+__global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
   constexpr int KR = K / 4;     // carry rows per wave
   constexpr int KT = KR / 16;   // 16-row tiles per wave (= K / 64)
   constexpr int VT = BV / 16;   // 16-col tiles

@@ -238,7 +238,7 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
 constexpr int kAS = 72;  // halves per row of the fp16 A tile in LDS
 
 template <bool GLA, bool USE_G, int K, int V>
-__global__ __launch_bounds__(256) void zoo_output_unrot_kernel(ZooOutParams p) {
+__global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p) {
   constexpr int QS = K + 16, VT = V / 16, RS = V + 8, VW = V + 4;
   __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];

@@ -65,7 +65,7 @@ LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl
 }
 
 template <int DECAY, int K, bool BF>
-__global__ __launch_bounds__(256) void zoo_wy_prep_kernel(WyParams p) {
+__global__ __launch_bounds__(256, 2) void zoo_wy_prep_kernel(WyParams p) {
   constexpr int LS = 64 + 8;  // floats per row of X: the T . X products run over 64 columns at a time
   static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
   __shared__ __align__(16) float T_s[64 * kGS];
