@@ -8,8 +8,8 @@
 // and tile 2*WAVES-1-w, an early and a late one, so every wave carries the same causal work.
 //
 // LDS holds two copies of the chunk's x tile, both "token-pair interleaved" (dword (kp, p) = {x[2kp][p],
-// x[2kp+1][p]}) so that an fp16 MFMA operand (8 tokens of one channel) is four 16-byte LDS reads covering the
-// four channels {4*(lane&15)+j} of the four MFMA calls at once, with no register shuffling:
+// x[2kp+1][p]}), four token pairs of a channel adjacent, so that an fp16 MFMA operand (8 tokens of one channel) is one
+// 16-byte LDS read:
 //   xP : x as stored
 //   xS : x[k] * exp(dA_e(k) - dA_k) * S_cb * dt_k, where e(k) is the last token of k's 32-token slab.
 // For 32-token slabs strictly before a wave's rows the causal weight factors as
@@ -25,7 +25,12 @@
 
 namespace {
 
-constexpr int kRow = 68;  // LDS row stride in dwords: 64 channels + 4 pad (272 B, keeps 16-byte alignment)
+// LDS layout of an x tile: dword (kp, p) = {x[2kp][p], x[2kp+1][p]} lives at [kp >> 2][slot(p)][kp & 3] with
+// slot(p) = (p & 3) * 16 + (p >> 2): the four token pairs of one MFMA contraction group are adjacent, so the operand of
+// channel 4 * (lane & 15) + j is ONE 16-byte read at slot j * 16 + (lane & 15) (16 lanes = 256 contiguous bytes) and
+// lands in four consecutive registers without any move.
+constexpr int kQuad = 260;  // dwords per row of four token pairs: 64 channels * 4 + 4 pad (the staging stores of the
+                            // two rows a wave touches fall in different banks)
 
 struct ScanParams {
   const int8_t* cb;
@@ -65,14 +70,19 @@ LQ_DEV uint32_t pack_h2(float a, float b) {
   return __builtin_bit_cast(uint32_t, v);
 }
 
-template <int WAVES>
+// WAVES = Q / 32 wavefronts; N64 = N / 64 contraction steps of the state path
+template <int WAVES, int N64>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void chunk_scan_kernel(ScanParams p) {
+  constexpr int N = 64 * N64;
+  constexpr int kSRow = N + 16;  // bytes per state row in LDS: 16 lanes reading 16 bytes of 16 consecutive rows hit 64 banks
+  constexpr int kSPieces = (4 * N + WAVES * 64 - 1) / (WAVES * 64);  // 16-byte pieces of the 64 x N state tile per thread
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int Q = p.Q;
-  uint32_t* xP = (uint32_t*)lds_raw;          // [Q/2][kRow]
-  uint32_t* xS = xP + (Q / 2) * kRow;         // [Q/2][kRow]
-  float* dA2_s = (float*)(xS + (Q / 2) * kRow);  // dA * log2(e)
+  uint32_t* xP = (uint32_t*)lds_raw;          // [Q/8][kQuad]
+  uint32_t* xS = xP + (Q / 8) * kQuad;        // [Q/8][kQuad]
+  float* dA2_s = (float*)(xS + (Q / 8) * kQuad);  // dA * log2(e)
   float* w_s = dA2_s + Q;                     // S_cb * dt
+  int8_t* S_s = (int8_t*)(w_s + Q);           // [64][kSRow] state tile of this (chunk, head), row p at (p & 3) * 16 + (p >> 2)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -86,10 +96,36 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   const int64_t cs = (((int64_t)b * p.nheads + h) * p.nchunks + c) * Q;
   const float scb = p.cb_scale[g];
 
-  // ---- stage dA*log2e, S_cb*dt, then both x tiles
-  for (int i = tid; i < Q; i += WAVES * 64) {
-    dA2_s[i] = p.dA[cs + i] * 1.44269504088896340736f;
-    w_s[i] = scb * p.dt[cs + i];
+  // Row tiles of this wave: 16w.. and 16(2*WAVES-1-w)..: an early and a late tile, so that every wave has the same
+  // number of causal slabs to process.
+  int rb[2];
+  rb[0] = 16 * wave;
+  rb[1] = 16 * (2 * WAVES - 1 - wave);
+
+  // ---- every global load of the prologue is issued here, oldest first in the order it is needed: the state tile
+  // (one 16-byte piece per thread, shared through LDS by all waves), this wave's C rows, dA / dt, then the x tile
+  const int8_t* Sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + p0) * (int64_t)N;
+  lq_v4i spiece[kSPieces];
+#pragma unroll
+  for (int k = 0; k < kSPieces; ++k) {
+    const int t = tid + k * WAVES * 64;
+    spiece[k] = lq_v4i{0, 0, 0, 0};
+    if (t < 4 * N) spiece[k] = *(const lq_v4i*)(Sp + t * 16);
+  }
+  lq_v4i cop[2][N64];
+  {
+    const int8_t* Cp = p.C + (int64_t)b * p.sC_b + (int64_t)c * Q * p.sC_l + (int64_t)g * p.sC_g;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int coff = min(rb[i] + rl, limit - 1) * (int)p.sC_l + kg * 16;  // fits 32 bits (checked by the launcher)
+#pragma unroll
+      for (int n = 0; n < N64; ++n) cop[i][n] = *(const lq_v4i*)(Cp + coff + 64 * n);
+    }
+  }
+  float dA_r = 0.0f, dt_r = 0.0f;  // Q <= WAVES * 64: one element per thread
+  if (tid < Q) {
+    dA_r = p.dA[cs + tid];
+    dt_r = p.dt[cs + tid];
   }
   const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0;
   lq_v8h r0[2], r1[2];
@@ -118,56 +154,43 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
         Dv[j] = dsc * (float)p.D[(int64_t)h * p.sD_h + (p.D_has_hdim ? p0 + 4 * rl + j : 0)];
     }
   }
-  // Row tiles of this wave: 16w.. and 16(2*WAVES-1-w)..: an early and a late tile, so that every wave has the same
-  // number of causal slabs to process.
-  int rb[2];
-  rb[0] = 16 * wave;
-  rb[1] = 16 * (2 * WAVES - 1 - wave);
-  // ---- state path (INT8 MFMA), issued before the staging barrier so its global loads overlap the x tile's
-  lq_v4i ai[2][4];
+  if (tid < Q) {
+    dA2_s[tid] = dA_r * 1.44269504088896340736f;
+    w_s[tid] = scb * dt_r;
+  }
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ai[i][j] = lq_v4i{0, 0, 0, 0};
-  if (rb[0] < limit) {
-    const int8_t* Cp = p.C + (int64_t)b * p.sC_b + (int64_t)c * Q * p.sC_l + (int64_t)g * p.sC_g;
-    const int8_t* Sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P) * p.N;
-    for (int n0 = 0; n0 < p.N; n0 += 64) {
-      const int nn = n0 + kg * 16;
-      lq_v4i cop[2], sop[4];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int m = min(rb[i] + rl, limit - 1);
-        cop[i] = *(const lq_v4i*)(Cp + (int64_t)m * p.sC_l + nn);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) sop[j] = *(const lq_v4i*)(Sp + (int64_t)(p0 + 4 * rl + j) * p.N + nn);
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) ai[i][j] = lq_mfma_i8(cop[i], sop[j], ai[i][j]);
-    }
+  for (int k = 0; k < kSPieces; ++k) {
+    const int t = tid + k * WAVES * 64;
+    const int pr = t / (N / 16), pc = t % (N / 16);
+    if (t < 4 * N) *(lq_v4i*)(S_s + ((pr & 3) * 16 + (pr >> 2)) * kSRow + pc * 16) = spiece[k];
   }
   __syncthreads();
+  // ---- state path (INT8 MFMA): C rows from registers, state rows from LDS
+  lq_v4i ai[2][4];
+#pragma unroll
+  for (int n = 0; n < N64; ++n) {
+    lq_v4i sop[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sop[j] = *(const lq_v4i*)(S_s + (j * 16 + rl) * kSRow + 64 * n + 16 * kg);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) ai[i][j] = lq_mfma_i8(cop[i][n], sop[j], n == 0 ? lq_v4i{0, 0, 0, 0} : ai[i][j]);
+  }
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
     const int kp = kp_of[it], c8 = c8_of[it];
     const int k = 2 * kp, ke = (k | 31);
     const float ae = dA2_s[ke];
     const lq_v2h g2 = {(_Float16)(fexp2(ae - dA2_s[k]) * w_s[k]), (_Float16)(fexp2(ae - dA2_s[k + 1]) * w_s[k + 1])};
-    lq_v4i plain[2], scaled[2];
+    const int base = (kp >> 2) * kQuad + (2 * c8) * 4 + (kp & 3);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const lq_v2h pr = {r0[it][e], r1[it][e]};
-      plain[e >> 2][e & 3] = (int)__builtin_bit_cast(uint32_t, pr);
-      scaled[e >> 2][e & 3] = (int)__builtin_bit_cast(uint32_t, pr * g2);
+      const int off = base + ((e & 3) * 16 + (e >> 2)) * 4;  // x_slot(8 c8 + e) * 4
+      xP[off] = __builtin_bit_cast(uint32_t, pr);
+      xS[off] = __builtin_bit_cast(uint32_t, pr * g2);
     }
-    uint32_t* d0 = xP + kp * kRow + c8 * 8;
-    uint32_t* d1 = xS + kp * kRow + c8 * 8;
-    *(lq_v4i*)d0 = plain[0];
-    *(lq_v4i*)(d0 + 4) = plain[1];
-    *(lq_v4i*)d1 = scaled[0];
-    *(lq_v4i*)(d1 + 4) = scaled[1];
   }
   __syncthreads();
 
@@ -206,14 +229,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
         const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
         const lq_v2h s2 = {sh, sh};
         const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
-        const int kp0 = 16 * J + 4 * kg;  // token pair index of this lane's first slot
-        lq_v4i xop[4];
+        lq_v4i xop[4];  // token pairs 16 J + 4 kg .. + 3 of channel 4 rl + j
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const lq_v4i v = *(const lq_v4i*)(xS + (kp0 + d) * kRow + 4 * rl);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
-        }
+        for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xS + (4 * J + kg) * kQuad + (j * 16 + rl) * 4);
         lq_v4i aw;
         uint32_t lo, hi;
         i8x4_to_f16x4((uint32_t)cw[0], s2, o2, lo, hi);
@@ -240,11 +258,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       const int kb = sbase + 8 * kg;
       lq_v4i xop[4];
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const lq_v4i v = *(const lq_v4i*)(xP + (kb / 2 + d) * kRow + 4 * rl);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xop[j][d] = v[j];
-      }
+      for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xP + (kb >> 3) * kQuad + (j * 16 + rl) * 4);
       const lq_v4f a0 = *(const lq_v4f*)(dA2_s + kb), a1 = *(const lq_v4f*)(dA2_s + kb + 4);
       const lq_v4f w0 = *(const lq_v4f*)(w_s + kb), w1 = *(const lq_v4f*)(w_s + kb + 4);
       const lq_v2i cw = *(const lq_v2i*)(crow + kb);
@@ -268,21 +282,25 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   // ---- D residual + store
   _Float16* op = p.out + (((int64_t)b * p.seqlen + (int64_t)c * Q) * p.nheads + h) * p.P + p0 + 4 * rl;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 2; ++i) {
+    // x[m][4 rl + j] for the lane's four rows m = rb + 4 kg + r: two adjacent token pairs of one quad row
+    lq_v2i xr2[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      xr2[j] = *(const lq_v2i*)(xP + ((rb[i] >> 3) + (kg >> 1)) * kQuad + (j * 16 + rl) * 4 + 2 * (kg & 1));
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int m = rb[i] + 4 * kg + r;
       if (m >= limit) continue;
-      const lq_v4i xv = *(const lq_v4i*)(xP + (m >> 1) * kRow + 4 * rl);
       lq_v4h o;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t wv = (uint32_t)xv[j];  // rows alternate low / high half: m & 1 == r & 1
-        const _Float16 xr = __builtin_bit_cast(_Float16, (uint16_t)((r & 1) ? (wv >> 16) : (wv & 0xffffu)));
-        o[j] = (_Float16)fmaf((float)xr, Dv[j], acc[i][j][r]);
+        const lq_v2h pr = __builtin_bit_cast(lq_v2h, (uint32_t)xr2[j][r >> 1]);
+        o[j] = (_Float16)fmaf((float)pr[r & 1], Dv[j], acc[i][j][r]);
       }
       *(lq_v4h*)(op + (int64_t)m * p.nheads * p.P) = o;
     }
+  }
 }
 
 bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
@@ -313,23 +331,33 @@ extern "C" int lq_chunk_scan(const lq_chunk_scan_args* a, hipStream_t stream) {
   p.nchunks = (p.seqlen + p.Q - 1) / p.Q;
   const int64_t by = (int64_t)p.batch * p.nchunks;
   if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
-  const size_t lds = (size_t)p.Q * kRow * 4 + (size_t)p.Q * 8;  // two [Q/2][kRow] dword tiles + dA2 + w
+  if ((int64_t)p.Q * p.sC_l >= (1ll << 31) || (int64_t)p.P * p.N >= (1ll << 31)) return LQ_ERR_SHAPE;  // 32-bit lane offsets
+  const size_t lds = (size_t)2 * (p.Q / 8) * kQuad * 4 + (size_t)p.Q * 8 + (size_t)64 * (p.N + 16);  // x tiles, dA2, w, states
   dim3 grid((p.P / 64) * p.nheads, (unsigned)by, 1);
   // more than 64 KB of dynamic LDS has to be opted into per kernel
-#define LQ_SCAN_LAUNCH(W)                                                                                   \
-  do {                                                                                                      \
-    if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&chunk_scan_kernel<W>),            \
+#define LQ_SCAN_LAUNCH(W, NN)                                                                                   \
+  do {                                                                                                          \
+    if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&chunk_scan_kernel<W, NN>),            \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
-      return LQ_ERR_LAUNCH;                                                                                 \
-    hipLaunchKernelGGL(chunk_scan_kernel<W>, grid, dim3(W * 64), lds, stream, p);                           \
+      return LQ_ERR_LAUNCH;                                                                                     \
+    hipLaunchKernelGGL((chunk_scan_kernel<W, NN>), grid, dim3(W * 64), lds, stream, p);                         \
   } while (0)
+#define LQ_SCAN_N(W)                                \
+  switch (p.N / 64) {                               \
+    case 1: LQ_SCAN_LAUNCH(W, 1); break;            \
+    case 2: LQ_SCAN_LAUNCH(W, 2); break;            \
+    case 3: LQ_SCAN_LAUNCH(W, 3); break;            \
+    case 4: LQ_SCAN_LAUNCH(W, 4); break;            \
+    default: return LQ_ERR_SHAPE; /* N 64 .. 256 */    \
+  }
   switch (p.Q / 32) {
-    case 2: LQ_SCAN_LAUNCH(2); break;
-    case 4: LQ_SCAN_LAUNCH(4); break;
-    case 8: LQ_SCAN_LAUNCH(8); break;
-    case 16: LQ_SCAN_LAUNCH(16); break;
+    case 2: LQ_SCAN_N(2); break;
+    case 4: LQ_SCAN_N(4); break;
+    case 8: LQ_SCAN_N(8); break;
+    case 16: LQ_SCAN_N(16); break;
     default: return LQ_ERR_SHAPE;  // chunk sizes 64, 128, 256, 512
   }
+#undef LQ_SCAN_N
 #undef LQ_SCAN_LAUNCH
   return lq_check_launch();
 }
