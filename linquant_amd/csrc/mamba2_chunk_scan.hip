@@ -29,8 +29,9 @@ namespace {
 // slot(p) = (p & 3) * 16 + (p >> 2): the four token pairs of one MFMA contraction group are adjacent, so the operand of
 // channel 4 * (lane & 15) + j is ONE 16-byte read at slot j * 16 + (lane & 15) (16 lanes = 256 contiguous bytes) and
 // lands in four consecutive registers without any move.
-constexpr int kQuad = 260;  // dwords per row of four token pairs: 64 channels * 4 + 4 pad (the staging stores of the
-                            // two rows a wave touches fall in different banks)
+constexpr int kQuad = 256;  // dwords per row of four token pairs: 64 channels * 4, unpadded: measured with the LDS
+                            // counters, the four 16-lane groups of an operand read (rows kQuad apart) take the
+                            // minimum two passes only when kQuad is a multiple of 64 dwords (260 took four)
 
 struct ScanParams {
   const int8_t* cb;
@@ -74,7 +75,8 @@ LQ_DEV uint32_t pack_h2(float a, float b) {
 template <int WAVES, int N64>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void chunk_scan_kernel(ScanParams p) {
   constexpr int N = 64 * N64;
-  constexpr int kSRow = N + 16;  // bytes per state row in LDS: 16 lanes reading 16 bytes of 16 consecutive rows hit 64 banks
+  constexpr int kSRow = N + 32;  // bytes per state row in LDS: the pitch at which an operand read (16 rows x 4 column
+                                 // groups) takes the minimum two passes (measured; N + 16 took four)
   constexpr int kSPieces = (4 * N + WAVES * 64 - 1) / (WAVES * 64);  // 16-byte pieces of the 64 x N state tile per thread
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int Q = p.Q;
@@ -332,7 +334,7 @@ extern "C" int lq_chunk_scan(const lq_chunk_scan_args* a, hipStream_t stream) {
   const int64_t by = (int64_t)p.batch * p.nchunks;
   if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
   if ((int64_t)p.Q * p.sC_l >= (1ll << 31) || (int64_t)p.P * p.N >= (1ll << 31)) return LQ_ERR_SHAPE;  // 32-bit lane offsets
-  const size_t lds = (size_t)2 * (p.Q / 8) * kQuad * 4 + (size_t)p.Q * 8 + (size_t)64 * (p.N + 16);  // x tiles, dA2, w, states
+  const size_t lds = (size_t)2 * (p.Q / 8) * kQuad * 4 + (size_t)p.Q * 8 + (size_t)64 * (p.N + 32);  // x tiles, dA2, w, states
   dim3 grid((p.P / 64) * p.nheads, (unsigned)by, 1);
   // more than 64 KB of dynamic LDS has to be opted into per kernel
 #define LQ_SCAN_LAUNCH(W, NN)                                                                                   \
