@@ -49,7 +49,7 @@ LQ_DEV float wy_wave_max(float m) {
   return m;
 }
 
-constexpr int kGS = 68;  // floats per row of the G / T tiles: 4*row + slot hits 64 distinct banks
+constexpr int kGS = 70;  // floats per row of the G / T tiles: measured, an A-operand read (16 rows, 4 adjacent slots) takes one LDS pass when the pitch is 2 mod 4 (68 took two)
 
 // D^T tile of T . X for row block I and 16 columns starting at col: lane (rl = token, kg) gets columns col + 4kg + r
 template <int LS>
@@ -66,7 +66,7 @@ LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl
 
 template <int DECAY, int K, bool BF>
 __global__ __launch_bounds__(256, 2) void zoo_wy_prep_kernel(WyParams p) {
-  constexpr int LS = 64 + 8;  // floats per row of X: the T . X products run over 64 columns at a time
+  constexpr int LS = 64 + 16;  // floats per row of X (the T . X products run over 64 columns at a time): measured, a B-operand read (4 rows, 16 adjacent columns) takes one LDS pass at 80 floats and two at 72
   static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
   __shared__ __align__(16) float T_s[64 * kGS];
   __shared__ __align__(16) float X_s[64 * LS];  // 36 KB of LDS in all: four workgroups per compute unit
