@@ -35,8 +35,7 @@ def stage_bytes(s, keyside):
     states = B * nc * H * P * N
     cb = B * nc * G * Q * Q
     return {
-        "prologue": 2 * bc_i8 * 2 + 2 * bc_i8,
-        "rotate_b_fp": (bc_i8 * 2 * 2) if keyside else 0,
+        "prologue": 2 * bc_i8 * 2 + 2 * bc_i8 + (bc_i8 * 2 if keyside else 0),  # B, C fp16 in; codes (+ rotated fp16 B) out
         "chunk_cumsum": B * L * H * 2 + dtda,
         "chunk_state": x + (bc_i8 * 2 if keyside else bc_i8) + dtda + states,
         "state_passing": 2 * states + B * H * P * N,
@@ -513,13 +512,14 @@ def main():
     torch.cuda.synchronize()
 
     def step():
-        x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
-                                                 sc["B_inv_scale"], sc["C_inv_scale"])
         kw = {}
-        if keyside:
-            b_view = xBC[..., s.d_ssm:s.d_ssm + gn].view(s.batch, s.seqlen, s.ngroups, s.dstate)
-            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=kronecker_hadamard_fwd(b_view, p["r_signs"], s.ngroups),
-                      b_gate_scale=sc["b_gate_scale"])
+        if keyside:  # one prologue launch also stores the rotated fp16 B of the key-side chunk state
+            x, qB, qC, b_fp = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                           sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True)
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"])
+        else:
+            x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                     sc["B_inv_scale"], sc["C_inv_scale"])
         out, _ = M._quant_mamba_chunk_scan_combined_fwd(
             x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
             p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
@@ -565,15 +565,17 @@ def main():
     saved = {n: getattr(M, n) for n in names}
     for n, label in names.items():
         setattr(M, n, timed(saved[n], label))
-    fused_t, rot_t = timed(Fs.fused_split_rotate_quant_xBC, "prologue"), timed(Hm.kronecker_hadamard_fwd, "rotate_b_fp")
+    fused_t = timed(Fs.fused_split_rotate_quant_xBC, "prologue")
 
     def step_staged():
-        x, qB, qC = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"], sc["C_inv_scale"])
         kw = {}
         if keyside:
-            b_view = xBC[..., s.d_ssm:s.d_ssm + gn].view(s.batch, s.seqlen, s.ngroups, s.dstate)
-            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=rot_t(b_view, p["r_signs"], s.ngroups),
-                      b_gate_scale=sc["b_gate_scale"])
+            x, qB, qC, b_fp = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"],
+                                      sc["C_inv_scale"], return_b_fp=True)
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"])
+        else:
+            x, qB, qC = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"],
+                                sc["C_inv_scale"])
         M._quant_mamba_chunk_scan_combined_fwd(
             x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
             p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],

@@ -178,6 +178,8 @@ typedef struct {
   int64_t xBC_stride_b, xBC_stride_t;
   int8_t* qB;                /* (B,T,G,N) int8 contiguous */
   int8_t* qC;                /* (B,T,G,N) int8 contiguous */
+  void* b_fp;                /* NULL, or (B,T,G,N) fp16 contiguous: the rotated fp16 B (what q_B is quantized from), i.e.
+                                kronecker_hadamard_fwd of the [dqk-scaled] B lanes, for the key-side chunk state */
   const void* signs;         /* (G,N) +-1 values of dtype signs_dtype, or NULL for no rotation */
   int32_t signs_dtype;       /* LQ_DT_F16 / LQ_DT_F32 / LQ_DT_I8 */
   const float* B_inv_scale;  /* (G,) */

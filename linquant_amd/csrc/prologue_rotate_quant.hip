@@ -63,7 +63,7 @@ LQ_DEV void fwht_row(float* v, int sub, float hb, float kron) {
 template <int N, bool QUANT>
 __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict__ src, int64_t s_b, int64_t s_t,
                                                      int64_t s_seg, int nseg_per_side, int64_t side_off,
-                                                     void* __restrict__ dst0, void* __restrict__ dst1,
+                                                     void* __restrict__ dst0, void* __restrict__ dst1, _Float16* __restrict__ fp0,
                                                      const void* __restrict__ signs, int signs_dtype,
                                                      const float* __restrict__ inv0, const float* __restrict__ inv1,
                                                      const float* __restrict__ dqk0, const float* __restrict__ dqk1,
@@ -106,6 +106,12 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
     o[0] = (int)lq_pack4(code[0], code[1], code[2], code[3]);
     o[1] = (int)lq_pack4(code[4], code[5], code[6], code[7]);
     *(lq_v2i*)dp = o;
+    if (fp0 && side == 0) {  // the rotated fp16 B itself, for the key-side chunk state
+      lq_v8h f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = (_Float16)v[i];
+      *(lq_v8h*)(fp0 + (((int64_t)b * T + t) * nseg_per_side + seg) * N + sub * 8) = f;
+    }
   } else {
     _Float16* dp = (_Float16*)dst0 + (((int64_t)b * T + t) * nseg_per_side + seg) * N + sub * 8;
     lq_v8h o;
@@ -139,6 +145,7 @@ extern "C" int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* a
   if (a->d_ssm % 8 || a->xBC_stride_b % 8 || a->xBC_stride_t % 8 || !al(a->xBC, 16) || !al(a->qB, 8) || !al(a->qC, 8))
     return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * 2 * G > 65535) return LQ_ERR_SHAPE;
+  if (a->b_fp && !al(a->b_fp, 16)) return LQ_ERR_SHAPE;
   const _Float16* src = (const _Float16*)a->xBC + a->d_ssm;
   const float hb = hblock_value(N / 2);
   const float kron = (float)(1.0 / sqrt(2.0));
@@ -146,11 +153,11 @@ extern "C" int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* a
   dim3 grid((a->seqlen + rpb - 1) / rpb, a->batch * 2 * G);
   if (N == 128)
     hipLaunchKernelGGL((rotate_kernel<128, true>), grid, dim3(256), 0, stream, src, a->xBC_stride_b, a->xBC_stride_t,
-                       (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, a->signs, a->signs_dtype, a->B_inv_scale,
+                       (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, (_Float16*)a->b_fp, a->signs, a->signs_dtype, a->B_inv_scale,
                        a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron);
   else
     hipLaunchKernelGGL((rotate_kernel<64, true>), grid, dim3(256), 0, stream, src, a->xBC_stride_b, a->xBC_stride_t,
-                       (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, a->signs, a->signs_dtype, a->B_inv_scale,
+                       (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, (_Float16*)a->b_fp, a->signs, a->signs_dtype, a->B_inv_scale,
                        a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron);
   return lq_check_launch();
 }
@@ -168,12 +175,12 @@ extern "C" int lq_kron_hadamard(const lq_kron_hadamard_args* a, hipStream_t stre
   dim3 grid((a->seqlen + rpb - 1) / rpb, a->batch * H);
   if (D == 128)
     hipLaunchKernelGGL((rotate_kernel<128, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
-                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, a->signs, a->signs_dtype,
+                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                        a->seqlen, hb, kron);
   else
     hipLaunchKernelGGL((rotate_kernel<64, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
-                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, a->signs, a->signs_dtype,
+                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                        a->seqlen, hb, kron);
   return lq_check_launch();

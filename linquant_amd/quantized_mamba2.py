@@ -22,7 +22,7 @@ import torch
 import torch.nn as nn
 
 from linquant_amd.hadamard_utils import qhad_transform
-from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd  # noqa: F401  (kept re-bindable like the reference's import)
 from linquant_amd.kernels.mamba2.causal_conv1d import causal_conv1d_fn
 from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC, prepare_dqk
 from linquant_amd.kernels.mamba2.ssd_combined import _quant_mamba_chunk_scan_combined_fwd
@@ -146,18 +146,18 @@ class QuantizedMamba2(nn.Module):
                 self._dqk_prepared = (prepare_dqk(dqk_b), prepare_dqk(dqk_c))
             dqk_b, dqk_c = self._dqk_prepared
         r_signs = getattr(self, "r_signs", None)
-        x_fp, q_B, q_C = fused_split_rotate_quant_xBC(xBC, r_signs, self.nheads, self.ngroups, self.d_state, self.headdim,
-                                                      self.B_inv_scale, self.C_inv_scale, dqk_b=dqk_b, dqk_c=dqk_c)
         keyside = getattr(self, "keyside", False)
         keyside_kwargs = {}
-        if keyside:  # the fp B of the key-side chunk state carries D_qk and the rotation q_B was quantized under
-            b_fp = xBC[..., self.d_ssm:self.d_ssm + gn]
-            if dqk_b is not None:
-                b_fp = b_fp * dqk_b.to(xBC.dtype)
-            b_fp = b_fp.reshape(xBC.shape[0], xBC.shape[1], self.ngroups, self.d_state).contiguous()
-            if r_signs is not None:
-                b_fp = kronecker_hadamard_fwd(b_fp, r_signs, self.ngroups)
+        if keyside:  # the fp B of the key-side chunk state carries D_qk and the rotation q_B was quantized under: the
+            # prologue kernel stores it next to the codes (one launch instead of the reference's two)
+            x_fp, q_B, q_C, b_fp = fused_split_rotate_quant_xBC(
+                xBC, r_signs, self.nheads, self.ngroups, self.d_state, self.headdim, self.B_inv_scale, self.C_inv_scale,
+                dqk_b=dqk_b, dqk_c=dqk_c, return_b_fp=True)
             keyside_kwargs = dict(keyside=True, x_scale_hp=self.x_quant_scale_hp, b_fp=b_fp, b_gate_scale=self.b_gate_scale)
+        else:
+            x_fp, q_B, q_C = fused_split_rotate_quant_xBC(xBC, r_signs, self.nheads, self.ngroups, self.d_state,
+                                                          self.headdim, self.B_inv_scale, self.C_inv_scale,
+                                                          dqk_b=dqk_b, dqk_c=dqk_c)
 
         # 4. INT8 SSD
         missing = [n for n in ("alpha_hp", "bscale_g", "static_state_scale", "static_cb_scale") if not hasattr(self, n)]

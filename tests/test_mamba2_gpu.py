@@ -372,3 +372,32 @@ def test_full_size_config5_slices(cuda):
     torch.cuda.synchronize()
     assert torch.equal(o[:, 1:], states[:, :-1].clamp(-127, 127)) and torch.equal(f, states[:, -1].clamp(-127, 127))
     assert int(o[:, 0].abs().max()) == 0
+
+
+@pytest.mark.parametrize("with_dqk", [False, True])
+def test_prologue_also_returns_rotated_fp_b(case, cuda, with_dqk):
+    """The optional fourth output of the prologue equals the separate rotation of the [dqk-scaled] B lanes bit for bit,
+    and leaves the three reference outputs unchanged."""
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    s = case["shape"]
+    xBC, dt_raw, p, sc = gpu_inputs(case, cuda)
+    gn = s.ngroups * s.dstate
+    kw = {}
+    if with_dqk:
+        gen = torch.Generator().manual_seed(5)
+        from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import prepare_dqk
+        kw = dict(dqk_b=prepare_dqk((0.5 + torch.rand(gn, generator=gen)).cuda()),      # fp16-rounded values, as the mixer holds them
+                  dqk_c=prepare_dqk((0.5 + torch.rand(gn, generator=gen)).cuda()))
+    x3, qB3, qC3 = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                sc["B_inv_scale"], sc["C_inv_scale"], **kw)
+    x4, qB4, qC4, b_fp = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                      sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True, **kw)
+    b_lanes = xBC[..., s.d_ssm:s.d_ssm + gn]
+    if with_dqk:
+        b_lanes = b_lanes * kw["dqk_b"].to(xBC.dtype)
+    ref = kronecker_hadamard_fwd(b_lanes.reshape(s.batch, s.seqlen, s.ngroups, s.dstate).contiguous(), p["r_signs"], s.ngroups)
+    torch.cuda.synchronize()
+    assert torch.equal(qB3, qB4) and torch.equal(qC3, qC4) and x4.data_ptr() == x3.data_ptr()
+    assert b_fp.shape == ref.shape and torch.equal(b_fp, ref)
