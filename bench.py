@@ -21,8 +21,8 @@ import time
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the default workload (key-side), from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by what the
 # same counters read for a plain 256 MiB copy (x2.0 / x1.0); summary in profiles/mamba2_ssd_c5_keyside_hbm_traffic.md
-C5_KEYSIDE_TRAFFIC_MB = {"chunk_scan": 860.2, "chunk_state": 509.1, "state_passing": 173.2, "chunk_cumsum": 63.1,
-                         "bmm_chunk": 42.2, "prologue": 25.2, "rotate_b_fp": 16.8}
+C5_KEYSIDE_TRAFFIC_MB = {"chunk_scan": 859.9, "chunk_state": 509.0, "state_passing": 181.0, "chunk_cumsum": 42.1,
+                         "bmm_chunk": 42.1, "prologue": 33.6}
 
 
 def stage_bytes(s, keyside):
