@@ -432,6 +432,30 @@ typedef struct {
 } lq_rmsnorm_gated_qhad_args;
 int lq_rmsnorm_gated_qhad(const lq_rmsnorm_gated_qhad_args* args, hipStream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Calibration: running absolute maxima of an activation tensor, on the device.
+ * ------------------------------------------------------------------------------------------ */
+
+/* replaces the calibrating branch of Quantizer.__call__ (linquant/invariances.py:77-81):
+ *   a = |x| [* gate];  a = amax over (batch, rows) keeping (H, D)  ("pc_static", mode 0)
+ *                      | amax over (batch, rows, D) keeping (H)     ("ph_static", mode 1)
+ *                      | amax over everything                        (per tensor,  mode 2)
+ *   out = max(out, a)   -- the running maximum over calibration batches; the caller zero-fills `out` once
+ * and the per-(H,P) / per-(H,N) SSD observers of scripts/nemotron_h_calibration.py (:293-345 x * scale_lut, :462-556
+ * gated B broadcast from its group to the heads, :558-600 plain x): `gate` is an optional fp32 factor per (batch, row,
+ * head) and `heads_per_group` > 1 reads x at head h / heads_per_group. */
+typedef struct {
+  const void* x;             /* (B, T, Hx, D) in any stride order, unit D stride; Hx = H / heads_per_group */
+  int32_t x_dtype;           /* LQ_DT_F16 / LQ_DT_BF16 / LQ_DT_F32 */
+  int64_t x_stride_b, x_stride_t, x_stride_h;
+  const float* gate;         /* NULL or (B, T, H) fp32 with the strides below */
+  int64_t gate_stride_b, gate_stride_t, gate_stride_h;
+  float* out;                /* mode 0: (H, D); mode 1: (H,); mode 2: (1,); fp32, updated in place */
+  int32_t batch, rows, nheads, dim, heads_per_group; /* dim a multiple of 8 */
+  int32_t mode;
+} lq_absmax_args;
+int lq_absmax(const lq_absmax_args* args, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

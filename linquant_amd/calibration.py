@@ -103,18 +103,29 @@ def calibrate_mamba2(shape: Mamba2Shape, xBC, dt_raw, params, head_block: int = 
     b_gate = torch.empty(H, N, device=dev)
     state_scale = torch.empty(H, P, device=dev)
     rep = H // G
+    on_gpu = xBC.is_cuda
+    if on_gpu:  # the three element-wise observers as device reductions straight from the fp16 view (no fp32 copy of x)
+        gate_blh = gate.reshape(B, L, H)
+        xs_hp, x_hp, bg_hn = (torch.zeros(n, device=dev) for n in (H * P, H * P, H * N))
+        x_view = xBC[..., :d_ssm].view(B, L, H, P)
+        absmax_update(xs_hp, x_view, "pc_static", gate=gate_blh)
+        absmax_update(x_hp, x_view, "pc_static")
+        absmax_update(bg_hn, Brot.contiguous(), "pc_static", gate=gate_blh, heads_per_group=rep)
     for h0 in range(0, H, head_block):
         h1 = min(H, h0 + head_block)
         xh = xBC[..., h0 * P:h1 * P].float().view(B, nc, Q, h1 - h0, P)
         gh = gate[..., h0:h1]
         xg = xh * gh[..., None]
-        alpha[h0:h1] = xg.abs().amax(dim=(0, 1, 2)) / 127.0
-        x_scale[h0:h1] = xh.abs().amax(dim=(0, 1, 2)) / 127.0
         gidx = torch.arange(h0, h1, device=dev) // rep
         Bh = Brot.view(B, nc, Q, G, N)[:, :, :, gidx]  # (B,nc,Q,hb,N)
-        b_gate[h0:h1] = (Bh * gh[..., None]).abs().amax(dim=(0, 1, 2))
+        if not on_gpu:
+            alpha[h0:h1] = xg.abs().amax(dim=(0, 1, 2)) / 127.0
+            x_scale[h0:h1] = xh.abs().amax(dim=(0, 1, 2)) / 127.0
+            b_gate[h0:h1] = (Bh * gh[..., None]).abs().amax(dim=(0, 1, 2))
         st = torch.einsum("bcqhp,bcqhn->bchpn", xg, Bh)
         state_scale[h0:h1] = st.abs().amax(dim=(0, 1, 4)) / 127.0
+    if on_gpu:
+        alpha, x_scale, b_gate = xs_hp.view(H, P) / 127.0, x_hp.view(H, P) / 127.0, bg_hn.view(H, N)
     tiny = 1e-8
     return dict(
         B_scale=B_scale.float().contiguous(), C_scale=C_scale.float().contiguous(),
@@ -123,3 +134,59 @@ def calibrate_mamba2(shape: Mamba2Shape, xBC, dt_raw, params, head_block: int = 
         x_scale_hp=x_scale.clamp_min(tiny).contiguous(), b_gate_scale=b_gate.clamp_min(tiny).view(1, 1, H, N).contiguous(),
         static_state_scale=state_scale.clamp_min(tiny).contiguous(), static_cb_scale=static_cb_scale.float().contiguous(),
     )
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Device-side absmax collectors (HIP): the calibrating half of the reference Quantizer and the amax SSD observers.
+# ---------------------------------------------------------------------------------------------------------------
+_ABSMAX_MODES = {"pc_static": 0, "ph_static": 1, "pt_static": 2}
+
+
+def absmax_update(out: torch.Tensor, x: torch.Tensor, scheme: str, gate: torch.Tensor | None = None,
+                  heads_per_group: int = 1) -> torch.Tensor:
+    """``out = max(out, amax |x [* gate]|)`` on the device, in place, without an fp32 copy of ``x``.
+
+    x: (B, T, Hx, D) view with unit stride along D (any other stride order), fp16 / bf16 / fp32; Hx = H // heads_per_group.
+    gate: optional fp32 (B, T, H) view (the per-token factor of the SSD observers).
+    scheme / out: "pc_static" -> (H, D), "ph_static" -> (H,), "pt_static" -> (1,), fp32; zero-filled by the caller before
+    the first batch (linquant/invariances.py:77-81 keeps the same running maximum)."""
+    from linquant_amd import _lib
+
+    codes = {torch.float16: _lib.LQ_DT_F16, torch.bfloat16: _lib.LQ_DT_BF16, torch.float32: _lib.LQ_DT_F32}
+    assert x.dim() == 4 and x.stride(3) == 1 and x.dtype in codes
+    B, T, Hx, D = x.shape
+    H = Hx * heads_per_group
+    mode = _ABSMAX_MODES[scheme]
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.numel() == (H * D, H, 1)[mode]
+    if gate is not None:
+        assert gate.dtype == torch.float32 and gate.shape == (B, T, H)
+    _lib.call("lq_absmax", x.device, x=_lib.ptr(x), x_dtype=codes[x.dtype], x_stride_b=x.stride(0), x_stride_t=x.stride(1),
+              x_stride_h=x.stride(2), gate=_lib.ptr(gate), gate_stride_b=0 if gate is None else gate.stride(0),
+              gate_stride_t=0 if gate is None else gate.stride(1), gate_stride_h=0 if gate is None else gate.stride(2),
+              out=_lib.ptr(out), batch=B, rows=T, nheads=H, dim=D, heads_per_group=heads_per_group, mode=mode)
+    return out
+
+
+class AbsmaxCollector:
+    """Calibrating half of linquant.invariances.Quantizer on the device: ``collector(role, x)`` with x [B, H, rows, D]
+    (the reference's operand layout; any view with unit D stride) keeps the running absolute maximum per role under the
+    role's scheme ("pc_static": per (H, D); "ph_static": per H; "pt_static": one value), ``scales(qmax)`` turns them
+    into static scales ``absmax / qmax`` clamped at 1e-12 like the reference."""
+
+    def __init__(self, scheme: str = "pc_static", scheme_by_role: dict | None = None):
+        self.scheme, self.scheme_by_role, self.absmax = scheme, dict(scheme_by_role or {}), {}
+
+    def __call__(self, role: str, x: torch.Tensor) -> torch.Tensor:
+        scheme = self.scheme_by_role.get(role, self.scheme)
+        B, H, rows, D = x.shape
+        if role not in self.absmax:
+            n = (H * D, H, 1)[_ABSMAX_MODES[scheme]]
+            self.absmax[role] = torch.zeros(n, dtype=torch.float32, device=x.device)
+        absmax_update(self.absmax[role], x.permute(0, 2, 1, 3), scheme)
+        return x
+
+    def scales(self, qmax: int = 127) -> dict:
+        out = {}
+        for role, a in self.absmax.items():
+            out[role] = (a / qmax).clamp_min(1e-12)
+        return out

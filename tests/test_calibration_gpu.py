@@ -1,0 +1,77 @@
+"""GPU test of the device-side absmax collectors: maxima are exact, so every comparison is bit for bit."""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("scheme", ["pc_static", "ph_static", "pt_static"])
+def test_absmax_schemes_and_running_maximum(cuda, dtype, scheme):
+    from linquant_amd.calibration import absmax_update
+
+    gen = torch.Generator().manual_seed(0)
+    B, T, H, D = 2, 300, 6, 64                      # a ragged last slab of rows
+    out = None
+    ref = None
+    for batch in range(3):                          # running maximum over calibration batches
+        big = (torch.randn(B, T, H, D + 16, generator=gen) * (1 + batch)).to(dtype).cuda()
+        x = big[..., 8:8 + D] if dtype != torch.float32 else big[..., 4:4 + D]      # strided, 16-byte aligned view
+        a = x.float().abs()
+        r = {"pc_static": a.amax(dim=(0, 1)).reshape(-1), "ph_static": a.amax(dim=(0, 1, 3)), "pt_static": a.amax().reshape(1)}[scheme]
+        ref = r if ref is None else torch.maximum(ref, r)
+        if out is None:
+            out = torch.zeros_like(r)
+        absmax_update(out, x, scheme)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+
+
+def test_absmax_reference_layout_gate_and_groups(cuda):
+    """The three SSD observers: plain x per (H, P), x * gate per (H, P), and B * gate per (H, N) with B broadcast from
+    its group to the heads -- against the torch expressions scripts/nemotron_h_calibration.py evaluates."""
+    from linquant_amd.calibration import AbsmaxCollector, absmax_update
+
+    gen = torch.Generator().manual_seed(1)
+    B, L, H, P, G, N = 2, 512, 8, 64, 2, 128
+    xBC = torch.randn(B, L, H * P + 2 * G * N, generator=gen).half().cuda()
+    x = xBC[..., :H * P].view(B, L, H, P)
+    Bm = xBC[..., H * P:H * P + G * N].view(B, L, G, N)
+    gate = torch.rand(B, H, L // 64, 64, generator=gen).cuda()           # (B, H, nchunks, Q) as the cumsum stage stores it
+    gate_blh = gate.permute(0, 2, 3, 1).reshape(B, L, H)                 # a view: no copy
+    x_hp = torch.zeros(H * P, device="cuda")
+    xs_hp = torch.zeros(H * P, device="cuda")
+    bg_hn = torch.zeros(H * N, device="cuda")
+    absmax_update(x_hp, x, "pc_static")
+    absmax_update(xs_hp, x, "pc_static", gate=gate_blh)
+    absmax_update(bg_hn, Bm, "pc_static", gate=gate_blh, heads_per_group=H // G)
+    torch.cuda.synchronize()
+    g = gate_blh.unsqueeze(-1)
+    assert torch.equal(x_hp.view(H, P), x.float().abs().amax(dim=(0, 1)))
+    assert torch.equal(xs_hp.view(H, P), (x.float() * g).abs().amax(dim=(0, 1)))
+    b_per_head = Bm[:, :, torch.arange(H, device="cuda") // (H // G)]
+    assert torch.equal(bg_hn.view(H, N), (b_per_head.float() * g).abs().amax(dim=(0, 1)))
+
+    # the reference's operand layout [B, H, rows, D] through the collector, two roles with different schemes
+    col = AbsmaxCollector("pc_static", {"q": "ph_static"})
+    q = torch.randn(B, H, L, P, generator=gen).half().cuda()
+    k = torch.randn(B, L, H, P, generator=gen).half().cuda().permute(0, 2, 1, 3)     # a permuted view with unit D stride
+    col("q", q), col("k", k), col("k", k * 2)
+    torch.cuda.synchronize()
+    sc = col.scales(127)
+    assert torch.equal(sc["q"], (q.float().abs().amax(dim=(0, 2, 3)) / 127).clamp_min(1e-12))
+    assert torch.equal(sc["k"].view(H, P), ((k * 2).float().abs().amax(dim=(0, 2)) / 127).clamp_min(1e-12))
+
+
+def test_absmax_rejections(cuda):
+    from linquant_amd import _lib
+    from linquant_amd.calibration import absmax_update
+
+    x = torch.zeros(1, 4, 2, 12, dtype=torch.float16, device="cuda")            # D not a multiple of 8
+    with pytest.raises(_lib.LinQuantHipError):
+        absmax_update(torch.zeros(24, device="cuda"), x, "pc_static")
+    x = torch.zeros(1, 4, 2, 24, dtype=torch.float16, device="cuda")[..., 4:20]  # misaligned view
+    with pytest.raises(_lib.LinQuantHipError):
+        absmax_update(torch.zeros(32, device="cuda"), x, "pc_static")
