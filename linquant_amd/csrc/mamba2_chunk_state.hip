@@ -25,6 +25,8 @@
 
 namespace {
 
+typedef uint32_t lq_v2u __attribute__((ext_vector_type(2)));
+
 constexpr int kXW = 64 + 4;    // dwords per token-quad row of the x slab (64 channels + pad: the four lane groups of an
 constexpr int kPad = 4;       // operand read land on bank offsets 0,16,32,48)
 
@@ -132,17 +134,20 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   lq_v2i xr[4];  // x: 4 tokens x 4 fp16
   lq_v4i br[4];  // key side: 4 tokens x 8 fp16; value side: only [t][0..1] used (8 int8)
 
+  // token * stride stays below 2^31 and both factors below 2^23 (checked by the launcher): a full-rate 24-bit multiply
+  // instead of the quarter-rate 64-bit one, eight times per slab
+  const int sxl = (int)p.sx_l, bst = (int)bstep;
   auto load_slab = [&](int k0) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int kx = min(k0 + 4 * kqx + t, last);
-      xr[t] = *(const lq_v2i*)(xg + (int64_t)kx * p.sx_l);
+      xr[t] = *(const lq_v2i*)(xg + __mul24(kx, sxl));
       if (has_b) {
         const int kb = min(k0 + 4 * kqb + t, last);
         if (KEYSIDE) {
-          br[t] = *(const lq_v4i*)(bg0 + (int64_t)kb * bstep);
+          br[t] = *(const lq_v4i*)(bg0 + __mul24(kb, bst));
         } else {
-          const lq_v2i v = *(const lq_v2i*)(bg0 + (int64_t)kb * bstep);
+          const lq_v2i v = *(const lq_v2i*)(bg0 + __mul24(kb, bst));
           br[t][0] = v[0], br[t][1] = v[1];
         }
       }
@@ -240,7 +245,8 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   const float so = p.oqs[(int64_t)h * p.soq_h + (int64_t)pr * p.soq_p];
   const float ratio = xs / so;
   const float req = KEYSIDE ? 0.0f : ratio * p.bscale_g[(int64_t)g * p.sbs_g];
-  int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + pr) * p.N + n0 + 4 * kg;
+  int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + pr) * p.N + n0;
+  uint32_t dq[NT / 16];  // dword q of this lane: codes of N = n0 + 16 q + 4 kg + {0..3}
 #pragma unroll
   for (int q = 0; q < NT / 16; ++q) {
     uint32_t cd[4];
@@ -255,7 +261,20 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
         cd[r] = (uint32_t)lq_q_rha(a * req, 127);
       }
     }
-    *(uint32_t*)(sp + 16 * q) = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
+    dq[q] = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
+  }
+  // The four lanes kg = 0..3 of one P row hold the four dwords of every 16-byte piece q of the row.  A 4 x 4 transpose
+  // between register index and lane group (two row-swap instructions per register pair) leaves lane kg with the whole
+  // piece q = 4 i + kg, stored as 16 bytes: a fourth of the store instructions, 64 contiguous bytes per row and store.
+#pragma unroll
+  for (int i = 0; i < NT / 64; ++i) {
+    uint32_t r0 = dq[4 * i], r1 = dq[4 * i + 1], r2 = dq[4 * i + 2], r3 = dq[4 * i + 3];
+    lq_v2u t;
+    t = __builtin_amdgcn_permlane32_swap(r0, r2, false, false), r0 = t[0], r2 = t[1];
+    t = __builtin_amdgcn_permlane32_swap(r1, r3, false, false), r1 = t[0], r3 = t[1];
+    t = __builtin_amdgcn_permlane16_swap(r0, r1, false, false), r0 = t[0], r1 = t[1];
+    t = __builtin_amdgcn_permlane16_swap(r2, r3, false, false), r2 = t[0], r3 = t[1];
+    *(lq_v4i*)(sp + 16 * (4 * i + kg)) = lq_v4i{(int)r0, (int)r1, (int)r2, (int)r3};
   }
 }
 
@@ -268,9 +287,12 @@ int launch(const Params& p, hipStream_t stream) {
   if (p.sx_b % 4 || p.sx_l % 4 || p.sx_h % 4 || !al(p.x, 8)) return LQ_ERR_SHAPE;
   const int bmod = KEYSIDE ? 8 : 8, balign = KEYSIDE ? 16 : 8;
   if (p.sB_b % bmod || p.sB_l % bmod || p.sB_g % bmod || !al(p.B, balign)) return LQ_ERR_SHAPE;
-  if (!al(p.states, 4)) return LQ_ERR_SHAPE;
+  if (!al(p.states, 16)) return LQ_ERR_SHAPE;
   const int64_t by = (int64_t)p.batch * p.nchunks;
   if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
+  if (p.sx_l < 0 || p.sB_l < 0 || p.sx_l >= (1 << 22) || p.sB_l >= (1 << 22) || (int64_t)p.Q * p.sx_l >= (1ll << 30) ||
+      (int64_t)p.Q * p.sB_l >= (1ll << 30))
+    return LQ_ERR_SHAPE;  // 24-bit token * stride products in the slab loads
   Params q = p;
   if (p.N % 128 == 0) {
     q.n_ntiles = p.N / 128;
