@@ -463,8 +463,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--workload", default="c5", choices=["c5", "c5_front", "c5_epilogue", "c5_layer"] + list(ZOO_WORKLOADS),
                     help="c5 (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on; others: zoo kernels")
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--value-side", action="store_true", help="value-side absorption instead of key-side")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
