@@ -7,7 +7,9 @@
 //     with qh = q8(q*scale, 1/sq) * sq and kh = q8(k, 1/sk) * sk  (fp32 reduction over the dequantized codes)
 //   entries above the diagonal are written as zero.
 //
-// One 4-wave workgroup per (chunk, batch*head); wave w owns the 16 rows of sub-block w.  Off-diagonal
+// One 4-wave workgroup per (pair of chunks, batch*head); wave w owns the 16 rows of sub-block w of the first chunk and
+// then those of sub-block 3 - w of the second one, so every wave does the same number of off-diagonal blocks (sub-block
+// I has I of them) and the rotation is staged once for both chunks.  Off-diagonal
 // operands are K-contiguous, so each lane builds its own 16-slot INT8 MFMA operand from plain global loads
 // (no LDS).  The diagonal block factorizes the decay weight around the block's first row whenever the decay spread
 // inside the block allows it and then runs as an fp32 MFMA product; otherwise lane (i = lane & 15, j-group =
@@ -55,40 +57,30 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
   const int c0 = NCH * kg;
   const int64_t off = ((row0 + rl) * H + h) * K + c0;
   const int64_t aoff = (row0 * H + h) * K + c0;
-  float gv[NCH], av[NCH];
+  // The factorized product is formed while the spread is still being measured (no arrays of operands stay live); when
+  // the spread turns out too large its result is dropped (overflowed operands are harmless there) and the exact path
+  // below runs instead.
   float spread = 0.0f;
+  lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int e4 = 0; e4 < NCH / 4; ++e4) {
-    const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4), a4 = *(const lq_v4f*)(p.g + aoff + 4 * e4);
+  for (int e8 = 0; e8 < NCH / 8; ++e8) {
+    const lq_v4f g0 = *(const lq_v4f*)(p.g + off + 8 * e8), g1 = *(const lq_v4f*)(p.g + off + 8 * e8 + 4);
+    const lq_v4f a0 = *(const lq_v4f*)(p.g + aoff + 8 * e8), a1 = *(const lq_v4f*)(p.g + aoff + 8 * e8 + 4);
+    float qv[8];
+    zoo_ld8(p.q + off + 8 * e8, bf, qv);
+    float kv[8];
+    zoo_ld8(p.k + off + 8 * e8, bf, kv);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      gv[4 * e4 + e] = g4[e];
-      av[4 * e4 + e] = a4[e];
-      spread = fmaxf(spread, __builtin_fabsf(g4[e] - a4[e]));
+    for (int e = 0; e < 8; ++e) {
+      const float d = (e < 4 ? g0[e & 3] : g1[e & 3]) - (e < 4 ? a0[e & 3] : a1[e & 3]);
+      spread = fmaxf(spread, __builtin_fabsf(d));
+      const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
+      const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
+      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * zoo_exp(d), kh * zoo_exp(-d), acc, 0, 0, 0);
     }
   }
   spread = wave_max(spread);
   if (spread <= 40.0f) {
-    float qa[NCH], ka[NCH];
-#pragma unroll
-    for (int e8 = 0; e8 < NCH / 8; ++e8) {
-      float qv[8];
-      zoo_ld8(p.q + off + 8 * e8, bf, qv);
-      float kv[8];
-      zoo_ld8(p.k + off + 8 * e8, bf, kv);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int n = 8 * e8 + e;
-        const float d = gv[n] - av[n];
-        const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
-        const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
-        qa[n] = qh * zoo_exp(d);
-        ka[n] = kh * zoo_exp(-d);
-      }
-    }
-    lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int n = 0; n < NCH; ++n) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[n], ka[n], acc, 0, 0, 0);
     // lane holds column j = rl, rows i = 4kg + r
 #pragma unroll
     for (int r = 0; r < 4; ++r)
@@ -131,21 +123,19 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
 }
 
 template <int K, bool ROT, bool BF>
-__global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
+__global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   constexpr int RS = K + 8;  // halves per row of the transposed rotation
   __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  const int ct = blockIdx.x;
   const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
   const int H = p.H;
-  const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
   const float sq = p.sq[h], sk = p.sk[h];
   const float inv_sq = 1.0f / sq, inv_sk = 1.0f / sk;
   const int qmax = p.qmax;
   constexpr bool bf = BF;
-  const int i0 = 16 * wave;
+  const int nchunks = p.T / 64;
 
   if constexpr (ROT) {
     // lanes walk m (coalesced rows of R), each thread gathers 8 consecutive n and writes one 16-byte piece of a row
@@ -157,6 +147,14 @@ __global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
       *(lq_v8h*)(RT + m * RS + 8 * n8) = rv;
     }
   }
+
+#pragma unroll 1
+  for (int pass = 0; pass < 2; ++pass) {
+  const int ct = 2 * blockIdx.x + pass;
+  if (ct >= nchunks) break;  // uniform over the workgroup
+  const int blk = pass ? 3 - wave : wave;  // sub-block of this wave in this chunk
+  const int i0 = 16 * blk;
+  const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
 
   // ---- state-read operand of the output kernel: codes of q * exp(g) * scale
   if (p.qg) {
@@ -187,8 +185,8 @@ __global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
   for (int J = 0; J < 3; ++J) acc[J] = lq_v4i{0, 0, 0, 0};
 
   if constexpr (!ROT) {
-    // ---- off-diagonal blocks J < wave: INT8 MFMA on anchored operands built from plain global loads
-    if (wave > 0) {
+    // ---- off-diagonal blocks J < blk: INT8 MFMA on anchored operands built from plain global loads
+    if (blk > 0) {
 #pragma unroll
       for (int ks = 0; ks < K / 64; ++ks) {
         const int kk = 64 * ks + 16 * kg;
@@ -227,7 +225,7 @@ __global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
         }
 #pragma unroll
         for (int J = 0; J < 3; ++J) {
-          if (J >= wave) continue;
+          if (J >= blk) continue;
           const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
           float k0[8];
           zoo_ld8(p.k + off, bf, k0);
@@ -256,78 +254,77 @@ __global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
     // Transposed product R^T . X^T: lane (rl, kg) receives, for token rl, channels 16mt + 4kg + r, which it packs
     // as dword mt of its INT8 operand; q and k operands share that channel -> slot map, so the INT8 dot is exact.
     constexpr int KS = K / 32, MT = K / 16;
-    // anchored fp16 operands: tensor 0 = q rows of this sub-block, tensor 1 + J = k rows of sub-block J < wave
-    lq_v8h xop[4][KS];
-    if (wave > 0) {
+    if (pass == 0) __syncthreads();  // R^T staged
+    // tensor 0 = q rows of this sub-block, tensor 1 + J = k rows of sub-block J < blk, all anchored at this sub-block's
+    // first row; two tensors share one sweep over R^T, and a k tensor meets the q codes as soon as it is quantized
+    uint32_t cq[MT];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int kk = 32 * ks + 8 * kg;
-        const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
-        const lq_v4f a0 = *(const lq_v4f*)ap, a1 = *(const lq_v4f*)(ap + 4);
-        {
-          const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
-          float qv[8];
-          zoo_ld8(p.q + off, bf, qv);
-          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+    for (int gp = 0; gp < 2; ++gp) {
+      if (2 * gp > blk || blk == 0) continue;  // uniform per wave
+      lq_v8h xop[2][KS];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            float x = qv[e] * zoo_exp(gg - an);
-            x = x * p.scale;
-            xop[0][ks][e] = (_Float16)x;
-          }
+      for (int u = 0; u < 2; ++u) {
+        const int t = 2 * gp + u;
+        if (t > blk) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) xop[u][ks] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
+          continue;
         }
+        const int64_t row = t == 0 ? t0 + i0 + rl : t0 + 16 * (t - 1) + rl;
+        const _Float16* src = t == 0 ? p.q : p.k;
 #pragma unroll
-        for (int J = 0; J < 3; ++J) {
-          if (J >= wave) continue;
-          const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
-          float kv[8];
-          zoo_ld8(p.k + off, bf, kv);
+        for (int ks = 0; ks < KS; ++ks) {
+          const int kk = 32 * ks + 8 * kg;
+          const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
+          const lq_v4f a0 = *(const lq_v4f*)ap, a1 = *(const lq_v4f*)(ap + 4);
+          const int64_t off = (row * H + h) * K + kk;
+          float xv[8];
+          zoo_ld8(src + off, bf, xv);
           const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            xop[1 + J][ks][e] = (_Float16)(kv[e] * zoo_exp(an - gg));
+            if (t == 0) {
+              float x = xv[e] * zoo_exp(gg - an);
+              x = x * p.scale;
+              xop[u][ks][e] = (_Float16)x;
+            } else {
+              xop[u][ks][e] = (_Float16)(xv[e] * zoo_exp(an - gg));
+            }
           }
         }
       }
-    }
-    __syncthreads();  // R^T staged
-    if (wave > 0) {
-      uint32_t cd[4][MT];
+      uint32_t cd[2][MT];
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        lq_v4f ra[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) ra[t] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+        lq_v4f ra[2];
+        ra[0] = ra[1] = lq_v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const lq_v8h rop = *(const lq_v8h*)(RT + (16 * mt + rl) * RS + 32 * ks + 8 * kg);
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            if (t > wave) continue;
-            ra[t] = lq_mfma_f16(rop, xop[t][ks], ra[t]);
-          }
+          ra[0] = lq_mfma_f16(rop, xop[0][ks], ra[0]);
+          ra[1] = lq_mfma_f16(rop, xop[1][ks], ra[1]);
         }
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          if (t > wave) continue;
-          const float inv = t == 0 ? inv_sq : inv_sk;
-          cd[t][mt] = zoo_pack_codes(zoo_q8(ra[t][0], inv, qmax), zoo_q8(ra[t][1], inv, qmax), zoo_q8(ra[t][2], inv, qmax),
-                                     zoo_q8(ra[t][3], inv, qmax));
+        for (int u = 0; u < 2; ++u) {
+          const float inv = (gp == 0 && u == 0) ? inv_sq : inv_sk;
+          cd[u][mt] = zoo_pack_codes(zoo_q8(ra[u][0], inv, qmax), zoo_q8(ra[u][1], inv, qmax), zoo_q8(ra[u][2], inv, qmax),
+                                     zoo_q8(ra[u][3], inv, qmax));
         }
       }
+      if (gp == 0) {
 #pragma unroll
-      for (int s = 0; s < K / 64; ++s) {
-        lq_v4i qop;
+        for (int mt = 0; mt < MT; ++mt) cq[mt] = cd[0][mt];
+      }
 #pragma unroll
-        for (int d = 0; d < 4; ++d) qop[d] = (int)cd[0][4 * s + d];
+      for (int u = (gp == 0 ? 1 : 0); u < 2; ++u) {
+        const int J = 2 * gp + u - 1;
+        if (J >= blk) continue;
 #pragma unroll
-        for (int J = 0; J < 3; ++J) {
-          if (J >= wave) continue;
-          lq_v4i kop;
+        for (int s = 0; s < K / 64; ++s) {
+          lq_v4i qop, kop;
 #pragma unroll
-          for (int d = 0; d < 4; ++d) kop[d] = (int)cd[1 + J][4 * s + d];
+          for (int d = 0; d < 4; ++d) qop[d] = (int)cq[4 * s + d], kop[d] = (int)cd[u][4 * s + d];
           acc[J] = lq_mfma_i8(qop, kop, acc[J]);
         }
       }
@@ -337,15 +334,16 @@ __global__ __launch_bounds__(256, 2) void zoo_gla_A_kernel(AParams p) {
   const float sqk = sq * sk;
 #pragma unroll
   for (int J = 0; J < 3; ++J) {
-    if (J >= wave) continue;
+    if (J >= blk) continue;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)((float)acc[J][r] * sqk);
   }
   // zero blocks above the diagonal
-  for (int J = wave + 1; J < 4; ++J)
+  for (int J = blk + 1; J < 4; ++J)
 #pragma unroll
     for (int r = 0; r < 4; ++r) p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)0.0f;
+  }  // pass
 }
 
 }  // namespace
@@ -365,7 +363,7 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.g = a->g, p.A = (_Float16*)a->A, p.qg = a->qg;
   p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
-  dim3 grid(a->seqlen / 64, a->batch * a->nheads);
+  dim3 grid((a->seqlen / 64 + 1) / 2, a->batch * a->nheads);
 #define LQ_A_LAUNCH(KV, ROTV)                                                                              \
   do {                                                                                                     \
     if (p.bf)                                                                                              \
