@@ -8,10 +8,10 @@
 //   W = T (L * exp(g)),  U = T (beta^sigma v),  Hw = beta^((1-sigma) tau) k,  fw = beta^((1-sigma)(1-tau))
 //
 // One 4-wave workgroup per (chunk, batch*head); every product runs on the fp32 MFMA (16x16x4).
-//   Gram: wave w owns row block w; operands come straight from global memory (lane (rl, kg) supplies 16 contiguous
-//     channels of token rl per 64-channel pass).  Per-channel decay is factorized around the first row of the row
-//     block (off-diagonal blocks: both factors <= 1; diagonal block: only when the decay spread inside the block is
-//     small, otherwise one exponential per (i, j, channel)).
+//   Gram: both operands are staged once per token as fp32 in LDS and the ten lower 16x16 blocks are spread 3/3/2/2
+//     over the waves.  Per-channel decay is factorized around the chunk's middle row; when the decay spread over the
+//     chunk is too large for that, each wave redoes its row block around the block's first row straight from global
+//     memory (diagonal block: one exponential per (i, j, channel) when even that spread is too large).
 //   Inverse: the four 16x16 diagonal blocks by forward substitution (lane per column), then block rows 1..3:
 //     T_IJ = -T_II . sum_{J <= M < I} G_IM . T_MJ.
 //   W, U: T . X with X staged in LDS as fp32; each wave takes row block w for the first half of the column tiles
@@ -64,36 +64,15 @@ LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl
   return acc;
 }
 
+// Gram of row block I = wave with the per-channel decay factorized around the first row of the row block (used when
+// the decay spread over the whole chunk is too large for one anchor): operands straight from global memory, lane
+// (rl, kg) supplies 16 contiguous channels of token rl per 64-channel pass; off-diagonal blocks: both factors <= 1;
+// diagonal block: only when the spread inside the block is small, otherwise one exponential per (i, j, channel).
 template <int DECAY, int K, bool BF>
-__global__ __launch_bounds__(256, 2) void zoo_wy_prep_kernel(WyParams p) {
-  constexpr int LS = 64 + 16;  // floats per row of X (the T . X products run over 64 columns at a time): measured, a B-operand read (4 rows, 16 adjacent columns) takes one LDS pass at 80 floats and two at 72
-  static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
-  __shared__ __align__(16) float T_s[64 * kGS];
-  __shared__ __align__(16) float X_s[64 * LS];  // 36 KB of LDS in all: four workgroups per compute unit
-  float* G_s = X_s;
-  __shared__ float gs_s[64], bs_s[64], bh_s[64];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rl = lane & 15, kg = lane >> 4;
-  const int ct = blockIdx.x;
-  const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
-  const int H = p.H, V = p.V;
-  const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
-  const float sigma = p.sigma, tau = p.tau;
+LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, const float* bh_s, const float* gs_s, int wave,
+                          int rl, int kg, int64_t t0, int h) {
+  const int H = p.H;
   constexpr bool bf = BF;
-
-  // ---- per-token factors; fw is written straight out
-  if (tid < 64) {
-    const float bt = p.beta[(t0 + tid) * H + h];
-    bs_s[tid] = powb(bt, sigma);
-    bh_s[tid] = powb(bt, 1.0f - sigma);
-    p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
-    if (DECAY == LQ_DECAY_SCALAR) gs_s[tid] = p.g[(t0 + tid) * H + h];
-  }
-  __syncthreads();
-
-  // ---- Gram, row block I = wave: G[i][j] for i > j
-  {
     const int I = wave;
     const int64_t irow = ((t0 + 16 * I + rl) * H + h) * K;
     const int64_t arow = ((t0 + 16 * I) * H + h) * K;
@@ -204,6 +183,131 @@ __global__ __launch_bounds__(256, 2) void zoo_wy_prep_kernel(WyParams p) {
       }
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) G_s[(16 * I + rl) * kGS + 16 * I + 4 * kg + jj] = (rl > 4 * kg + jj) ? sacc[jj] : 0.0f;
+    }
+}
+
+template <int DECAY, int K, bool BF>
+__global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
+  constexpr int LS = 64 + 16;  // floats per row of X (the T . X products run over 64 columns at a time): measured, a B-operand read (4 rows, 16 adjacent columns) takes one LDS pass at 80 floats and two at 72
+  static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
+  __shared__ __align__(16) float lds_f[64 * kGS + 64 * LS];  // 38 KB of LDS: four workgroups per compute unit
+  float* T_s = lds_f;
+  float* X_s = lds_f + 64 * kGS;
+  float* G_s = X_s;
+  constexpr int kOP = 72;  // floats per row of the staged Gram operands: a 16-byte read of 16 rows x 4 adjacent pieces takes the minimum two LDS passes at 40 or 72
+  static_assert(2 * 64 * kOP <= 64 * kGS + 64 * LS, "the Gram operands live in the T / X buffers until G is written");
+  float* Lg_s = lds_f;
+  float* Hg_s = lds_f + 64 * kOP;
+  __shared__ float gs_s[64], bs_s[64], bh_s[64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
+  const int ct = blockIdx.x;
+  const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+  const int H = p.H, V = p.V;
+  const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
+  const float sigma = p.sigma, tau = p.tau;
+  constexpr bool bf = BF;
+
+  // ---- per-token factors; fw is written straight out
+  if (tid < 64) {
+    const float bt = p.beta[(t0 + tid) * H + h];
+    bs_s[tid] = powb(bt, sigma);
+    bh_s[tid] = powb(bt, 1.0f - sigma);
+    p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
+    if (DECAY == LQ_DECAY_SCALAR) gs_s[tid] = p.g[(t0 + tid) * H + h];
+  }
+  __syncthreads();
+
+  // ---- Gram G[i][j] for i > j.  Operands are staged once per token, 64 channels at a time, as fp32 in LDS:
+  //   Lg = beta^sigma k e^(g - a),  Hg = beta^(1-sigma) k e^(a - g),  a = g of the chunk's middle row (one anchor for the
+  //   whole chunk: |g - a| <= 40 keeps every factor and product a normal fp32 number; checked, see below),
+  // and the ten 16x16 blocks are spread 3/3/2/2 over the waves.  An operand read is 16 bytes: lane (rl, kg) takes
+  // channels 16s + 4kg .. + 3 of row rl, and its element e feeds MFMA step e of both operands alike.
+  {
+    // wave 0: (3,0) (3,1) (3,2); wave 1: (2,0) (2,1) (2,2); wave 2: (1,0) (1,1); wave 3: (3,3) (0,0)
+    const int nb = wave < 2 ? 3 : 2;
+    auto blk_i = [&](int q) { return wave < 3 ? 3 - wave : (q == 0 ? 3 : 0); };
+    auto blk_j = [&](int q) { return wave < 3 ? q : (q == 0 ? 3 : 0); };
+    lq_v4f acc[3];
+#pragma unroll
+    for (int q = 0; q < 3; ++q) acc[q] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+    float spread = 0.0f;
+    const int64_t arow = ((t0 + 32) * H + h) * K;
+#pragma unroll 1
+    for (int ps = 0; ps < K / 64; ++ps) {
+      if (ps > 0) __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int it = tid + 256 * q;
+        const int r = it >> 3, c8 = it & 7;
+        const int64_t off = ((t0 + r) * H + h) * K + 64 * ps + 8 * c8;
+        float kv[8];
+        zoo_ld8(p.k + off, bf, kv);
+        const float bs = bs_s[r], bh = bh_s[r];
+        lq_v4f l0, l1, h0, h1;
+        if (DECAY == LQ_DECAY_DIAGONAL) {
+          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+          const lq_v4f a0 = *(const lq_v4f*)(p.g + arow + 64 * ps + 8 * c8), a1 = *(const lq_v4f*)(p.g + arow + 64 * ps + 8 * c8 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float d0 = g0[e] - a0[e], d1 = g1[e] - a1[e];
+            spread = fmaxf(spread, fmaxf(__builtin_fabsf(d0), __builtin_fabsf(d1)));
+            l0[e] = (bs * kv[e]) * zoo_exp(d0);
+            l1[e] = (bs * kv[4 + e]) * zoo_exp(d1);
+            h0[e] = (bh * kv[e]) * zoo_exp(-d0);
+            h1[e] = (bh * kv[4 + e]) * zoo_exp(-d1);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            l0[e] = bs * kv[e];
+            l1[e] = bs * kv[4 + e];
+            h0[e] = bh * kv[e];
+            h1[e] = bh * kv[4 + e];
+          }
+        }
+        *(lq_v4f*)(Lg_s + r * kOP + 8 * c8) = l0;
+        *(lq_v4f*)(Lg_s + r * kOP + 8 * c8 + 4) = l1;
+        *(lq_v4f*)(Hg_s + r * kOP + 8 * c8) = h0;
+        *(lq_v4f*)(Hg_s + r * kOP + 8 * c8 + 4) = h1;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int q = 0; q < 3; ++q) {
+        if (q >= nb) continue;
+        const float* lp = Lg_s + (16 * blk_i(q) + rl) * kOP + 4 * kg;
+        const float* hp = Hg_s + (16 * blk_j(q) + rl) * kOP + 4 * kg;
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+          const lq_v4f la = *(const lq_v4f*)(lp + 16 * s4), hb = *(const lq_v4f*)(hp + 16 * s4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[q] = mfma_f32(la[e], hb[e], acc[q]);
+        }
+      }
+    }
+    bool one_anchor = true;
+    if (DECAY == LQ_DECAY_DIAGONAL) one_anchor = __syncthreads_or(spread > 40.0f) == 0;
+    else __syncthreads();
+    // the operand buffers are dead: G overlays them
+    if (one_anchor) {
+      // lane holds column j = rl of block J, rows i = 4kg + r of block I
+#pragma unroll
+      for (int q = 0; q < 3; ++q) {
+        if (q >= nb) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = 16 * blk_i(q) + 4 * kg + r, j = 16 * blk_j(q) + rl;
+          float v = 0.0f;
+          if (i > j) {
+            v = acc[q][r];
+            if (DECAY == LQ_DECAY_SCALAR) v = v * zoo_exp(gs_s[i] - gs_s[j]);
+          }
+          G_s[i * kGS + j] = v;
+        }
+      }
+    } else {
+      gram_rowblock<DECAY, K, BF>(p, G_s, bs_s, bh_s, gs_s, wave, rl, kg, t0, h);
     }
   }
   __syncthreads();

@@ -200,10 +200,11 @@ def _wy_reference(k, v, beta, gc, decay, sigma, tau):
 
 @pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet", "kda"])
 @pytest.mark.parametrize("sigma,tau", [(1.0, 1.0), (0.5, 0.5), (0.0, 1.0)])
-@pytest.mark.parametrize("K,gscale", [(64, 1.0), (128, 1.0), (64, 40.0)])
+@pytest.mark.parametrize("K,gscale", [(64, 1.0), (128, 1.0), (64, 40.0), (128, 4.0), (128, 40.0)])
 def test_wy_prep_kernel(cuda, cell, sigma, tau, K, gscale):
     """The fp32-MFMA WY prep (Gram, blocked triangular inverse, T.X) against the float64 transform, including the
-    strongly decaying regime that takes the per-element path of the diagonal Gram blocks."""
+    strongly decaying regimes that leave the one-anchor Gram for the per-row-block one and for the per-element path of
+    the diagonal Gram blocks."""
     from linquant_amd.kernels.zoo import _common as C
 
     decay = zc.CELLS[cell][1]
