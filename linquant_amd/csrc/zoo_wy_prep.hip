@@ -7,15 +7,16 @@
 //   T = (I + G)^-1  (unit lower triangular, forward substitution)
 //   W = T (L * exp(g)),  U = T (beta^sigma v),  Hw = beta^((1-sigma) tau) k,  fw = beta^((1-sigma)(1-tau))
 //
-// One 4-wave workgroup per (chunk, batch*head); every product runs on the fp32 MFMA (16x16x4).
+// One 4-wave workgroup per (chunk, batch*head); the Gram and the inverse run on the fp32 MFMA (16x16x4).
 //   Gram: both operands are staged once per token as fp32 in LDS and the ten lower 16x16 blocks are spread 3/3/2/2
 //     over the waves.  Per-channel decay is factorized around the chunk's middle row; when the decay spread over the
 //     chunk is too large for that, each wave redoes its row block around the block's first row straight from global
 //     memory (diagonal block: one exponential per (i, j, channel) when even that spread is too large).
 //   Inverse: the four 16x16 diagonal blocks by forward substitution (lane per column), then block rows 1..3:
 //     T_IJ = -T_II . sum_{J <= M < I} G_IM . T_MJ.
-//   W, U: T . X with X staged in LDS as fp32; each wave takes row block w for the first half of the column tiles
-//     and row block 3 - w for the second half (equal work), and stores four adjacent channels per lane.
+//   W, U: T . X on the bf16 MFMA with T and X each split in three bf16 pieces (six products per step); X is staged
+//     transposed in LDS, each wave takes row block w for the first half of the column tiles and row block 3 - w for
+//     the second half (equal work), and stores four adjacent channels per lane.
 #include "zoo_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -51,16 +52,67 @@ LQ_DEV float wy_wave_max(float m) {
 
 constexpr int kGS = 70;  // floats per row of the G / T tiles: measured, an A-operand read (16 rows, 4 adjacent slots) takes one LDS pass when the pitch is 2 mod 4 (68 took two)
 
-// D^T tile of T . X for row block I and 16 columns starting at col: lane (rl = token, kg) gets columns col + 4kg + r
-template <int LS>
-LQ_DEV lq_v4f tx_tile(const float* T_s, const float* X_s, int I, int col, int rl, int kg) {
-  lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
-  for (int J = 0; J <= I; ++J)
+// ---- T . X on the bf16 MFMA with both factors split in three bf16 pieces, x = hi + mid + lo (each the upper 16 bits
+// of what the pieces before it leave, so hi + mid + lo has 24 significant bits): the six products down to 2^-16 of the
+// leading one (hi.hi, hi.mid, mid.hi, mid.mid, hi.lo, lo.hi) reproduce the fp32 product to about 2^-23 at 3/8 of the
+// fp32 MFMA's issue time.  (Two pieces per factor, 2^-16, moved stored state codes by two steps in places.)
+typedef __bf16 wy_v8bf __attribute__((ext_vector_type(8)));
+typedef float wy_v2f __attribute__((ext_vector_type(2)));
+
+LQ_DEV lq_v4f mfma_bf16(lq_v4i a, lq_v4i b, lq_v4f c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(wy_v8bf, a), __builtin_bit_cast(wy_v8bf, b), c, 0, 0, 0);
+}
+
+// two fp32 values -> one dword each of their hi, mid and lo pieces (first value in the low half)
+LQ_DEV void split3(float x0, float x1, uint32_t& hi, uint32_t& mid, uint32_t& lo) {
+  const uint32_t b0 = __float_as_uint(x0), b1 = __float_as_uint(x1);
+  hi = __builtin_amdgcn_perm(b1, b0, 0x07060302u);
+  const float r0 = x0 - __uint_as_float(b0 & 0xffff0000u), r1 = x1 - __uint_as_float(b1 & 0xffff0000u);  // exact
+  const uint32_t c0 = __float_as_uint(r0), c1 = __float_as_uint(r1);
+  mid = __builtin_amdgcn_perm(c1, c0, 0x07060302u);
+  const float q0 = r0 - __uint_as_float(c0 & 0xffff0000u), q1 = r1 - __uint_as_float(c1 & 0xffff0000u);  // exact
+  lo = __builtin_amdgcn_perm(__float_as_uint(q1), __float_as_uint(q0), 0x07060302u);
+}
+
+constexpr int kXP = 36;  // dwords per column of the transposed X tiles (32 token pairs + pad)
+constexpr int kXT = 64 * kXP;  // dwords per tile (64 columns)
+
+// X tiles in LDS: one tile per piece, [column][token pair] dwords (even token in the low half), 64 columns; the token-pair index is
+// XOR-ed with 8 * ((column >> 4) & 3) so that the transposing writes of one wave (8 pairs x 8 column groups) spread
+// over all banks while a 16-byte operand piece (4 pairs) stays whole.
+LQ_DEV int xt_index(int col, int pair) { return col * kXP + (pair ^ (((col >> 4) & 3) << 3)); }
+
+// T operand of row block I for contraction step st (tokens 32st + 8kg .. + 7): lane (rl, kg) holds T[16I + rl][those],
+// zero where the block column lies right of the diagonal block (never written)
+LQ_DEV void t_operand(const float* T_s, int I, int st, int rl, int kg, lq_v4i& th, lq_v4i& tm, lq_v4i& tl) {
+  const int m0 = 32 * st + 8 * kg;
+  const float* tp = T_s + (16 * I + rl) * kGS + m0;
+  const bool live = m0 < 16 * (I + 1);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int m = 16 * J + 4 * s + kg;
-      acc = mfma_f32(X_s[m * LS + col + rl], T_s[(16 * I + rl) * kGS + m], acc);
-    }
+  for (int d = 0; d < 4; ++d) {
+    const wy_v2f t2 = *(const wy_v2f*)(tp + 2 * d);
+    uint32_t h, m, l;
+    split3(live ? t2[0] : 0.0f, live ? t2[1] : 0.0f, h, m, l);
+    th[d] = (int)h, tm[d] = (int)m, tl[d] = (int)l;
+  }
+}
+
+// D^T tile of T . X for row block I and the 16 columns of tile nt: lane (rl = token, kg) gets columns 16nt + 4kg + r
+LQ_DEV lq_v4f tx_tile(const uint32_t* Xt, const lq_v4i (&th)[2], const lq_v4i (&tm)[2], const lq_v4i (&tl)[2], int I,
+                      int nt, int rl, int kg) {
+  lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int st = 0; st < 2; ++st) {
+    if (st > (I >> 1)) continue;
+    const int at = xt_index(16 * nt + rl, 16 * st + 4 * kg);
+    const lq_v4i xh = *(const lq_v4i*)(Xt + at), xm = *(const lq_v4i*)(Xt + kXT + at), xl = *(const lq_v4i*)(Xt + 2 * kXT + at);
+    acc = mfma_bf16(xl, th[st], acc);
+    acc = mfma_bf16(xh, tl[st], acc);
+    acc = mfma_bf16(xm, tm[st], acc);
+    acc = mfma_bf16(xm, th[st], acc);
+    acc = mfma_bf16(xh, tm[st], acc);
+    acc = mfma_bf16(xh, th[st], acc);
+  }
   return acc;
 }
 
@@ -188,12 +240,14 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
 
 template <int DECAY, int K, bool BF>
 __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
-  constexpr int LS = 64 + 16;  // floats per row of X (the T . X products run over 64 columns at a time): measured, a B-operand read (4 rows, 16 adjacent columns) takes one LDS pass at 80 floats and two at 72
+  constexpr int LS = 64 + 16;  // floats per row of the buffer that holds the Gram tile and then the X tiles
   static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
+  static_assert(3 * kXT <= 64 * kGS + 64 * LS, "the three bf16 pieces of a 64-column X tile overlay the T and X buffers");
   __shared__ __align__(16) float lds_f[64 * kGS + 64 * LS];  // 38 KB of LDS: four workgroups per compute unit
   float* T_s = lds_f;
   float* X_s = lds_f + 64 * kGS;
   float* G_s = X_s;
+  uint32_t* Xt = (uint32_t*)lds_f;  // overlays T once its operands sit in registers
   constexpr int kOP = 72;  // floats per row of the staged Gram operands: a 16-byte read of 16 rows x 4 adjacent pieces takes the minimum two LDS passes at 40 or 72
   static_assert(2 * 64 * kOP <= 64 * kGS + 64 * LS, "the Gram operands live in the T / X buffers until G is written");
   float* Lg_s = lds_f;
@@ -348,48 +402,71 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
     __syncthreads();
   }
 
+  // ---- T operands of this wave's two row blocks (w for the first half of the column tiles, 3 - w for the second:
+  // equal work), split once and kept in registers
+  lq_v4i th[2][2], tm[2][2], tl[2][2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int st = 0; st < 2; ++st) t_operand(T_s, u ? 3 - wave : wave, st, rl, kg, th[u][st], tm[u][st], tl[u][st]);
+  __syncthreads();  // T is dead from here on: the X tiles overlay it
+
+  // each thread stages two adjacent tokens x 8 columns of a 64-column tile: a dword of the transposed tile is a token pair
+  const int rp = tid >> 3, c8 = tid & 7;
+  const int64_t tok0 = t0 + 2 * rp;
+  auto stage = [&](const float (&xa)[8], const float (&xb)[8]) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      uint32_t hi, mid, lo;
+      split3(xa[e], xb[e], hi, mid, lo);
+      const int at = xt_index(8 * c8 + e, rp);
+      Xt[at] = hi, Xt[kXT + at] = mid, Xt[2 * kXT + at] = lo;
+    }
+  };
+
   // ---- Hw is written straight out; X = beta^sigma k exp(g) is staged 64 columns at a time (over the dead Gram tile)
   for (int kc = 0; kc < K; kc += 64) {
     if (kc > 0) __syncthreads();
-    for (int it = tid; it < 64 * 8; it += 256) {
-      const int r = it >> 3, c8 = it & 7;
-      const int64_t off = ((t0 + r) * H + h) * K + kc + 8 * c8;
-      float kv[8];
-      zoo_ld8(p.k + off, bf, kv);
-      const float bt = p.beta[(t0 + r) * H + h];
-      const float bw = powb(bt, (1.0f - sigma) * tau);
-      float bl = powb(bt, sigma);
-      if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(p.g[(t0 + r) * H + h]);
-      float ge[8];
-      if (DECAY == LQ_DECAY_DIAGONAL) {
-        const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+    {
+      float xr[2][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-      }
-      float hw[8];
-      lq_v4f x0, x1;
+      for (int u = 0; u < 2; ++u) {
+        const int64_t off = ((tok0 + u) * H + h) * K + kc + 8 * c8;
+        float kv[8];
+        zoo_ld8(p.k + off, bf, kv);
+        const float bt = p.beta[(tok0 + u) * H + h];
+        const float bw = powb(bt, (1.0f - sigma) * tau);
+        float bl = bs_s[2 * rp + u];
+        if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(gs_s[2 * rp + u]);
+        float ge[8];
+        if (DECAY == LQ_DECAY_DIAGONAL) {
+          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float kf = kv[e];
-        float x = bl * kf;
-        if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
-        if (e < 4) x0[e] = x; else x1[e - 4] = x;
-        hw[e] = bw * kf;
-      }
-      {
+          for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+        }
+        float hw[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float kf = kv[e];
+          float x = bl * kf;
+          if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
+          xr[u][e] = x;
+          hw[e] = bw * kf;
+        }
         lq_v4i o;
 #pragma unroll
         for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
         *(lq_v4i*)(p.Hw + off) = o;
       }
-      *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
-      *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
+      stage(xr[0], xr[1]);
     }
     __syncthreads();
     // W = T . X for these 64 columns
+#pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
-      const int I = nt < 2 ? wave : 3 - wave;
-      const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
+      const int u = nt < 2 ? 0 : 1;
+      const int I = u ? 3 - wave : wave;
+      const lq_v4f a = tx_tile(Xt, th[u], tm[u], tl[u], I, nt, rl, kg);
       lq_v2i o;
       o[0] = (int)zoo_enc2(a[0], a[1], bf);
       o[1] = (int)zoo_enc2(a[2], a[3], bf);
@@ -399,27 +476,25 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
 
   // ---- U = T . (beta^sigma v), 64 value columns per pass through the X buffer
   for (int vc = 0; vc < V; vc += 64) {
-    constexpr int pw = 64;
     __syncthreads();
-    for (int it = tid; it < 64 * (pw / 8); it += 256) {
-      const int r = it / (pw / 8), c8 = it % (pw / 8);
-      float vv[8];
-      zoo_ld8(p.v + ((t0 + r) * H + h) * V + vc + 8 * c8, bf, vv);
-      const float bsr = bs_s[r];
-      lq_v4f x0, x1;
+    {
+      float xr[2][8];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        x0[e] = bsr * vv[e];
-        x1[e] = bsr * vv[4 + e];
+      for (int u = 0; u < 2; ++u) {
+        float vv[8];
+        zoo_ld8(p.v + ((tok0 + u) * H + h) * V + vc + 8 * c8, bf, vv);
+        const float bsr = bs_s[2 * rp + u];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xr[u][e] = bsr * vv[e];
       }
-      *(lq_v4f*)(X_s + r * LS + 8 * c8) = x0;
-      *(lq_v4f*)(X_s + r * LS + 8 * c8 + 4) = x1;
+      stage(xr[0], xr[1]);
     }
     __syncthreads();
-    const int ntl = pw / 16;
-    for (int nt = 0; nt < ntl; ++nt) {
-      const int I = nt < ntl / 2 ? wave : 3 - wave;
-      const lq_v4f a = tx_tile<LS>(T_s, X_s, I, 16 * nt, rl, kg);
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int u = nt < 2 ? 0 : 1;
+      const int I = u ? 3 - wave : wave;
+      const lq_v4f a = tx_tile(Xt, th[u], tm[u], tl[u], I, nt, rl, kg);
       lq_v2i o;
       o[0] = (int)zoo_enc2(a[0], a[1], bf);
       o[1] = (int)zoo_enc2(a[2], a[3], bf);
