@@ -15,7 +15,7 @@
 // the full contraction).  The carry lives in registers: wave w owns K/4 rows.  The stored state goes through
 // LDS V-major so that it is copied out coalesced and read back as the K-contiguous operand of the state read;
 // the pseudo-value codes go through LDS channel-major so that they are the token-contiguous operand of the
-// write product.  All global operands of chunk c+1 are fetched into registers while chunk c is computed.
+// write product.  All global operands of chunk c+2 are fetched into registers while chunk c is computed.
 #include "zoo_params.h"
 #include "../../include/linquant_hip.h"
 
@@ -33,8 +33,10 @@ struct StepOps {
   float fw[DELTA ? 4 : 1], ev[DELTA ? 4 : 1];
 };
 
-template <bool DELTA, int K, int BV>
-__global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
+// BF (bf16 activations) is a template parameter: as a run-time flag every decode / encode of U and E in the chunk loop
+// became a branch of its own.
+template <bool DELTA, int K, int BV, bool BF>
+__global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StateParams p) {
   constexpr int KR = K / 4;     // carry rows per wave
   constexpr int KT = KR / 16;   // 16-row tiles per wave (= K / 64)
   constexpr int VT = BV / 16;   // 16-col tiles
@@ -48,11 +50,23 @@ __global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  const int v0 = blockIdx.x * BV;
-  const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+  // Workgroups are dealt to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The V tiles of one
+  // (batch, head) read the same key, state-read and decay operands at the same time, so they are renumbered onto one
+  // XCD (consecutive slots of it) whenever the grid divides evenly; otherwise each tile fetches its own copy from HBM.
+  int vtile = blockIdx.x, bh = blockIdx.y;
+  {
+    const int nv = gridDim.x, total = gridDim.x * gridDim.y;
+    if (total % 8 == 0 && (total / 8) % nv == 0) {
+      const int lid = blockIdx.x + nv * blockIdx.y;
+      const int vid = (lid % 8) * (total / 8) + lid / 8;
+      vtile = vid % nv, bh = vid / nv;
+    }
+  }
+  const int v0 = vtile * BV;
+  const int b = bh / p.H, h = bh % p.H;
   const int H = p.H, V = p.V, T = p.T, NT = p.NT;
   const int qmax = p.qmax;
-  const bool bf = p.bf != 0;
+  constexpr bool bf = BF;
 
   // per-lane scales of the carry tile: rows k = KR*wave + 16kt + 4kg + r, cols v = v0 + 16vt + rl
   float skw_r[KT][4], svw_c[VT], inv_ss_c[VT];
@@ -118,11 +132,11 @@ __global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) hc[kt][vt][r] = 0.0f;
 
-  StepOps<DELTA, K, BV> cur, nxt;
-  load_step(0, cur);
-  nxt = cur;
-
-  for (int ct = 0; ct < NT; ++ct) {
+  // One chunk step; the operands of chunk ct + 2 are requested into `pre` at its start.  Vector memory operations
+  // retire in issue order, loads and stores alike, so a load issued behind the stores of the previous step is not seen
+  // complete before those stores are acknowledged: with one step of look-ahead that acknowledgement sat on the critical
+  // path of every step, with two it has a whole step to arrive.
+  auto do_step = [&](int ct, StepOps<DELTA, K, BV>& cur, StepOps<DELTA, K, BV>& pre) {
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
     unsigned char* hTb = hT + (DELTA ? 0 : (ct & 1) * BV * HS);
     // ---- stored copy of the incoming state -> LDS (V-major)
@@ -135,7 +149,7 @@ __global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
         for (int r = 0; r < 4; ++r) cd[r] = zoo_q8(hc[kt][vt][r], inv_ss_c[vt], 127);
         *(uint32_t*)(hTb + (16 * vt + rl) * HS + KR * wave + 16 * kt + 4 * kg) = zoo_pack_codes(cd[0], cd[1], cd[2], cd[3]);
       }
-    if (ct + 1 < NT) load_step(ct + 1, nxt);
+    if (ct + 2 < NT) load_step(ct + 2, pre);
     __syncthreads();
 
     // ---- copy the stored state out, coalesced: h_i8[b][ct][h][v0 + v][k]
@@ -211,7 +225,16 @@ __global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
         }
       }
     }
-    cur = nxt;
+  };
+
+  StepOps<DELTA, K, BV> s0, s1, s2;
+  load_step(0, s0);
+  s2 = s1 = s0;
+  if (NT > 1) load_step(1, s1);
+  for (int ct = 0; ct < NT; ct += 3) {
+    do_step(ct, s0, s2);
+    if (ct + 1 < NT) do_step(ct + 1, s1, s0);
+    if (ct + 2 < NT) do_step(ct + 2, s2, s1);
   }
 
   if (p.ht) {
@@ -228,12 +251,21 @@ __global__ __launch_bounds__(256, 2) void zoo_state_kernel(StateParams p) {
 template <bool DELTA, int K>
 int launch_bv(const StateParams& p, int BV, int B, hipStream_t stream) {
   dim3 grid(p.V / BV, B * p.H);
+  constexpr bool D = DELTA;  // the linear family touches no half-precision tensor: one instantiation serves both dtypes
+#define LQ_STATE_LAUNCH(BVV)                                                                                  \
+  do {                                                                                                        \
+    if (D && p.bf)                                                                                            \
+      hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, BVV, D>), grid, dim3(256), 0, stream, p);                \
+    else                                                                                                      \
+      hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, BVV, false>), grid, dim3(256), 0, stream, p);            \
+  } while (0)
   if (BV == 64)
-    hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, 64>), grid, dim3(256), 0, stream, p);
+    LQ_STATE_LAUNCH(64);
   else if (BV == 32)
-    hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, 32>), grid, dim3(256), 0, stream, p);
+    LQ_STATE_LAUNCH(32);
   else
-    hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, 16>), grid, dim3(256), 0, stream, p);
+    LQ_STATE_LAUNCH(16);
+#undef LQ_STATE_LAUNCH
   return lq_check_launch();
 }
 
