@@ -35,9 +35,21 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  const int v0 = blockIdx.x * BV;
-  const int ct = blockIdx.y;
-  const int b = blockIdx.z / p.H, h = blockIdx.z % p.H;
+  // Workgroups go to the 8 XCDs round-robin by linear id and each XCD has its own L2: the V tiles of one (chunk,
+  // batch, head) read the same q / k / A rows, so they are renumbered onto one XCD when the grid divides evenly.
+  int vtile = blockIdx.x, ct = blockIdx.y, bh = blockIdx.z;
+  {
+    const int nv = gridDim.x, total = gridDim.x * gridDim.y * gridDim.z;
+    if (nv > 1 && total % 8 == 0 && (total / 8) % nv == 0) {
+      const int lid = blockIdx.x + nv * (blockIdx.y + gridDim.y * blockIdx.z);
+      const int vid = (lid % 8) * (total / 8) + lid / 8;
+      vtile = vid % nv;
+      ct = (vid / nv) % gridDim.y;
+      bh = vid / (nv * gridDim.y);
+    }
+  }
+  const int v0 = vtile * BV;
+  const int b = bh / p.H, h = bh % p.H;
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
   const float sq = p.sq[h];
