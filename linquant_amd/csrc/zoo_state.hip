@@ -149,16 +149,27 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
         for (int r = 0; r < 4; ++r) cd[r] = zoo_q8(hc[kt][vt][r], inv_ss_c[vt], 127);
         *(uint32_t*)(hTb + (16 * vt + rl) * HS + KR * wave + 16 * kt + 4 * kg) = zoo_pack_codes(cd[0], cd[1], cd[2], cd[3]);
       }
-    if (ct + 2 < NT) load_step(ct + 2, pre);
+    // requested unconditionally (the last chunks re-request the final one): a branch around the loads would make the
+    // compiler's count of outstanding memory operations path-dependent, and it then waits for the newest loads as well
+    load_step(min(ct + 2, NT - 1), pre);
     __syncthreads();
 
     // ---- copy the stored state out, coalesced: h_i8[b][ct][h][v0 + v][k]
     {
       int8_t* dst = p.h_i8 + ((((int64_t)b * NT + ct) * H + h) * V + v0) * K;
       constexpr int SEG = K / 16;
-      for (int it = tid; it < BV * SEG; it += 256) {
-        const int vr = it / SEG, sg = it % SEG;
-        *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hTb + vr * HS + sg * 16);
+      if constexpr (BV * SEG % 256 == 0) {
+#pragma unroll
+        for (int i = 0; i < BV * SEG / 256; ++i) {
+          const int it = tid + 256 * i;
+          const int vr = it / SEG, sg = it % SEG;
+          *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hTb + vr * HS + sg * 16);
+        }
+      } else {
+        for (int it = tid; it < BV * SEG; it += 256) {
+          const int vr = it / SEG, sg = it % SEG;
+          *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hTb + vr * HS + sg * 16);
+        }
       }
     }
 
@@ -230,12 +241,29 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
   StepOps<DELTA, K, BV> s0, s1, s2;
   load_step(0, s0);
   s2 = s1 = s0;
-  if (NT > 1) load_step(1, s1);
-  for (int ct = 0; ct < NT; ct += 3) {
-    do_step(ct, s0, s2);
-    if (ct + 1 < NT) do_step(ct + 1, s1, s0);
-    if (ct + 2 < NT) do_step(ct + 2, s2, s1);
+  load_step(min(1, NT - 1), s1);
+  // Everything requested so far (scales, the first two operand sets) is waited for here, once.  The compiler places its
+  // waits from a count of the memory operations issued after a load; a load still outstanding at loop entry has few
+  // operations behind it on the entry path, and the merged count would make every iteration wait until almost nothing
+  // is in flight, the look-ahead loads included.
+  asm volatile("" ::: "memory");  // keeps the requests above on this side of the wait
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), as an instruction the compiler's own wait placement accounts for
+  asm volatile("" ::: "memory");
+  // Six steps per trip.  The operand sets rotate with period three; what the compiler cannot do is carry a set that is
+  // still being loaded across the loop's back edge without copying it (the copy waits for loads issued only a step
+  // earlier), so the back edge is met every sixth step (every twelfth was slower again: instruction cache).
+#define LQ_STEP3(base)                   \
+  do_step(ct + (base), s0, s2);          \
+  if (ct + (base) + 1 >= NT) break;      \
+  do_step(ct + (base) + 1, s1, s0);      \
+  if (ct + (base) + 2 >= NT) break;      \
+  do_step(ct + (base) + 2, s2, s1);      \
+  if (ct + (base) + 3 >= NT) break;
+  for (int ct = 0; ct < NT; ct += 6) {
+    LQ_STEP3(0)
+    LQ_STEP3(3)
   }
+#undef LQ_STEP3
 
   if (p.ht) {
 #pragma unroll
