@@ -84,7 +84,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   uint32_t* xS = xP + (Q / 8) * kQuad;        // [Q/8][kQuad]
   float* dA2_s = (float*)(xS + (Q / 8) * kQuad);  // dA * log2(e)
   float* w_s = dA2_s + Q;                     // S_cb * dt
-  int8_t* S_s = (int8_t*)(w_s + Q);           // [64][kSRow] state tile of this (chunk, head), row p at (p & 3) * 16 + (p >> 2)
+  float* ssl_s = w_s + Q;                     // [64] C scale * state scale of the tile's channels
+  float* Dl_s = ssl_s + 64;                   // [64] dequantized D of the tile's channels
+  int8_t* S_s = (int8_t*)(Dl_s + 64);           // [64][kSRow] state tile of this (chunk, head), row p at (p & 3) * 16 + (p >> 2)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -111,8 +113,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
   for (int k = 0; k < kSPieces; ++k) {
     const int t = tid + k * WAVES * 64;
-    spiece[k] = lq_v4i{0, 0, 0, 0};
-    if (t < 4 * N) spiece[k] = *(const lq_v4i*)(Sp + t * 16);
+    spiece[k] = *(const lq_v4i*)(Sp + min(t, 4 * N - 1) * 16);  // unconditional: a surplus thread re-reads the last piece
   }
   lq_v4i cop[2][N64];
   {
@@ -124,11 +125,19 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       for (int n = 0; n < N64; ++n) cop[i][n] = *(const lq_v4i*)(Cp + coff + 64 * n);
     }
   }
-  float dA_r = 0.0f, dt_r = 0.0f;  // Q <= WAVES * 64: one element per thread
-  if (tid < Q) {
-    dA_r = p.dA[cs + tid];
-    dt_r = p.dt[cs + tid];
-  }
+  // Q <= WAVES * 64: one element per thread; requested without a branch (a conditional request is waited for where
+  // the branches join, which here is before the x tile has even been requested)
+  const float dA_r = p.dA[cs + min(tid, Q - 1)];
+  const float dt_r = p.dt[cs + min(tid, Q - 1)];
+  // per-channel scale and D of channel p0 + (tid & 63): they go through LDS with the other small operands (requested
+  // before the bulk of the prologue so that waiting for them does not wait for the x tile: memory operations retire in
+  // issue order)
+  const float ss_r = p.ss[(int64_t)h * p.sss_h + (int64_t)(p0 + (tid & 63)) * p.sss_p];
+  // without D the request goes to a valid dummy address and dsc = 0 discards it: no branch around a request
+  const int8_t* Dp = p.D ? p.D + (int64_t)h * p.sD_h + (p.D_has_hdim ? p0 + (tid & 63) : 0) : p.states;
+  const int D_r = (int)*Dp;
+  const float gscale = p.C_scale[g];
+  const float dsc = p.D ? *p.D_scale : 0.0f;
   const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0;
   lq_v8h r0[2], r1[2];
   int kp_of[2], c8_of[2];
@@ -137,28 +146,31 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     const int item = tid + it * WAVES * 64;  // Q*4 items in total, 2 per thread
     const int kp = item >> 3, c8 = item & 7;
     kp_of[it] = kp, c8_of[it] = c8;
-    lq_v8h z = {0, 0, 0, 0, 0, 0, 0, 0};
-    r0[it] = z, r1[it] = z;
-    if (2 * kp < limit) r0[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp) * p.sx_l + c8 * 8);
-    if (2 * kp + 1 < limit) r1[it] = *(const lq_v8h*)(xg + (int64_t)(2 * kp + 1) * p.sx_l + c8 * 8);
+    // rows past the sequence end re-read its last row and are zeroed when staged (no branch around a request)
+    r0[it] = *(const lq_v8h*)(xg + (int64_t)min(2 * kp, limit - 1) * p.sx_l + c8 * 8);
+    r1[it] = *(const lq_v8h*)(xg + (int64_t)min(2 * kp + 1, limit - 1) * p.sx_l + c8 * 8);
   }
-  // Small per-head operands of the epilogues are fetched now: issued where they are used, each would expose a full
-  // memory round trip behind the barriers.
-  float ssv[4], Dv[4] = {0.f, 0.f, 0.f, 0.f};
-  {
-    const float gscale = p.C_scale[g];
+  // CB codes of this wave's off-diagonal slabs.  The early tile has ne = rb[0] / 32 of them, the late one the rest of
+  // NS = WAVES - 1 (the same total for every wave), so they are walked as one flat list of NS steps whose loads run four
+  // steps ahead through a ring of four registers: every request is unconditional and its position in the instruction
+  // stream is fixed, which keeps the compiler's wait counts exact (a one-ahead prefetch inside `if (J + 1 < nslab)`
+  // was waited for in full at every step).  The codes of the two own slabs are requested here as well.
+  constexpr int NS = WAVES - 1;
+  const int8_t* cbp = p.cb + ((((int64_t)b * p.nchunks + c) * p.G + g) * Q) * Q;
+  const int ne = __builtin_amdgcn_readfirstlane(rb[0] >> 5);
+  const int8_t* crow0 = cbp + (rb[0] + rl) * Q + 8 * kg;
+  const int8_t* crow1 = cbp + (rb[1] + rl) * Q + 8 * kg;
+  auto cb_slab = [&](int s) { return *(const lq_v2i*)(s < ne ? crow0 + 32 * s : crow1 + 32 * (s - ne)); };
+  lq_v2i cwr[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) ssv[j] = gscale * p.ss[(int64_t)h * p.sss_h + (int64_t)(p0 + 4 * rl + j) * p.sss_p];
-    if (p.D) {
-      const float dsc = *p.D_scale;
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        Dv[j] = dsc * (float)p.D[(int64_t)h * p.sD_h + (p.D_has_hdim ? p0 + 4 * rl + j : 0)];
-    }
-  }
+  for (int s = 0; s < 4; ++s) cwr[s] = cb_slab(s < NS ? s : NS - 1);
   if (tid < Q) {
     dA2_s[tid] = dA_r * 1.44269504088896340736f;
     w_s[tid] = scb * dt_r;
+  }
+  if (tid < 64) {
+    ssl_s[tid] = gscale * ss_r;
+    Dl_s[tid] = dsc * (float)D_r;
   }
 #pragma unroll
   for (int k = 0; k < kSPieces; ++k) {
@@ -167,6 +179,10 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     if (t < 4 * N) *(lq_v4i*)(S_s + ((pr & 3) * 16 + (pr >> 2)) * kSRow + pc * 16) = spiece[k];
   }
   __syncthreads();
+  // codes of the two own slabs: needed after the state path and the off-diagonal slabs
+  lq_v2i cwo[2];
+  cwo[0] = *(const lq_v2i*)(crow0 + (rb[0] & ~31));
+  cwo[1] = *(const lq_v2i*)(crow1 + (rb[1] & ~31));
   // ---- state path (INT8 MFMA): C rows from registers, state rows from LDS
   lq_v4i ai[2][4];
 #pragma unroll
@@ -186,9 +202,10 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     const float ae = dA2_s[ke];
     const lq_v2h g2 = {(_Float16)(fexp2(ae - dA2_s[k]) * w_s[k]), (_Float16)(fexp2(ae - dA2_s[k + 1]) * w_s[k + 1])};
     const int base = (kp >> 2) * kQuad + (2 * c8) * 4 + (kp & 3);
+    const bool in0 = k < limit, in1 = k + 1 < limit;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const lq_v2h pr = {r0[it][e], r1[it][e]};
+      const lq_v2h pr = {in0 ? r0[it][e] : (_Float16)0.0f, in1 ? r1[it][e] : (_Float16)0.0f};
       const int off = base + ((e & 3) * 16 + (e >> 2)) * 4;  // x_slot(8 c8 + e) * 4
       xP[off] = __builtin_bit_cast(uint32_t, pr);
       xS[off] = __builtin_bit_cast(uint32_t, pr * g2);
@@ -201,6 +218,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   // ---- state read dequantized and gated: float(acc) * (sC * ss[p]) * exp(dA_m)
   lq_v4f acc[2][4];  // [row tile][channel call j]
   {
+    const lq_v4f ssv = *(const lq_v4f*)(ssl_s + 4 * rl);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -211,77 +229,80 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       }
   }
 
-  const int8_t* cbp = p.cb + ((((int64_t)b * p.nchunks + c) * p.G + g) * Q) * Q;
-
+  // ---- slabs before each tile's own slab: (scaled CB codes) x (anchor-scaled x), row factor applied once per tile.
+  // A tile past the sequence end is processed like any other (its rows are never stored).
+  {
+    // anchor of a tile = last token before its own slab
+    const float aE0 = dA2_s[max(rb[0] & ~31, 1) - 1], aE1 = dA2_s[(rb[1] & ~31) - 1];
+    lq_v4f off[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    if (rb[i] >= limit) continue;
-    const int nslab = rb[i] >> 5;      // 32-token slabs strictly before the slab that holds this tile
-    const int sbase = 32 * nslab;      // first token of the tile's own slab
-    const int8_t* crow = cbp + (int64_t)(rb[i] + rl) * Q;
-    // ---- slabs before the tile's own slab: (scaled CB codes) x (anchor-scaled x), row factor applied once
-    if (nslab > 0) {
-      lq_v4f off[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) off[j] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-      const float aE = dA2_s[sbase - 1];
-      lq_v2i cw = *(const lq_v2i*)(crow + 8 * kg), cwn = cw;
-      for (int J = 0; J < nslab; ++J) {
-        if (J + 1 < nslab) cwn = *(const lq_v2i*)(crow + 32 * (J + 1) + 8 * kg);
-        const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
-        const lq_v2h s2 = {sh, sh};
-        const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
-        lq_v4i xop[4];  // token pairs 16 J + 4 kg .. + 3 of channel 4 rl + j
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xS + (4 * J + kg) * kQuad + (j * 16 + rl) * 4);
-        lq_v4i aw;
-        uint32_t lo, hi;
-        i8x4_to_f16x4((uint32_t)cw[0], s2, o2, lo, hi);
-        aw[0] = (int)lo, aw[1] = (int)hi;
-        i8x4_to_f16x4((uint32_t)cw[1], s2, o2, lo, hi);
-        aw[2] = (int)lo, aw[3] = (int)hi;
-        const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) off[j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[j]);
-        cw = cwn;
-      }
+    for (int j = 0; j < 4; ++j) off[j] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+    auto flush = [&](int i, float aE) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float rf = fexp2(dA2_s[rb[i] + 4 * kg + r] - aE);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j][r] = fmaf(off[j][r], rf, acc[i][j][r]);
+        for (int j = 0; j < 4; ++j) acc[i][j][r] = fmaf(off[j][r], rf, acc[i][j][r]), off[j][r] = 0.0f;
       }
-    }
-
-    // ---- the tile's own 32-token slab: per-element weights exp2(dA2_m - (dA2_k - log2(S_cb dt_k))), k <= m
-    {
-      const int m = rb[i] + rl;
-      const float dAm = dA2_s[m];
-      const int kb = sbase + 8 * kg;
-      lq_v4i xop[4];
+    };
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xP + (kb >> 3) * kQuad + (j * 16 + rl) * 4);
-      const lq_v4f a0 = *(const lq_v4f*)(dA2_s + kb), a1 = *(const lq_v4f*)(dA2_s + kb + 4);
-      const lq_v4f w0 = *(const lq_v4f*)(w_s + kb), w1 = *(const lq_v4f*)(w_s + kb + 4);
-      const lq_v2i cw = *(const lq_v2i*)(crow + kb);
-      float v[8];
+    for (int s = 0; s < NS; ++s) {
+      if (s > 0 && s <= (WAVES - 1) / 2 && s == ne) flush(0, aE0);  // the early tile's slabs are done (wave-uniform)
+      const bool late = s >= ne;
+      const int J = late ? s - ne : s;
+      const float aE = late ? aE1 : aE0;
+      const lq_v2i cw = cwr[s & 3];
+      if (s + 4 < NS) cwr[s & 3] = cb_slab(s + 4);
+      const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
+      const lq_v2h s2 = {sh, sh};
+      const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
+      lq_v4i xop[4];  // token pairs 16 J + 4 kg .. + 3 of channel 4 rl + j
 #pragma unroll
-      for (int t = 0; t < 8; ++t) {
-        const float akw = (t < 4 ? a0[t & 3] : a1[t & 3]) - __builtin_amdgcn_logf(t < 4 ? w0[t & 3] : w1[t & 3]);
-        const float cf = (float)lq_sbyte((uint32_t)cw[t >> 2], t & 3);
-        v[t] = cf * fexp2(dAm - akw);
-        if (kb + t > m) v[t] = 0.0f;
-      }
+      for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xS + (4 * J + kg) * kQuad + (j * 16 + rl) * 4);
       lq_v4i aw;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) aw[d] = (int)pack_h2(v[2 * d], v[2 * d + 1]);
+      uint32_t lo, hi;
+      i8x4_to_f16x4((uint32_t)cw[0], s2, o2, lo, hi);
+      aw[0] = (int)lo, aw[1] = (int)hi;
+      i8x4_to_f16x4((uint32_t)cw[1], s2, o2, lo, hi);
+      aw[2] = (int)lo, aw[3] = (int)hi;
       const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), acc[i][j]);
+      for (int j = 0; j < 4; ++j) off[j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[j]);
     }
+    if (NS > 0) flush(1, aE1);
+  }
+
+  // ---- each tile's own 32-token slab: per-element weights exp2(dA2_m - (dA2_k - log2(S_cb dt_k))), k <= m
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int sbase = rb[i] & ~31;  // first token of the tile's own slab
+    const int m = rb[i] + rl;
+    const float dAm = dA2_s[m];
+    const int kb = sbase + 8 * kg;
+    lq_v4i xop[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xP + (kb >> 3) * kQuad + (j * 16 + rl) * 4);
+    const lq_v4f a0 = *(const lq_v4f*)(dA2_s + kb), a1 = *(const lq_v4f*)(dA2_s + kb + 4);
+    const lq_v4f w0 = *(const lq_v4f*)(w_s + kb), w1 = *(const lq_v4f*)(w_s + kb + 4);
+    const lq_v2i cw = cwo[i];
+    float v[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      const float akw = (t < 4 ? a0[t & 3] : a1[t & 3]) - __builtin_amdgcn_logf(t < 4 ? w0[t & 3] : w1[t & 3]);
+      const float cf = (float)lq_sbyte((uint32_t)cw[t >> 2], t & 3);
+      v[t] = cf * fexp2(dAm - akw);
+      if (kb + t > m) v[t] = 0.0f;
+    }
+    lq_v4i aw;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) aw[d] = (int)pack_h2(v[2 * d], v[2 * d + 1]);
+    const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), acc[i][j]);
   }
 
   // ---- D residual + store
+  const lq_v4f Dv = *(const lq_v4f*)(Dl_s + 4 * rl);
   _Float16* op = p.out + (((int64_t)b * p.seqlen + (int64_t)c * Q) * p.nheads + h) * p.P + p0 + 4 * rl;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
@@ -334,7 +355,7 @@ extern "C" int lq_chunk_scan(const lq_chunk_scan_args* a, hipStream_t stream) {
   const int64_t by = (int64_t)p.batch * p.nchunks;
   if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
   if ((int64_t)p.Q * p.sC_l >= (1ll << 31) || (int64_t)p.P * p.N >= (1ll << 31)) return LQ_ERR_SHAPE;  // 32-bit lane offsets
-  const size_t lds = (size_t)2 * (p.Q / 8) * kQuad * 4 + (size_t)p.Q * 8 + (size_t)64 * (p.N + 32);  // x tiles, dA2, w, states
+  const size_t lds = (size_t)2 * (p.Q / 8) * kQuad * 4 + (size_t)p.Q * 8 + 512 + (size_t)64 * (p.N + 32);  // x tiles, dA2, w, per-channel scales, states
   dim3 grid((p.P / 64) * p.nheads, (unsigned)by, 1);
   // more than 64 KB of dynamic LDS has to be opted into per kernel
 #define LQ_SCAN_LAUNCH(W, NN)                                                                                   \
