@@ -70,7 +70,12 @@ LQ_DEV float mul_half(uint32_t w, float f) {
   return __builtin_fmaf((float)h[HI], f, 0.0f);
 }
 
-template <bool KEYSIDE, int NT>
+// NSLAB = number of 64-token slabs of a chunk when it is one of the unrolled counts (2, 4), else 0 (run-time loop).
+// With a known count the slab loop is fully unrolled over two register sets: the next slab is requested before the
+// current one is quantized, no request sits inside a run-time branch, and the compiler's wait counts stay exact.
+// Measured at B4 L8192 H80 P64 N128 Q256: value side 115 -> 108 us; key side 146 -> 150 us (its slabs are bound by the
+// per-head quantization arithmetic of B, not by the loads), so the key side keeps the run-time loop.
+template <bool KEYSIDE, int NT, int NSLAB>
 __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int Q = p.Q;
@@ -93,76 +98,94 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   const int limit = min(Q, p.seqlen - c * Q);
   const int64_t cs = (((int64_t)b * p.nheads + h) * p.nchunks + c) * Q;
 
-  // ---- gates of the whole chunk
-  {
-    const float dA_last = p.dA[cs + Q - 1];
-    for (int k = tid; k < Q; k += 256) gate_s[k] = k < limit ? lq_expf(dA_last - p.dA[cs + k]) * p.dt[cs + k] : 0.0f;
-    if (KEYSIDE && tid < NT) {
-      const int n = n0 + tid;
-      bdeq_s[tid] = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n] / 127.0f;
-    }
-  }
+  // ---- Every global request of the prologue is issued first, oldest first in the order of first use, and none sits
+  // inside a branch: memory operations retire in issue order, a request inside a branch is waited for where the branches
+  // join, and arithmetic on a loaded value is a wait for it.  (The gates were computed by a loop that waited for dA and
+  // for dt in turn, followed by a wait for the B scales: three memory round trips before the first slab was requested.)
+  // Tokens past the sequence end carry a zero gate, which zeroes the gated operand's codes; their loads are redirected
+  // to the last valid token so no access leaves the tensor.
+  const float dA_last = p.dA[cs + Q - 1];
+  const int kg0 = min(tid, Q - 1);  // gate of token kg0 (threads past a short chunk repeat its last token)
+  const float dA_k = p.dA[cs + kg0];
+  const float dt_k = p.dt[cs + kg0];
+  float bg_t = 1.0f;
+  if (KEYSIDE)
+    bg_t = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)(n0 + (tid & (NT - 1))) * p.sbg_n];
 
-  // ---- fixed thread -> work mapping of the quantize phase: x slab = 16 token quads x 16 groups of 4 channels
-  // (all 256 threads), B slab = 16 token quads x NT/8 groups of 8 channels.  Tokens past the sequence end
-  // carry a zero gate, which zeroes the gated operand's codes; their loads are redirected to the last valid
-  // token so no access leaves the tensor.
+  // fixed thread -> work mapping of the quantize phase: x slab = 16 token quads x 16 groups of 4 channels (all 256
+  // threads), B slab = 16 token quads x NT/8 groups of 8 channels (threads without a B item load a clamped address)
   const int kqx = tid >> 4, c4x = tid & 15;
   constexpr int kBItems = NT / 8;
   const bool has_b = (NT == 128) || (tid < 16 * kBItems);
   const int kqb = (NT == 128) ? (tid >> 4) : (tid / kBItems);
   const int cb8 = (NT == 128) ? (tid & 15) : (tid % kBItems);
 
-  float xinv[4], binv[8];
+  float xs_raw[4], bg_raw[8];
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    const float sc = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 4 * c4x + e) * p.sxs_p];
-    xinv[e] = KEYSIDE ? 1.0f / fmaxf(sc, 1e-10f) : 1.0f / sc;
-  }
-  if (KEYSIDE && has_b) {
+  for (int e = 0; e < 4; ++e) xs_raw[e] = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 4 * c4x + e) * p.sxs_p];
+  if (KEYSIDE) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int n = n0 + 8 * cb8 + e;
-      binv[e] = 127.0f / p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)n * p.sbg_n];
-    }
+    for (int e = 0; e < 8; ++e)
+      bg_raw[e] = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)(n0 + 8 * cb8 + e) * p.sbg_n];
   }
+  // scales of the epilogue (requested here: at their point of use they would expose one more round trip)
+  const int pr = p0 + 16 * wave + rl;
+  const float xs_ep = p.xs[(int64_t)h * p.sxs_h + (int64_t)pr * p.sxs_p];
+  const float so_ep = p.oqs[(int64_t)h * p.soq_h + (int64_t)pr * p.soq_p];
+  const float bs_ep = KEYSIDE ? 0.0f : p.bscale_g[(int64_t)g * p.sbs_g];
 
   const int last = limit - 1;
   const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0 + 4 * c4x;
   const char* bg0 = (const char*)p.B + ((int64_t)b * p.sB_b + (int64_t)c * Q * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8) * (KEYSIDE ? 2 : 1);
   const int64_t bstep = p.sB_l * (KEYSIDE ? 2 : 1);  // bytes per token
-  lq_v2i xr[4];  // x: 4 tokens x 4 fp16
-  lq_v4i br[4];  // key side: 4 tokens x 8 fp16; value side: only [t][0..1] used (8 int8)
+  lq_v2i xrA[4], xrB[4];  // x: 4 tokens x 4 fp16 (two sets: the slab being quantized and the one in flight)
+  lq_v4i brA[4], brB[4];  // key side: 4 tokens x 8 fp16; value side: only [t][0..1] used (8 int8)
 
   // token * stride stays below 2^31 and both factors below 2^23 (checked by the launcher): a full-rate 24-bit multiply
   // instead of the quarter-rate 64-bit one, eight times per slab
   const int sxl = (int)p.sx_l, bst = (int)bstep;
-  auto load_slab = [&](int k0) {
+  auto load_slab = [&](int k0, lq_v2i (&xr)[4], lq_v4i (&br)[4]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int kx = min(k0 + 4 * kqx + t, last);
       xr[t] = *(const lq_v2i*)(xg + __mul24(kx, sxl));
-      if (has_b) {
-        const int kb = min(k0 + 4 * kqb + t, last);
-        if (KEYSIDE) {
-          br[t] = *(const lq_v4i*)(bg0 + __mul24(kb, bst));
-        } else {
-          const lq_v2i v = *(const lq_v2i*)(bg0 + __mul24(kb, bst));
-          br[t][0] = v[0], br[t][1] = v[1];
-        }
+      const int kb = min(k0 + 4 * kqb + t, last);
+      if (KEYSIDE) {
+        br[t] = *(const lq_v4i*)(bg0 + __mul24(kb, bst));
+      } else {
+        const lq_v2i v = *(const lq_v2i*)(bg0 + __mul24(kb, bst));
+        br[t][0] = v[0], br[t][1] = v[1];
       }
     }
   };
+  load_slab(0, xrA, brA);
+
+  // ---- gates of the whole chunk, dequantization scales of B, reciprocal operand scales
+  // (written by every thread, duplicates included: a store under `if (tid < Q)` lets the compiler sink the requests
+  // above into that branch, which puts their round trip back on the critical path)
+  {
+    const float gv = lq_expf(dA_last - dA_k) * dt_k;
+    gate_s[kg0] = kg0 < limit ? gv : 0.0f;
+  }
+  for (int k = tid + 256; k < Q; k += 256)  // chunks longer than the workgroup
+    gate_s[k] = k < limit ? lq_expf(dA_last - p.dA[cs + k]) * p.dt[cs + k] : 0.0f;
+  if (KEYSIDE) bdeq_s[tid & (NT - 1)] = bg_t / 127.0f;
+  float xinv[4], binv[8];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) xinv[e] = KEYSIDE ? 1.0f / fmaxf(xs_raw[e], 1e-10f) : 1.0f / xs_raw[e];
+  if (KEYSIDE) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) binv[e] = 127.0f / bg_raw[e];
+  }
 
   lq_v4i acc[NT / 16];
 #pragma unroll
   for (int q = 0; q < NT / 16; ++q) acc[q] = lq_v4i{0, 0, 0, 0};
 
-  load_slab(0);
   __syncthreads();  // gates visible
 
   const int nslab = Q >> 6;
-  for (int s = 0; s < nslab; ++s) {
+  auto slab = [&](int s, lq_v2i (&xr)[4], lq_v4i (&br)[4], auto post) {
     const int k0 = s * 64;
     uint32_t* xb = xq + (s & 1) * 16 * kXW;
     uint32_t* bb = bq + (s & 1) * 16 * kBW;
@@ -224,7 +247,7 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
       *(lq_v4i*)dst = bo[0];
       *(lq_v4i*)(dst + 4) = bo[1];
     }
-    if (s + 1 < nslab) load_slab(k0 + 64);
+    post();  // the run-time loop requests the next slab here, into the registers just consumed
     __syncthreads();
     // ---- MFMA from LDS: rows = N (this tile), cols = the wave's 16 P rows
     lq_v4i xop;
@@ -237,14 +260,28 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
       for (int i = 0; i < 4; ++i) bop[i] = (int)bb[(4 * kg + i) * kBW + 16 * q + rl];
       acc[q] = lq_mfma_i8(bop, xop, acc[q]);
     }
+  };
+  if constexpr (NSLAB > 0) {
+#pragma unroll
+    for (int s = 0; s < NSLAB; ++s) {
+      if (s & 1) {
+        if (s + 1 < NSLAB) load_slab(64 * (s + 1), xrA, brA);
+        asm volatile("" ::: "memory");  // the requests stay ahead of the LDS traffic below
+        slab(s, xrB, brB, [] {});
+      } else {
+        if (s + 1 < NSLAB) load_slab(64 * (s + 1), xrB, brB);
+        asm volatile("" ::: "memory");
+        slab(s, xrA, brA, [] {});
+      }
+    }
+  } else {
+    for (int s = 0; s < nslab; ++s)
+      slab(s, xrA, brA, [&] { if (s + 1 < nslab) load_slab(64 * (s + 1), xrA, brA); });
   }
 
   // ---- epilogue: lane holds N = n0 + 16q + 4kg + {0..3} of P row p0 + 16*wave + rl
-  const int pr = p0 + 16 * wave + rl;
-  const float xs = p.xs[(int64_t)h * p.sxs_h + (int64_t)pr * p.sxs_p];
-  const float so = p.oqs[(int64_t)h * p.soq_h + (int64_t)pr * p.soq_p];
-  const float ratio = xs / so;
-  const float req = KEYSIDE ? 0.0f : ratio * p.bscale_g[(int64_t)g * p.sbs_g];
+  const float ratio = xs_ep / so_ep;
+  const float req = KEYSIDE ? 0.0f : ratio * bs_ep;
   int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + pr) * p.N + n0;
   uint32_t dq[NT / 16];  // dword q of this lane: codes of N = n0 + 16 q + 4 kg + {0..3}
 #pragma unroll
@@ -298,12 +335,22 @@ int launch(const Params& p, hipStream_t stream) {
     q.n_ntiles = p.N / 128;
     const size_t lds = (size_t)p.Q * 4 + 128 * 4 + (2 * 16 * kXW + 2 * 16 * (128 + kPad)) * 4;
     dim3 grid((p.P / 64) * q.n_ntiles * p.nheads, (unsigned)by, 1);
-    hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128>), grid, dim3(256), lds, stream, q);
+    if (!KEYSIDE && p.Q == 256)
+      hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128, 4>), grid, dim3(256), lds, stream, q);
+    else if (!KEYSIDE && p.Q == 128)
+      hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128, 2>), grid, dim3(256), lds, stream, q);
+    else
+      hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128, 0>), grid, dim3(256), lds, stream, q);
   } else {
     q.n_ntiles = p.N / 64;
     const size_t lds = (size_t)p.Q * 4 + 64 * 4 + (2 * 16 * kXW + 2 * 16 * (64 + kPad)) * 4;
     dim3 grid((p.P / 64) * q.n_ntiles * p.nheads, (unsigned)by, 1);
-    hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64>), grid, dim3(256), lds, stream, q);
+    if (!KEYSIDE && p.Q == 256)
+      hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64, 4>), grid, dim3(256), lds, stream, q);
+    else if (!KEYSIDE && p.Q == 128)
+      hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64, 2>), grid, dim3(256), lds, stream, q);
+    else
+      hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64, 0>), grid, dim3(256), lds, stream, q);
   }
   return lq_check_launch();
 }
