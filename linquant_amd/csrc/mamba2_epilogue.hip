@@ -151,27 +151,30 @@ __global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel
       }
       __syncthreads();
     }
+    // Weights without a branch on their dtype (a load inside a branch is waited for inside it: one memory round trip per
+    // piece): two 16-byte requests per piece, the whole fp16 piece twice or the two halves of the fp32 piece, and a
+    // select per element.  (float)h * f rounds once either way, so both dtypes share y = (a * rstd) * w.
+    const bool wf32 = p.weight_f32;
+    const char* wbase = (const char*)p.weight;
 #pragma unroll
     for (int it = 0; it < kIt; ++it) {
-      if (p.weight_f32) {
-        const lq_v4f w0 = *(const lq_v4f*)((const float*)p.weight + pcc[it] * 8);
-        const lq_v4f w1 = *(const lq_v4f*)((const float*)p.weight + pcc[it] * 8 + 4);
+      const char* wp = wbase + (int64_t)pcc[it] * (wf32 ? 32 : 16);
+      const lq_v4i wa = *(const lq_v4i*)wp;
+      const lq_v4i wb = *(const lq_v4i*)(wp + (wf32 ? 16 : 0));
+      const lq_v8h wh = __builtin_bit_cast(lq_v8h, wa);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float y = (v[it][e] * rstd[it]) * (e < 4 ? w0[e & 3] : w1[e & 3]);
-          asm volatile("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
-          xv[it][e] = (_Float16)y;
-        }
-      } else {
-        const lq_v8h wh = *(const lq_v8h*)((const _Float16*)p.weight + pcc[it] * 8);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float y = mul_half(wh[e], v[it][e] * rstd[it]);
-          asm volatile("" : "+v"(y));  // as above
-          xv[it][e] = (_Float16)y;
-        }
+      for (int e = 0; e < 8; ++e) {
+        const float w32 = __int_as_float(e < 4 ? wa[e & 3] : wb[e & 3]);
+        const float w = wf32 ? w32 : (float)wh[e];
+        float y = (v[it][e] * rstd[it]) * w;
+        asm("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
+        xv[it][e] = (_Float16)y;
       }
-      if (p.norm_out && live && valid[it]) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + (it * 64 + lane) * 8) = xv[it];
+    }
+    if (p.norm_out && live) {
+#pragma unroll
+      for (int it = 0; it < kIt; ++it)
+        if (valid[it]) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + (it * 64 + lane) * 8) = xv[it];
     }
   } else if constexpr (!EXACT) {
 #pragma unroll
@@ -213,9 +216,9 @@ __global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel
           lq_v4i hb;
 #pragma unroll
           for (int hw = 0; hw < 2; ++hw) {
-            uint32_t wd = 0;
             const bool ok = cp < g && c0 + 4 * hw < g;
-            if (ok) wd = *(const uint32_t*)(p.had + cp * g + c0 + 4 * hw);
+            // requested without a branch (entries outside the matrix read a clamped address and are zeroed below)
+            const uint32_t wd = *(const uint32_t*)(p.had + min(cp, g - 1) * g + min(c0 + 4 * hw, g - 4));
             const uint32_t lo = 0x3C003C00u | ((wd & 0x80u) << 8) | ((wd & 0x8000u) << 16);
             const uint32_t hi = 0x3C003C00u | ((wd & 0x800000u) >> 8) | (wd & 0x80000000u);
             hb[2 * hw] = ok ? (int)lo : 0;
