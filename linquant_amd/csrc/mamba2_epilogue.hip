@@ -58,11 +58,19 @@ LQ_DEV float wave_sum(float v) {
   return v;
 }
 
+// A 16-byte global load issued as an instruction (the compiler neither moves nor repeats it), and the wait that makes
+// its result usable: every value requested this way passes through arrived() before its first use.
+LQ_DEV void request16(lq_v4i& dst, const void* ptr) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+}
+LQ_DEV void arrived(lq_v4i& v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v)::"memory"); }
+
 // IT = 16-byte pieces per lane (g <= 4 IT); NT = 16-column tiles of had, KS = 32-chunk contraction steps that follow
 // NORM: gate + RMSNorm in front; QHAD: Hadamard + INT8 behind (false: the kernel ends after storing the normalized row)
 // GATE: z is given; EXACT: g = 4 IT, every lane owns IT whole pieces and no access needs a guard
 template <int IT, bool NORM, bool QHAD, bool GATE, bool EXACT>
-__global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel(EpiParams p) {
+__global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(IT <= 10 ? 3 : 2, IT <= 10 ? 3 : 2))) void epilogue_kernel(
+    EpiParams p) {
   constexpr int kIt = IT, NT = (IT + 3) / 4, KS = (IT + 7) / 8;
   extern __shared__ __align__(16) unsigned char smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -85,36 +93,59 @@ __global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel
     valid[it] = EXACT || pc < pieces;
     pcc[it] = EXACT ? pc : min(pc, pieces - 1);
   }
+  // The row's requests are written as instructions: as plain loads the compiler sinks them next to their uses (or drops
+  // and repeats them) to save registers, and the row then arrives two pieces at a time, one memory round trip after the
+  // other.  All of them are issued back to back and waited for once; no other vector memory operation is outstanding at
+  // this point, and the compiler's own wait counts are unaffected by operations older than the ones it tracks.
   lq_v8h xv[kIt];
+  lq_v8h zv[(NORM && GATE) ? kIt : 1];
   {
+    lq_v4i xraw[kIt], zraw[(NORM && GATE) ? kIt : 1];
     const _Float16* xr = p.x + (int64_t)row * p.x_stride;
 #pragma unroll
-    for (int it = 0; it < kIt; ++it) xv[it] = *(const lq_v8h*)(xr + pcc[it] * 8);
+    for (int it = 0; it < kIt; ++it) request16(xraw[it], xr + pcc[it] * 8);
+    if constexpr (NORM && GATE) {
+      const _Float16* zr = p.z + (int64_t)row * p.z_stride;
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) request16(zraw[it], zr + pcc[it] * 8);
+    }
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) arrived(xraw[it]);
+    if constexpr (NORM && GATE) {
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) arrived(zraw[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < kIt; ++it) xv[it] = __builtin_bit_cast(lq_v8h, xraw[it]);
+    if constexpr (NORM && GATE) {
+#pragma unroll
+      for (int it = 0; it < kIt; ++it) zv[it] = __builtin_bit_cast(lq_v8h, zraw[it]);
+    }
   }
 
   if constexpr (NORM) {
-    lq_v8h zv[GATE ? kIt : 1];
-    if constexpr (GATE) {
-      const _Float16* zr = p.z + (int64_t)row * p.z_stride;
-#pragma unroll
-      for (int it = 0; it < kIt; ++it) zv[it] = *(const lq_v8h*)(zr + pcc[it] * 8);
-    }
-    float v[kIt][8];
+    // The gated value is evaluated twice, for the sum of squares and again for the normalized output, instead of being
+    // kept: an fp32 copy of the row (8 IT registers) next to the packed x and z made the scheduler sink the row's
+    // requests next to their uses, and the row then arrived two pieces at a time, one memory round trip after the other.
+    // Without the copy all 2 IT requests are in flight together; the second evaluation costs 2 IT quarter-rate
+    // instructions per lane and returns the same bits.
+    auto gated = [&](int it, int e) -> float {
+      float a;
+      if constexpr (GATE) {
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(mul_half(zv[it][e], -1.44269504088896340736f)));
+        a = mul_half(xv[it][e], mul_half(zv[it][e], sg));
+      } else {
+        a = (float)xv[it][e];
+      }
+      return valid[it] ? a : 0.0f;
+    };
     float part[kIt];
 #pragma unroll
     for (int it = 0; it < kIt; ++it) {
       float s = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        float a;
-        if constexpr (GATE) {
-          const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(mul_half(zv[it][e], -1.44269504088896340736f)));
-          a = mul_half(xv[it][e], mul_half(zv[it][e], sg));
-        } else {
-          a = (float)xv[it][e];
-        }
-        if (!valid[it]) a = 0.0f;
-        v[it][e] = a;
+        const float a = gated(it, e);
         s = __builtin_fmaf(a, a, s);
       }
       part[it] = s;
@@ -166,7 +197,7 @@ __global__ __launch_bounds__(64 * kWaves, IT <= 10 ? 3 : 2) void epilogue_kernel
       for (int e = 0; e < 8; ++e) {
         const float w32 = __int_as_float(e < 4 ? wa[e & 3] : wb[e & 3]);
         const float w = wf32 ? w32 : (float)wh[e];
-        float y = (v[it][e] * rstd[it]) * w;
+        float y = (gated(it, e) * rstd[it]) * w;
         asm("" : "+v"(y));  // keeps the fp32 rounding of the product: no multiply fused into the fp16 conversion
         xv[it][e] = (_Float16)y;
       }
