@@ -49,17 +49,32 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
   extern __shared__ int gate_lds[];
   const int b = blockIdx.z, h = blockIdx.y;
   const float fs = (float)(1 << shift);
-  for (int c = threadIdx.x; c < nchunks; c += blockDim.x) {
-    const float g = lq_expf(dA[(int64_t)b * sd_b + (int64_t)h * sd_h + (int64_t)c * sd_c]) * fs;
-    gate_lds[c] = lq_q_rha(g, 127);
-  }
-  __syncthreads();
-  const int64_t d0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
-  if (d0 >= dim) return;
+  // (a surplus lane keeps working on a clamped, in-range slice and stores nothing: no early exit before the barrier, and
+  // the first states are requested before the gates are computed, so the two round trips overlap)
+  const int64_t d_raw = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  const bool live = d_raw < dim;
+  const int64_t d0 = live ? d_raw : 0;
   const int8_t* sp = states + (int64_t)b * ss_b + (int64_t)h * ss_h + d0;
   int8_t* op = out + (int64_t)b * so_b + (int64_t)h * so_h + d0;
   int8_t* fp = fin ? fin + (int64_t)b * sf_b + (int64_t)h * sf_h + d0 : nullptr;
   const int half = (1 << shift) >> 1;
+  const bool even = nchunks % DEPTH == 0;  // uniform: the branch-free loop below needs whole groups of DEPTH chunks
+
+  // the gate's request goes first: memory operations retire in issue order, so waiting for it then does not wait for the
+  // states requested behind it
+  const int cg = min((int)threadIdx.x, nchunks - 1);
+  const float dA0 = dA[(int64_t)b * sd_b + (int64_t)h * sd_h + (int64_t)cg * sd_c];
+  V buf[DEPTH];
+#pragma unroll
+  for (int j = 0; j < DEPTH; ++j) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)min(j, nchunks - 1) * ss_c));
+
+  gate_lds[cg] = lq_q_rha(lq_expf(dA0) * fs, 127);  // surplus threads rewrite the last gate with the same value
+  for (int c = threadIdx.x + blockDim.x; c < nchunks; c += blockDim.x) {
+    const float g = lq_expf(dA[(int64_t)b * sd_b + (int64_t)h * sd_h + (int64_t)c * sd_c]) * fs;
+    gate_lds[c] = lq_q_rha(g, 127);
+  }
+  __syncthreads();
+  if (!live) return;
 
   int s[VEC];
 #pragma unroll
@@ -67,10 +82,40 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
   V zero = {};
   __builtin_nontemporal_store(zero, (V*)op);
 
-  V buf[DEPTH];
+  auto step = [&](const V& cur, int c) {
+    const int gq = gate_lds[c];
+    V res;
+    const uint32_t* cw = (const uint32_t*)&cur;
+    uint32_t* rw = (uint32_t*)&res;
 #pragma unroll
-  for (int j = 0; j < DEPTH; ++j)
-    if (j < nchunks) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)j * ss_c));
+    for (int w = 0; w < W; ++w) rw[w] = step_word(cw[w], s + 4 * w, gq, shift, half);
+    return res;
+  };
+
+  if (even) {
+    // whole groups: every request and every store of the steady state is unconditional, which keeps the compiler's
+    // count of outstanding operations exact (with guards around them it drained the whole ring once per group)
+    for (int c0 = 0; c0 + DEPTH < nchunks; c0 += DEPTH) {
+#pragma unroll
+      for (int j = 0; j < DEPTH; ++j) {
+        const int c = c0 + j;
+        const V cur = buf[j];
+        buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)(c + DEPTH) * ss_c));
+        __builtin_nontemporal_store(step(cur, c), (V*)(op + (int64_t)(c + 1) * so_c));
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) {  // last group: nothing left to request
+      const int c = nchunks - DEPTH + j;
+      const V res = step(buf[j], c);
+      if (j < DEPTH - 1) {
+        __builtin_nontemporal_store(res, (V*)(op + (int64_t)(c + 1) * so_c));
+      } else if (fp) {
+        __builtin_nontemporal_store(res, (V*)fp);
+      }
+    }
+    return;
+  }
 
   for (int c0 = 0; c0 < nchunks; c0 += DEPTH) {
 #pragma unroll
@@ -79,12 +124,7 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
       if (c < nchunks) {
         V cur = buf[j];
         if (c + DEPTH < nchunks) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)(c + DEPTH) * ss_c));
-        const int gq = gate_lds[c];
-        V res;
-        uint32_t* cw = (uint32_t*)&cur;
-        uint32_t* rw = (uint32_t*)&res;
-#pragma unroll
-        for (int w = 0; w < W; ++w) rw[w] = step_word(cw[w], s + 4 * w, gq, shift, half);
+        const V res = step(cur, c);
         if (c < nchunks - 1) {
           __builtin_nontemporal_store(res, (V*)(op + (int64_t)(c + 1) * so_c));
         } else if (fp) {
