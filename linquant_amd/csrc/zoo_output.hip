@@ -59,51 +59,80 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   const int qmax = p.qmax;
   constexpr bool bf = BF;
 
+  // ---- every global request of the workgroup is issued here, before the first use and outside any branch, oldest first
+  // in the order of use.  (Issued where they were used they formed a chain of about nine exposed round trips: one per
+  // iteration of the code loop, one for v, one per contraction step of the state read, one per scale vector.)
+  constexpr int NQ = K / 32;  // 16-byte pieces of q (and of k) per thread: 64 tokens x K / 8 pieces over 256 threads
+  lq_v4i qraw[GLA ? 1 : NQ], kraw[GLA ? 1 : NQ];
+  if constexpr (!GLA) {
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      const int it = tid + 256 * i;
+      const int t = it / (K / 8), c8 = it % (K / 8);
+      const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
+      qraw[i] = *(const lq_v4i*)(p.q + off);
+      kraw[i] = *(const lq_v4i*)(p.k + off);
+    }
+  }
+  const int tp = tid >> 3, c8v = tid & 7;  // value tile: 32 token pairs x 8 groups of 8 channels
+  const int64_t voff = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8v;
+  const lq_v4i va_raw = *(const lq_v4i*)(p.v + voff), vb_raw = *(const lq_v4i*)(p.v + voff + (int64_t)H * V);
+  const lq_v4f sv0 = *(const lq_v4f*)(p.svl + h * V + v0 + 8 * c8v), sv1 = *(const lq_v4f*)(p.svl + h * V + v0 + 8 * c8v + 4);
+  const float g_raw = (USE_G && !GLA) ? p.g[(t0 + (tid & 63)) * H + h] : 0.0f;
+  const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
+  lq_v4i hop[K / 64][4];
+  lq_v4i qgop[GLA ? K / 64 : 1];
+#pragma unroll
+  for (int ks = 0; ks < K / 64; ++ks) {
+    if constexpr (GLA) qgop[ks] = *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) hop[ks][jj] = *(const lq_v4i*)(hp + (4 * rl + jj) * K + 64 * ks + 16 * kg);
+  }
+  const lq_v4f ss4 = *(const lq_v4f*)(p.ss + h * V + v0 + 4 * rl);
+  const lq_v4f svl4 = *(const lq_v4f*)(p.svl + h * V + v0 + 4 * rl);
+
   // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
-  if (!GLA)
-  for (int it = tid; it < 64 * (K / 8); it += 256) {
-    const int t = it / (K / 8), c8 = it % (K / 8);
-    const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
-    float qv[8];
-    zoo_ld8(p.q + off, bf, qv);
-    int cq[8];
+  if constexpr (!GLA) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) cq[e] = zoo_q8(qv[e] * p.scale, inv_sq, qmax);
-    lq_v2i o;
-    o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
-    o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
-    *(lq_v2i*)(qc + t * QS + 8 * c8) = o;
-    {
-      float kv[8];
-      zoo_ld8(p.k + off, bf, kv);
-      int ck[8];
+    for (int i = 0; i < NQ; ++i) {
+      const int it = tid + 256 * i;
+      const int t = it / (K / 8), c8 = it % (K / 8);
+      lq_v2i oq, ok;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) ck[e] = zoo_q8(kv[e], inv_sk, qmax);
-      o[0] = (int)zoo_pack_codes(ck[0], ck[1], ck[2], ck[3]);
-      o[1] = (int)zoo_pack_codes(ck[4], ck[5], ck[6], ck[7]);
-      *(lq_v2i*)(kc + t * QS + 8 * c8) = o;
+      for (int hf = 0; hf < 2; ++hf) {
+        int cq[4], ck[4];
+#pragma unroll
+        for (int d = 0; d < 2; ++d) {
+          float q0, q1, k0, k1;
+          zoo_dec2((uint32_t)qraw[i][2 * hf + d], bf, q0, q1);
+          zoo_dec2((uint32_t)kraw[i][2 * hf + d], bf, k0, k1);
+          cq[2 * d] = zoo_q8(q0 * p.scale, inv_sq, qmax), cq[2 * d + 1] = zoo_q8(q1 * p.scale, inv_sq, qmax);
+          ck[2 * d] = zoo_q8(k0, inv_sk, qmax), ck[2 * d + 1] = zoo_q8(k1, inv_sk, qmax);
+        }
+        oq[hf] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
+        ok[hf] = (int)zoo_pack_codes(ck[0], ck[1], ck[2], ck[3]);
+      }
+      *(lq_v2i*)(qc + t * QS + 8 * c8) = oq;
+      *(lq_v2i*)(kc + t * QS + 8 * c8) = ok;
     }
   }
   {
-    const int tp = tid >> 3, c8 = tid & 7;  // 32 token pairs x 8 groups of 8 channels
-    const int64_t off = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8;
-    float va[8];
-    zoo_ld8(p.v + off, bf, va);
-    float vb[8];
-    zoo_ld8(p.v + off + (int64_t)H * V, bf, vb);
     lq_v4i o0, o1;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float inv = 1.0f / p.svl[h * V + v0 + 8 * c8 + e];
-      const float ca = (float)zoo_q8(va[e], inv, qmax);
-      const float cb = (float)zoo_q8(vb[e], inv, qmax);
-      const int w = (int)zoo_pack_h2(ca, cb);
-      if (e < 4) o0[e] = w; else o1[e - 4] = w;
+    for (int d = 0; d < 4; ++d) {
+      float a0, a1, b0, b1;
+      zoo_dec2((uint32_t)va_raw[d], bf, a0, a1);
+      zoo_dec2((uint32_t)vb_raw[d], bf, b0, b1);
+      const float s0 = d < 2 ? sv0[2 * d] : sv1[2 * d - 4], s1 = d < 2 ? sv0[2 * d + 1] : sv1[2 * d - 3];
+      const float i0 = 1.0f / s0, i1 = 1.0f / s1;
+      const int w0 = (int)zoo_pack_h2((float)zoo_q8(a0, i0, qmax), (float)zoo_q8(b0, i0, qmax));
+      const int w1 = (int)zoo_pack_h2((float)zoo_q8(a1, i1, qmax), (float)zoo_q8(b1, i1, qmax));
+      if (d < 2) o0[2 * d] = w0, o0[2 * d + 1] = w1; else o1[2 * d - 4] = w0, o1[2 * d - 3] = w1;
     }
-    *(lq_v4i*)(vP + tp * kVW + 8 * c8) = o0;
-    *(lq_v4i*)(vP + tp * kVW + 8 * c8 + 4) = o1;
+    *(lq_v4i*)(vP + tp * kVW + 8 * c8v) = o0;
+    *(lq_v4i*)(vP + tp * kVW + 8 * c8v + 4) = o1;
   }
-  if (USE_G && !GLA && tid < 64) g_s[tid] = p.g[(t0 + tid) * H + h];
+  if (USE_G && !GLA) g_s[tid & 63] = g_raw;  // four threads per token write the same value
   __syncthreads();
 
   // ---- phase 2: INT8 contractions of this wave's 16 rows
@@ -113,16 +142,15 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   lq_v4i a32[4];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
-  const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
-    const lq_v4i qop = GLA ? *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg)
-                           : *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+    lq_v4i qop;
+    if constexpr (GLA)
+      qop = qgop[ks];
+    else
+      qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const lq_v4i hop = *(const lq_v4i*)(hp + (4 * rl + jj) * K + 64 * ks + 16 * kg);
-      o32[jj] = lq_mfma_i8(qop, hop, o32[jj]);
-    }
+    for (int jj = 0; jj < 4; ++jj) o32[jj] = lq_mfma_i8(qop, hop[ks][jj], o32[jj]);
     if (!GLA) {
 #pragma unroll
       for (int jt = 0; jt < 4; ++jt) {
@@ -136,9 +164,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   // ---- phase 3: dequantize; A -> fp16 in operand layout
   float of[4][4];  // [jj][r]: rows 16w + 4kg + r, channels v0 + 4rl + jj
   {
-    float ssv[4];
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) ssv[jj] = p.ss[h * V + v0 + 4 * rl + jj];
+    const lq_v4f ssv = ss4;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + 4 * kg + r]) : 1.0f;
@@ -192,9 +218,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) loc[jj] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[jj]), loc[jj]);
   }
-  float svl[4];
-#pragma unroll
-  for (int jj = 0; jj < 4; ++jj) svl[jj] = p.svl[h * V + v0 + 4 * rl + jj];
+  const lq_v4f svl = svl4;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + 4 * rl;
@@ -244,7 +268,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
-  if ((a->q && !zoo_al(a->q, 16)) || (a->qg && !zoo_al(a->qg, 16)) || (a->A && !zoo_al(a->A, 16)) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16))
+  if ((a->q && !zoo_al(a->q, 16)) || (a->qg && !zoo_al(a->qg, 16)) || (a->A && !zoo_al(a->A, 16)) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16) || !zoo_al(a->ss, 16) || !zoo_al(a->svl, 16))
     return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535 || a->seqlen / 64 > 65535) return LQ_ERR_SHAPE;
   OutParams p = {};
