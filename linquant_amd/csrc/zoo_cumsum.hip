@@ -40,7 +40,12 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
   const int64_t tstride = (int64_t)H * K;
   float v[16];
 #pragma unroll
-  for (int t = 0; t < 16; ++t) v[t] = t < SEG ? g[base + t * tstride] : 0.0f;
+  for (int t = 0; t < 16; ++t) {
+    // requested without a branch (a load under `t < SEG` is waited for inside its branch: sixteen round trips in a row);
+    // tokens past the segment re-read its last one and count as zero
+    const float x = g[base + min(t, SEG - 1) * tstride];
+    v[t] = t < SEG ? x : 0.0f;
+  }
   double run = 0.0, pre[16];
 #pragma unroll
   for (int t = 0; t < 16; ++t) {
