@@ -82,45 +82,66 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
 #pragma unroll
     for (int e = 0; e < CK; ++e) inv_skw[e] = 1.0f / p.skw[h * K + CK * cg + e];
     const float inv_sw = p.w ? 1.0f / p.sw[h] : 0.0f;
+    // every request of the thread's four tokens is issued before the first is used (with the loads inside the token
+    // loop, next to a run-time `if (p.w)`, each token cost its own memory round trips)
+    typedef int raw_t __attribute__((ext_vector_type(CK / 2)));  // CK half-precision values
+    typedef float gf_t __attribute__((ext_vector_type(4)));
+    raw_t kraw[4], wraw[4];
+    gf_t graw[4][CK / 4], glast[CK / 4];
+    int64_t offs[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      offs[t] = ((t0 + 4 * tq + t) * H + h) * K + CK * cg;
+      kraw[t] = *(const raw_t*)(p.key + offs[t]);
+      if (DECAY == LQ_DECAY_DIAGONAL) {
+#pragma unroll
+        for (int d = 0; d < CK / 4; ++d) graw[t][d] = *(const gf_t*)(p.g + offs[t] + 4 * d);
+      }
+    }
+    if (DECAY == LQ_DECAY_DIAGONAL) {
+#pragma unroll
+      for (int d = 0; d < CK / 4; ++d) glast[d] = *(const gf_t*)(p.g + ((t0 + 63) * H + h) * K + CK * cg + 4 * d);
+    }
+    if (p.w) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) wraw[t] = *(const raw_t*)(p.w + offs[t]);
+    }
     uint32_t kcode[CK][4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int tl = 4 * tq + t;
-      const int64_t off = ((t0 + tl) * H + h) * K + CK * cg;
       float kv[CK];
-      if constexpr (CK == 8)
-        zoo_ld8(p.key + off, bf, kv);
-      else
-        zoo_ld4(p.key + off, bf, kv);
+#pragma unroll
+      for (int d = 0; d < CK / 2; ++d) zoo_dec2((uint32_t)kraw[t][d], bf, kv[2 * d], kv[2 * d + 1]);
       if (DECAY == LQ_DECAY_SCALAR) {
         const float f = ek_s[tl];
 #pragma unroll
         for (int e = 0; e < CK; ++e) kv[e] = kv[e] * f;
       } else if (DECAY == LQ_DECAY_DIAGONAL) {
-        const float* gr = p.g + off;
-        const float* gl = p.g + ((t0 + 63) * H + h) * K + CK * cg;
         const float el = ek_s[tl];
 #pragma unroll
-        for (int e = 0; e < CK; ++e) kv[e] = kv[e] * zoo_exp(gl[e] - gr[e] - el);
+        for (int e = 0; e < CK; ++e) kv[e] = kv[e] * zoo_exp(glast[e >> 2][e & 3] - graw[t][e >> 2][e & 3] - el);
       }
 #pragma unroll
       for (int e = 0; e < CK; ++e) kcode[e][t] = (uint32_t)zoo_q8(kv[e], inv_skw[e], qmax);
-      if (p.w) {
-        int wc[CK];
-        float wv[CK];
-        if constexpr (CK == 8) {
-          zoo_ld8(p.w + off, bf, wv);
+    }
+    if (p.w) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) wc[e] = zoo_q8(wv[e], inv_sw, qmax);
+      for (int t = 0; t < 4; ++t) {
+        int wc[CK];
+#pragma unroll
+        for (int d = 0; d < CK / 2; ++d) {
+          float w0, w1;
+          zoo_dec2((uint32_t)wraw[t][d], bf, w0, w1);
+          wc[2 * d] = zoo_q8(w0, inv_sw, qmax), wc[2 * d + 1] = zoo_q8(w1, inv_sw, qmax);
+        }
+        if constexpr (CK == 8) {
           lq_v2i o;
           o[0] = (int)zoo_pack_codes(wc[0], wc[1], wc[2], wc[3]);
           o[1] = (int)zoo_pack_codes(wc[4], wc[5], wc[6], wc[7]);
-          *(lq_v2i*)(p.wq + off) = o;
+          *(lq_v2i*)(p.wq + offs[t]) = o;
         } else {
-          zoo_ld4(p.w + off, bf, wv);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) wc[e] = zoo_q8(wv[e], inv_sw, qmax);
-          *(uint32_t*)(p.wq + off) = zoo_pack_codes(wc[0], wc[1], wc[2], wc[3]);
+          *(uint32_t*)(p.wq + offs[t]) = zoo_pack_codes(wc[0], wc[1], wc[2], wc[3]);
         }
       }
     }
