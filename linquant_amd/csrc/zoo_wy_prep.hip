@@ -424,34 +424,56 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
     }
   };
 
-  // ---- Hw is written straight out; X = beta^sigma k exp(g) is staged 64 columns at a time (over the dead Gram tile)
+  // ---- W and U passes, 64 columns at a time through the X tiles.  The global operands of a pass are requested while the
+  // products of the pass before it run (requested at their point of use, each pass exposed a memory round trip between
+  // two barriers).
+  lq_v4i kraw[2], vraw[2];
+  lq_v4f graw[2][2];
+  float btr[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) btr[u] = p.beta[(tok0 + u) * H + h];
+  auto request_k = [&](int kc) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int64_t off = ((tok0 + u) * H + h) * K + kc + 8 * c8;
+      kraw[u] = *(const lq_v4i*)(p.k + off);
+      if (DECAY == LQ_DECAY_DIAGONAL) graw[u][0] = *(const lq_v4f*)(p.g + off), graw[u][1] = *(const lq_v4f*)(p.g + off + 4);
+    }
+  };
+  auto request_v = [&](int vc) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) vraw[u] = *(const lq_v4i*)(p.v + ((tok0 + u) * H + h) * V + vc + 8 * c8);
+  };
+  // (per-channel decay: its kernel sits at the register limit of four waves per SIMD, and holding a pass of k and g
+  // across the products spilled: 272 -> 316 us; it requests at the point of use)
+  constexpr bool kAhead = DECAY != LQ_DECAY_DIAGONAL;
+  if (kAhead) request_k(0);
+
+  // Hw is written straight out; X = beta^sigma k exp(g) is staged (over the dead Gram tile)
+#pragma unroll
   for (int kc = 0; kc < K; kc += 64) {
     if (kc > 0) __syncthreads();
+    if (!kAhead) request_k(kc);
     {
       float xr[2][8];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int64_t off = ((tok0 + u) * H + h) * K + kc + 8 * c8;
-        float kv[8];
-        zoo_ld8(p.k + off, bf, kv);
-        const float bt = p.beta[(tok0 + u) * H + h];
-        const float bw = powb(bt, (1.0f - sigma) * tau);
+        const float bw = powb(btr[u], (1.0f - sigma) * tau);
         float bl = bs_s[2 * rp + u];
         if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(gs_s[2 * rp + u]);
-        float ge[8];
-        if (DECAY == LQ_DECAY_DIAGONAL) {
-          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) ge[e] = zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-        }
         float hw[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float kf = kv[e];
-          float x = bl * kf;
-          if (DECAY == LQ_DECAY_DIAGONAL) x = x * ge[e];
-          xr[u][e] = x;
-          hw[e] = bw * kf;
+        for (int d = 0; d < 4; ++d) {
+          float k0, k1;
+          zoo_dec2((uint32_t)kraw[u][d], bf, k0, k1);
+          float x0 = bl * k0, x1 = bl * k1;
+          if (DECAY == LQ_DECAY_DIAGONAL) {
+            x0 = x0 * zoo_exp(graw[u][d >> 1][(2 * d) & 3]);
+            x1 = x1 * zoo_exp(graw[u][d >> 1][(2 * d + 1) & 3]);
+          }
+          xr[u][2 * d] = x0, xr[u][2 * d + 1] = x1;
+          hw[2 * d] = bw * k0, hw[2 * d + 1] = bw * k1;
         }
         lq_v4i o;
 #pragma unroll
@@ -461,6 +483,11 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
       stage(xr[0], xr[1]);
     }
     __syncthreads();
+    if (kc + 64 < K) {
+      if (kAhead) request_k(kc + 64);
+    } else if (kAhead) {
+      request_v(0);
+    }
     // W = T . X for these 64 columns
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
@@ -474,22 +501,26 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
     }
   }
 
-  // ---- U = T . (beta^sigma v), 64 value columns per pass through the X buffer
+  // ---- U = T . (beta^sigma v)
   for (int vc = 0; vc < V; vc += 64) {
     __syncthreads();
+    if (!kAhead) request_v(vc);
     {
       float xr[2][8];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        float vv[8];
-        zoo_ld8(p.v + ((tok0 + u) * H + h) * V + vc + 8 * c8, bf, vv);
         const float bsr = bs_s[2 * rp + u];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) xr[u][e] = bsr * vv[e];
+        for (int d = 0; d < 4; ++d) {
+          float v0, v1;
+          zoo_dec2((uint32_t)vraw[u][d], bf, v0, v1);
+          xr[u][2 * d] = bsr * v0, xr[u][2 * d + 1] = bsr * v1;
+        }
       }
       stage(xr[0], xr[1]);
     }
     __syncthreads();
+    if (kAhead) request_v(min(vc + 64, V - 64));  // unconditional: the last pass requests its own columns once more
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       const int u = nt < 2 ? 0 : 1;
