@@ -66,23 +66,18 @@ __global__ __launch_bounds__(256) void causal_conv1d_kernel(const _Float16* __re
   const int t0 = tb * kTL;
   if (t0 >= L) return;
   const int c = cg * 8;
-  float w[W][8], bv[8];
+  // Every request of the thread is issued before the first use and outside any branch: the taps of its 8 channels are
+  // 8 W contiguous halves (W 16-byte pieces; element-wise loads, a branch on `bias` and one on `t >= 0` per halo row
+  // made a chain of about eight memory round trips in front of the x rows), the bias piece comes from a valid dummy
+  // address when there is none, halo rows before the sequence start re-read row 0 and are zeroed in registers.
+  lq_v8h wraw[W];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    bv[e] = bias ? (float)bias[c + e] : 0.0f;
-#pragma unroll
-    for (int j = 0; j < W; ++j) w[j][e] = (float)weight[(int64_t)(c + e) * W + j];
-  }
+  for (int j = 0; j < W; ++j) wraw[j] = *(const lq_v8h*)(weight + (int64_t)c * W + 8 * j);
+  const lq_v8h braw = *(const lq_v8h*)(bias ? bias + c : weight + (int64_t)c * W);
   const _Float16* xp = x + (int64_t)b * sx_b + c;
-  float win[W][8];  // sliding window: win[j] = x[t - (W-1) + j]
+  lq_v8h halo[W - 1];
 #pragma unroll
-  for (int j = 0; j < W - 1; ++j) {
-    const int t = t0 - (W - 1) + j;
-    lq_v8h v = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (t >= 0) v = *(const lq_v8h*)(xp + (int64_t)t * sx_l);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) win[j + 1][e] = (float)v[e];
-  }
+  for (int j = 0; j < W - 1; ++j) halo[j] = *(const lq_v8h*)(xp + (int64_t)max(t0 - (W - 1) + j, 0) * sx_l);
   _Float16* op = out + ((int64_t)b * L) * D + c;
   // all rows of the block are requested before the first one is used (the clamped row index keeps a ragged last block
   // inside the sequence; its surplus rows are computed and not stored)
@@ -91,6 +86,20 @@ __global__ __launch_bounds__(256) void causal_conv1d_kernel(const _Float16* __re
   for (int i = 0; i < kTL; ++i) {
     const int t = t0 + i < L ? t0 + i : L - 1;
     rows[i] = *(const lq_v8h*)(xp + (int64_t)t * sx_l);
+  }
+  float w[W][8], bv[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    bv[e] = bias ? (float)braw[e] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < W; ++j) w[j][e] = (float)wraw[(e * W + j) >> 3][(e * W + j) & 7];  // weight[(c + e) * W + j]
+  }
+  float win[W][8];  // sliding window: win[j] = x[t - (W-1) + j]
+#pragma unroll
+  for (int j = 0; j < W - 1; ++j) {
+    const bool in = t0 - (W - 1) + j >= 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) win[j + 1][e] = in ? (float)halo[j][e] : 0.0f;
   }
 #pragma unroll
   for (int i = 0; i < kTL; ++i) {
@@ -137,6 +146,7 @@ extern "C" int lq_causal_conv1d(const lq_causal_conv1d_args* a, hipStream_t stre
   if (a->batch <= 0 || a->seqlen <= 0 || a->dim <= 0 || a->dim % 8 != 0 || a->batch > 65535) return LQ_ERR_SHAPE;
   if (a->width < 2 || a->width > 4) return LQ_ERR_SHAPE;
   if (a->x_stride_b % 8 != 0 || a->x_stride_l % 8 != 0 || !al(a->x, 16) || !al(a->out, 16)) return LQ_ERR_SHAPE;
+  if (!al(a->weight, 16) || (a->bias && !al(a->bias, 16))) return LQ_ERR_SHAPE;  // taps and bias are read as 16-byte pieces
   const int64_t items = (int64_t)(a->dim / 8) * ((a->seqlen + kTL - 1) / kTL);
   if (items > 0x7fffffff) return LQ_ERR_SHAPE;
   dim3 grid((unsigned)((items + 255) / 256), a->batch);
