@@ -60,7 +60,10 @@ LQ_DEV void fwht_row(float* v, int sub, float hb, float kron) {
   }
 }
 
-template <int N, bool QUANT>
+// VEC: signs and dqk are 16-byte aligned, so a lane's eight entries are fetched as whole pieces, requested together with
+// its row piece before anything is used (element by element, behind a run-time dtype switch, they formed a chain of
+// memory round trips several times longer than the transform itself).
+template <int N, bool QUANT, bool VEC>
 __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict__ src, int64_t s_b, int64_t s_t,
                                                      int64_t s_seg, int nseg_per_side, int64_t side_off,
                                                      void* __restrict__ dst0, void* __restrict__ dst1, _Float16* __restrict__ fp0,
@@ -83,17 +86,47 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
   const _Float16* sp = src + (int64_t)b * s_b + (int64_t)tt * s_t + side * side_off + (int64_t)seg * s_seg + sub * 8;
   const lq_v8h hv = *(const lq_v8h*)sp;
   float v[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = (float)hv[i];
   const float* dqk = side ? dqk1 : dqk0;
-  if (QUANT && dqk) {
+  if constexpr (VEC) {
+    // absent operands are read from a valid dummy address (the start of the row) and ignored
+    const int64_t e0 = (int64_t)seg * N + sub * 8;
+    const float* dq = (QUANT && dqk) ? dqk + e0 : (const float*)(sp - sub * 8);
+    const lq_v4f d0 = *(const lq_v4f*)dq, d1 = *(const lq_v4f*)(dq + 4);
+    const int es = signs_dtype == LQ_DT_F16 ? 2 : (signs_dtype == LQ_DT_F32 ? 4 : 1);
+    const char* sgp = signs ? (const char*)signs + e0 * es : (const char*)(sp - sub * 8);
+    const lq_v4i s0 = *(const lq_v4i*)(es == 1 ? sgp - ((uintptr_t)sgp & 8) : sgp);          // int8: the aligned 16 bytes around the 8
+    const lq_v4i s1 = *(const lq_v4i*)(es == 4 ? sgp + 16 : sgp - ((uintptr_t)sgp & 15));    // fp32: second half
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (float)(_Float16)(v[i] * dqk[seg * N + sub * 8 + i]);
-  }
-  if (signs) {
+    for (int i = 0; i < 8; ++i) v[i] = (float)hv[i];
+    if (QUANT && dqk) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = bf16_round(v[i] * load_sign(signs, (int64_t)seg * N + sub * 8 + i, signs_dtype));
-    fwht_row<LPH>(v, sub, hb, kron);
+      for (int i = 0; i < 8; ++i) v[i] = (float)(_Float16)(v[i] * (i < 4 ? d0[i & 3] : d1[i & 3]));
+    }
+    if (signs) {
+      const lq_v8h sh = __builtin_bit_cast(lq_v8h, s0);
+      const int boff = (int)((uintptr_t)sgp & 8) >> 2;  // int8: dword index of the lane's 8 bytes inside s0
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float f16v = (float)sh[i];
+        const float f32v = __int_as_float(i < 4 ? s0[i & 3] : s1[i & 3]);
+        const float i8v = (float)lq_sbyte((uint32_t)(boff ? s0[2 + (i >> 2)] : s0[i >> 2]), i & 3);
+        const float sg = es == 2 ? f16v : (es == 4 ? f32v : i8v);
+        v[i] = bf16_round(v[i] * sg);
+      }
+      fwht_row<LPH>(v, sub, hb, kron);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)hv[i];
+    if (QUANT && dqk) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = (float)(_Float16)(v[i] * dqk[seg * N + sub * 8 + i]);
+    }
+    if (signs) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = bf16_round(v[i] * load_sign(signs, (int64_t)seg * N + sub * 8 + i, signs_dtype));
+      fwht_row<LPH>(v, sub, hb, kron);
+    }
   }
   if (!live) return;
   if (QUANT) {
@@ -151,14 +184,17 @@ extern "C" int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* a
   const float kron = (float)(1.0 / sqrt(2.0));
   const int rpb = 256 / (N / 8);
   dim3 grid((a->seqlen + rpb - 1) / rpb, a->batch * 2 * G);
-  if (N == 128)
-    hipLaunchKernelGGL((rotate_kernel<128, true>), grid, dim3(256), 0, stream, src, a->xBC_stride_b, a->xBC_stride_t,
-                       (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, (_Float16*)a->b_fp, a->signs, a->signs_dtype, a->B_inv_scale,
-                       a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron);
-  else
-    hipLaunchKernelGGL((rotate_kernel<64, true>), grid, dim3(256), 0, stream, src, a->xBC_stride_b, a->xBC_stride_t,
-                       (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, (_Float16*)a->b_fp, a->signs, a->signs_dtype, a->B_inv_scale,
-                       a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron);
+  const bool vec = (!a->signs || al(a->signs, 16)) && (!a->dqk_b || (al(a->dqk_b, 16) && al(a->dqk_c, 16)));
+#define LQ_ROT_LAUNCH(NN, VV)                                                                                          \
+  hipLaunchKernelGGL((rotate_kernel<NN, true, VV>), grid, dim3(256), 0, stream, src, a->xBC_stride_b, a->xBC_stride_t, \
+                     (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, (_Float16*)a->b_fp, a->signs, a->signs_dtype,         \
+                     a->B_inv_scale, a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron)
+  if (N == 128) {
+    if (vec) LQ_ROT_LAUNCH(128, true); else LQ_ROT_LAUNCH(128, false);
+  } else {
+    if (vec) LQ_ROT_LAUNCH(64, true); else LQ_ROT_LAUNCH(64, false);
+  }
+#undef LQ_ROT_LAUNCH
   return lq_check_launch();
 }
 
@@ -173,13 +209,24 @@ extern "C" int lq_kron_hadamard(const lq_kron_hadamard_args* a, hipStream_t stre
   const float kron = (float)(1.0 / sqrt(2.0));
   const int rpb = 256 / (D / 8);
   dim3 grid((a->seqlen + rpb - 1) / rpb, a->batch * H);
-  if (D == 128)
-    hipLaunchKernelGGL((rotate_kernel<128, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
+  const bool vec = al(a->signs, 16);
+  if (D == 128 && vec)
+    hipLaunchKernelGGL((rotate_kernel<128, false, true>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
+                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       a->seqlen, hb, kron);
+  else if (vec)
+    hipLaunchKernelGGL((rotate_kernel<64, false, true>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
+                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
+                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       a->seqlen, hb, kron);
+  else if (D == 128)
+    hipLaunchKernelGGL((rotate_kernel<128, false, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
                        a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                        a->seqlen, hb, kron);
   else
-    hipLaunchKernelGGL((rotate_kernel<64, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
+    hipLaunchKernelGGL((rotate_kernel<64, false, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
                        a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                        a->seqlen, hb, kron);
