@@ -36,9 +36,10 @@ typedef _Float16 lq_v2h __attribute__((ext_vector_type(2)));
 // x <= -86 returns 0 (keeps every result a normal number), x > 88 returns +inf, NaN propagates.
 LQ_DEV float lq_expf(float x) {
 #pragma clang fp contract(off)
-  if (x != x) return x;
-  if (!(x > -86.0f)) return 0.0f;
-  if (x > 88.0f) return __builtin_inff();
+  // evaluated without a branch on a clamped argument, the special cases selected at the end: as early returns they
+  // became a branch per call, and a load whose value feeds a branch is waited for on the spot
+  const float xin = x;
+  x = fminf(fmaxf(x, -86.0f), 88.0f);  // NaN -> -86, replaced below
   float t = x * 1.44269502162933349609375f;
   float n = __builtin_rintf(t);
   float r = x - n * 0.693145751953125f;
@@ -52,7 +53,10 @@ LQ_DEV float lq_expf(float x) {
   p = p * r + 1.0f;
   p = p * r + 1.0f;
   int e = ((int)n + 127) << 23;
-  return p * __int_as_float(e);
+  float y = p * __int_as_float(e);
+  y = xin > 88.0f ? __builtin_inff() : y;
+  y = !(xin > -86.0f) ? 0.0f : y;
+  return xin != xin ? xin : y;
 }
 
 // log(y) for normal y > 0: y = m * 2^e with m in [sqrt(1/2), sqrt(2)), s = (m-1)/(m+1),
