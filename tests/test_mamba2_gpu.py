@@ -184,7 +184,43 @@ def test_chunk_state_scalar_scales_and_ragged(cuda):
     assert_same_codes(st, rs, "states (scalar scales, ragged)")
 
 
-@pytest.mark.parametrize("dim,shift,nc", [(8192, 7, 32), (4096 + 16, 7, 5), (1000, 7, 9), (999, 5, 3), (64 * 64, 7, 1)])
+@pytest.mark.parametrize("sign_dtype", [torch.float32, torch.float16, torch.int8])
+@pytest.mark.parametrize("offset", [0, 1])
+def test_prologue_sign_dtypes_and_alignment(cuda, sign_dtype, offset):
+    """Signs in each accepted dtype, 16-byte aligned (fetched as whole pieces) and one element off (element-wise path),
+    with and without dqk: same codes as the oracle either way."""
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC, prepare_dqk
+
+    s = Mamba2Shape(batch=1, seqlen=77, nheads=2, headdim=64, dstate=128, ngroups=2, chunk=64)
+    say("prologue sign dtype / alignment", sign_dtype, offset)
+    g = torch.Generator().manual_seed(23)
+    xBC = torch.randn(s.batch, s.seqlen, s.xbc_dim, generator=g).half()
+    signs = (torch.randint(0, 2, (s.ngroups, s.dstate), generator=g) * 2 - 1).float()
+    dq = torch.rand(s.ngroups, s.dstate, generator=g) + 0.5
+    binv, cinv = torch.tensor([20.0, 35.0]), torch.tensor([28.0, 31.0])
+
+    def shifted(t):  # the same values in a buffer whose data pointer is `offset` elements past a 256-byte boundary
+        buf = torch.empty(t.numel() + offset, dtype=t.dtype, device=cuda)
+        view = buf[offset:].view(t.shape)
+        view.copy_(t)
+        return view
+
+    for use_dqk in (False, True):
+        sg = shifted(signs.to(sign_dtype).to(cuda))
+        kw = {}
+        if use_dqk:
+            kw = {"dqk_b": shifted((1 / dq).half().to(cuda)), "dqk_c": shifted(prepare_dqk(dq).to(cuda))}
+        _, qB, qC = fused_split_rotate_quant_xBC(xBC.to(cuda), sg, s.nheads, s.ngroups, s.dstate, s.headdim, binv.to(cuda),
+                                                 cinv.to(cuda), **kw)
+        torch.cuda.synchronize()
+        _, rB, rC = O.split_rotate_quant_xBC(npy(xBC), npy(signs), s.nheads, s.ngroups, s.dstate, s.headdim, npy(binv), npy(cinv),
+                                             npy(prepare_dqk(1 / dq)) if use_dqk else None, npy(prepare_dqk(dq)) if use_dqk else None)
+        assert_same_codes(qB, rB, f"q_B {sign_dtype} offset={offset} dqk={use_dqk}")
+        assert_same_codes(qC, rC, f"q_C {sign_dtype} offset={offset} dqk={use_dqk}")
+
+
+@pytest.mark.parametrize("dim,shift,nc", [(8192, 7, 32), (4096 + 16, 7, 5), (1000, 7, 9), (999, 5, 3), (64 * 64, 7, 1), (2048, 7, 8),
+                                          (2048, 6, 16)])
 def test_state_passing(cuda, dim, shift, nc):
     from linquant_amd.kernels.mamba2.state_passing import _fixedpoint_state_passing_fwd
 
