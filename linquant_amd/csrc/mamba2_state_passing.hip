@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
         const int c = c0 + j;
         const V cur = buf[j];
         buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)(c + DEPTH) * ss_c));
-        __builtin_nontemporal_store(step(cur, c), (V*)(op + (int64_t)(c + 1) * so_c));
+        *(V*)(op + (int64_t)(c + 1) * so_c) = step(cur, c);  // cached store: the chunk scan reads it two launches later
       }
     }
 #pragma unroll
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
       const int c = nchunks - DEPTH + j;
       const V res = step(buf[j], c);
       if (j < DEPTH - 1) {
-        __builtin_nontemporal_store(res, (V*)(op + (int64_t)(c + 1) * so_c));
+        *(V*)(op + (int64_t)(c + 1) * so_c) = res;
       } else if (fp) {
         __builtin_nontemporal_store(res, (V*)fp);
       }
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
         if (c + DEPTH < nchunks) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)(c + DEPTH) * ss_c));
         const V res = step(cur, c);
         if (c < nchunks - 1) {
-          __builtin_nontemporal_store(res, (V*)(op + (int64_t)(c + 1) * so_c));
+          *(V*)(op + (int64_t)(c + 1) * so_c) = res;
         } else if (fp) {
           __builtin_nontemporal_store(res, (V*)fp);
         }
