@@ -61,7 +61,7 @@ LQ_DEV float wave_sum(float v) {
 // A 16-byte global load issued as an instruction (the compiler neither moves nor repeats it), and the wait that makes
 // its result usable: every value requested this way passes through arrived() before its first use.
 LQ_DEV void request16(lq_v4i& dst, const void* ptr) {
-  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory");
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(ptr) : "memory");  // streamed once
 }
 LQ_DEV void arrived(lq_v4i& v) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(v)::"memory"); }
 
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(IT 
     if (p.norm_out && live) {
 #pragma unroll
       for (int it = 0; it < kIt; ++it)
-        if (valid[it]) *(lq_v8h*)(p.norm_out + (int64_t)row * p.dim + (it * 64 + lane) * 8) = xv[it];
+        if (valid[it]) __builtin_nontemporal_store(xv[it], (lq_v8h*)(p.norm_out + (int64_t)row * p.dim + (it * 64 + lane) * 8));
     }
   } else if constexpr (!EXACT) {
 #pragma unroll
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(IT 
         const int pc = it * 64 + lane;  // 16-byte pieces of the INT8 row: 8 per chunk
         if (pc < 8 * g) {
           const lq_v4i o = *(const lq_v4i*)(Os + (pc >> 3) * kOS + (pc & 7) * 16);
-          *(lq_v4i*)(p.out + (int64_t)row * p.dim + pc * 16) = o;
+          __builtin_nontemporal_store(o, (lq_v4i*)(p.out + (int64_t)row * p.dim + pc * 16));
         }
       }
     }

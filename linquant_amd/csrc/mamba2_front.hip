@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void causal_conv1d_kernel(const _Float16* __re
       if (silu) a = a * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(a * -1.44269504088896340736f));
       o[e] = (_Float16)a;
     }
-    if (t < L) *(lq_v8h*)(op + (int64_t)t * D) = o;
+    if (t < L) __builtin_nontemporal_store(o, (lq_v8h*)(op + (int64_t)t * D));
   }
 }
 
