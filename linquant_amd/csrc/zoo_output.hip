@@ -226,12 +226,12 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) res[jj] = of[jj][r] + loc[jj][r] * svl[jj];
     if (p.o_is_f32) {
-      *(lq_v4f*)((float*)p.o + off) = lq_v4f{res[0], res[1], res[2], res[3]};
+      __builtin_nontemporal_store(lq_v4f{res[0], res[1], res[2], res[3]}, (lq_v4f*)((float*)p.o + off));
     } else {
       lq_v2i w;
       w[0] = (int)zoo_enc2(res[0], res[1], bf);
       w[1] = (int)zoo_enc2(res[2], res[3], bf);
-      *(lq_v2i*)((_Float16*)p.o + off) = w;
+      __builtin_nontemporal_store(w, (lq_v2i*)((_Float16*)p.o + off));
     }
   }
 }
