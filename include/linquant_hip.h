@@ -298,8 +298,8 @@ typedef struct {
   int32_t o_is_f32;
   const float* sq;           /* (H,) */
   const float* sk;           /* (H,) (no / scalar decay) */
-  const float* svl;          /* (H,V) */
-  const float* ss;           /* (H,V) */
+  const float* svl;          /* (H,V), 16-byte aligned */
+  const float* ss;           /* (H,V), 16-byte aligned */
   const void* unrot;         /* (V,V) fp16 or NULL */
   float scale;
   int32_t qmax;
@@ -371,8 +371,8 @@ int lq_fp16_to_int8(const lq_fp16_to_int8_args* args, hipStream_t stream);
 typedef struct {
   const void* x;             /* (B,L,D) fp16, unit D stride */
   int64_t x_stride_b, x_stride_l;
-  const void* weight;        /* (D,W) fp16 contiguous */
-  const void* bias;          /* (D,) fp16 or NULL */
+  const void* weight;        /* (D,W) fp16 contiguous, 16-byte aligned */
+  const void* bias;          /* (D,) fp16 or NULL, 16-byte aligned */
   void* out;                 /* (B,L,D) fp16 contiguous */
   int32_t batch, seqlen, dim, width; /* dim a multiple of 8, width 2..4 */
   int32_t silu;              /* 1: SiLU activation, 0: none */
