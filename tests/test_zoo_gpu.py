@@ -235,7 +235,7 @@ def test_wy_prep_kernel(cuda, cell, sigma, tau, K, gscale):
 
 
 def test_reference_mamba2_cell_config(cuda):
-    """BASELINE configs[0]: the Mamba-2 cell through chunk_simple_gla (q = C, k = B broadcast to heads, v = x*dt,
+    """The benchmark's first configuration (the CPU-runnable one): the Mamba-2 cell through chunk_simple_gla (q = C, k = B broadcast to heads, v = x*dt,
     g = dt*A, scale = 1), B1 T2048 H8 K = V = 64, per-head / per-channel static scales."""
     from linquant_amd.kernels import zoo
     from oracle import zoo_reference as Z
