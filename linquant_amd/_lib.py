@@ -92,6 +92,12 @@ def ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def aligned(t, nbytes=16):
+    """``t`` itself when its first byte sits on an ``nbytes`` boundary (or it is None), else a fresh copy: kernels that
+    fetch small parameter tables as whole 16-byte pieces need this, and a view into a larger tensor need not have it."""
+    return t if t is None or t.data_ptr() % nbytes == 0 else t.clone()
+
+
 def current_stream(device):
     import torch
 

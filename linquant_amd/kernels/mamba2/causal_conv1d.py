@@ -16,8 +16,8 @@ def causal_conv1d_fn(x, weight, bias=None, activation=None):
     B, D, L = x.shape
     W = weight.shape[1]
     assert weight.shape == (D, W) and 2 <= W <= 4 and D % 8 == 0
-    weight = weight.to(torch.float16).contiguous()
-    bias = None if bias is None else bias.to(torch.float16).contiguous()
+    weight = _lib.aligned(weight.to(torch.float16).contiguous())
+    bias = None if bias is None else _lib.aligned(bias.to(torch.float16).contiguous())
     out = torch.empty(B, L, D, dtype=torch.float16, device=x.device)
     _lib.call("lq_causal_conv1d", x.device, x=_lib.ptr(x), x_stride_b=x.stride(0), x_stride_l=x.stride(2),
               weight=_lib.ptr(weight), bias=_lib.ptr(bias), out=_lib.ptr(out), batch=B, seqlen=L, dim=D, width=W,

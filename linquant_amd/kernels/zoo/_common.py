@@ -93,6 +93,7 @@ def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims,
     """``A`` (fp16) and ``qg`` (INT8 codes of the decayed query) come from run_gla_A under per-channel decay; q and key
     are only read under no / scalar decay."""
     B, T, H, K, V = dims
+    svl, ss = _lib.aligned(svl), _lib.aligned(ss)
     _lib.call("lq_zoo_output", value.device, q=_lib.ptr(q), qg=_lib.ptr(qg), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
               g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
               sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),

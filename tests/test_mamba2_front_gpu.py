@@ -70,3 +70,26 @@ def test_causal_conv1d(cuda, width, bias, act, L):
         diff = np.abs(got.astype(np.float64) - ref.astype(np.float64))
         assert (diff <= np.spacing(np.abs(ref)).astype(np.float64)).all(), "more than one fp16 ulp apart"
         assert (got != ref).mean() < 1e-2
+
+
+def test_causal_conv1d_parameter_views(cuda):
+    """Taps and bias that are views into a larger parameter tensor (first byte off the 16-byte grid) give the same output
+    as freshly allocated ones through the wrapper, and the C entry point itself rejects such pointers with LQ_E_SHAPE."""
+    from linquant_amd import _lib
+    from linquant_amd.kernels.mamba2.causal_conv1d import causal_conv1d_fn
+
+    gen = torch.Generator().manual_seed(2)
+    B, L, D, W = 1, 96, 256, 4
+    x = torch.randn(B, L, D, generator=gen).half().cuda()
+    wbig = (torch.randn(D + 1, W, generator=gen) * 0.5).half().cuda()
+    bbig = (torch.randn(D + 4, generator=gen) * 0.1).half().cuda()
+    w_view, b_view = wbig[1:], bbig[4:]                              # 8 bytes past a 16-byte boundary
+    assert w_view.data_ptr() % 16 == 8 and b_view.data_ptr() % 16 == 8 and w_view.is_contiguous()
+    ref = causal_conv1d_fn(x.transpose(1, 2), w_view.clone(), b_view.clone(), activation="silu")
+    got = causal_conv1d_fn(x.transpose(1, 2), w_view, b_view, activation="silu")
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref)
+    out = torch.empty(B, L, D, dtype=torch.float16, device="cuda")
+    with pytest.raises(_lib.LinQuantHipError):
+        _lib.call("lq_causal_conv1d", x.device, x=_lib.ptr(x), x_stride_b=x.stride(0), x_stride_l=x.stride(1),
+                  weight=_lib.ptr(w_view), bias=None, out=_lib.ptr(out), batch=B, seqlen=L, dim=D, width=W, silu=1)
