@@ -78,6 +78,17 @@ def zoo_stage_bytes(fam, dec, B, T, H, K, V):
     return out
 
 
+def copy_probe(dev):
+    """One plain device-to-device copy of 256 MiB: what the HBM byte counters read for it calibrates them."""
+    import torch
+
+    probe = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+    probe.zero_()
+    probe_dst = torch.empty_like(probe)
+    probe_dst.copy_(probe)
+    torch.cuda.synchronize()
+
+
 def hadamard_signed(n, seed, device):
     import torch
 
@@ -153,6 +164,8 @@ def bench_zoo(args):
     del dbg, ht
     torch.cuda.synchronize()
 
+    if args.copy_probe:
+        copy_probe(dev)
     for _ in range(args.warmup):
         call(sc)
     torch.cuda.synchronize()
@@ -527,12 +540,7 @@ def main():
         return out
 
     if args.copy_probe:
-        probe = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
-        probe.zero_()
-        probe_dst = torch.empty_like(probe)
-        probe_dst.copy_(probe)
-        torch.cuda.synchronize()
-        del probe, probe_dst
+        copy_probe(dev)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -16,6 +16,8 @@
 // lane >> 4) accumulates four (i, j) pairs with one exponential per (i, j, channel).
 // With a local R_QK (rot, (K,K) fp16, x -> x.R) the anchored off-diagonal operands are rounded to fp16 and rotated
 // on the fp16 MFMA before quantization (gla.py:53-57); the diagonal blocks are not rotated.
+#include <type_traits>
+
 #include "zoo_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -40,6 +42,47 @@ LQ_DEV float wave_max(float m) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   return m;
+}
+
+// Diagonal block, every (i, j, n) weight evaluated on its own and masked before use (any decay spread):
+// lane (i = rl, j = 4kg + jj), 8 channels per step.
+template <int K, bool BF>
+LQ_DEV void diag_exact(const AParams& p, float sq, float sk, float inv_sq, float inv_sk, int rl, int kg, int64_t row0, int h,
+                       int i0) {
+  const int H = p.H, qmax = p.qmax;
+  constexpr bool bf = BF;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  const int64_t irow = ((row0 + rl) * H + h) * K;
+  for (int n8 = 0; n8 < K; n8 += 8) {
+    float qv[8];
+    zoo_ld8(p.q + irow + n8, bf, qv);
+    const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int j = 4 * kg + jj;
+      const int64_t jrow = ((row0 + j) * H + h) * K;
+      float kv[8];
+      zoo_ld8(p.k + jrow + n8, bf, kv);
+      const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
+        const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
+        const float gi = e < 4 ? gi0[e & 3] : gi1[e & 3], gj = e < 4 ? gj0[e & 3] : gj1[e & 3];
+        const float w = (j <= rl) ? zoo_exp(gi - gj) : 0.0f;
+        s[jj] = s[jj] + (qh * kh) * w;
+      }
+    }
+  }
+  lq_v4f o;
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) o[jj] = (4 * kg + jj <= rl) ? s[jj] : 0.0f;
+  {
+    lq_v2i oh;
+    oh[0] = (int)zoo_pack_h2(o[0], o[1]);
+    oh[1] = (int)zoo_pack_h2(o[2], o[3]);
+    *(lq_v2i*)(p.A + ((row0 + rl) * H + h) * 64 + i0 + 4 * kg) = oh;
+  }
 }
 
 // Diagonal 16x16 block of one wave (rows row0 .. row0+15), written to A[row][i0 + j].
@@ -87,45 +130,17 @@ LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float
       p.A[((row0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((rl <= 4 * kg + r) ? acc[r] : 0.0f);
     return;
   }
-  // exact path: lane (i = rl, j = 4kg + jj), 8 channels per step
-  float s[4] = {0.f, 0.f, 0.f, 0.f};
-  const int64_t irow = ((row0 + rl) * H + h) * K;
-  for (int n8 = 0; n8 < K; n8 += 8) {
-    float qv[8];
-    zoo_ld8(p.q + irow + n8, bf, qv);
-    const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const int j = 4 * kg + jj;
-      const int64_t jrow = ((row0 + j) * H + h) * K;
-      float kv[8];
-      zoo_ld8(p.k + jrow + n8, bf, kv);
-      const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
-        const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
-        const float gi = e < 4 ? gi0[e & 3] : gi1[e & 3], gj = e < 4 ? gj0[e & 3] : gj1[e & 3];
-        const float w = (j <= rl) ? zoo_exp(gi - gj) : 0.0f;
-        s[jj] = s[jj] + (qh * kh) * w;
-      }
-    }
-  }
-  lq_v4f o;
-#pragma unroll
-  for (int jj = 0; jj < 4; ++jj) o[jj] = (4 * kg + jj <= rl) ? s[jj] : 0.0f;
-  {
-    lq_v2i oh;
-    oh[0] = (int)zoo_pack_h2(o[0], o[1]);
-    oh[1] = (int)zoo_pack_h2(o[2], o[3]);
-    *(lq_v2i*)(p.A + ((row0 + rl) * H + h) * 64 + i0 + 4 * kg) = oh;
-  }
+  diag_exact<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, row0, h, i0);
 }
 
-template <int K, bool ROT, bool BF>
+// QG (rotated path only): the state-read codes are wanted (p.qg is set); a compile-time flag keeps the own-rows loop
+// one basic block.
+template <int K, bool ROT, bool BF, bool QG>
 __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   constexpr int RS = K + 8;  // halves per row of the transposed rotation
   __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
+  // rotated query codes of sub-blocks 1..3 of both chunks: [pass][I - 1][lane][dword]
+  __shared__ __align__(16) uint32_t QC[ROT ? 2 * 3 * 64 * (K / 16) : 4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -156,188 +171,275 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   const int i0 = 16 * blk;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
 
-  // ---- state-read operand of the output kernel: codes of q * exp(g) * scale
-  if (p.qg) {
-    for (int it = tid; it < 64 * (K / 8); it += 256) {
-      const int t = it / (K / 8), c8 = it % (K / 8);
-      const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
-      float qv[8];
-      zoo_ld8(p.q + off, bf, qv);
-      const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
-      int cq[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-        x = x * p.scale;
-        cq[e] = zoo_q8(x, inv_sq, qmax);
-      }
-      lq_v2i o;
-      o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
-      o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
-      *(lq_v2i*)(p.qg + off) = o;
-    }
-  }
-
-  diag_block<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
-
-  lq_v4i acc[3];
-#pragma unroll
-  for (int J = 0; J < 3; ++J) acc[J] = lq_v4i{0, 0, 0, 0};
-
-  if constexpr (!ROT) {
-    // ---- off-diagonal blocks J < blk: INT8 MFMA on anchored operands built from plain global loads
-    if (blk > 0) {
-#pragma unroll
-      for (int ks = 0; ks < K / 64; ++ks) {
-        const int kk = 64 * ks + 16 * kg;
-        float an[16];
-        {
-          const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
-#pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) {
-            const lq_v4f a4 = *(const lq_v4f*)(ap + 4 * e4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) an[4 * e4 + e] = a4[e];
-          }
-        }
-        lq_v4i qop;
-        {
-          const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
-          float q0[8];
-          zoo_ld8(p.q + off, bf, q0);
-          float q1[8];
-          zoo_ld8(p.q + off + 8, bf, q1);
-          int cd[16];
-#pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) {
-            const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int n = 4 * e4 + e;
-              const float qf = n < 8 ? q0[n & 7] : q1[n & 7];
-              float x = qf * zoo_exp(g4[e] - an[n]);
-              x = x * p.scale;
-              cd[n] = zoo_q8(x, inv_sq, qmax);
-            }
-          }
-#pragma unroll
-          for (int d = 0; d < 4; ++d) qop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
-        }
-#pragma unroll
-        for (int J = 0; J < 3; ++J) {
-          if (J >= blk) continue;
-          const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
-          float k0[8];
-          zoo_ld8(p.k + off, bf, k0);
-          float k1[8];
-          zoo_ld8(p.k + off + 8, bf, k1);
-          int cd[16];
-#pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) {
-            const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int n = 4 * e4 + e;
-              const float kf = n < 8 ? k0[n & 7] : k1[n & 7];
-              cd[n] = zoo_q8(kf * zoo_exp(an[n] - g4[e]), inv_sk, qmax);
-            }
-          }
-          lq_v4i kop;
-#pragma unroll
-          for (int d = 0; d < 4; ++d) kop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
-          acc[J] = lq_mfma_i8(qop, kop, acc[J]);
-        }
-      }
-    }
-  } else {
-    // ---- local R_QK: the anchored operands are rotated (fp16 MFMA, fp32 accumulate) before quantization.
-    // Transposed product R^T . X^T: lane (rl, kg) receives, for token rl, channels 16mt + 4kg + r, which it packs
-    // as dword mt of its INT8 operand; q and k operands share that channel -> slot map, so the INT8 dot is exact.
+  if constexpr (ROT) {
+    // ---- local R_QK: column-wise.  The wave loads its own sub-block (q, k, g rows) once, in the layout of the rotation
+    // operand (lane (rl, kg) = token rl, channels 32ks + 8kg + e), and takes everything that needs those rows from
+    // the registers: the state-read codes q*exp(g)*scale, the diagonal block, the query operand anchored at this
+    // sub-block's first row (rotated, quantized, handed to the other waves through LDS) and the key operands anchored
+    // at the first row of each later sub-block I (rotated, quantized, met with sub-block I's query codes from LDS).
+    // The rotation is the transposed product R^T . X^T: lane (rl, kg) receives, for token rl, channels 16mt + 4kg + r,
+    // which it packs as dword mt of its INT8 operand; q and k operands share that channel -> slot map, so the INT8
+    // dot is exact and a consumer lane needs exactly the dwords the same lane of the producer wave holds.
     constexpr int KS = K / 32, MT = K / 16;
     if (pass == 0) __syncthreads();  // R^T staged
-    // tensor 0 = q rows of this sub-block, tensor 1 + J = k rows of sub-block J < blk, all anchored at this sub-block's
-    // first row; two tensors share one sweep over R^T, and a k tensor meets the q codes as soon as it is quantized
-    uint32_t cq[MT];
+    const int64_t roff = ((t0 + i0 + rl) * H + h) * K + 8 * kg;
+    // One step (32 channels, 8 per lane) of raw operands: own rows of q / k / g and the first rows of g of two
+    // sub-blocks (anchors; the address stays inside the chunk for every sub-block <= 3).  Steps are requested one ahead
+    // of their use.
+    struct Step {
+      lq_v4i q, k;
+      lq_v4f g[2], a[2], b[2];
+    };
+    auto request = [&](auto with_q, int Ia, int Ib, int ks, Step& r) {
+      if constexpr (decltype(with_q)::value) r.q = *(const lq_v4i*)(p.q + roff + 32 * ks);
+      r.k = *(const lq_v4i*)(p.k + roff + 32 * ks);
+      const float* gp = p.g + roff + 32 * ks;
+      r.g[0] = *(const lq_v4f*)gp, r.g[1] = *(const lq_v4f*)(gp + 4);
+      const float* ap = p.g + ((t0 + 16 * Ia) * H + h) * K + 32 * ks + 8 * kg;
+      r.a[0] = *(const lq_v4f*)ap, r.a[1] = *(const lq_v4f*)(ap + 4);
+      const float* bp = p.g + ((t0 + 16 * Ib) * H + h) * K + 32 * ks + 8 * kg;
+      r.b[0] = *(const lq_v4f*)bp, r.b[1] = *(const lq_v4f*)(bp + 4);
+    };
+    auto unpack = [&](const lq_v4i& raw, float (&o)[8]) {
 #pragma unroll
-    for (int gp = 0; gp < 2; ++gp) {
-      if (2 * gp > blk || blk == 0) continue;  // uniform per wave
-      lq_v8h xop[2][KS];
+      for (int d = 0; d < 4; ++d) zoo_dec2((uint32_t)raw[d], bf, o[2 * d], o[2 * d + 1]);
+    };
+    // key rows of this sub-block anchored at the first rows of sub-blocks Ia and Ib, as fp16 rotation operands (the
+    // rows are fetched again here rather than held in registers across the first sweep: they are cache hits)
+    auto build_k2 = [&](int Ia, int Ib, lq_v8h (&xa)[KS], lq_v8h (&xb)[KS]) {
+      Step st[2];
+      request(std::false_type{}, Ia, Ib, 0, st[0]);
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int t = 2 * gp + u;
-        if (t > blk) {
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 1 < KS) request(std::false_type{}, Ia, Ib, ks + 1, st[(ks + 1) & 1]);
+        const Step& r = st[ks & 1];
+        float kf[8];
+        unpack(r.k, kf);
 #pragma unroll
-          for (int ks = 0; ks < KS; ++ks) xop[u][ks] = lq_v8h{0, 0, 0, 0, 0, 0, 0, 0};
-          continue;
+        for (int e = 0; e < 8; ++e) {
+          const float gg = r.g[e >> 2][e & 3];
+          xa[ks][e] = (_Float16)(kf[e] * zoo_exp(r.a[e >> 2][e & 3] - gg));
+          xb[ks][e] = (_Float16)(kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg));
         }
-        const int64_t row = t == 0 ? t0 + i0 + rl : t0 + 16 * (t - 1) + rl;
-        const _Float16* src = t == 0 ? p.q : p.k;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const int kk = 32 * ks + 8 * kg;
-          const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
-          const lq_v4f a0 = *(const lq_v4f*)ap, a1 = *(const lq_v4f*)(ap + 4);
-          const int64_t off = (row * H + h) * K + kk;
-          float xv[8];
-          zoo_ld8(src + off, bf, xv);
-          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float gg = e < 4 ? g0[e & 3] : g1[e & 3], an = e < 4 ? a0[e & 3] : a1[e & 3];
-            if (t == 0) {
-              float x = xv[e] * zoo_exp(gg - an);
-              x = x * p.scale;
-              xop[u][ks][e] = (_Float16)x;
-            } else {
-              xop[u][ks][e] = (_Float16)(xv[e] * zoo_exp(an - gg));
-            }
-          }
-        }
+        __builtin_amdgcn_sched_barrier(0);  // keeps the look-ahead at one step
       }
-      uint32_t cd[2][MT];
+    };
+    // one sweep over R^T for one or two operands; codes of token rl, dword mt = channels 16mt + 4kg + r
+    auto sweep = [&](auto two, const lq_v8h (&x0)[KS], const lq_v8h (&x1)[KS], float inv0, float inv1, uint32_t (&c0)[MT],
+                     uint32_t (&c1)[MT]) {
+      constexpr bool kTwo = decltype(two)::value;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        lq_v4f ra[2];
-        ra[0] = ra[1] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+        lq_v4f r0 = {0.f, 0.f, 0.f, 0.f}, r1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const lq_v8h rop = *(const lq_v8h*)(RT + (16 * mt + rl) * RS + 32 * ks + 8 * kg);
-          ra[0] = lq_mfma_f16(rop, xop[0][ks], ra[0]);
-          ra[1] = lq_mfma_f16(rop, xop[1][ks], ra[1]);
+          r0 = lq_mfma_f16(rop, x0[ks], r0);
+          if constexpr (kTwo) r1 = lq_mfma_f16(rop, x1[ks], r1);
         }
+        c0[mt] = zoo_pack_codes(zoo_q8(r0[0], inv0, qmax), zoo_q8(r0[1], inv0, qmax), zoo_q8(r0[2], inv0, qmax),
+                                zoo_q8(r0[3], inv0, qmax));
+        if constexpr (kTwo)
+          c1[mt] = zoo_pack_codes(zoo_q8(r1[0], inv1, qmax), zoo_q8(r1[1], inv1, qmax), zoo_q8(r1[2], inv1, qmax),
+                                  zoo_q8(r1[3], inv1, qmax));
+      }
+    };
+    const float sqk = sq * sk;
+    // key codes of this sub-block against the query codes of sub-block I (from LDS) -> A[rows of I][columns of blk]
+    auto meet = [&](int I, const uint32_t (&ck)[MT]) {
+      const uint32_t* qc = QC + (((pass * 3 + I - 1) * 64 + lane) * MT);
+      lq_v4i acc = {0, 0, 0, 0};
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const float inv = (gp == 0 && u == 0) ? inv_sq : inv_sk;
-          cd[u][mt] = zoo_pack_codes(zoo_q8(ra[u][0], inv, qmax), zoo_q8(ra[u][1], inv, qmax), zoo_q8(ra[u][2], inv, qmax),
-                                     zoo_q8(ra[u][3], inv, qmax));
+      for (int s = 0; s < K / 64; ++s) {
+        const lq_v4i qop = *(const lq_v4i*)(qc + 4 * s);
+        lq_v4i kop;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) kop[d] = (int)ck[4 * s + d];
+        acc = lq_mfma_i8(qop, kop, acc);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p.A[((t0 + 16 * I + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((float)acc[r] * sqk);
+    };
+
+    // own rows, fetched once: state-read codes, diagonal block (factorized around the first row while the spread is
+    // measured) and the two operands of the first sweep
+    lq_v8h xq[KS], xk[KS];
+    float spread = 0.0f;
+    lq_v4f dacc = {0.f, 0.f, 0.f, 0.f};
+    const int inext = blk < 3 ? blk + 1 : 3;
+    Step st[2];
+    request(std::true_type{}, blk, inext, 0, st[0]);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 1 < KS) request(std::true_type{}, blk, inext, ks + 1, st[(ks + 1) & 1]);
+      const Step& r = st[ks & 1];
+      float qf[8], kf[8];
+      unpack(r.q, qf);
+      unpack(r.k, kf);
+      int cs[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float gg = r.g[e >> 2][e & 3];
+        const float d = gg - r.a[e >> 2][e & 3];
+        spread = fmaxf(spread, __builtin_fabsf(d));
+        const float ed = zoo_exp(d);
+        const float qh = (float)zoo_q8(qf[e] * p.scale, inv_sq, qmax) * sq;
+        const float kh = (float)zoo_q8(kf[e], inv_sk, qmax) * sk;
+        dacc = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * ed, kh * zoo_exp(-d), dacc, 0, 0, 0);
+        float x = qf[e] * ed;
+        x = x * p.scale;
+        xq[ks][e] = (_Float16)x;
+        xk[ks][e] = (_Float16)(kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg));
+        float y = qf[e] * zoo_exp(gg);
+        y = y * p.scale;
+        cs[e] = zoo_q8(y, inv_sq, qmax);
+      }
+      if constexpr (QG) {
+        lq_v2i o;
+        o[0] = (int)zoo_pack_codes(cs[0], cs[1], cs[2], cs[3]);
+        o[1] = (int)zoo_pack_codes(cs[4], cs[5], cs[6], cs[7]);
+        *(lq_v2i*)(p.qg + roff + 32 * ks) = o;
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keeps the look-ahead at one step
+    }
+    // first sweep: query operand of this sub-block (none for sub-block 0) and key operand for sub-block blk + 1 (none
+    // for sub-block 3)
+    uint32_t cq[MT], ck[MT];
+    sweep(std::true_type{}, xq, xk, inv_sq, inv_sk, cq, ck);  // sub-block 0 has no use for cq, sub-block 3 none for ck
+    if (blk > 0) {
+      uint32_t* qc = QC + (((pass * 3 + blk - 1) * 64 + lane) * MT);
+#pragma unroll
+      for (int s = 0; s < MT / 4; ++s) {
+        lq_v4i o;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) o[d] = (int)cq[4 * s + d];
+        *(lq_v4i*)(qc + 4 * s) = o;
+      }
+    }
+    __syncthreads();  // query codes of the chunk are in LDS (the two passes use separate buffers)
+    if (blk < 3) meet(blk + 1, ck);
+    // second sweep: key operands for sub-blocks blk + 2 and blk + 3
+    if (blk <= 1) {
+      build_k2(2, 3, xq, xk);
+      sweep(std::true_type{}, xq, xk, inv_sk, inv_sk, cq, ck);
+      if (blk == 0) meet(2, cq);
+      meet(3, ck);
+    }
+    // diagonal block, last: its rare exact path is kept away from the registers of the sweeps
+    spread = wave_max(spread);
+    if (spread <= 40.0f) {
+      // lane holds column j = rl, rows i = 4kg + r
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((rl <= 4 * kg + r) ? dacc[r] : 0.0f);
+    } else {
+      diag_exact<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
+    }
+  } else {
+    // ---- state-read operand of the output kernel: codes of q * exp(g) * scale
+    if (p.qg) {
+      for (int it = tid; it < 64 * (K / 8); it += 256) {
+        const int t = it / (K / 8), c8 = it % (K / 8);
+        const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
+        float qv[8];
+        zoo_ld8(p.q + off, bf, qv);
+        const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+        int cq[8];
+  #pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
+          x = x * p.scale;
+          cq[e] = zoo_q8(x, inv_sq, qmax);
         }
+        lq_v2i o;
+        o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
+        o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
+        *(lq_v2i*)(p.qg + off) = o;
       }
-      if (gp == 0) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) cq[mt] = cd[0][mt];
-      }
-#pragma unroll
-      for (int u = (gp == 0 ? 1 : 0); u < 2; ++u) {
-        const int J = 2 * gp + u - 1;
-        if (J >= blk) continue;
-#pragma unroll
-        for (int s = 0; s < K / 64; ++s) {
-          lq_v4i qop, kop;
-#pragma unroll
-          for (int d = 0; d < 4; ++d) qop[d] = (int)cq[4 * s + d], kop[d] = (int)cd[u][4 * s + d];
-          acc[J] = lq_mfma_i8(qop, kop, acc[J]);
+    }
+
+    diag_block<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
+
+    lq_v4i acc[3];
+  #pragma unroll
+    for (int J = 0; J < 3; ++J) acc[J] = lq_v4i{0, 0, 0, 0};
+
+    {
+      // ---- off-diagonal blocks J < blk: INT8 MFMA on anchored operands built from plain global loads
+      if (blk > 0) {
+  #pragma unroll
+        for (int ks = 0; ks < K / 64; ++ks) {
+          const int kk = 64 * ks + 16 * kg;
+          float an[16];
+          {
+            const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
+  #pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+              const lq_v4f a4 = *(const lq_v4f*)(ap + 4 * e4);
+  #pragma unroll
+              for (int e = 0; e < 4; ++e) an[4 * e4 + e] = a4[e];
+            }
+          }
+          lq_v4i qop;
+          {
+            const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
+            float q0[8];
+            zoo_ld8(p.q + off, bf, q0);
+            float q1[8];
+            zoo_ld8(p.q + off + 8, bf, q1);
+            int cd[16];
+  #pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+              const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
+  #pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int n = 4 * e4 + e;
+                const float qf = n < 8 ? q0[n & 7] : q1[n & 7];
+                float x = qf * zoo_exp(g4[e] - an[n]);
+                x = x * p.scale;
+                cd[n] = zoo_q8(x, inv_sq, qmax);
+              }
+            }
+  #pragma unroll
+            for (int d = 0; d < 4; ++d) qop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
+          }
+  #pragma unroll
+          for (int J = 0; J < 3; ++J) {
+            if (J >= blk) continue;
+            const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
+            float k0[8];
+            zoo_ld8(p.k + off, bf, k0);
+            float k1[8];
+            zoo_ld8(p.k + off + 8, bf, k1);
+            int cd[16];
+  #pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+              const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
+  #pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int n = 4 * e4 + e;
+                const float kf = n < 8 ? k0[n & 7] : k1[n & 7];
+                cd[n] = zoo_q8(kf * zoo_exp(an[n] - g4[e]), inv_sk, qmax);
+              }
+            }
+            lq_v4i kop;
+  #pragma unroll
+            for (int d = 0; d < 4; ++d) kop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
+            acc[J] = lq_mfma_i8(qop, kop, acc[J]);
+          }
         }
       }
     }
-  }
 
-  const float sqk = sq * sk;
-#pragma unroll
-  for (int J = 0; J < 3; ++J) {
-    if (J >= blk) continue;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)((float)acc[J][r] * sqk);
+    const float sqk = sq * sk;
+  #pragma unroll
+    for (int J = 0; J < 3; ++J) {
+      if (J >= blk) continue;
+  #pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)((float)acc[J][r] * sqk);
+    }
   }
   // zero blocks above the diagonal
   for (int J = blk + 1; J < 4; ++J)
@@ -364,24 +466,27 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
   dim3 grid((a->seqlen / 64 + 1) / 2, a->batch * a->nheads);
-#define LQ_A_LAUNCH(KV, ROTV)                                                                              \
+#define LQ_A_LAUNCH2(KV, ROTV, QGV)                                                                        \
   do {                                                                                                     \
     if (p.bf)                                                                                              \
-      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, true>), grid, dim3(256), 0, stream, p);               \
+      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, true, QGV>), grid, dim3(256), 0, stream, p);          \
     else                                                                                                   \
-      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, false>), grid, dim3(256), 0, stream, p);              \
+      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, false, QGV>), grid, dim3(256), 0, stream, p);         \
   } while (0)
-  if (a->kdim == 128) {
-    if (a->rot)
-      LQ_A_LAUNCH(128, true);
-    else
-      LQ_A_LAUNCH(128, false);
-  } else {
-    if (a->rot)
-      LQ_A_LAUNCH(64, true);
-    else
-      LQ_A_LAUNCH(64, false);
-  }
+#define LQ_A_LAUNCH(KV)                 \
+  do {                                  \
+    if (a->rot && p.qg)                 \
+      LQ_A_LAUNCH2(KV, true, true);     \
+    else if (a->rot)                    \
+      LQ_A_LAUNCH2(KV, true, false);    \
+    else                                \
+      LQ_A_LAUNCH2(KV, false, false);   \
+  } while (0)
+  if (a->kdim == 128)
+    LQ_A_LAUNCH(128);
+  else
+    LQ_A_LAUNCH(64);
+#undef LQ_A_LAUNCH2
 #undef LQ_A_LAUNCH
   return lq_check_launch();
 }
