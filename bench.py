@@ -57,6 +57,17 @@ ZOO_CELLS = {"linear_none": ("linear", "none"), "mamba2": ("linear", "scalar"), 
              "deltanet": ("delta", "none"), "gated_deltanet": ("delta", "scalar"), "kda": ("delta", "diagonal")}
 
 
+# HBM bytes per launch of the zoo stages at the benchmark shapes, from rocprofv3 FETCH_SIZE / WRITE_SIZE scaled by what the
+# same counters read for a plain 256 MiB copy in the same run (x2.0 / x1.0); summary in profiles/zoo_c2_c3_c4_hbm_traffic.md
+# (c3_deltanet was not collected: its stages are those of c3_gdn without the decay)
+ZOO_TRAFFIC_MB = {
+    "c2_la": {"write_codes": 205.2, "state": 136.8, "output": 335.8},
+    "c2_gla": {"cumsum": 277.3, "gla_A": 464.0, "write_codes": 341.7, "state": 136.8, "output": 268.6},
+    "c3_gdn": {"cumsum": 2.1, "wy_prep": 385.5, "write_codes": 206.5, "state": 275.5, "output": 344.4},
+    "c4_kda": {"cumsum": 555.2, "wy_prep": 1428.2, "gla_A": 951.2, "write_codes": 693.9, "state": 558.6, "output": 537.7},
+}
+
+
 def zoo_stage_bytes(fam, dec, B, T, H, K, V):
     """Algorithmic HBM bytes per zoo stage: every tensor the stage must read or write, counted once."""
     qk, vv, tok = B * T * H * K * 2, B * T * H * V * 2, B * T * H * 4
@@ -214,6 +225,8 @@ def bench_zoo(args):
     roofline = {"kernel": "zoo_" + dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "avg_ms": round(avg_dom, 4),
                 "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
+    if dom in ZOO_TRAFFIC_MB.get(args.workload, {}):
+        roofline["traffic"] = int(ZOO_TRAFFIC_MB[args.workload][dom] * 1e6)
 
     cpu = None
     if not args.no_cpu_baseline:

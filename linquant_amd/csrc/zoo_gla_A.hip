@@ -7,15 +7,17 @@
 //     with qh = q8(q*scale, 1/sq) * sq and kh = q8(k, 1/sk) * sk  (fp32 reduction over the dequantized codes)
 //   entries above the diagonal are written as zero.
 //
-// One 4-wave workgroup per (pair of chunks, batch*head); wave w owns the 16 rows of sub-block w of the first chunk and
-// then those of sub-block 3 - w of the second one, so every wave does the same number of off-diagonal blocks (sub-block
-// I has I of them) and the rotation is staged once for both chunks.  Off-diagonal
-// operands are K-contiguous, so each lane builds its own 16-slot INT8 MFMA operand from plain global loads
-// (no LDS).  The diagonal block factorizes the decay weight around the block's first row whenever the decay spread
-// inside the block allows it and then runs as an fp32 MFMA product; otherwise lane (i = lane & 15, j-group =
+// One 4-wave workgroup per (pair of chunks, batch*head); wave w owns sub-block w of the first chunk and then sub-block
+// 3 - w of the second one, so every wave does the same amount of off-diagonal work and the rotation is staged once
+// for both chunks.  The diagonal block factorizes the decay weight around the block's first row whenever the decay
+// spread inside the block allows it and then runs as an fp32 MFMA product; otherwise lane (i = lane & 15, j-group =
 // lane >> 4) accumulates four (i, j) pairs with one exponential per (i, j, channel).
+// Without a rotation the wave of sub-block I (row-wise) builds its anchored query operand and the key operand of
+// every earlier sub-block from plain K-contiguous global loads, 16 INT8 slots per lane (no LDS).
 // With a local R_QK (rot, (K,K) fp16, x -> x.R) the anchored off-diagonal operands are rounded to fp16 and rotated
-// on the fp16 MFMA before quantization (gla.py:53-57); the diagonal blocks are not rotated.
+// on the fp16 MFMA before quantization (gla.py:53-57); the diagonal blocks are not rotated.  That path is column-wise:
+// the wave of sub-block J fetches its own rows once, hands its anchored query codes to the other waves through LDS and
+// builds its key operand once per later sub-block I (anchored at I's first row), meeting I's query codes from LDS.
 #include <type_traits>
 
 #include "zoo_common.h"
