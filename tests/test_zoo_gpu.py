@@ -124,7 +124,7 @@ def test_strong_decay_stays_finite(cuda, cell, eta):
 
 
 @pytest.mark.parametrize("cell", ["gla", "kda"])
-@pytest.mark.parametrize("n,K", [(128, 64), (512, 64), (256, 128)])
+@pytest.mark.parametrize("n,K", [(128, 64), (512, 64), (256, 128), (64, 128), (192, 128), (192, 64)])
 def test_local_rqk_rotation(cuda, cell, n, K):
     """R_QK on a diagonal-decay cell is local: only the anchored operands of the off-diagonal sub-blocks are rotated
     (/root/reference tests/test_kernel_gla.py:47-60)."""
