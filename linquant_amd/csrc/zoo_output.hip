@@ -7,7 +7,8 @@
 //   diagonal decay:     qq = q8(q*exp(g)*scale, 1/sq);  of = float(qq . h_i8) * sq * ss[v];  Af = A (fp32 input)
 //   both:               o  = of + (fp16(Af) . fp16(q8(v, 1/svl))) * svl[v]
 //
-// One 4-wave workgroup per (64-column V tile, chunk, batch*head); wave w owns rows 16w..16w+15 of the chunk.
+// One 4-wave workgroup per (one or two 64-column V tiles, chunk, batch*head); wave w owns rows 16w..16w+15 of the
+// chunk.  With two tiles (V a multiple of 128) the q / k codes and the A tile are made once for both.
 // q / k codes are produced once per workgroup into LDS (K-contiguous rows: plain 16-byte INT8 MFMA operands);
 // the stored state is V-major in HBM, so its operand is a plain 16-byte global load.  The local value
 // operand goes to LDS as token-pair interleaved fp16 (dword = two consecutive tokens of one channel), the
@@ -24,13 +25,15 @@ constexpr int kVW = 68;  // dwords per token-pair row of the value tile
 
 using OutParams = ZooOutParams;
 
-template <bool GLA, bool USE_G, int K, bool BF>
+// NV: 64-column V tiles per workgroup (2 when V is a multiple of 128: the q / k codes and the A tile are then made once
+// for both tiles)
+template <bool GLA, bool USE_G, int K, bool BF, int NV>
 __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   constexpr int QS = K + 16;  // byte stride of a code row
   __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) _Float16 Afl[GLA ? 8 : 64 * kAS];
-  __shared__ __align__(16) uint32_t vP[32 * kVW];
+  __shared__ __align__(16) uint32_t vP[NV * 32 * kVW];
   __shared__ float g_s[64];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -48,7 +51,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       bh = vid / (nv * gridDim.y);
     }
   }
-  const int v0 = vtile * BV;
+  const int v0 = vtile * BV * NV;
   const int b = bh / p.H, h = bh % p.H;
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
@@ -76,20 +79,31 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
   const int tp = tid >> 3, c8v = tid & 7;  // value tile: 32 token pairs x 8 groups of 8 channels
   const int64_t voff = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8v;
-  const lq_v4i va_raw = *(const lq_v4i*)(p.v + voff), vb_raw = *(const lq_v4i*)(p.v + voff + (int64_t)H * V);
-  const lq_v4f sv0 = *(const lq_v4f*)(p.svl + h * V + v0 + 8 * c8v), sv1 = *(const lq_v4f*)(p.svl + h * V + v0 + 8 * c8v + 4);
+  lq_v4i va_raw[NV], vb_raw[NV];
+  lq_v4f sv0[NV], sv1[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    va_raw[n] = *(const lq_v4i*)(p.v + voff + BV * n), vb_raw[n] = *(const lq_v4i*)(p.v + voff + BV * n + (int64_t)H * V);
+    sv0[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 8 * c8v), sv1[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 8 * c8v + 4);
+  }
   const float g_raw = (USE_G && !GLA) ? p.g[(t0 + (tid & 63)) * H + h] : 0.0f;
   const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
-  lq_v4i hop[K / 64][4];
+  lq_v4i hop[NV][K / 64][4];
   lq_v4i qgop[GLA ? K / 64 : 1];
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
     if constexpr (GLA) qgop[ks] = *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) hop[ks][jj] = *(const lq_v4i*)(hp + (4 * rl + jj) * K + 64 * ks + 16 * kg);
+    for (int n = 0; n < NV; ++n)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) hop[n][ks][jj] = *(const lq_v4i*)(hp + (BV * n + 4 * rl + jj) * K + 64 * ks + 16 * kg);
   }
-  const lq_v4f ss4 = *(const lq_v4f*)(p.ss + h * V + v0 + 4 * rl);
-  const lq_v4f svl4 = *(const lq_v4f*)(p.svl + h * V + v0 + 4 * rl);
+  lq_v4f ss4[NV], svl4[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    ss4[n] = *(const lq_v4f*)(p.ss + h * V + v0 + BV * n + 4 * rl);
+    svl4[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 4 * rl);
+  }
 
   // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
   if constexpr (!GLA) {
@@ -116,29 +130,32 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       *(lq_v2i*)(kc + t * QS + 8 * c8) = ok;
     }
   }
-  {
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
     lq_v4i o0, o1;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       float a0, a1, b0, b1;
-      zoo_dec2((uint32_t)va_raw[d], bf, a0, a1);
-      zoo_dec2((uint32_t)vb_raw[d], bf, b0, b1);
-      const float s0 = d < 2 ? sv0[2 * d] : sv1[2 * d - 4], s1 = d < 2 ? sv0[2 * d + 1] : sv1[2 * d - 3];
+      zoo_dec2((uint32_t)va_raw[n][d], bf, a0, a1);
+      zoo_dec2((uint32_t)vb_raw[n][d], bf, b0, b1);
+      const float s0 = d < 2 ? sv0[n][2 * d] : sv1[n][2 * d - 4], s1 = d < 2 ? sv0[n][2 * d + 1] : sv1[n][2 * d - 3];
       const float i0 = 1.0f / s0, i1 = 1.0f / s1;
       const int w0 = (int)zoo_pack_h2((float)zoo_q8(a0, i0, qmax), (float)zoo_q8(b0, i0, qmax));
       const int w1 = (int)zoo_pack_h2((float)zoo_q8(a1, i1, qmax), (float)zoo_q8(b1, i1, qmax));
       if (d < 2) o0[2 * d] = w0, o0[2 * d + 1] = w1; else o1[2 * d - 4] = w0, o1[2 * d - 3] = w1;
     }
-    *(lq_v4i*)(vP + tp * kVW + 8 * c8v) = o0;
-    *(lq_v4i*)(vP + tp * kVW + 8 * c8v + 4) = o1;
+    *(lq_v4i*)(vP + (32 * n + tp) * kVW + 8 * c8v) = o0;
+    *(lq_v4i*)(vP + (32 * n + tp) * kVW + 8 * c8v + 4) = o1;
   }
   if (USE_G && !GLA) g_s[tid & 63] = g_raw;  // four threads per token write the same value
   __syncthreads();
 
   // ---- phase 2: INT8 contractions of this wave's 16 rows
-  lq_v4i o32[4];
+  lq_v4i o32[NV][4];
 #pragma unroll
-  for (int jj = 0; jj < 4; ++jj) o32[jj] = lq_v4i{0, 0, 0, 0};
+  for (int n = 0; n < NV; ++n)
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) o32[n][jj] = lq_v4i{0, 0, 0, 0};
   lq_v4i a32[4];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
@@ -150,7 +167,9 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
     else
       qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) o32[jj] = lq_mfma_i8(qop, hop[ks][jj], o32[jj]);
+    for (int n = 0; n < NV; ++n)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) o32[n][jj] = lq_mfma_i8(qop, hop[n][ks][jj], o32[n][jj]);
     if (!GLA) {
 #pragma unroll
       for (int jt = 0; jt < 4; ++jt) {
@@ -162,19 +181,18 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
 
   // ---- phase 3: dequantize; A -> fp16 in operand layout
-  float of[4][4];  // [jj][r]: rows 16w + 4kg + r, channels v0 + 4rl + jj
-  {
-    const lq_v4f ssv = ss4;
+  float of[NV][4][4];  // [tile][jj][r]: rows 16w + 4kg + r, channels v0 + 64 tile + 4rl + jj
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + 4 * kg + r]) : 1.0f;
+  for (int r = 0; r < 4; ++r) {
+    const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + 4 * kg + r]) : 1.0f;
+#pragma unroll
+    for (int n = 0; n < NV; ++n)
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
-        float x = (float)o32[jj][r] * sq;
-        x = x * ssv[jj];
-        of[jj][r] = (USE_G && !GLA) ? x * eg : x;
+        float x = (float)o32[n][jj][r] * sq;
+        x = x * ss4[n][jj];
+        of[n][jj][r] = (USE_G && !GLA) ? x * eg : x;
       }
-    }
   }
   if (!GLA) {
     const float sqk = sq * sk;
@@ -197,9 +215,11 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
 
   // ---- phase 4: local product on the fp16 MFMA and store
-  lq_v4f loc[4];
+  lq_v4f loc[NV][4];
 #pragma unroll
-  for (int jj = 0; jj < 4; ++jj) loc[jj] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < NV; ++n)
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) loc[n][jj] = lq_v4f{0.f, 0.f, 0.f, 0.f};
   const int nslab = (16 * wave + 15) / 32 + 1;
   for (int js = 0; js < nslab; ++js) {
     lq_v8h aop;
@@ -208,23 +228,27 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
     } else {
       aop = *(const lq_v8h*)(Afl + (16 * wave + rl) * kAS + 32 * js + 8 * kg);
     }
-    lq_v4i xop[4];
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const lq_v4i vv = *(const lq_v4i*)(vP + (16 * js + 4 * kg + d) * kVW + 4 * rl);
+    for (int n = 0; n < NV; ++n) {
+      lq_v4i xop[4];
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) xop[jj][d] = vv[jj];
+      for (int d = 0; d < 4; ++d) {
+        const lq_v4i vv = *(const lq_v4i*)(vP + (32 * n + 16 * js + 4 * kg + d) * kVW + 4 * rl);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) xop[jj][d] = vv[jj];
+      }
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) loc[n][jj] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[jj]), loc[n][jj]);
     }
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) loc[jj] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[jj]), loc[jj]);
   }
-  const lq_v4f svl = svl4;
+#pragma unroll
+  for (int n = 0; n < NV; ++n)
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + 4 * rl;
+    const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + BV * n + 4 * rl;
     float res[4];
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) res[jj] = of[jj][r] + loc[jj][r] * svl[jj];
+    for (int jj = 0; jj < 4; ++jj) res[jj] = of[n][jj][r] + loc[n][jj][r] * svl4[n][jj];
     if (p.o_is_f32) {
       __builtin_nontemporal_store(lq_v4f{res[0], res[1], res[2], res[3]}, (lq_v4f*)((float*)p.o + off));
     } else {
@@ -236,20 +260,29 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
 }
 
-template <bool GLA, bool USE_G, int K>
+template <bool GLA, bool USE_G, int K, int NV>
 void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
   if (p.bf)
-    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true, NV>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false, NV>), grid, dim3(256), 0, stream, p);
 }
 
 template <bool GLA, bool USE_G>
-int launch(const OutParams& p, int K, dim3 grid, hipStream_t stream) {
-  if (K == 128)
-    launch_bf<GLA, USE_G, 128>(p, grid, stream);
-  else
-    launch_bf<GLA, USE_G, 64>(p, grid, stream);
+int launch(const OutParams& p, int K, hipStream_t stream) {
+  const bool two = p.V % (2 * BV) == 0;  // two V tiles per workgroup
+  const dim3 grid(p.V / (two ? 2 * BV : BV), p.NT, p.B * p.H);
+  if (K == 128) {
+    if (two)
+      launch_bf<GLA, USE_G, 128, 2>(p, grid, stream);
+    else
+      launch_bf<GLA, USE_G, 128, 1>(p, grid, stream);
+  } else {
+    if (two)
+      launch_bf<GLA, USE_G, 64, 2>(p, grid, stream);
+    else
+      launch_bf<GLA, USE_G, 64, 1>(p, grid, stream);
+  }
   return lq_check_launch();
 }
 
@@ -278,8 +311,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   p.unrot = (const _Float16*)a->unrot;
   if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
-  dim3 grid(a->vdim / BV, p.NT, a->batch * a->nheads);
-  if (gla) return launch<true, true>(p, a->kdim, grid, stream);
-  if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, grid, stream);
-  return launch<false, false>(p, a->kdim, grid, stream);
+  if (gla) return launch<true, true>(p, a->kdim, stream);
+  if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, stream);
+  return launch<false, false>(p, a->kdim, stream);
 }
