@@ -124,6 +124,18 @@ def test_strong_decay_stays_finite(cuda, cell, eta):
 
 
 @pytest.mark.parametrize("cell", ["gla", "kda"])
+@pytest.mark.parametrize("gscale", [4.0, 40.0])
+def test_local_rqk_rotation_strong_decay(cuda, cell, gscale):
+    """The rotated A kernel under decay spreads that rule out the factorized diagonal block (its exact path runs) and
+    push the anchored operands toward zero: same criterion, nothing non-finite."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell, K=128, H=2, gscale=gscale, seed=2), 256)
+    out, _, qz, run = _go(cell, tensors, rot=signed_hadamard(128, 3))
+    zc.check(out, run, qz, f"{cell} local R_QK gscale={gscale}")
+
+
+@pytest.mark.parametrize("cell", ["gla", "kda"])
 @pytest.mark.parametrize("n,K", [(128, 64), (512, 64), (256, 128), (64, 128), (192, 128), (192, 64)])
 def test_local_rqk_rotation(cuda, cell, n, K):
     """R_QK on a diagonal-decay cell is local: only the anchored operands of the off-diagonal sub-blocks are rotated
