@@ -12,12 +12,13 @@
 // for both chunks.  The diagonal block factorizes the decay weight around the block's first row whenever the decay
 // spread inside the block allows it and then runs as an fp32 MFMA product; otherwise lane (i = lane & 15, j-group =
 // lane >> 4) accumulates four (i, j) pairs with one exponential per (i, j, channel).
-// Without a rotation the wave of sub-block I (row-wise) builds its anchored query operand and the key operand of
-// every earlier sub-block from plain K-contiguous global loads, 16 INT8 slots per lane (no LDS).
+// Column-wise: the wave of sub-block J fetches its own rows once, hands its anchored query codes to the other waves
+// through LDS and builds its key operand once per later sub-block I (anchored at I's first row), meeting I's query codes
+// from LDS on the INT8 MFMA; a lane's 16 INT8 slots per contraction step hold the same channels in the query and the key
+// operand, so the dot product is exact whatever the channel -> slot map.
 // With a local R_QK (rot, (K,K) fp16, x -> x.R) the anchored off-diagonal operands are rounded to fp16 and rotated
-// on the fp16 MFMA before quantization (gla.py:53-57); the diagonal blocks are not rotated.  That path is column-wise:
-// the wave of sub-block J fetches its own rows once, hands its anchored query codes to the other waves through LDS and
-// builds its key operand once per later sub-block I (anchored at I's first row), meeting I's query codes from LDS.
+// on the fp16 MFMA before quantization (gla.py:53-57); without one they are quantized as they are built.  The diagonal
+// blocks are never rotated.
 #include <type_traits>
 
 #include "zoo_common.h"
@@ -87,62 +88,14 @@ LQ_DEV void diag_exact(const AParams& p, float sq, float sk, float inv_sq, float
   }
 }
 
-// Diagonal 16x16 block of one wave (rows row0 .. row0+15), written to A[row][i0 + j].
-//   A[i][j] = sum_n qh[i][n] kh[j][n] exp(g[i][n] - g[j][n]),  j <= i,  qh / kh the dequantized codes.
-// When the decay spread inside the block is small (every |g[r][n] - g[first][n]| <= 40) the weight factorizes
-// safely around the first row: the operands qh*exp(g_i - a) and kh*exp(a - g_j) stay normal fp32 numbers and
-// the sum is an fp32 16x16xK matrix product (lane (rl, kg) owns K/4 contiguous channels of token rl).
-// Otherwise every (i, j, n) weight is evaluated on its own, masked before use, as the reference does.
-template <int K, bool BF>
-LQ_DEV void diag_block(const AParams& p, float sq, float sk, float inv_sq, float inv_sk, int rl, int kg, int64_t row0, int h,
-                       int i0) {
-  constexpr int NCH = K / 4;
-  const int H = p.H, qmax = p.qmax;
-  constexpr bool bf = BF;
-  const int c0 = NCH * kg;
-  const int64_t off = ((row0 + rl) * H + h) * K + c0;
-  const int64_t aoff = (row0 * H + h) * K + c0;
-  // The factorized product is formed while the spread is still being measured (no arrays of operands stay live); when
-  // the spread turns out too large its result is dropped (overflowed operands are harmless there) and the exact path
-  // below runs instead.
-  float spread = 0.0f;
-  lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int e8 = 0; e8 < NCH / 8; ++e8) {
-    const lq_v4f g0 = *(const lq_v4f*)(p.g + off + 8 * e8), g1 = *(const lq_v4f*)(p.g + off + 8 * e8 + 4);
-    const lq_v4f a0 = *(const lq_v4f*)(p.g + aoff + 8 * e8), a1 = *(const lq_v4f*)(p.g + aoff + 8 * e8 + 4);
-    float qv[8];
-    zoo_ld8(p.q + off + 8 * e8, bf, qv);
-    float kv[8];
-    zoo_ld8(p.k + off + 8 * e8, bf, kv);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float d = (e < 4 ? g0[e & 3] : g1[e & 3]) - (e < 4 ? a0[e & 3] : a1[e & 3]);
-      spread = fmaxf(spread, __builtin_fabsf(d));
-      const float qh = (float)zoo_q8(qv[e] * p.scale, inv_sq, qmax) * sq;
-      const float kh = (float)zoo_q8(kv[e], inv_sk, qmax) * sk;
-      acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * zoo_exp(d), kh * zoo_exp(-d), acc, 0, 0, 0);
-    }
-  }
-  spread = wave_max(spread);
-  if (spread <= 40.0f) {
-    // lane holds column j = rl, rows i = 4kg + r
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      p.A[((row0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((rl <= 4 * kg + r) ? acc[r] : 0.0f);
-    return;
-  }
-  diag_exact<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, row0, h, i0);
-}
-
-// QG (rotated path only): the state-read codes are wanted (p.qg is set); a compile-time flag keeps the own-rows loop
+// QG: the state-read codes are wanted (p.qg is set); a compile-time flag keeps the own-rows loop
 // one basic block.
 template <int K, bool ROT, bool BF, bool QG>
 __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   constexpr int RS = K + 8;  // halves per row of the transposed rotation
   __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
   // rotated query codes of sub-blocks 1..3 of both chunks: [pass][I - 1][lane][dword]
-  __shared__ __align__(16) uint32_t QC[ROT ? 2 * 3 * 64 * (K / 16) : 4];
+  __shared__ __align__(16) uint32_t QC[2 * 3 * 64 * (K / 16)];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -173,8 +126,8 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   const int i0 = 16 * blk;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
 
-  if constexpr (ROT) {
-    // ---- local R_QK: column-wise.  The wave loads its own sub-block (q, k, g rows) once, in the layout of the rotation
+  {
+    // ---- The wave loads its own sub-block (q, k, g rows) once, in the layout of the rotation
     // operand (lane (rl, kg) = token rl, channels 32ks + 8kg + e), and takes everything that needs those rows from
     // the registers: the state-read codes q*exp(g)*scale, the diagonal block, the query operand anchored at this
     // sub-block's first row (rotated, quantized, handed to the other waves through LDS) and the key operands anchored
@@ -183,7 +136,7 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
     // which it packs as dword mt of its INT8 operand; q and k operands share that channel -> slot map, so the INT8
     // dot is exact and a consumer lane needs exactly the dwords the same lane of the producer wave holds.
     constexpr int KS = K / 32, MT = K / 16;
-    if (pass == 0) __syncthreads();  // R^T staged
+    if (ROT && pass == 0) __syncthreads();  // R^T staged
     const int64_t roff = ((t0 + i0 + rl) * H + h) * K + 8 * kg;
     // One step (32 channels, 8 per lane) of raw operands: own rows of q / k / g and the first rows of g of two
     // sub-blocks (anchors; the address stays inside the chunk for every sub-block <= 3).  Steps are requested one ahead
@@ -208,7 +161,8 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
     };
     // key rows of this sub-block anchored at the first rows of sub-blocks Ia and Ib, as fp16 rotation operands (the
     // rows are fetched again here rather than held in registers across the first sweep: they are cache hits)
-    auto build_k2 = [&](int Ia, int Ib, lq_v8h (&xa)[KS], lq_v8h (&xb)[KS]) {
+    // (without a rotation they are quantized on the spot into ca / cb)
+    auto build_k2 = [&](int Ia, int Ib, lq_v8h (&xa)[KS], lq_v8h (&xb)[KS], uint32_t (&ca)[MT], uint32_t (&cb)[MT]) {
       Step st[2];
       request(std::false_type{}, Ia, Ib, 0, st[0]);
 #pragma unroll
@@ -217,11 +171,23 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
         const Step& r = st[ks & 1];
         float kf[8];
         unpack(r.k, kf);
+        int ia[8], ib[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float gg = r.g[e >> 2][e & 3];
-          xa[ks][e] = (_Float16)(kf[e] * zoo_exp(r.a[e >> 2][e & 3] - gg));
-          xb[ks][e] = (_Float16)(kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg));
+          const float va = kf[e] * zoo_exp(r.a[e >> 2][e & 3] - gg), vb = kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg);
+          if constexpr (ROT) {
+            xa[ks][e] = (_Float16)va, xb[ks][e] = (_Float16)vb;
+          } else {
+            ia[e] = zoo_q8(va, inv_sk, qmax), ib[e] = zoo_q8(vb, inv_sk, qmax);
+          }
+        }
+        if constexpr (!ROT) {
+          ca[2 * ks] = zoo_pack_codes(ia[0], ia[1], ia[2], ia[3]), ca[2 * ks + 1] = zoo_pack_codes(ia[4], ia[5], ia[6], ia[7]);
+          cb[2 * ks] = zoo_pack_codes(ib[0], ib[1], ib[2], ib[3]), cb[2 * ks + 1] = zoo_pack_codes(ib[4], ib[5], ib[6], ib[7]);
+          // the codes are next used after the loop: without this anchor their arithmetic sinks there and every step's
+          // raw operands stay in registers
+          asm volatile("" : "+v"(ca[2 * ks]), "+v"(ca[2 * ks + 1]), "+v"(cb[2 * ks]), "+v"(cb[2 * ks + 1]));
         }
         __builtin_amdgcn_sched_barrier(0);  // keeps the look-ahead at one step
       }
@@ -267,6 +233,7 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
     // own rows, fetched once: state-read codes, diagonal block (factorized around the first row while the spread is
     // measured) and the two operands of the first sweep
     lq_v8h xq[KS], xk[KS];
+    uint32_t cq[MT], ck[MT];
     float spread = 0.0f;
     lq_v4f dacc = {0.f, 0.f, 0.f, 0.f};
     const int inext = blk < 3 ? blk + 1 : 3;
@@ -279,7 +246,7 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
       float qf[8], kf[8];
       unpack(r.q, qf);
       unpack(r.k, kf);
-      int cs[8];
+      int cs[8], iq[8], ik[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float gg = r.g[e >> 2][e & 3];
@@ -291,8 +258,12 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
         dacc = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * ed, kh * zoo_exp(-d), dacc, 0, 0, 0);
         float x = qf[e] * ed;
         x = x * p.scale;
-        xq[ks][e] = (_Float16)x;
-        xk[ks][e] = (_Float16)(kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg));
+        const float xn = kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg);
+        if constexpr (ROT) {
+          xq[ks][e] = (_Float16)x, xk[ks][e] = (_Float16)xn;
+        } else {
+          iq[e] = zoo_q8(x, inv_sq, qmax), ik[e] = zoo_q8(xn, inv_sk, qmax);
+        }
         float y = qf[e] * zoo_exp(gg);
         y = y * p.scale;
         cs[e] = zoo_q8(y, inv_sq, qmax);
@@ -303,12 +274,16 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
         o[1] = (int)zoo_pack_codes(cs[4], cs[5], cs[6], cs[7]);
         *(lq_v2i*)(p.qg + roff + 32 * ks) = o;
       }
+      if constexpr (!ROT) {
+        cq[2 * ks] = zoo_pack_codes(iq[0], iq[1], iq[2], iq[3]), cq[2 * ks + 1] = zoo_pack_codes(iq[4], iq[5], iq[6], iq[7]);
+        ck[2 * ks] = zoo_pack_codes(ik[0], ik[1], ik[2], ik[3]), ck[2 * ks + 1] = zoo_pack_codes(ik[4], ik[5], ik[6], ik[7]);
+        asm volatile("" : "+v"(cq[2 * ks]), "+v"(cq[2 * ks + 1]), "+v"(ck[2 * ks]), "+v"(ck[2 * ks + 1]));  // as in build_k2
+      }
       __builtin_amdgcn_sched_barrier(0);  // keeps the look-ahead at one step
     }
     // first sweep: query operand of this sub-block (none for sub-block 0) and key operand for sub-block blk + 1 (none
     // for sub-block 3)
-    uint32_t cq[MT], ck[MT];
-    sweep(std::true_type{}, xq, xk, inv_sq, inv_sk, cq, ck);  // sub-block 0 has no use for cq, sub-block 3 none for ck
+    if constexpr (ROT) sweep(std::true_type{}, xq, xk, inv_sq, inv_sk, cq, ck);  // sub-block 0 has no use for cq, sub-block 3 none for ck
     if (blk > 0) {
       uint32_t* qc = QC + (((pass * 3 + blk - 1) * 64 + lane) * MT);
 #pragma unroll
@@ -323,8 +298,8 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
     if (blk < 3) meet(blk + 1, ck);
     // second sweep: key operands for sub-blocks blk + 2 and blk + 3
     if (blk <= 1) {
-      build_k2(2, 3, xq, xk);
-      sweep(std::true_type{}, xq, xk, inv_sk, inv_sk, cq, ck);
+      build_k2(2, 3, xq, xk, cq, ck);
+      if constexpr (ROT) sweep(std::true_type{}, xq, xk, inv_sk, inv_sk, cq, ck);
       if (blk == 0) meet(2, cq);
       meet(3, ck);
     }
@@ -337,110 +312,6 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
         p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((rl <= 4 * kg + r) ? dacc[r] : 0.0f);
     } else {
       diag_exact<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
-    }
-  } else {
-    // ---- state-read operand of the output kernel: codes of q * exp(g) * scale
-    if (p.qg) {
-      for (int it = tid; it < 64 * (K / 8); it += 256) {
-        const int t = it / (K / 8), c8 = it % (K / 8);
-        const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
-        float qv[8];
-        zoo_ld8(p.q + off, bf, qv);
-        const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
-        int cq[8];
-  #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float x = qv[e] * zoo_exp(e < 4 ? g0[e & 3] : g1[e & 3]);
-          x = x * p.scale;
-          cq[e] = zoo_q8(x, inv_sq, qmax);
-        }
-        lq_v2i o;
-        o[0] = (int)zoo_pack_codes(cq[0], cq[1], cq[2], cq[3]);
-        o[1] = (int)zoo_pack_codes(cq[4], cq[5], cq[6], cq[7]);
-        *(lq_v2i*)(p.qg + off) = o;
-      }
-    }
-
-    diag_block<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
-
-    lq_v4i acc[3];
-  #pragma unroll
-    for (int J = 0; J < 3; ++J) acc[J] = lq_v4i{0, 0, 0, 0};
-
-    {
-      // ---- off-diagonal blocks J < blk: INT8 MFMA on anchored operands built from plain global loads
-      if (blk > 0) {
-  #pragma unroll
-        for (int ks = 0; ks < K / 64; ++ks) {
-          const int kk = 64 * ks + 16 * kg;
-          float an[16];
-          {
-            const float* ap = p.g + ((t0 + i0) * H + h) * K + kk;
-  #pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-              const lq_v4f a4 = *(const lq_v4f*)(ap + 4 * e4);
-  #pragma unroll
-              for (int e = 0; e < 4; ++e) an[4 * e4 + e] = a4[e];
-            }
-          }
-          lq_v4i qop;
-          {
-            const int64_t off = ((t0 + i0 + rl) * H + h) * K + kk;
-            float q0[8];
-            zoo_ld8(p.q + off, bf, q0);
-            float q1[8];
-            zoo_ld8(p.q + off + 8, bf, q1);
-            int cd[16];
-  #pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-              const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
-  #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int n = 4 * e4 + e;
-                const float qf = n < 8 ? q0[n & 7] : q1[n & 7];
-                float x = qf * zoo_exp(g4[e] - an[n]);
-                x = x * p.scale;
-                cd[n] = zoo_q8(x, inv_sq, qmax);
-              }
-            }
-  #pragma unroll
-            for (int d = 0; d < 4; ++d) qop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
-          }
-  #pragma unroll
-          for (int J = 0; J < 3; ++J) {
-            if (J >= blk) continue;
-            const int64_t off = ((t0 + 16 * J + rl) * H + h) * K + kk;
-            float k0[8];
-            zoo_ld8(p.k + off, bf, k0);
-            float k1[8];
-            zoo_ld8(p.k + off + 8, bf, k1);
-            int cd[16];
-  #pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-              const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
-  #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int n = 4 * e4 + e;
-                const float kf = n < 8 ? k0[n & 7] : k1[n & 7];
-                cd[n] = zoo_q8(kf * zoo_exp(an[n] - g4[e]), inv_sk, qmax);
-              }
-            }
-            lq_v4i kop;
-  #pragma unroll
-            for (int d = 0; d < 4; ++d) kop[d] = (int)zoo_pack_codes(cd[4 * d], cd[4 * d + 1], cd[4 * d + 2], cd[4 * d + 3]);
-            acc[J] = lq_mfma_i8(qop, kop, acc[J]);
-          }
-        }
-      }
-    }
-
-    const float sqk = sq * sk;
-  #pragma unroll
-    for (int J = 0; J < 3; ++J) {
-      if (J >= blk) continue;
-  #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + 16 * J + rl] = (_Float16)((float)acc[J][r] * sqk);
     }
   }
   // zero blocks above the diagonal
@@ -481,6 +352,8 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
       LQ_A_LAUNCH2(KV, true, true);     \
     else if (a->rot)                    \
       LQ_A_LAUNCH2(KV, true, false);    \
+    else if (p.qg)                      \
+      LQ_A_LAUNCH2(KV, false, true);    \
     else                                \
       LQ_A_LAUNCH2(KV, false, false);   \
   } while (0)
