@@ -72,10 +72,14 @@ struct UStepOps {
   float fw, ev;
 };
 
-template <bool DELTA, int K, int V>
+// KP: workgroups per (batch, head) along K.  The key rows of the linear family are independent recurrences, so a
+// workgroup may own K / KP of them (the delta family reads the whole state per step: KP = 1).
+template <bool DELTA, int K, int V, int KP>
 __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) {
-  constexpr int KR = K / 4, KT = KR / 16, VT = V / 16;
-  constexpr int HS = K + 16, ES = 64 + 16, RS = V + 8;
+  static_assert(KP == 1 || !DELTA, "the delta family needs all of K in one workgroup");
+  constexpr int KW = K / KP, KR = KW / 4, KT = KR / 16, VT = V / 16;
+  static_assert(KT >= 1, "a wave owns at least one 16-row tile");
+  constexpr int HS = KW + 16, ES = 64 + 16, RS = V + 8;
   __shared__ __align__(16) unsigned char hT[V * HS];
   __shared__ __align__(16) unsigned char eT[DELTA ? V * ES : 16];
   __shared__ __align__(16) _Float16 RuT_s[V * RS];          // RuT_s[v'][v] = Ru[v][v']: x . Ru
@@ -85,6 +89,7 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
   const int b = blockIdx.x / p.H, h = blockIdx.x % p.H;
+  const int kb = blockIdx.y * KW;  // first key row of this workgroup
   const int H = p.H, T = p.T, NT = p.NT;
   const int qmax = p.qmax;
   const bool bf = p.bf != 0;
@@ -97,7 +102,7 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
   }
   float skw_c[KT];
 #pragma unroll
-  for (int kt = 0; kt < KT; ++kt) skw_c[kt] = p.skw[h * K + KR * wave + 16 * kt + rl];
+  for (int kt = 0; kt < KT; ++kt) skw_c[kt] = p.skw[h * K + kb + KR * wave + 16 * kt + rl];
   const float sw = DELTA ? p.sw[h] : 0.0f;
 
   auto load_step = [&](int ct, UStepOps<DELTA, K, V>& o) {
@@ -105,8 +110,8 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
-      o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + KR * wave + 16 * kt + rl) * 64 + 16 * kg);
-      o.gam[kt] = p.gam[cb * K + KR * wave + 16 * kt + rl];
+      o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + kb + KR * wave + 16 * kt + rl) * 64 + 16 * kg);
+      o.gam[kt] = p.gam[cb * K + kb + KR * wave + 16 * kt + rl];
     }
     if constexpr (!DELTA) {
 #pragma unroll
@@ -151,8 +156,8 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
     if (ct + 1 < NT) load_step(ct + 1, nxt);
     __syncthreads();
     {
-      int8_t* dst = p.h_i8 + (((int64_t)b * NT + ct) * H + h) * V * K;
-      constexpr int SEG = K / 16;
+      int8_t* dst = p.h_i8 + (((int64_t)b * NT + ct) * H + h) * V * K + kb;
+      constexpr int SEG = KW / 16;
       for (int it = tid; it < V * SEG; it += 256) {
         const int vr = it / SEG, sg = it % SEG;
         *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hT + vr * HS + sg * 16);
@@ -230,7 +235,7 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
     for (int vt = 0; vt < VT; ++vt)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
-        *(lq_v4f*)(p.ht + (((int64_t)b * H + h) * K + KR * wave + 16 * kt + rl) * V + 16 * vt + 4 * kg) =
+        *(lq_v4f*)(p.ht + (((int64_t)b * H + h) * K + kb + KR * wave + 16 * kt + rl) * V + 16 * vt + 4 * kg) =
             lq_v4f{hc[vt][kt][0], hc[vt][kt][1], hc[vt][kt][2], hc[vt][kt][3]};
   }
 }
@@ -410,11 +415,12 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
 
 template <bool DELTA, int K>
 int launch_state(const ZooStateParams& p, int batch, hipStream_t stream) {
-  dim3 grid(batch * p.H);
+  constexpr int KP = (!DELTA && K == 128) ? 2 : 1;
+  dim3 grid(batch * p.H, KP);
   if (p.V == 128)
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP>), grid, dim3(256), 0, stream, p);
   return lq_check_launch();
 }
 

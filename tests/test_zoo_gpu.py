@@ -149,7 +149,7 @@ def test_local_rqk_rotation(cuda, cell, n, K):
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))
-@pytest.mark.parametrize("n,K,V", [(128, 64, 128), (512, 64, 128), (256, 128, 64)])
+@pytest.mark.parametrize("n,K,V", [(128, 64, 128), (512, 64, 128), (256, 128, 64), (256, 128, 128)])
 def test_canonical_storage_rv(cuda, cell, n, K, V):
     """R_V with canonical storage: v rotated outside, every product un-rotated in-kernel before it joins the fp32
     carry / the output (/root/reference tests/test_kernel_simple_gla.py:84-104, test_kernel_gla.py:63-75)."""
