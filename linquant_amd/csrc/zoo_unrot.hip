@@ -265,6 +265,18 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
   const int qmax = p.qmax;
   const bool bf = p.bf != 0;
 
+  // state-read operands (and the stored query codes) are requested first: they are not needed before phase 2 and
+  // arrive while phase 1 stages the codes
+  const int8_t* hp = p.h_i8 + (((int64_t)b * p.NT + ct) * H + h) * V * K;
+  lq_v4i hop[K / 64][VT];
+  lq_v4i qgop[GLA ? K / 64 : 1];
+#pragma unroll
+  for (int ks = 0; ks < K / 64; ++ks) {
+    if constexpr (GLA) qgop[ks] = *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
+#pragma unroll
+    for (int vt = 0; vt < VT; ++vt) hop[ks][vt] = *(const lq_v4i*)(hp + (16 * vt + rl) * K + 64 * ks + 16 * kg);
+  }
+
   // ---- phase 1: codes and tables -> LDS
   stage_rotation<V, true>(RuT_s, p.unrot, tid);
   if (tid < V) ss_s[tid] = p.ss[h * V + tid], svl_s[tid] = p.svl[h * V + tid];
@@ -299,10 +311,11 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
     zoo_ld8(p.v + off, bf, va);
     float vb[8];
     zoo_ld8(p.v + off + (int64_t)H * V, bf, vb);
+    const lq_v4f s0 = *(const lq_v4f*)(p.svl + h * V + 8 * c8), s1 = *(const lq_v4f*)(p.svl + h * V + 8 * c8 + 4);
     lq_v4i o0, o1;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const float inv = 1.0f / p.svl[h * V + 8 * c8 + e];
+      const float inv = 1.0f / (e < 4 ? s0[e & 3] : s1[e & 3]);
       const int w = (int)zoo_pack_h2((float)zoo_q8(va[e], inv, qmax), (float)zoo_q8(vb[e], inv, qmax));
       if (e < 4) o0[e] = w; else o1[e - 4] = w;
     }
@@ -319,14 +332,15 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
   lq_v4i a32[4];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
-  const int8_t* hp = p.h_i8 + (((int64_t)b * p.NT + ct) * H + h) * V * K;
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
-    const lq_v4i qop = GLA ? *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg)
-                           : *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+    lq_v4i qop;
+    if constexpr (GLA)
+      qop = qgop[ks];
+    else
+      qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
 #pragma unroll
-    for (int vt = 0; vt < VT; ++vt)
-      o32[vt] = lq_mfma_i8(*(const lq_v4i*)(hp + (16 * vt + rl) * K + 64 * ks + 16 * kg), qop, o32[vt]);
+    for (int vt = 0; vt < VT; ++vt) o32[vt] = lq_mfma_i8(hop[ks][vt], qop, o32[vt]);
     if (!GLA) {
 #pragma unroll
       for (int jt = 0; jt < 4; ++jt) {
