@@ -24,6 +24,24 @@ __global__ __launch_bounds__(256) void cumsum_scalar_kernel(const float* __restr
   }
 }
 
+// The same scan for the chunk size every caller uses: all 64 values of a thread are requested before the first is added
+// (the loop above waits for each load in turn: 64 round trips), summed in the same order.
+__global__ __launch_bounds__(256) void cumsum_scalar64_kernel(const float* __restrict__ g, float* __restrict__ gc, int H,
+                                                              int64_t total) {
+  const int64_t idx = min((int64_t)blockIdx.x * 256 + threadIdx.x, total - 1);  // (b, chunk, h); the tail repeats the last
+  const int h = idx % H;
+  const int64_t base = (idx / H) * 64 * H + h;
+  float v[64];
+#pragma unroll
+  for (int t = 0; t < 64; ++t) v[t] = g[base + (int64_t)t * H];
+  double run = 0.0;
+#pragma unroll
+  for (int t = 0; t < 64; ++t) {
+    run += (double)v[t];
+    gc[base + (int64_t)t * H] = (float)run;
+  }
+}
+
 // one workgroup per (batch, chunk, head); 4*K threads: thread (k, q) scans tokens q*C/4 .. of channel k (all of its
 // loads are independent and issued up front), the four partial totals are combined through LDS; LDS tile [C][K+1]
 // for the envelope reduction
@@ -91,8 +109,12 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
   const int NT = a->seqlen / a->chunk_size;
   if (a->kdim == 0) {
     const int64_t total = (int64_t)a->batch * NT * a->nheads;
-    hipLaunchKernelGGL(cumsum_scalar_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g, a->gc,
-                       a->seqlen, a->nheads, a->chunk_size, total);
+    if (a->chunk_size == 64)
+      hipLaunchKernelGGL(cumsum_scalar64_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g, a->gc,
+                         a->nheads, total);
+    else
+      hipLaunchKernelGGL(cumsum_scalar_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g, a->gc,
+                         a->seqlen, a->nheads, a->chunk_size, total);
   } else {
     if (!a->logenv) return LQ_ERR_NULL;
     if (a->kdim > 256 || a->kdim % 16 != 0 || a->chunk_size % 16 != 0 || a->chunk_size > 64) return LQ_ERR_SHAPE;
