@@ -13,7 +13,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 HEADER = ROOT.parent / "include" / "linquant_hip.h"
 LIB_PATH = ROOT / "csrc" / "liblinquant_hip.so"
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 LQ_DT_F16, LQ_DT_F32, LQ_DT_I8, LQ_DT_BF16 = 0, 1, 2, 3
 
@@ -90,6 +90,14 @@ def load():
 def ptr(t):
     """Device pointer of a torch tensor (None -> NULL)."""
     return None if t is None else t.data_ptr()
+
+
+def f32(t):
+    """``t`` itself when it is fp32 (or None), else an fp32 copy: the kernels read scale tensors as fp32, where the
+    reference's kernels convert on load, so an fp16 / fp64 scale buffer must not be reinterpreted."""
+    import torch
+
+    return t if t is None or t.dtype == torch.float32 else t.float()
 
 
 def aligned(t, nbytes=16):

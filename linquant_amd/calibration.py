@@ -47,20 +47,21 @@ def hadamard(n: int, device=None, dtype=torch.float32) -> torch.Tensor:
     return H / math.sqrt(n)
 
 
-def mamba2_synthetic(shape: Mamba2Shape, seed: int, device="cpu"):
-    """Seeded synthetic activations of one Mamba-2 SSD layer: xBC ~ N(0,1) fp16, raw dt ~ N(-2, 0.5) fp16
-    (softplus applied in-kernel), drawn on the CPU generator in this order then moved to ``device``."""
+def mamba2_synthetic(shape: Mamba2Shape, seed: int, device="cpu", dt_mean: float = -2.0):
+    """Seeded synthetic activations of one Mamba-2 SSD layer: xBC ~ N(0,1) fp16, raw dt ~ N(dt_mean, 0.5) fp16
+    (softplus applied in-kernel), drawn on the CPU generator in this order then moved to ``device``.  The default
+    dt_mean = -2 gives dt ~ 0.13; -4.5 gives the weak-decay regime dt ~ 0.011 of trained Mamba-2 layers."""
     g = torch.Generator().manual_seed(seed)
     xBC = torch.randn(shape.batch, shape.seqlen, shape.xbc_dim, generator=g).to(torch.float16)
-    dt_raw = (torch.randn(shape.batch, shape.seqlen, shape.nheads, generator=g) * 0.5 - 2.0).to(torch.float16)
+    dt_raw = (torch.randn(shape.batch, shape.seqlen, shape.nheads, generator=g) * 0.5 + dt_mean).to(torch.float16)
     return xBC.to(device), dt_raw.to(device)
 
 
-def mamba2_params(shape: Mamba2Shape, seed: int, device="cpu"):
-    """Per-layer parameters: A = -exp(U(log 1, log 16)) as INT8 A_log codes, D ~ N(0,1) as INT8 codes, zero
+def mamba2_params(shape: Mamba2Shape, seed: int, device="cpu", a_max: float = 16.0):
+    """Per-layer parameters: A = -exp(U(log 1, log a_max)) as INT8 A_log codes, D ~ N(0,1) as INT8 codes, zero
     dt_bias, +-1 rotation signs (G,N)."""
     g = torch.Generator().manual_seed(seed)
-    a_log = torch.rand(shape.nheads, generator=g) * math.log(16.0)
+    a_log = torch.rand(shape.nheads, generator=g) * math.log(a_max)
     D = torch.randn(shape.nheads, generator=g)
     signs = (torch.randint(0, 2, (shape.ngroups, shape.dstate), generator=g) * 2 - 1).to(torch.float32)
     A_log_scale = (a_log.abs().amax() / 127.0).clamp_min(1e-8)
@@ -190,3 +191,43 @@ class AbsmaxCollector:
         for role, a in self.absmax.items():
             out[role] = (a / qmax).clamp_min(1e-12)
         return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Zoo cells: synthetic inputs of the benchmark configurations and the diagonal q/k rescaling D_QK.
+# ---------------------------------------------------------------------------------------------------------------
+ZOO_CELLS = {"linear_none": ("linear", "none"), "mamba2": ("linear", "scalar"), "gla": ("linear", "diagonal"),
+             "deltanet": ("delta", "none"), "gated_deltanet": ("delta", "scalar"), "kda": ("delta", "diagonal")}
+
+
+def zoo_synthetic(cell: str, B: int, T: int, H: int, K: int, V: int, seed: int):
+    """Seeded fp32 CPU inputs (q, k, v, g, beta) of one zoo cell in the benchmark recipes: q, v ~ N(0,1); k ~ N(0,1),
+    L2-normalized for the delta family; beta = sigmoid(N(0,1)); log decay g = logsigmoid(N(0,1)) / 16 per channel (GLA),
+    logsigmoid(N(1,1)) per channel (KDA), logsigmoid(N(2,1)) per head (Gated DeltaNet), -softplus(N(-2,0.5)) * A with
+    A = exp(U(0, log 16)) (the Mamba-2 cell).  Draw order: q, k, v, beta, g."""
+    fam, dec = ZOO_CELLS[cell]
+    gen = torch.Generator().manual_seed(seed)
+    rn = lambda *shape: torch.randn(*shape, generator=gen)  # noqa: E731
+    q, k = rn(B, T, H, K), rn(B, T, H, K)
+    if fam == "delta":
+        k = Fn.normalize(k, dim=-1)
+    v = rn(B, T, H, V)
+    beta = torch.sigmoid(rn(B, T, H)) if fam == "delta" else None
+    g = None
+    if cell == "gla":
+        g = Fn.logsigmoid(rn(B, T, H, K)) / 16
+    elif cell == "kda":
+        g = Fn.logsigmoid(rn(B, T, H, K) + 1.0)
+    elif cell == "gated_deltanet":
+        g = Fn.logsigmoid(rn(B, T, H) + 2.0)
+    elif cell == "mamba2":
+        g = -Fn.softplus(rn(B, T, H) * 0.5 - 2.0) * torch.exp(torch.rand(H, generator=gen) * 2.77)
+    return q, k, v, (None if g is None else g.float()), beta
+
+
+def dqk_from_absmax(q: torch.Tensor, k: torch.Tensor, alpha: float = 0.5) -> torch.Tensor:
+    """Diagonal rescaling D_QK per (H, K) from a calibration batch: D = (max|k| / max|q|)^alpha with the maxima over
+    batch and tokens, clamped at 1e-8; applied as q' = q * D, k' = k / D (linquant/harness.py:68-88)."""
+    aq = q.detach().abs().amax(dim=(0, 1)).double().clamp_min(1e-8)
+    ak = k.detach().abs().amax(dim=(0, 1)).double().clamp_min(1e-8)
+    return ((ak / aq) ** alpha).float()

@@ -11,7 +11,8 @@
 // x[2kp+1][p]}), four token pairs of a channel adjacent, so that an fp16 MFMA operand (8 tokens of one channel) is one
 // 16-byte LDS read:
 //   xP : x as stored
-//   xS : x[k] * exp(dA_e(k) - dA_k) * S_cb * dt_k, where e(k) is the last token of k's 32-token slab.
+//   xS : x[k] * exp(dA_e(k) - dA_k) * S_cb * dt_k * 2^-kf, where e(k) is the last token of k's 32-token slab and
+//        2^kf is the power-of-two part of S_cb (returned by the row factor).
 // For 32-token slabs strictly before a wave's rows the causal weight factors as
 //   exp(dA_m - dA_k) = exp(dA_m - dA_E) * exp(dA_E - dA_e) * exp(dA_e - dA_k),   all exponents <= 0,
 // (E = last token before the tile's own 32-token slab), so those slabs need no per-element exponential: the B operand is
@@ -56,14 +57,17 @@ struct ScanParams {
 
 LQ_DEV float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// 4 int8 codes (one dword) -> 4 exact fp16 values as two packed dwords: 0x6400 | (b ^ 0x80) is 1024 + (b + 128).
-// With (s2, o2) = (s, -1152 s) the result is s * code (one packed fma: exact for s = 1, fp16-rounded otherwise).
-LQ_DEV void i8x4_to_f16x4(uint32_t w, lq_v2h s2, lq_v2h o2, uint32_t& lo, uint32_t& hi) {
+// 4 int8 codes (one dword) -> fp16(code * s) as two packed dwords: 0x6400 | (b ^ 0x80) is 1024 + (b + 128), from which
+// 1152 is subtracted exactly (the code itself, exact in fp16) before the one rounded multiply by s.  Folding the bias
+// into a fused multiply-add as (1152 + code) * s - fp16(1152 s) would shift every weight of the slab by the rounding
+// error of fp16(1152 s), up to half a code step: a bias, not noise.
+LQ_DEV void i8x4_to_f16x4(uint32_t w, lq_v2h s2, uint32_t& lo, uint32_t& hi) {
   const uint32_t u = w ^ 0x80808080u;
   const uint32_t a = __builtin_amdgcn_perm(0x64646464u, u, 0x05010400u);
   const uint32_t b = __builtin_amdgcn_perm(0x64646464u, u, 0x05030402u);
-  lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(lq_v2h, a), s2, o2));
-  hi = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(lq_v2h, b), s2, o2));
+  const lq_v2h bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+  lo = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(lq_v2h, a) - bias) * s2);
+  hi = __builtin_bit_cast(uint32_t, (__builtin_bit_cast(lq_v2h, b) - bias) * s2);
 }
 
 LQ_DEV uint32_t pack_h2(float a, float b) {
@@ -99,6 +103,9 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   const int limit = min(Q, p.seqlen - c * Q);
   const int64_t cs = (((int64_t)b * p.nheads + h) * p.nchunks + c) * Q;
   const float scb = p.cb_scale[g];
+  // power-of-two part of S_cb, as an exponent: kept out of the fp16 operand xS (whose values would drift into the
+  // fp16 subnormal range with a small S_cb) and returned in fp32 by the row factor of the off-diagonal slabs
+  const float kf = (float)(lq_clampi((__float_as_int(scb) >> 23) & 0xff, 2, 252) - 127);
 
   // Row tiles of this wave: 16w.. and 16(2*WAVES-1-w)..: an early and a late tile, so that every wave has the same
   // number of causal slabs to process.
@@ -201,7 +208,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   for (int it = 0; it < 2; ++it) {
     const int kp = kp_of[it], c8 = c8_of[it];
     const int k = 2 * kp, ke = (k | 31);
-    const float ae = dA2_s[ke];
+    const float ae = dA2_s[ke] - kf;
     const lq_v2h g2 = {(_Float16)(fexp2(ae - dA2_s[k]) * w_s[k]), (_Float16)(fexp2(ae - dA2_s[k + 1]) * w_s[k + 1])};
     const int base = (kp >> 2) * kQuad + (2 * c8) * 4 + (kp & 3);
     const bool in0 = k < limit, in1 = k + 1 < limit;
@@ -249,7 +256,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     };
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
-      if (s > 0 && s <= (WAVES - 1) / 2 && s == ne) flush(0, aE0);  // the early tile's slabs are done (wave-uniform)
+      if (s > 0 && s <= (WAVES - 1) / 2 && s == ne) flush(0, aE0 - kf);  // the early tile's slabs are done (wave-uniform)
       const bool late = s >= ne;
       const int J = late ? s - ne : s;
       const float aE = late ? aE1 : aE0;
@@ -257,21 +264,20 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       if (s + 4 < NS) cwr[s & 3] = cb_slab(s + 4);
       const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
       const lq_v2h s2 = {sh, sh};
-      const lq_v2h o2 = s2 * lq_v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
       lq_v4i xop[4];  // token pairs 16 J + 4 kg .. + 3 of channel 4 rl + j
 #pragma unroll
       for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xS + (4 * J + kg) * kQuad + (j * 16 + rl) * 4);
       lq_v4i aw;
       uint32_t lo, hi;
-      i8x4_to_f16x4((uint32_t)cw[0], s2, o2, lo, hi);
+      i8x4_to_f16x4((uint32_t)cw[0], s2, lo, hi);
       aw[0] = (int)lo, aw[1] = (int)hi;
-      i8x4_to_f16x4((uint32_t)cw[1], s2, o2, lo, hi);
+      i8x4_to_f16x4((uint32_t)cw[1], s2, lo, hi);
       aw[2] = (int)lo, aw[3] = (int)hi;
       const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
 #pragma unroll
       for (int j = 0; j < 4; ++j) off[j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[j]);
     }
-    if (NS > 0) flush(1, aE1);
+    if (NS > 0) flush(1, aE1 - kf);
   }
 
   // ---- each tile's own 32-token slab: per-element weights exp2(dA2_m - (dA2_k - log2(S_cb dt_k))), k <= m

@@ -182,6 +182,9 @@ extern "C" int lq_state_passing(const lq_state_passing_args* a, hipStream_t stre
   if (a->batch <= 0 || a->nheads <= 0 || a->nchunks <= 0 || a->dim <= 0) return LQ_ERR_SHAPE;
   if (a->batch > 65535 || a->nheads > 65535) return LQ_ERR_SHAPE;
   if (a->gate_shift < 0 || a->gate_shift > 15) return LQ_ERR_SHAPE;
+  // the running INT32 state is multiplied as a 24-bit quantity: with a gate of 127/128 or less (shift >= 7) it stays
+  // below 127 * 128; with fewer fractional bits the gate can be exactly 1 and the state grows by up to 127 per chunk
+  if (a->gate_shift < 7 && a->nchunks > 65536) return LQ_ERR_SHAPE;
   if (a->nchunks > 12288) return LQ_ERR_SHAPE;                      // gate table lives in LDS
 
   int vec = a->vec_hint;

@@ -19,7 +19,8 @@ def _quant_chunk_scan_fwd(cb_i8, x_fp, dt, dA_cumsum, q_C, C_scale, states, q_D,
     assert x_fp.dtype == torch.float16 and x_fp.stride(3) == 1, "x must be fp16 with unit headdim stride"
     assert q_C.dtype == torch.int8 and q_C.stride(3) == 1
     cb_i8, states = cb_i8.contiguous(), states.contiguous()
-    dt, dA_cumsum = dt.contiguous(), dA_cumsum.contiguous()
+    dt, dA_cumsum = _lib.f32(dt).contiguous(), _lib.f32(dA_cumsum).contiguous()
+    C_scale, cb_scale, state_dequant_scale = _lib.f32(C_scale), _lib.f32(cb_scale), _lib.f32(state_dequant_scale)
     out = torch.empty(batch, seqlen, nheads, headdim, device=dev, dtype=torch.float16)
     d_scale = None if q_D is None else _as_f32_scalar(D_scale, dev)
     if q_D is not None:

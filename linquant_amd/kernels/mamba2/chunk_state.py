@@ -16,7 +16,8 @@ def _quant_chunk_state_fwd_xfp_static_int8(x_fp, q_B, dt, dA_cumsum, alpha_hp, b
     batch, seqlen, nheads, headdim = x_fp.shape
     assert x_fp.dtype == torch.float16 and x_fp.stride(3) == 1, "x must be fp16 with unit headdim stride"
     assert q_B.dtype == torch.int8 and q_B.stride(3) == 1
-    dt, dA_cumsum = dt.contiguous(), dA_cumsum.contiguous()
+    dt, dA_cumsum = _lib.f32(dt).contiguous(), _lib.f32(dA_cumsum).contiguous()
+    alpha_hp, bscale_g, out_qscale = _lib.f32(alpha_hp), _lib.f32(bscale_g), _lib.f32(out_qscale)
     states = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x_fp.device, dtype=torch.int8)
     _lib.call("lq_chunk_state_value", x_fp.device,
               x=_lib.ptr(x_fp), x_stride_b=x_fp.stride(0), x_stride_l=x_fp.stride(1), x_stride_h=x_fp.stride(2),

@@ -21,8 +21,9 @@ def _chunk_state_keyside_fwd(x_fp, x_scale_hp, b_fp, dt, dA_cumsum, out_qscale, 
     batch, seqlen, nheads, headdim = x_fp.shape
     assert x_fp.dtype == torch.float16 and x_fp.stride(3) == 1, "x must be fp16 with unit headdim stride"
     assert b_fp.dtype == torch.float16 and b_fp.stride(3) == 1, "b_fp must be fp16 with unit dstate stride"
+    x_scale_hp, out_qscale, b_gate_scale = _lib.f32(x_scale_hp), _lib.f32(out_qscale), _lib.f32(b_gate_scale)
     bgs = _bgs_strides(b_gate_scale)
-    dt, dA_cumsum = dt.contiguous(), dA_cumsum.contiguous()
+    dt, dA_cumsum = _lib.f32(dt).contiguous(), _lib.f32(dA_cumsum).contiguous()
     states = torch.empty((batch, nchunks, nheads, headdim, dstate), device=x_fp.device, dtype=torch.int8)
     _lib.call("lq_chunk_state_key", x_fp.device,
               x=_lib.ptr(x_fp), x_stride_b=x_fp.stride(0), x_stride_l=x_fp.stride(1), x_stride_h=x_fp.stride(2),

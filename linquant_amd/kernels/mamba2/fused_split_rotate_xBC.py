@@ -51,7 +51,7 @@ def fused_split_rotate_quant_xBC(xBC, r_signs, nheads, ngroups, d_state, headdim
               xBC=_lib.ptr(xBC), xBC_stride_b=xBC.stride(0), xBC_stride_t=xBC.stride(1),
               qB=_lib.ptr(q_B), qC=_lib.ptr(q_C), b_fp=_lib.ptr(b_fp), signs=_lib.ptr(signs),
               signs_dtype=0 if signs is None else _SIGN_CODES[signs.dtype],
-              B_inv_scale=_lib.ptr(B_inv_scale), C_inv_scale=_lib.ptr(C_inv_scale),
+              B_inv_scale=_lib.ptr(_lib.f32(B_inv_scale)), C_inv_scale=_lib.ptr(_lib.f32(C_inv_scale)),
               dqk_b=_lib.ptr(dqk_b) if has_dqk else None, dqk_c=_lib.ptr(dqk_c) if has_dqk else None,
               batch=batch, seqlen=seq_len, d_ssm=d_ssm, ngroups=ngroups, dstate=d_state)
     if return_b_fp:

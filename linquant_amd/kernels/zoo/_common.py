@@ -87,6 +87,7 @@ def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, fa
     """``value`` is v (linear family) or U (delta family)."""
     c = write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay)
     state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile, unrot)
+    return c
 
 
 def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None, qg=None):
@@ -130,8 +131,13 @@ def out_buffer(v, out_dtype):
     return torch.empty(v.shape, dtype=dt, device=v.device)
 
 
-def export_debug(debug, h_i8, **extra):
-    """Optional hook for tests: the stored INT8 state in the reference's (B,NT,H,K,V) orientation."""
+def export_debug(debug, h_i8, codes=None, **extra):
+    """Optional hook for tests: the stored INT8 state in the reference's (B,NT,H,K,V) orientation and the INT8
+    operand codes of the pre-pass in token-major orientation (kq (B,T,H,K), vq (B,T,H,V), wq (B,T,H,K))."""
     if debug is not None:
         debug["h_i8"] = h_i8.transpose(-1, -2)
+        if codes is not None:
+            B, NT, H = codes["kqT"].shape[:3]
+            tok = lambda t: None if t is None else t.permute(0, 1, 4, 2, 3).reshape(B, NT * CHUNK, H, t.shape[3])  # noqa: E731
+            debug.update(kq=tok(codes["kqT"]), vq=tok(codes["vqT"]), wq=codes["wq"])
         debug.update(extra)

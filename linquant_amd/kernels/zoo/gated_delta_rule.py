@@ -35,8 +35,8 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
+    codes = C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
                 w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru)
     C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
-    C.export_debug(_debug, h_i8, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
+    C.export_debug(_debug, h_i8, codes, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return o, ht

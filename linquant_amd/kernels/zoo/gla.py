@@ -32,9 +32,9 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
+    codes = C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
                 C.DECAY_DIAGONAL, unrot=Ru)
     C.run_output(None, None, v, h_i8, None, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
-    C.export_debug(_debug, h_i8, A=A, g=gc, logenv=logenv)
+    C.export_debug(_debug, h_i8, codes, A=A, qg=qg, g=gc, logenv=logenv)
     return o, ht

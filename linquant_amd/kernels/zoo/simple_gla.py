@@ -32,7 +32,7 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
-    C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru)
+    codes = C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru)
     C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
-    C.export_debug(_debug, h_i8, g=gg)
+    C.export_debug(_debug, h_i8, codes, g=gg)
     return o, ht

@@ -57,6 +57,7 @@ class ZooQuantizer:
         self.calibrating, self.layer, self.disabled = False, 0, False
         self.absmax, self.scales = {}, {}
         self.trace = None  # optional list collecting the stored INT8 state codes of every chunk
+        self.code_trace = None  # optional dict role -> list of the INT8 operand codes of every call (one per chunk)
 
     @classmethod
     def kernel_profile(cls, policy="kernel_static", bits=8):
@@ -109,6 +110,8 @@ class ZooQuantizer:
             codes = self.round((x.float() * (1.0 / scale.float())).double())
         else:
             codes = self.round(x / scale)
+        if self.code_trace is not None:
+            self.code_trace.setdefault(role, []).append(codes.clamp(-qmax, qmax).to(torch.int8))
         return codes.clamp(-qmax, qmax) * scale
 
     def finalize(self):

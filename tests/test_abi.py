@@ -83,3 +83,24 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
     with pytest.raises(_lib.LinQuantHipError):
         _lib.load()
+
+
+def binding_example():
+    """The ctypes binding example of the integration notes (the fenced block that defines lq_state_passing_args), as
+    source text."""
+    text = (ROOT / "INTEGRATION.md").read_text()
+    blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
+    (block,) = [b for b in blocks if "class lq_state_passing_args" in b]
+    return block
+
+
+def test_documented_binding_example_matches_the_library(monkeypatch):
+    """The documented stub is executed as written: it loads the library by its in-tree path, checks the ABI version
+    and passes its own lq_args_size assertion; its struct has the header's field names in the header's order."""
+    monkeypatch.chdir(ROOT)
+    ns = {}
+    exec(compile(binding_example(), "binding_example", "exec"), ns)
+    st = ns["lq_state_passing_args"]
+    assert [n for n, _ in st._fields_] == [n for n, _ in _lib.STRUCTS["lq_state_passing_args"]._fields_]
+    assert ctypes.sizeof(st) == ctypes.sizeof(_lib.STRUCTS["lq_state_passing_args"])
+    assert callable(ns["_fixedpoint_state_passing_fwd"])

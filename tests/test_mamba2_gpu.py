@@ -40,15 +40,19 @@ def assert_close_out(got, ref, name, tol=1e-3):
 
 
 SHAPES = [
-    Mamba2Shape(batch=2, seqlen=512, nheads=4, headdim=64, dstate=128, ngroups=1, chunk=256),
-    Mamba2Shape(batch=1, seqlen=256, nheads=8, headdim=64, dstate=64, ngroups=2, chunk=64),
-    Mamba2Shape(batch=2, seqlen=384, nheads=2, headdim=128, dstate=128, ngroups=2, chunk=128),
+    (Mamba2Shape(batch=2, seqlen=512, nheads=4, headdim=64, dstate=128, ngroups=1, chunk=256), "strong"),
+    (Mamba2Shape(batch=1, seqlen=256, nheads=8, headdim=64, dstate=64, ngroups=2, chunk=64), "strong"),
+    (Mamba2Shape(batch=2, seqlen=384, nheads=2, headdim=128, dstate=128, ngroups=2, chunk=128), "strong"),
+    # weak decay (dt ~ 0.011, A ~ -1): the slab factors of the scan's off-diagonal path lie strictly inside (0, 1)
+    (Mamba2Shape(batch=1, seqlen=512, nheads=4, headdim=64, dstate=128, ngroups=1, chunk=256), "weak"),
+    (Mamba2Shape(batch=1, seqlen=384, nheads=2, headdim=64, dstate=64, ngroups=1, chunk=128), "weak"),
 ]
 
 
-@pytest.fixture(scope="module", params=range(len(SHAPES)))
+@pytest.fixture(scope="module", params=range(len(SHAPES)), ids=lambda i: f"{SHAPES[i][1]}{i}")
 def case(request):
-    c = build_case(SHAPES[request.param])
+    shape, regime = SHAPES[request.param]
+    c = build_case(shape, regime=regime)
     c["oracle"] = {False: oracle_pipeline(c, False), True: oracle_pipeline(c, True)}
     return c
 
@@ -254,6 +258,24 @@ def test_state_passing_noncontiguous(cuda):
     assert_same_codes(fin, rfin, "final")
 
 
+def test_documented_binding_example_runs(cuda, monkeypatch):
+    """The stand-alone ctypes binding shown in the integration notes, executed as written, gives the wrapper's result."""
+    from linquant_amd.kernels.mamba2.state_passing import _fixedpoint_state_passing_fwd
+    from tests.test_abi import ROOT, binding_example
+
+    say("documented ctypes binding of lq_state_passing")
+    monkeypatch.chdir(ROOT)
+    ns = {}
+    exec(compile(binding_example(), "binding_example", "exec"), ns)
+    rng = np.random.default_rng(1)
+    states = dev(rng.integers(-128, 128, size=(2, 5, 3, 512)).astype(np.int8), cuda)
+    dA = dev(-rng.random((2, 3, 5)).astype(np.float32), cuda)
+    out, fin = ns["_fixedpoint_state_passing_fwd"](states, dA)
+    rout, rfin = _fixedpoint_state_passing_fwd(states, dA)
+    torch.cuda.synchronize()
+    assert torch.equal(out, rout) and torch.equal(fin, rfin)
+
+
 @pytest.mark.parametrize("keyside", [False, True])
 def test_bmm_chunk(case, cuda, keyside):
     from linquant_amd.kernels.mamba2.bmm_chunk import _quant_bmm_chunk_fwd
@@ -291,6 +313,15 @@ def test_chunk_scan(case, cuda, keyside):
     r2 = O.chunk_scan(ref["cb"], ref["x"], ref["dt"], ref["dA_cumsum"], ref["q_C"], npy(sc["C_scale"]), ref["passed"],
                       None, None, npy(sc["static_state_scale"]), npy(sc["static_cb_scale"]))
     assert_close_out(out2, r2, "out (no D)")
+    # a small static CB scale (the chunk scan is defined for any codes and scale): S_cb * dt ~ 1e-4 is at the edge of the
+    # fp16 normal range, where the reference's own fp16 weights are still accurate for all but the smallest codes
+    small = (sc["static_cb_scale"] * (1.37 * 2.0 ** -6)).contiguous()
+    out3 = _quant_chunk_scan_fwd(dev(ref["cb"], cuda), x, dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda),
+                                 dev(ref["q_C"], cuda), sc["C_scale"], torch.zeros_like(dev(ref["passed"], cuda)), None, None,
+                                 sc["static_state_scale"], small)
+    r3 = O.chunk_scan(ref["cb"], ref["x"], ref["dt"], ref["dA_cumsum"], ref["q_C"], npy(sc["C_scale"]),
+                      np.zeros_like(ref["passed"]), None, None, npy(sc["static_state_scale"]), npy(small))
+    assert_close_out(out3, r3, "out (small S_cb, causal path only)")
 
 
 @pytest.mark.parametrize("keyside", [False, True])

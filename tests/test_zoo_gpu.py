@@ -54,31 +54,34 @@ def test_eta_split(cuda, cell, eta):
     zc.check(out, run, qz, f"{cell} eta={eta}")
 
 
-FULL_SIZE = {"linear_none": (4, 4096, 16), "gla": (4, 4096, 16), "deltanet": (4, 4096, 16), "gated_deltanet": (4, 4096, 16),
-             "kda": (2, 8192, 32)}
-
-
-@pytest.mark.parametrize("cell", list(FULL_SIZE))
-def test_full_size_slices(cuda, cell):
-    """The benchmark's shapes (K = V = 128, chunk 64; local R_QK on the diagonal-decay cells, sigma = 0.5 on the delta
-    cells). Every (batch row, head) is an independent recurrence, so the full-size launch must reproduce, bit for bit,
-    a launch on one batch row and two non-adjacent heads cut out of the same inputs; that cut is small enough for the
-    float64 oracle and is held to the reference's criterion over the whole 64- or 128-chunk horizon."""
+@pytest.mark.parametrize("name", list(zc.CONFIGS))
+def test_full_size_slices(cuda, name):
+    """The benchmark configurations as they are stated, at full size (K = V = 128, chunk 64): c2 linear attention and
+    GLA under kernel_pt with N(0,1) queries, c3 DeltaNet / Gated DeltaNet under kernel_ptk with the write gate at
+    sigma = 0.5, c4 KDA under per-channel static scales with D_QK (alpha = 0.5) and the local R_QK; static scales from a
+    separate seed-1 batch.  Every (batch row, head) is an independent recurrence, so the full-size launch must reproduce,
+    bit for bit, a launch on one batch row and two non-adjacent heads cut out of the same inputs; that cut is small
+    enough for the float64 oracle and is held to the reference's criterion over the whole 64- or 128-chunk horizon."""
     import sys
 
-    from oracle.zoo_reference import signed_hadamard
+    from linquant_amd.calibration import dqk_from_absmax
 
-    B, T, H = FULL_SIZE[cell]
+    cfg = zc.CONFIGS[name]
+    cell, B, T, H = cfg["cell"], cfg["B"], cfg["T"], cfg["H"]
     K = V = 128
-    print("full size", cell, B, T, H, flush=True, file=sys.stderr)
-    tensors = zc.inputs(cell, B=B, T=T, H=H, K=K, V=V, seed=7)
+    print("full size", name, cfg, flush=True, file=sys.stderr)
     b, hs = B - 1, [5, H - 3]
+    tensors, rot = zc.config_inputs(name, 0)
+    calib, _ = zc.config_inputs(name, 1, heads=hs, batch_row=b)
+    if cfg["dqk"]:
+        cal_full, _ = zc.config_inputs(name, 1)
+        D = dqk_from_absmax(cal_full[0].float(), cal_full[1].float(), 0.5)  # (H, K)
+        del cal_full
+        tensors, calib = zc.apply_dqk(tensors, D), zc.apply_dqk(calib, D[hs])
     part = [t[b:b + 1, :, hs].contiguous() if t is not None else None for t in tensors]
     fam, dec = zc.CELLS[cell]
-    rot = signed_hadamard(K, 3) if dec == "diagonal" else None
-    rho = 0.5 if fam == "delta" else 1.0
-    eta = DEFAULT_ETA[cell]
-    qz, run = zc.calibrated(cell, part, eta=eta, rho=rho, rot_qk=rot)
+    eta, rho = cfg["eta"], cfg["rho"]
+    qz, run = zc.calibrated(cell, part, policy=cfg["policy"], eta=eta, rho=rho, rot_qk=rot, calib_tensors=calib)
     sc = qz.kernel_scales(0, 2, K, V, delta=fam == "delta")
     pick = torch.zeros(H, dtype=torch.long)
     pick[hs[1]] = 1                                                  # every other head borrows the first cut head's scales
@@ -86,8 +89,9 @@ def test_full_size_slices(cuda, cell):
     out_part, _ = zc.run_kernel(cell, part, sc, eta=eta, rho=rho, rot=rot)
     torch.cuda.synchronize()
     assert torch.isfinite(out_full).all()
-    assert torch.equal(out_full[b:b + 1][:, :, hs], out_part), f"{cell}: the full-size launch differs from the launch on its cut"
-    zc.check(out_part, run, qz, f"{cell} full-size cut")
+    assert torch.equal(out_full[b:b + 1][:, :, hs], out_part), f"{name}: the full-size launch differs from the launch on its cut"
+    e_max, e_mean = zc.check(out_part, run, qz, f"{name} full-size cut")
+    print(f"[full size] {name}: rel err max {e_max:.2e} mean {e_mean:.2e}", flush=True)
 
 
 @pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet", "kda"])
@@ -181,12 +185,13 @@ def test_bf16_activations(cuda, cell, variant):
 @pytest.mark.parametrize("cell", list(zc.CELLS))
 @pytest.mark.parametrize("seed", [4, 3])
 def test_stored_state_codes_and_final_state(cuda, cell, seed):
-    """Stored INT8 state codes against the oracle's: within one step.  The delta-rule cells carry one caveat: W and U
-    are half-precision roundings of fp32 sums, and where such a sum lies within fp32 noise of a rounding boundary the
-    kernel and the float64 oracle round apart (about one element in 10^4, for the fp32 MFMA and for the split-bf16
-    product alike); the pseudo-value code that flips with it shifts a column of the state by one more step.  Seed 3
-    shows one such code with either product, so the bar is: never more than two steps, two steps in fewer than 5e-5 of
-    the codes, any difference in fewer than 2 %."""
+    """Stored INT8 state codes against the oracle's: within one step, and different at all in fewer than 1e-3 of the
+    codes (measured: none for linear attention and the Mamba-2 cell, 1.6e-4 GLA, 8e-5 KDA, 5e-6 Gated DeltaNet,
+    3e-4 DeltaNet).  DeltaNet carries one caveat: W and U are half-precision roundings of fp32 sums, and where such a
+    sum lies within fp32 noise of a rounding boundary the kernel and the float64 oracle round apart (about one element
+    in 10^4, for the fp32 MFMA and for the split-bf16 product alike); the pseudo-value code that flips with it shifts a
+    column of the state by one more step.  Measured: 2 and 1 of 196608 codes two steps apart (1.0e-5, 5e-6) at the two
+    seeds, for DeltaNet only; the bound asserted for it is 3e-5, and one step for every other cell."""
     tensors = zc.cut(zc.inputs(cell, seed=seed), 256)
     dbg = {}
     out, ht, qz, run = _go(cell, tensors, debug=dbg, final_state=True)
@@ -195,14 +200,68 @@ def test_stored_state_codes_and_final_state(cuda, cell, seed):
     assert (got[:, 0] == 0).all()
     NT = codes.shape[0]
     diff = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
-    limit = 2 if zc.CELLS[cell][0] == "delta" else 1
+    limit = 2 if cell == "deltanet" else 1
+    print(f"[state codes] {cell} seed {seed}: differ {(diff != 0).float().mean().item():.3e}, off by two "
+          f"{(diff > 1).float().mean().item():.3e} ({int((diff > 1).sum())} of {diff.numel()}), max {int(diff.max())}", flush=True)
     assert diff.max().item() <= limit, f"{cell}: stored state code off by {diff.max().item()}"
-    assert (diff > 1).float().mean().item() < 5e-5, f"{cell}: {(diff > 1).sum().item()} codes off by two"
-    assert (diff != 0).float().mean().item() < 0.02, f"{cell}: {(diff != 0).float().mean().item():.3%} codes differ"
+    assert (diff > 1).float().mean().item() <= 3e-5, f"{cell}: {(diff > 1).sum().item()} codes off by two"
+    assert (diff != 0).float().mean().item() < 1e-3, f"{cell}: {(diff != 0).float().mean().item():.3%} codes differ"
     # the final fp32 carry quantizes to the last stored code
     sc = qz.kernel_scales(0, *tensors[0].shape[2:], tensors[2].shape[-1])["state"]
     last = torch.round(ht.cpu() / sc[None, :, None, :]).clamp(-127, 127)
     assert (last - codes[-1]).abs().max().item() <= limit
+
+
+# Measured on MI355X (T = 256, B2, H4 / H2, 131072 .. 262144 codes per role): no code of any role differs from the
+# oracle's, in any of the six cells, at K = 64 and K = 128.  A tie between the fp32 and the float64 evaluation of an
+# exponentially weighted operand is possible in principle (about 1e-5 per code), so the bound is not zero.
+CODE_FLIP_BOUND = 1e-4
+
+
+@pytest.mark.parametrize("K", [64, 128])
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+def test_operand_codes_per_role(cuda, cell, K):
+    """INT8 operand codes of every role the kernels materialize (key / value write codes, state-read codes of W, codes
+    of the decayed query) against the oracle's codes for the same role: never more than one step apart, and the
+    fraction that differs is the rate of fp32-vs-float64 rounding ties (the oracle forms q*scale, k*Omega etc. in
+    float64 and casts; the kernels form them in fp32).  Operands that carry no exponential weight and a power-of-two
+    `scale` must match bit for bit."""
+    tensors = zc.cut(zc.inputs(cell, K=K, H=2 if K == 128 else 4, seed=9), 256)
+    dbg = {}
+    out, _, qz, run = _go(cell, tensors, debug=dbg)
+    ref = zc.operand_codes(qz, run)
+    fam, dec = zc.CELLS[cell]
+    pairs = [("k_write", "kq")]
+    pairs.append(("v_write", "vq") if fam == "linear" else ("w_read", "wq"))
+    if dec == "diagonal":
+        pairs.append(("q_read", "qg"))
+    for role, name in pairs:
+        got, want = dbg[name].cpu().int(), ref[role].int()
+        assert got.shape == want.shape, (role, got.shape, want.shape)
+        diff = (got - want).abs()
+        rate = (diff != 0).float().mean().item()
+        print(f"[codes] {cell} K={K} {role}: {int((diff != 0).sum())} of {diff.numel()} differ ({rate:.2e}), max {int(diff.max())}",
+              flush=True)
+        assert diff.max().item() <= 1, f"{cell} {role}: code off by {diff.max().item()}"
+        assert rate <= CODE_FLIP_BOUND, f"{cell} {role}: {rate:.2e} of the codes differ"
+        if dec == "none" and role in ("k_write", "v_write"):
+            assert rate == 0.0, f"{cell} {role}: un-weighted operand codes must be bit-exact"
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+def test_output_error_distribution(cuda, cell):
+    """Dequantized outputs against the float64 oracle at the 1e-3 bar over a four-chunk horizon: every output within
+    1e-3 of the output's maximum (measured worst case over the six cells: 3.3e-4).  Over longer horizons a stored state
+    code that rounds the other way (test_stored_state_codes_and_final_state measures how often) moves the outputs it
+    feeds by a code step, 3e-3 .. 1.5e-2 of the maximum, which is why the long tests use the reference's own criterion."""
+    tensors = zc.cut(zc.inputs(cell, seed=11), 256)
+    out, _, qz, run = _go(cell, tensors)
+    ref = run().float()
+    d = (out.float().cpu() - ref).abs() / ref.abs().max()
+    frac, worst = (d > 1e-3).float().mean().item(), d.max().item()
+    print(f"[output 1e-3] {cell}: {frac:.3e} of the outputs beyond 1e-3 of the maximum, worst {worst:.2e}, "
+          f"median {d.median().item():.1e}", flush=True)
+    assert worst <= 1e-3, f"{cell}: output {worst:.2e} of the maximum away from the float64 oracle"
 
 
 @pytest.mark.parametrize("cell", ["mamba2", "kda"])

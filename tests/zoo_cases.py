@@ -24,28 +24,68 @@ def inputs(cell, B=2, T=512, H=4, K=64, V=128, seed=0, gscale=1.0, dtype=torch.f
     return q, k, v, g, beta
 
 
+# The benchmark configurations (shape, cell, policy, placements) as they are stated: per-tensor operands for linear
+# attention / GLA, per-token-tensor key roles with the write gate placed at sigma = 0.5 for the delta rules, per-channel
+# static scales with D_QK (alpha = 0.5) for KDA; R_QK persistent on q, k (no / scalar decay) or local (diagonal decay).
+CONFIGS = {
+    "c2_la": dict(cell="linear_none", B=4, T=4096, H=16, policy="kernel_pt", eta=1.0, rho=1.0, dqk=False),
+    "c2_gla": dict(cell="gla", B=4, T=4096, H=16, policy="kernel_pt", eta=0.0, rho=1.0, dqk=False),
+    "c3_deltanet": dict(cell="deltanet", B=4, T=4096, H=16, policy="kernel_ptk", eta=1.0, rho=0.5, dqk=False),
+    "c3_gdn": dict(cell="gated_deltanet", B=4, T=4096, H=16, policy="kernel_ptk", eta=1.0, rho=0.5, dqk=False),
+    "c4_kda": dict(cell="kda", B=2, T=8192, H=32, policy="kernel_static", eta=0.0, rho=0.5, dqk=True),
+}
+
+
+def config_inputs(name, seed, K=128, V=128, heads=None, batch_row=None):
+    """fp16 inputs of a benchmark configuration as the kernels receive them, optionally cut to one batch row and a list of
+    heads (the cut commutes with every step here: all of them are per (batch, head)):
+    (tensors, rot) with rot the local R_QK of the diagonal-decay cells (None otherwise: there q, k arrive rotated,
+    materialized in fp16, as the oracle's `mat(q @ R)` does)."""
+    from linquant_amd.calibration import zoo_synthetic
+
+    cfg = CONFIGS[name]
+    q, k, v, g, beta = zoo_synthetic(cfg["cell"], cfg["B"], cfg["T"], cfg["H"], K, V, seed)
+    if batch_row is not None:
+        sel = lambda t: None if t is None else t[batch_row:batch_row + 1][:, :, heads].contiguous()  # noqa: E731
+        q, k, v, g, beta = sel(q), sel(k), sel(v), sel(g), sel(beta)
+    R = Z.signed_hadamard(K, 1)
+    q, k, v = q.half(), k.half(), v.half()
+    if CELLS[cfg["cell"]][1] != "diagonal":
+        q, k = (q.double() @ R).half(), (k.double() @ R).half()
+        R = None
+    return (q, k, v, g, beta), R
+
+
+def apply_dqk(tensors, D):
+    """q' = fp16(q * D), k' = fp16(k / D) with D (H, K) fp32: products formed in fp32, rounded once to fp16."""
+    q, k, v, g, beta = tensors
+    return ((q.float() * D[None, None]).half(), (k.float() * (1.0 / D)[None, None]).half(), v, g, beta)
+
+
 def cut(tensors, n):
     return [t[:, :n].contiguous() if t is not None else None for t in tensors]
 
 
-def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None, out_dtype=None):
-    """Returns (qz, run): the oracle's quantizer with scales calibrated on these inputs, and a closure that
-    evaluates the oracle under the quantizer's current arithmetic mode; like the kernels, the oracle materializes its
-    output in the activation dtype unless ``out_dtype`` says otherwise."""
+def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None, out_dtype=None,
+               calib_tensors=None):
+    """Returns (qz, run): the oracle's quantizer with scales calibrated on these inputs (or on ``calib_tensors``, a
+    separate batch), and a closure that evaluates the oracle on ``tensors`` under the quantizer's current arithmetic
+    mode; like the kernels, the oracle materializes its output in the activation dtype unless ``out_dtype`` says
+    otherwise."""
     fam, dec = CELLS[cell]
-    q, k, v, g, beta = tensors
-    K = q.shape[-1]
+    K = tensors[0].shape[-1]
     qz = Z.ZooQuantizer.kernel_profile(policy, bits)
 
-    def run():
+    def forward(t):
+        q, k, v, g, beta = t
         return Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=qz, eta=eta, rho=rho,
                                tau=tau, read_post=True, C=64, out_dtype=out_dtype, rot_qk=rot_qk, rot_v=rot_v,
                                storage="canonical" if rot_v is not None else "rotated")
 
     qz.calibrating = True
-    run()
+    forward(tensors if calib_tensors is None else calib_tensors)
     qz.finalize()
-    return qz, run
+    return qz, lambda: forward(tensors)
 
 
 def run_kernel(cell, tensors, scales, *, eta=1.0, rho=1.0, tau=1.0, bits=8, out_dtype=None, final_state=False,
@@ -99,3 +139,17 @@ def state_codes(qz, run):
     codes = torch.stack([c.to(torch.int8) for c in qz.trace])
     qz.trace = None
     return codes
+
+
+def operand_codes(qz, run):
+    """INT8 operand codes the oracle formed, per role, token-major: role -> (B, T, H, D) int8 (one call per chunk and
+    role; roles called more than once per chunk, like the anchored sub-block operands, are left out)."""
+    qz.code_trace = {}
+    run()
+    trace, qz.code_trace = qz.code_trace, None
+    nt = len(trace["k_write"])
+    out = {}
+    for role, calls in trace.items():
+        if len(calls) == nt:  # [B,H,C,D] per chunk -> (B,T,H,D)
+            out[role] = torch.cat([c.permute(0, 2, 1, 3) for c in calls], dim=1)
+    return out
