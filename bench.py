@@ -122,35 +122,37 @@ def bench_zoo(args):
     dev = torch.device("cuda:0")
     cell, B, T, H, K, V, desc = ZOO_WORKLOADS[args.workload]
     fam, dec = ZOO_CELLS[cell]
-    gen = torch.Generator().manual_seed(0)
-    rn = lambda *shape: torch.randn(*shape, generator=gen)  # noqa: E731
-    q = rn(B, T, H, K)
-    k = rn(B, T, H, K)
-    if fam == "delta":
-        k = torch.nn.functional.normalize(k, dim=-1)
-    v = rn(B, T, H, V)
-    beta = torch.sigmoid(rn(B, T, H)).to(dev) if fam == "delta" else None
-    g = None
-    if cell == "gla":
-        g = torch.nn.functional.logsigmoid(rn(B, T, H, K)) / 16
-    elif cell == "kda":
-        g = torch.nn.functional.logsigmoid(rn(B, T, H, K) + 1.0)
-    elif cell == "gated_deltanet":
-        g = torch.nn.functional.logsigmoid(rn(B, T, H) + 2.0)
-    elif cell == "mamba2":
-        g = -torch.nn.functional.softplus(rn(B, T, H) * 0.5 - 2.0) * torch.exp(torch.rand(H, generator=gen) * 2.77)
+    from linquant_amd.calibration import dqk_from_absmax, zoo_synthetic
+
+    q, k, v, g, beta = zoo_synthetic(cell, B, T, H, K, V, seed=0)
     R = hadamard_signed(K, 1, dev)
     rot = R if dec == "diagonal" else None
-    q, k, v = q.to(dev), k.to(dev), v.to(dev)
-    if dec != "diagonal" and args.workload != "c1":  # persistent R_QK: folded into the projections in deployment
-        q, k = (q.double() @ R).float(), (k.double() @ R).float()
-    q, k, v = q.half(), k.half(), v.half()
-    g = g.float().to(dev) if g is not None else None
+    q0, k0, v = q.to(dev).half(), k.to(dev).half(), v.to(dev).half()
+    beta = beta.to(dev) if beta is not None else None
+    g = g.to(dev) if g is not None else None
+    # operand prologue, part of the timed step: persistent R_QK on q, k (no / scalar decay; the diagonal-decay cells rotate
+    # locally inside the A kernel) and, for the KDA configuration, D_QK (alpha = 0.5) from a seed-1 calibration batch
+    persistent = dec != "diagonal" and args.workload != "c1"
+    sq = zoo.rotation_signs(R) if persistent else None
+    dqk = None
+    if args.workload == "c4_kda":
+        cq, ck, *_ = zoo_synthetic(cell, 1, 2048, H, K, V, seed=1)
+        dqk = dqk_from_absmax(cq.half().float(), ck.half().float(), 0.5).to(dev)
+    has_prologue = persistent or dqk is not None
+    qr, kr = torch.empty_like(q0), torch.empty_like(k0)
+
+    def prologue():
+        if has_prologue:
+            zoo.rotate_qkv(q0, k0, None, signs_qk=sq, dqk=dqk, out=(qr, kr, None))
+            return qr, kr
+        return q0, k0
+
+    q, k = prologue()
     scale = 1.0 if args.workload == "c1" else K ** -0.5
     sigma = 0.5 if args.workload.startswith("c3") else 1.0
     eta = 0.0 if dec == "diagonal" else 1.0
 
-    def call(sc, **kw):
+    def kernels(sc, **kw):
         if fam == "linear" and dec == "diagonal":
             return zoo.chunk_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, rot=rot, **kw)
         if fam == "linear":
@@ -158,6 +160,10 @@ def bench_zoo(args):
         if dec == "diagonal":
             return zoo.chunk_kda_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, rot=rot, **kw)
         return zoo.chunk_delta_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, **kw)
+
+    def call(sc, **kw):
+        prologue()
+        return kernels(sc, **kw)
 
     # static scales: operand roles from the inputs' absmax (decay factors are <= 1), state / pseudo-value roles from a
     # pilot run of the kernels themselves with a coarse state grid
@@ -205,13 +211,17 @@ def bench_zoo(args):
     try:
         for n, label in names.items():
             setattr(C, n, timed(saved[n], label))
+        tp = timed(prologue, "prologue")
         for _ in range(max(10, args.steps)):
-            call(sc)
+            if has_prologue:
+                tp()
+            kernels(sc)
         torch.cuda.synchronize()
     finally:
         for n, f in saved.items():
             setattr(C, n, f)
     nbytes = zoo_stage_bytes(fam, dec, B, T, H, K, V)
+    nbytes["prologue"] = 2 * (B * T * H * K * 2) * 2  # q and k, read and written once
     stages = {}
     for label, evs in records.items():
         ts = sorted(a.elapsed_time(b) for a, b in evs)
@@ -256,7 +266,10 @@ def bench_zoo(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{args.workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
-                   "tokens_per_step": tokens},
+                   "tokens_per_step": tokens,
+                   "prologue": ("in the timed step: " + ("R_QK on q, k" if persistent else "") +
+                                (" D_QK (alpha 0.5) on q, k" if dqk is not None else "")) if has_prologue else
+                               "none (local R_QK inside the A kernel)" if rot is not None else "none"},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
     }
     print(json.dumps(line), flush=True)

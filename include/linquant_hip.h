@@ -166,6 +166,61 @@ typedef struct {
 } lq_chunk_scan_args;
 int lq_chunk_scan(const lq_chunk_scan_args* args, hipStream_t stream);
 
+/* replaces _quant_mamba_chunk_scan_combined_fwd, linquant/kernels/mamba2/ssd_combined.py:19-131, as one call: the five
+ * stages above launched back to back on `stream` (cumsum -> chunk state -> state passing -> C.B^T -> chunk scan), with
+ * the intermediates the reference allocates per call (dt, dA_cumsum, chunk states, passed states, CB) laid out in one
+ * caller-supplied workspace.  Field meanings as in the per-stage structs; keyside selects lq_chunk_state_key (x_scale_hp,
+ * b_fp, b_gate_scale) or lq_chunk_state_value (qB, alpha_hp, bscale_g), and the B operand of C.B^T with it. */
+typedef struct {
+  const void* x;             /* (B,L,H,P) fp16, unit P stride */
+  int64_t x_stride_b, x_stride_l, x_stride_h;
+  const void* dt;            /* (B,L,H) raw dt */
+  int32_t dt_dtype;
+  int64_t dt_stride_b, dt_stride_l, dt_stride_h;
+  const float* dt_scale;     /* device scalar */
+  const int8_t* A_log;       /* (H,) */
+  int64_t A_log_stride_h;
+  const float* A_log_scale;  /* device scalar */
+  const float* dt_bias;      /* (H,) or NULL */
+  int64_t dt_bias_stride_h;
+  int32_t dt_softplus;
+  float dt_min, dt_max;
+  const int8_t* qB;          /* (B,L,G,N) int8 (value side), unit N stride */
+  int64_t qB_stride_b, qB_stride_l, qB_stride_g;
+  const void* b_fp;          /* (B,L,G,N) fp16 (key side), unit N stride */
+  int64_t bfp_stride_b, bfp_stride_l, bfp_stride_g;
+  const int8_t* qC;          /* (B,L,G,N) int8, unit N stride */
+  int64_t qC_stride_b, qC_stride_l, qC_stride_g;
+  const float* B_scale;      /* (G,) */
+  const float* C_scale;      /* (G,) */
+  const int8_t* D;           /* (H,) or (H,P) int8, or NULL */
+  int64_t D_stride_h;
+  int32_t D_has_hdim;
+  const float* D_scale;      /* device scalar */
+  const float* state_scale;  /* (H,P) view: static_state_scale */
+  int64_t ss_stride_h, ss_stride_p;
+  const float* cb_scale;     /* (G,): static_cb_scale */
+  const float* alpha_hp;     /* value side: (H,P) view */
+  int64_t alpha_stride_h, alpha_stride_p;
+  const float* bscale_g;     /* value side: (G,) */
+  int64_t bscale_stride_g;
+  const float* x_scale_hp;   /* key side: (H,P) view */
+  int64_t xs_stride_h, xs_stride_p;
+  const float* b_gate_scale; /* key side: 4-D broadcastable (B,nc,H,N) */
+  int64_t bgs_stride_b, bgs_stride_c, bgs_stride_h, bgs_stride_n;
+  int32_t keyside;
+  int32_t gate_shift;        /* fractional bits of the state-passing gate (reference: 7) */
+  void* out;                 /* (B,L,H,P) fp16 contiguous */
+  int8_t* final_states;      /* (B,H,P*N) int8 contiguous, or NULL */
+  void* workspace;           /* device memory, 256-byte aligned, lq_ssd_combined_workspace_bytes() bytes; contents undefined
+                                on entry and on return */
+  int64_t workspace_bytes;
+  int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+} lq_ssd_combined_args;
+int lq_ssd_combined(const lq_ssd_combined_args* args, hipStream_t stream);
+/* workspace size for the dims in `args` (pointers are not read), written to *bytes */
+int lq_ssd_combined_workspace_bytes(const lq_ssd_combined_args* args, int64_t* bytes);
+
 /* ------------------------------------------------------------------------------------------
  * Rotation + quantize prologue.
  * ------------------------------------------------------------------------------------------ */
@@ -348,6 +403,30 @@ typedef struct {
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
 } lq_zoo_wy_prep_args;
 int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
+
+/* replaces the operand rotations in front of a zoo call: the three GEMMs q @ R_QK, k @ R_QK, v @ R_V of
+ * bench/zoo_kernels.py:135-140 (the oracle's entry rotation, linquant/reference.py:42-46) and the diagonal q / k
+ * rescaling D_QK of linquant/harness.py:68-88, in one launch:
+ *   q_out = act((q * dq) . H_K / sqrt(K) * signs_qk),  k_out likewise with dk (= 1 / dq),  v_out = act(v . H_V / sqrt(V) * signs_v)
+ * with the Sylvester Hadamard matrix H_n (linquant/reference.py:232-239: R = H_n / sqrt(n) . diag(signs)), evaluated as a
+ * fast Walsh-Hadamard transform in fp32 and rounded once to the activation dtype.  A tensor whose input pointer is NULL
+ * is skipped; NULL signs leave out the rotation (diagonal-decay cells rotate locally inside lq_zoo_gla_A); NULL dq / dk
+ * leave out the rescaling.  In place (q_out == q) is allowed. */
+typedef struct {
+  const void* q;             /* (B,T,H,K) fp16/bf16 contiguous, or NULL */
+  const void* k;             /* (B,T,H,K), or NULL */
+  const void* v;             /* (B,T,H,V), or NULL */
+  void* q_out;               /* same shape and dtype as the input */
+  void* k_out;
+  void* v_out;
+  const float* dq;           /* (H,K) fp32 factor on q (D_QK), or NULL */
+  const float* dk;           /* (H,K) fp32 factor on k (1 / D_QK), or NULL */
+  const float* signs_qk;     /* (K,) fp32 +-1 column signs of R_QK, or NULL */
+  const float* signs_v;      /* (V,) fp32 +-1 column signs of R_V, or NULL */
+  int32_t batch, seqlen, nheads, kdim, vdim; /* kdim, vdim in {64, 128} */
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16 */
+} lq_zoo_rotate_qkv_args;
+int lq_zoo_rotate_qkv(const lq_zoo_rotate_qkv_args* args, hipStream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Element-wise stages in front of the Mamba-2 SSD prologue.

@@ -54,6 +54,9 @@ _structs, _funcs = parse_header()
 STRUCTS = {name: type(name, (ctypes.Structure,), {"_fields_": fields}) for name, fields in _structs.items()}
 FUNCTIONS = tuple(_funcs)
 
+# entry points whose first argument is another function's args struct
+_SHARED_ARGS = {"lq_ssd_combined_workspace_bytes": "lq_ssd_combined_args"}
+
 _lib = None
 
 
@@ -69,7 +72,7 @@ def load():
     for fn in FUNCTIONS:
         f = getattr(lib, fn)
         f.restype = ctypes.c_int
-        sname = fn + "_args"
+        sname = _SHARED_ARGS.get(fn, fn + "_args")
         if sname in STRUCTS:
             f.argtypes = [ctypes.POINTER(STRUCTS[sname]), ctypes.c_void_p]
         elif fn == "lq_args_size":
@@ -112,10 +115,32 @@ def current_stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
+def fill(struct_name: str, **fields):
+    """An instance of the named args struct with the given fields set (unknown names raise KeyError)."""
+    st = STRUCTS[struct_name]()
+    known = {n for n, _ in st._fields_}
+    for k, v in fields.items():
+        if k not in known:
+            raise KeyError(f"{struct_name} has no field {k!r}")
+        setattr(st, k, v)
+    return st
+
+
+def launch(fn: str, device, st):
+    """Call entry point ``fn`` with an already filled args struct on the current stream of ``device``."""
+    lib = load()
+    import torch
+
+    with torch.cuda.device(device):
+        rc = getattr(lib, fn)(ctypes.byref(st), current_stream(device))
+    if rc != 0:
+        raise LinQuantHipError(f"{fn} failed with code {rc}: {_ERRORS.get(rc, 'unknown error')}")
+
+
 def call(fn: str, device, **fields):
     """Fill ``<fn>_args`` from keyword fields and launch on the current stream of ``device``."""
     lib = load()
-    st = STRUCTS[fn + "_args"]()
+    st = STRUCTS[_SHARED_ARGS.get(fn, fn + "_args")]()
     known = {n for n, _ in st._fields_}
     for k, v in fields.items():
         if k not in known:

@@ -17,6 +17,7 @@ Follows (reference file:line):
   _linear_chunk           linquant/reference.py:190-199
   _delta_chunk            linquant/reference.py:202-229
   signed_hadamard         linquant/reference.py:232-239 (sign stream from torch's CPU generator)
+  rotate_operands         linquant/reference.py:40-46 (entry rotations), linquant/harness.py:84-87 (D_QK)
 
 Pinned by tests/test_oracle_zoo.py: golden vectors written by the reference itself (tests/golden/zoo_golden.npz,
 generator tests/golden/make_zoo_golden.py) for every cell x policy incl. calibrated scales, rotations, canonical
@@ -159,6 +160,24 @@ def signed_hadamard(n, seed, device=None):
     gen = torch.Generator().manual_seed(seed)
     signs = torch.randint(0, 2, (n,), generator=gen).double() * 2 - 1
     return (Hm / n ** 0.5 * signs).to(device)
+
+
+def rotate_operands(q, k, v, rot_qk=None, rot_v=None, dqk=None):
+    """The operand prologue in front of a kernel call: q' = mat((q D) @ R_QK), k' = mat((k / D) @ R_QK),
+    v' = mat(v @ R_V) with mat = float64 -> fp32 -> activation dtype (linquant/reference.py:40-46; D_QK as
+    linquant/harness.py:84-87 applies it, the reciprocal formed in fp32 as the kernels receive it).  Any of rot_qk,
+    rot_v, dqk (H,K) may be None.  Returns tensors in the inputs' dtype."""
+    def mat(t, like):
+        return t.float().to(like.dtype)
+
+    qq, kk = q.double(), k.double()
+    if dqk is not None:
+        d = dqk.float()
+        qq, kk = qq * d.double()[None, None], kk * (1.0 / d).double()[None, None]
+    if rot_qk is not None:
+        qq, kk = qq @ rot_qk.double(), kk @ rot_qk.double()
+    vv = v.double() if rot_v is None else v.double() @ rot_v.double()
+    return mat(qq, q), mat(kk, k), mat(vv, v)
 
 
 # ----------------------------------------------------------------------------------------- pieces

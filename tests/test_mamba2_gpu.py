@@ -372,6 +372,100 @@ def test_pipeline_end_to_end(case, cuda, keyside):
     assert_close_out(out, ref["out"], "out")
 
 
+@pytest.mark.parametrize("keyside", [False, True])
+def test_one_call_equals_stage_by_stage(case, cuda, keyside):
+    """With no stage re-bound the combined forward is one C call (lq_ssd_combined) over one workspace; it must give
+    the stage-by-stage path's output bit for bit (same kernels, same order)."""
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    s = case["shape"]
+    say("one call vs staged", "key" if keyside else "value", s)
+    xBC, dt_raw, p, sc = gpu_inputs(case, cuda)
+    x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                             sc["B_inv_scale"], sc["C_inv_scale"])
+    kw = {}
+    if keyside:
+        gn = s.ngroups * s.dstate
+        b_fp = xBC[..., s.d_ssm:s.d_ssm + gn].reshape(s.batch, s.seqlen, s.ngroups, s.dstate).contiguous()
+        kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=kronecker_hadamard_fwd(b_fp, p["r_signs"], s.ngroups),
+                  b_gate_scale=sc["b_gate_scale"])
+
+    def fwd():
+        return M._quant_mamba_chunk_scan_combined_fwd(
+            x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], **kw)[0]
+
+    assert not M._stages_rebound()
+    one = fwd()
+    orig = M._chunk_scan_v2
+    M._chunk_scan_v2 = lambda *a: orig(*a)  # any re-bound stage selects the stage-by-stage path
+    try:
+        assert M._stages_rebound()
+        staged = fwd()
+    finally:
+        M._chunk_scan_v2 = orig
+    torch.cuda.synchronize()
+    assert torch.equal(one, staged)
+    assert_close_out(one, case["oracle"][keyside]["out"], "out (one call)")
+
+
+def test_hip_graph_capture_and_replay(cuda):
+    """The whole key-side step (prologue + combined forward: seven launches, no allocation or synchronisation inside
+    the library) captured once in a HIP graph and replayed: every replay must equal the eager result bit for bit, with
+    eager work and synchronisations between the replays and with new input values written into the captured buffers."""
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    s = Mamba2Shape(batch=2, seqlen=1024, nheads=8, headdim=64, dstate=128, ngroups=1, chunk=256)
+    say("HIP graph capture", s)
+    c = build_case(s)
+    p = {k: v.to(cuda) for k, v in c["params"].items()}
+    sc = {k: v.to(cuda) for k, v in c["scales"].items()}
+    xBC, dt_raw = c["xBC"].to(cuda), c["dt_raw"].to(cuda)
+
+    def step():
+        x, qB, qC, b_fp = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                       sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True)
+        return M._quant_mamba_chunk_scan_combined_fwd(
+            x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], keyside=True,
+            x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"])[0]
+
+    eager = step().clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    torch.cuda.synchronize()
+    for i in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"replay {i} differs from the eager result"
+        again = step()  # eager work of the program itself between replays
+        torch.cuda.synchronize()
+        assert torch.equal(again, eager)
+    other = build_case(s, seed=5)
+    xBC.copy_(other["xBC"].to(cuda))
+    dt_raw.copy_(other["dt_raw"].to(cuda))
+    eager2 = step().clone()
+    torch.cuda.synchronize()
+    assert not torch.equal(eager2, eager)
+    for i in range(2):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager2), f"replay {i} on new inputs differs from the eager result"
+
+
 def test_full_size_config5_slices(cuda):
     """Mamba-2 2.7B-shape layer (B4 L8192 H80 P64 N128 Q256) on the GPU; every integer stage is checked
     bit-exactly against the oracle on head / batch slices the oracle finishes in seconds, the output on the

@@ -153,3 +153,34 @@ def test_kernel_profile_is_close_to_exact_and_policies_differ():
         assert sc["q"].shape == (H,) and sc["kw"].shape == (H, K) and sc["state"].shape == (H, V) and sc["ew"].shape == (H, V)
         assert all(t.dtype == torch.float32 for t in sc.values())
     assert errs["kernel_static"] < 0.05 and errs["kernel_pt"] < 0.1
+
+
+def test_rotate_operands_is_the_entry_rotation_of_chunk_forward():
+    """The stand-alone operand prologue hands chunk_forward exactly what chunk_forward would have formed itself:
+    forward(q, k, v, rot_qk=R, rot_v=Rv) == forward(*rotate_operands(q, k, v, R, Rv)) under kernel arithmetic, bit
+    for bit (linquant/reference.py:40-46), and the rotation is orthogonal; D_QK scales q up and k down by the same
+    factor, so the unquantized q.k products do not move (linquant/harness.py:84-87)."""
+    import torch
+
+    from oracle import zoo_reference as Z
+    from tests import zoo_cases as zc
+
+    q, k, v, g, beta = zc.cut(zc.inputs("mamba2", B=1, H=2, K=64, V=64, seed=3), 128)
+    R, Rv = Z.signed_hadamard(64, 1), Z.signed_hadamard(64, 2)
+    assert torch.allclose(R @ R.T, torch.eye(64, dtype=torch.float64), atol=1e-12)
+    qz = Z.ZooQuantizer.kernel_profile("kernel_static", 8)
+    fw = lambda a, b, c, **kw: Z.chunk_forward(a, b, c, g, None, family="linear", decay="scalar", scale=0.125, qz=qz,  # noqa: E731
+                                               eta=1.0, read_post=True, C=64, **kw)
+    qz.calibrating = True
+    fw(q, k, v, rot_qk=R, rot_v=Rv)
+    qz.finalize()
+    qr, kr, vr = Z.rotate_operands(q, k, v, R, Rv)
+    assert qr.dtype == q.dtype
+    a = fw(q, k, v, rot_qk=R, rot_v=Rv, out_dtype=torch.float64)
+    b = fw(qr, kr, vr, out_dtype=torch.float64) @ Rv.T  # rotated storage: the caller un-rotates the output
+    assert torch.equal(a, b)
+    D = torch.rand(2, 64) + 0.5
+    qd, kd, _ = Z.rotate_operands(q, k, v, None, None, D)
+    dots = (q.double() * k.double()).sum(-1)
+    assert torch.allclose((qd.double() * kd.double()).sum(-1), dots, atol=5e-3)
+    assert torch.equal(qd, (q.float() * D[None, None]).half()) and torch.equal(kd, (k.float() * (1.0 / D)[None, None]).half())
