@@ -213,13 +213,23 @@ typedef struct {
   void* out;                 /* (B,L,H,P) fp16 contiguous */
   int8_t* final_states;      /* (B,H,P*N) int8 contiguous, or NULL */
   void* workspace;           /* device memory, 256-byte aligned, lq_ssd_combined_workspace_bytes() bytes; contents undefined
-                                on entry and on return */
+                                on entry and on return (ignored by lq_ssd_combined_static) */
   int64_t workspace_bytes;
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
 } lq_ssd_combined_args;
 int lq_ssd_combined(const lq_ssd_combined_args* args, hipStream_t stream);
 /* workspace size for the dims in `args` (pointers are not read), written to *bytes */
 int lq_ssd_combined_workspace_bytes(const lq_ssd_combined_args* args, int64_t* bytes);
+
+/* No counterpart in the reference.  lq_ssd_combined for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid it): the intermediates live in a device array of
+ * LQ_SSD_STATIC_WORKSPACE_BYTES that is part of the library image (one per GPU, held until the process ends), so the
+ * call takes inputs and outputs only (`workspace` is ignored) and allocates nothing.  Returns LQ_E_SHAPE when the dims
+ * need more than that.  Every call on one GPU shares the array: calls that overlap on one GPU race (serialize them on
+ * one stream or with events); nothing in it needs clearing between calls, every byte a stage reads was written by an
+ * earlier stage of the same call. */
+#define LQ_SSD_STATIC_WORKSPACE_BYTES (64ll << 20)
+int lq_ssd_combined_static(const lq_ssd_combined_args* args, hipStream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Rotation + quantize prologue.

@@ -55,7 +55,7 @@ STRUCTS = {name: type(name, (ctypes.Structure,), {"_fields_": fields}) for name,
 FUNCTIONS = tuple(_funcs)
 
 # entry points whose first argument is another function's args struct
-_SHARED_ARGS = {"lq_ssd_combined_workspace_bytes": "lq_ssd_combined_args"}
+_SHARED_ARGS = {"lq_ssd_combined_static": "lq_ssd_combined_args", "lq_ssd_combined_workspace_bytes": "lq_ssd_combined_args"}
 
 _lib = None
 

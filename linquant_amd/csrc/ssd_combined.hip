@@ -1,6 +1,9 @@
 // The Mamba-2 INT8 SSD forward as one C call: cumsum -> chunk state -> state passing -> C.B^T -> chunk scan launched
 // back to back on the caller's stream.  Replaces the orchestration of linquant/kernels/mamba2/ssd_combined.py:58-131;
-// the intermediates that function allocates per call live in one caller-supplied workspace.
+// the intermediates that function allocates per call live in one workspace: caller-supplied (lq_ssd_combined) or a
+// device array that is part of the library image (lq_ssd_combined_static, for callers that cannot allocate).
+#include <mutex>
+
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -132,6 +135,32 @@ int check(const lq_ssd_combined_args* a) {
 
 }  // namespace
 
+// Scratch of the allocation-free entry point: one copy per GPU, inside the library's code object.  Its name is a
+// host-side stand-in, not a device address: the address on each device comes from hipGetSymbolAddress, once per device,
+// and only that address is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[LQ_SSD_STATIC_WORKSPACE_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+char* scratch_ptr[kMaxDevices];  // by device ordinal; nullptr until resolved
+
+int static_workspace(char** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return LQ_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return LQ_ERR_LAUNCH;
+    scratch_ptr[dev] = (char*)p;
+  }
+  *out = scratch_ptr[dev];
+  return LQ_OK;
+}
+
+}  // namespace
+
 extern "C" int lq_ssd_combined_workspace_bytes(const lq_ssd_combined_args* a, int64_t* bytes) {
   if (!a || !bytes) return LQ_ERR_NULL;
   Layout l;
@@ -149,4 +178,15 @@ extern "C" int lq_ssd_combined(const lq_ssd_combined_args* a, hipStream_t stream
   if ((rc = plan(a, &l)) != LQ_OK) return rc;
   if (a->workspace_bytes < l.total || ((uintptr_t)a->workspace % kAlign) != 0) return LQ_ERR_SHAPE;
   return run(a, (char*)a->workspace, l, stream);
+}
+
+extern "C" int lq_ssd_combined_static(const lq_ssd_combined_args* a, hipStream_t stream) {
+  int rc = check(a);
+  if (rc != LQ_OK) return rc;
+  Layout l;
+  if ((rc = plan(a, &l)) != LQ_OK) return rc;
+  if (l.total > LQ_SSD_STATIC_WORKSPACE_BYTES) return LQ_ERR_SHAPE;  // larger than the built-in scratch: use lq_ssd_combined
+  char* ws = nullptr;
+  if ((rc = static_workspace(&ws)) != LQ_OK) return rc;
+  return run(a, ws, l, stream);
 }

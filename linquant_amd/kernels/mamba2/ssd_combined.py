@@ -130,15 +130,17 @@ def workspace_bytes(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size)
 
 def _one_call(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale, chunk_size, q_D, D_scale, dt_bias,
               dt_softplus, dt_limit, static_state_scale, static_cb_scale, alpha_hp, bscale_g, keyside, x_scale_hp, b_fp,
-              b_gate_scale):
+              b_gate_scale, static=False):
     batch, seqlen, nheads, headdim = x_fp.shape
     _, _, ngroups, dstate = q_C.shape
     out = torch.empty(batch, seqlen, nheads, headdim, device=x_fp.device, dtype=torch.float16)
-    ws = torch.empty(workspace_bytes(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size), dtype=torch.uint8,
-                     device=x_fp.device)
+    ws = None
+    if not static:
+        ws = torch.empty(workspace_bytes(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size), dtype=torch.uint8,
+                         device=x_fp.device)
     st, keep = combined_args(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale, chunk_size, q_D, D_scale,
                              dt_bias, dt_softplus, dt_limit, static_state_scale, static_cb_scale, alpha_hp, bscale_g, keyside,
                              x_scale_hp, b_fp, b_gate_scale, out, ws)
-    _lib.launch("lq_ssd_combined", x_fp.device, st)
+    _lib.launch("lq_ssd_combined_static" if static else "lq_ssd_combined", x_fp.device, st)
     del keep
     return out
