@@ -47,7 +47,12 @@ struct Params {
   int64_t sbg_b, sbg_c, sbg_h, sbg_n;
   int8_t* states;
   int batch, seqlen, nheads, P, G, N, Q, nchunks, n_ntiles;
+  // floor(2^32 / d) + 1 for d = heads per group, tiles per (batch, chunk, head), N tiles per P tile; 0 when d == 1:
+  // x / d == umulhi(x, magic) for x, d < 2^16
+  uint32_t hpg_magic, tiles_magic, nt_magic;
 };
+
+LQ_DEV int div_magic(uint32_t x, uint32_t magic) { return magic ? (int)__umulhi(x, magic) : (int)x; }
 
 // clamp to [-127, 127] then round half even; returns a dword whose low byte is the INT8 code
 LQ_DEV uint32_t rint_code(float y) {
@@ -73,27 +78,32 @@ LQ_DEV float mul_half(uint32_t w, float f) {
 // NSLAB = number of 64-token slabs of a chunk when it is one of the unrolled counts (2, 4), else 0 (run-time loop).
 // With a known count the slab loop is fully unrolled over two register sets: the next slab is requested before the
 // current one is quantized, no request sits inside a run-time branch, and the compiler's wait counts stay exact.
-// Measured at B4 L8192 H80 P64 N128 Q256: value side 115 -> 108 us; key side 146 -> 150 us (its slabs are bound by the
-// per-head quantization arithmetic of B, not by the loads), so the key side keeps the run-time loop.
+// Measured at B4 L8192 H80 P64 N128 Q256: value side 115 -> 108 us; key side 146 -> 150 us, and 123 -> 128 us after the
+// prologue was slimmed (its slabs are bound by the per-head quantization arithmetic of B, not by the loads), so the key
+// side keeps the run-time loop.
 template <bool KEYSIDE, int NT, int NSLAB>
 __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
   const int Q = p.Q;
   float* gate_s = (float*)lds_raw;                    // [Q]
   float* bdeq_s = gate_s + Q;                         // [NT] b_gate / 127 (key side)
+  float* binv_s = bdeq_s + NT;                        // [NT] 127 / b_gate (key side)
+  float* xinv_s = binv_s + NT;                        // [64] reciprocal operand scale of the tile's P rows
+  float* req_s = xinv_s + 64;                         // [64] epilogue factor of the tile's P rows
   constexpr int kBW = NT + kPad;
-  uint32_t* xq = (uint32_t*)(bdeq_s + NT);            // [2][16][kXW]
+  uint32_t* xq = (uint32_t*)(req_s + 64);             // [2][16][kXW]
   uint32_t* bq = xq + 2 * 16 * kXW;                   // [2][16][kBW]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
   // heads vary fastest across consecutive workgroups: the B tile of a (batch, chunk) is shared by the heads of
   // a group and stays in L2 while they are swept
-  const int h = blockIdx.x % p.nheads;
-  const int tile = blockIdx.x / p.nheads;
-  const int ptile = tile / p.n_ntiles, ntile = tile % p.n_ntiles;
-  const int b = blockIdx.y / p.nchunks, c = blockIdx.y % p.nchunks;
-  const int g = h / (p.nheads / p.G);
+  // (grid = heads x chunks x (batch * tiles): no run-time integer division in front of the first request)
+  const int h = blockIdx.x, c = blockIdx.y;
+  const int b = div_magic(blockIdx.z, p.tiles_magic);
+  const int tile = (int)blockIdx.z - b * (p.P >> 6) * p.n_ntiles;
+  const int ptile = div_magic((uint32_t)tile, p.nt_magic), ntile = tile - ptile * p.n_ntiles;
+  const int g = div_magic((uint32_t)h, p.hpg_magic);
   const int p0 = ptile * 64, n0 = ntile * NT;
   const int limit = min(Q, p.seqlen - c * Q);
   const int64_t cs = (((int64_t)b * p.nheads + h) * p.nchunks + c) * Q;
@@ -108,9 +118,16 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   const int kg0 = min(tid, Q - 1);  // gate of token kg0 (threads past a short chunk repeat its last token)
   const float dA_k = p.dA[cs + kg0];
   const float dt_k = p.dt[cs + kg0];
+  // Scales: every distinct value of the tile is requested by one thread and turned into its reciprocal / ratio once,
+  // then shared through LDS (each thread used to fetch and divide its own 4 + 8 + 2 copies: fourteen IEEE divisions and as
+  // many 64-bit address computations per thread, a quarter of the kernel's instructions).
   float bg_t = 1.0f;
   if (KEYSIDE)
     bg_t = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)(n0 + (tid & (NT - 1))) * p.sbg_n];
+  const int prow = p0 + (tid & 63);
+  const float xs_t = p.xs[(int64_t)h * p.sxs_h + (int64_t)prow * p.sxs_p];
+  const float so_t = p.oqs[(int64_t)h * p.soq_h + (int64_t)prow * p.soq_p];
+  const float bs_t = KEYSIDE ? 0.0f : p.bscale_g[(int64_t)g * p.sbs_g];
 
   // fixed thread -> work mapping of the quantize phase: x slab = 16 token quads x 16 groups of 4 channels (all 256
   // threads), B slab = 16 token quads x NT/8 groups of 8 channels (threads without a B item load a clamped address)
@@ -120,40 +137,39 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   const int kqb = (NT == 128) ? (tid >> 4) : (tid / kBItems);
   const int cb8 = (NT == 128) ? (tid & 15) : (tid % kBItems);
 
-  float xs_raw[4], bg_raw[8];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) xs_raw[e] = p.xs[(int64_t)h * p.sxs_h + (int64_t)(p0 + 4 * c4x + e) * p.sxs_p];
-  if (KEYSIDE) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      bg_raw[e] = p.bgs[(int64_t)b * p.sbg_b + (int64_t)c * p.sbg_c + (int64_t)h * p.sbg_h + (int64_t)(n0 + 8 * cb8 + e) * p.sbg_n];
-  }
-  // scales of the epilogue (requested here: at their point of use they would expose one more round trip)
   const int pr = p0 + 16 * wave + rl;
-  const float xs_ep = p.xs[(int64_t)h * p.sxs_h + (int64_t)pr * p.sxs_p];
-  const float so_ep = p.oqs[(int64_t)h * p.soq_h + (int64_t)pr * p.soq_p];
-  const float bs_ep = KEYSIDE ? 0.0f : p.bscale_g[(int64_t)g * p.sbs_g];
 
   const int last = limit - 1;
-  const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0 + 4 * c4x;
-  const char* bg0 = (const char*)p.B + ((int64_t)b * p.sB_b + (int64_t)c * Q * p.sB_l + (int64_t)g * p.sB_g + n0 + 8 * cb8) * (KEYSIDE ? 2 : 1);
+  // wave-uniform 64-bit bases; the lane's own channel offset goes into the 32-bit part
+  const _Float16* xg = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h * p.sx_h + p0;
+  const char* bg0 = (const char*)p.B + ((int64_t)b * p.sB_b + (int64_t)c * Q * p.sB_l + (int64_t)g * p.sB_g + n0) * (KEYSIDE ? 2 : 1);
+  const uint32_t xlane = (uint32_t)c4x * 8u, blane = (uint32_t)cb8 * (KEYSIDE ? 16u : 8u);
   const int64_t bstep = p.sB_l * (KEYSIDE ? 2 : 1);  // bytes per token
   lq_v2i xrA[4], xrB[4];  // x: 4 tokens x 4 fp16 (two sets: the slab being quantized and the one in flight)
   lq_v4i brA[4], brB[4];  // key side: 4 tokens x 8 fp16; value side: only [t][0..1] used (8 int8)
 
   // token * stride stays below 2^31 and both factors below 2^23 (checked by the launcher): a full-rate 24-bit multiply
-  // instead of the quarter-rate 64-bit one, eight times per slab
+  // instead of the quarter-rate 64-bit one.  A full chunk needs no clamping of the token index, so its row offsets are
+  // formed once and advanced by a scalar per slab; a ragged last chunk (wave-uniform) multiplies the clamped index.
   const int sxl = (int)p.sx_l, bst = (int)bstep;
+  const bool ragged = limit < Q;
+  uint32_t xo[4], bo4[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    xo[t] = (uint32_t)__mul24(4 * kqx + t, sxl) * 2u + xlane;
+    bo4[t] = (uint32_t)__mul24(4 * kqb + t, bst) + blane;
+  }
   auto load_slab = [&](int k0, lq_v2i (&xr)[4], lq_v4i (&br)[4]) {
+    const uint32_t xk = (uint32_t)(k0 * sxl) * 2u, bk = (uint32_t)(k0 * bst);  // scalar
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      const int kx = min(k0 + 4 * kqx + t, last);
-      xr[t] = *(const lq_v2i*)(xg + __mul24(kx, sxl));
-      const int kb = min(k0 + 4 * kqb + t, last);
+      const uint32_t ox = ragged ? (uint32_t)__mul24(min(k0 + 4 * kqx + t, last), sxl) * 2u + xlane : xo[t] + xk;
+      const uint32_t ob = ragged ? (uint32_t)__mul24(min(k0 + 4 * kqb + t, last), bst) + blane : bo4[t] + bk;
+      xr[t] = *(const lq_v2i*)((const char*)xg + ox);
       if (KEYSIDE) {
-        br[t] = *(const lq_v4i*)(bg0 + __mul24(kb, bst));
+        br[t] = *(const lq_v4i*)(bg0 + ob);
       } else {
-        const lq_v2i v = *(const lq_v2i*)(bg0 + __mul24(kb, bst));
+        const lq_v2i v = *(const lq_v2i*)(bg0 + ob);
         br[t][0] = v[0], br[t][1] = v[1];
       }
     }
@@ -169,20 +185,32 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   }
   for (int k = tid + 256; k < Q; k += 256)  // chunks longer than the workgroup
     gate_s[k] = k < limit ? lq_expf(dA_last - p.dA[cs + k]) * p.dt[cs + k] : 0.0f;
-  if (KEYSIDE) bdeq_s[tid & (NT - 1)] = bg_t / 127.0f;
-  float xinv[4], binv[8];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) xinv[e] = KEYSIDE ? 1.0f / fmaxf(xs_raw[e], 1e-10f) : 1.0f / xs_raw[e];
   if (KEYSIDE) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) binv[e] = 127.0f / bg_raw[e];
+    bdeq_s[tid & (NT - 1)] = bg_t / 127.0f;
+    binv_s[tid & (NT - 1)] = 127.0f / bg_t;
+  }
+  xinv_s[tid & 63] = KEYSIDE ? 1.0f / fmaxf(xs_t, 1e-10f) : 1.0f / xs_t;
+  {
+    const float ratio = xs_t / so_t;
+    req_s[tid & 63] = KEYSIDE ? ratio : ratio * bs_t;
   }
 
   lq_v4i acc[NT / 16];
 #pragma unroll
   for (int q = 0; q < NT / 16; ++q) acc[q] = lq_v4i{0, 0, 0, 0};
 
-  __syncthreads();  // gates visible
+  __syncthreads();  // gates and scale tables visible
+  float xinv[4], binv[8];
+  {
+    const lq_v4f xv = *(const lq_v4f*)(xinv_s + 4 * c4x);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) xinv[e] = xv[e];
+    if (KEYSIDE) {
+      const lq_v4f b0 = *(const lq_v4f*)(binv_s + 8 * cb8), b1 = *(const lq_v4f*)(binv_s + 8 * cb8 + 4);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) binv[e] = e < 4 ? b0[e & 3] : b1[e & 3];
+    }
+  }
 
   const int nslab = Q >> 6;
   auto slab = [&](int s, lq_v2i (&xr)[4], lq_v4i (&br)[4], auto post) {
@@ -280,8 +308,8 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   }
 
   // ---- epilogue: lane holds N = n0 + 16q + 4kg + {0..3} of P row p0 + 16*wave + rl
-  const float ratio = xs_ep / so_ep;
-  const float req = KEYSIDE ? 0.0f : ratio * bs_ep;
+  const float ratio = req_s[16 * wave + rl];  // key side: x_scale / S_out; value side: (alpha / S_out) * bscale
+  const float req = ratio;
   int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + pr) * p.N + n0;
   uint32_t dq[NT / 16];  // dword q of this lane: codes of N = n0 + 16 q + 4 kg + {0..3}
 #pragma unroll
@@ -325,16 +353,19 @@ int launch(const Params& p, hipStream_t stream) {
   const int bmod = KEYSIDE ? 8 : 8, balign = KEYSIDE ? 16 : 8;
   if (p.sB_b % bmod || p.sB_l % bmod || p.sB_g % bmod || !al(p.B, balign)) return LQ_ERR_SHAPE;
   if (!al(p.states, 16)) return LQ_ERR_SHAPE;
-  const int64_t by = (int64_t)p.batch * p.nchunks;
-  if (by > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
+  if (p.nchunks > 65535 || p.nheads > 65535) return LQ_ERR_SHAPE;
+  auto magic = [](uint32_t d) { return d == 1 ? 0u : (uint32_t)(0x100000000ull / d) + 1u; };
   if (p.sx_l < 0 || p.sB_l < 0 || p.sx_l >= (1 << 22) || p.sB_l >= (1 << 22) || (int64_t)p.Q * p.sx_l >= (1ll << 30) ||
       (int64_t)p.Q * p.sB_l >= (1ll << 30))
     return LQ_ERR_SHAPE;  // 24-bit token * stride products in the slab loads
   Params q = p;
   if (p.N % 128 == 0) {
     q.n_ntiles = p.N / 128;
-    const size_t lds = (size_t)p.Q * 4 + 128 * 4 + (2 * 16 * kXW + 2 * 16 * (128 + kPad)) * 4;
-    dim3 grid((p.P / 64) * q.n_ntiles * p.nheads, (unsigned)by, 1);
+    const size_t lds = (size_t)p.Q * 4 + (2 * 128 + 128) * 4 + (2 * 16 * kXW + 2 * 16 * (128 + kPad)) * 4;
+    const int tiles = (p.P / 64) * q.n_ntiles;
+    if ((int64_t)p.batch * tiles > 65535) return LQ_ERR_SHAPE;
+    q.hpg_magic = magic((uint32_t)(p.nheads / p.G)), q.tiles_magic = magic((uint32_t)tiles), q.nt_magic = magic((uint32_t)q.n_ntiles);
+    dim3 grid(p.nheads, p.nchunks, p.batch * tiles);
     if (!KEYSIDE && p.Q == 256)
       hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128, 4>), grid, dim3(256), lds, stream, q);
     else if (!KEYSIDE && p.Q == 128)
@@ -343,8 +374,11 @@ int launch(const Params& p, hipStream_t stream) {
       hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128, 0>), grid, dim3(256), lds, stream, q);
   } else {
     q.n_ntiles = p.N / 64;
-    const size_t lds = (size_t)p.Q * 4 + 64 * 4 + (2 * 16 * kXW + 2 * 16 * (64 + kPad)) * 4;
-    dim3 grid((p.P / 64) * q.n_ntiles * p.nheads, (unsigned)by, 1);
+    const size_t lds = (size_t)p.Q * 4 + (2 * 64 + 128) * 4 + (2 * 16 * kXW + 2 * 16 * (64 + kPad)) * 4;
+    const int tiles = (p.P / 64) * q.n_ntiles;
+    if ((int64_t)p.batch * tiles > 65535) return LQ_ERR_SHAPE;
+    q.hpg_magic = magic((uint32_t)(p.nheads / p.G)), q.tiles_magic = magic((uint32_t)tiles), q.nt_magic = magic((uint32_t)q.n_ntiles);
+    dim3 grid(p.nheads, p.nchunks, p.batch * tiles);
     if (!KEYSIDE && p.Q == 256)
       hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64, 4>), grid, dim3(256), lds, stream, q);
     else if (!KEYSIDE && p.Q == 128)
