@@ -11,79 +11,116 @@
 
 namespace {
 
-template <bool B_IS_FP>
+typedef uint32_t lq_v2u __attribute__((ext_vector_type(2)));
+
+// clamp to [-127, 127] then round half even; returns a dword whose low byte is the INT8 code
+LQ_DEV uint32_t rint_code(float y) {
+  const float c = __builtin_amdgcn_fmed3f(y, -127.0f, 127.0f);
+  return __float_as_uint(c + 12582912.0f);
+}
+
+LQ_DEV uint32_t pack_low_bytes(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+  const uint32_t lo = __builtin_amdgcn_perm(b, a, 0x0c0c0400u);  // {a.b0, b.b0, 0, 0}
+  const uint32_t hi = __builtin_amdgcn_perm(d, c, 0x04000c0cu);  // {0, 0, c.b0, d.b0}
+  return lo | hi;
+}
+
+// One wavefront per 64 x 64 output tile.  N64 = N / 64 contraction steps, all of whose operands are requested before
+// the first is used, from clamped (always valid) rows: a request inside `if (row < limit)` is waited for where the
+// branches join, and a run-time loop over N put a second memory round trip behind the first.  Rows past the sequence
+// end are zeroed after the fact.  The epilogue transposes each lane's 4 x 4 block of code dwords across the four lane
+// groups so that a lane stores 16 contiguous bytes: 4 stores per lane instead of 16, 64 contiguous bytes per row.
+template <bool B_IS_FP, int N64>
 __global__ __launch_bounds__(64, 2) void bmm_chunk_kernel(const int8_t* __restrict__ a, int64_t sa_b, int64_t sa_l,
                                                        int64_t sa_g, const void* __restrict__ bv, int64_t sb_b,
                                                        int64_t sb_l, int64_t sb_g, const float* __restrict__ a_scale,
                                                        const float* __restrict__ b_scale,
                                                        const float* __restrict__ cb_scale, int8_t* __restrict__ out,
-                                                       int seqlen, int G, int N, int Q, int nchunks) {
+                                                       int seqlen, int G, int Q, int nchunks, uint32_t tiles_magic,
+                                                       uint32_t g_magic) {
   const int lane = threadIdx.x, rl = lane & 15, kg = lane >> 4;
-  const int tiles = Q >> 6;
-  const int mt64 = blockIdx.x / tiles, kt64 = blockIdx.x % tiles;
+  // floor(2^32 / d) + 1 multipliers (0 for d == 1) stand in for the run-time divisions by tiles per row and groups
+  const int mt64 = tiles_magic ? (int)__umulhi(blockIdx.x, tiles_magic) : (int)blockIdx.x;
+  const int kt64 = (int)blockIdx.x - mt64 * (Q >> 6);
   const int b = blockIdx.y;
-  const int c = blockIdx.z / G, g = blockIdx.z % G;
+  const int c = g_magic ? (int)__umulhi(blockIdx.z, g_magic) : (int)blockIdx.z;
+  const int g = (int)blockIdx.z - c * G;
   const int limit = min(Q, seqlen - c * Q);
-  const float a_sc = a_scale[g], b_sc = b_scale[g];
+  const float a_sc = a_scale[g], b_sc = b_scale[g], cb_sc = cb_scale[g];
+
+  const int8_t* ap = a + (int64_t)b * sa_b + (int64_t)c * Q * sa_l + (int64_t)g * sa_g;
+  const char* bp = (const char*)bv + ((int64_t)b * sb_b + (int64_t)c * Q * sb_l + (int64_t)g * sb_g) * (B_IS_FP ? 2 : 1);
+  const uint32_t sal = (uint32_t)sa_l, sbl = (uint32_t)sb_l * (B_IS_FP ? 2u : 1u);
+  lq_v4i cop[N64][4], braw[N64][4][B_IS_FP ? 2 : 1];
+  bool mlive[4], klive[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = mt64 * 64 + i * 16 + rl, k = kt64 * 64 + i * 16 + rl;
+    mlive[i] = m < limit, klive[i] = k < limit;
+    const uint32_t mo = __umul24((uint32_t)min(m, limit - 1), sal) + (uint32_t)kg * 16u;
+    const uint32_t ko = __umul24((uint32_t)min(k, limit - 1), sbl) + (uint32_t)kg * (B_IS_FP ? 32u : 16u);
+#pragma unroll
+    for (int n = 0; n < N64; ++n) {
+      cop[n][i] = *(const lq_v4i*)(ap + mo + 64u * n);
+      braw[n][i][0] = *(const lq_v4i*)(bp + ko + (B_IS_FP ? 128u : 64u) * n);
+      if (B_IS_FP) braw[n][i][1] = *(const lq_v4i*)(bp + ko + 128u * n + 16u);
+    }
+  }
   const float b_inv = 1.0f / b_sc;
+  const float inv_scb = (a_sc * b_sc) / cb_sc;
 
   lq_v4i acc[4][4];  // [k tile][m tile]
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = lq_v4i{0, 0, 0, 0};
-
-  const int8_t* ap = a + (int64_t)b * sa_b + (int64_t)c * Q * sa_l + (int64_t)g * sa_g;
-  for (int n0 = 0; n0 < N; n0 += 64) {
-    const int nn = n0 + kg * 16;
-    lq_v4i cop[4], bop[4];
+#pragma unroll
+  for (int n = 0; n < N64; ++n) {
+    lq_v4i bop[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int m = mt64 * 64 + i * 16 + rl;
-      cop[i] = lq_v4i{0, 0, 0, 0};
-      if (m < limit) cop[i] = *(const lq_v4i*)(ap + (int64_t)m * sa_l + nn);
-      const int k = kt64 * 64 + i * 16 + rl;
-      bop[i] = lq_v4i{0, 0, 0, 0};
-      if (k < limit) {
-        if (B_IS_FP) {
-          const _Float16* bp = (const _Float16*)bv + (int64_t)b * sb_b + ((int64_t)c * Q + k) * sb_l + (int64_t)g * sb_g + nn;
-          const lq_v8h h0 = *(const lq_v8h*)bp;
-          const lq_v8h h1 = *(const lq_v8h*)(bp + 8);
-          int code[16];
+      if (!mlive[i]) cop[n][i] = lq_v4i{0, 0, 0, 0};
+      if (B_IS_FP) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            code[e] = lq_q_rint((float)h0[e] * b_inv, -127, 127);
-            code[8 + e] = lq_q_rint((float)h1[e] * b_inv, -127, 127);
-          }
+        for (int d = 0; d < 4; ++d) {
+          const lq_v8h hv = __builtin_bit_cast(lq_v8h, braw[n][i][d >> 1]);
+          uint32_t cd[4];
 #pragma unroll
-          for (int d = 0; d < 4; ++d)
-            bop[i][d] = (int)lq_pack4(code[4 * d], code[4 * d + 1], code[4 * d + 2], code[4 * d + 3]);
-        } else {
-          const int8_t* bp = (const int8_t*)bv + (int64_t)b * sb_b + ((int64_t)c * Q + k) * sb_l + (int64_t)g * sb_g + nn;
-          bop[i] = *(const lq_v4i*)bp;
+          for (int e = 0; e < 4; ++e) cd[e] = rint_code((float)hv[4 * (d & 1) + e] * b_inv);
+          bop[i][d] = (int)pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
         }
+      } else {
+        bop[i] = braw[n][i][0];
       }
+      if (!klive[i]) bop[i] = lq_v4i{0, 0, 0, 0};
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = lq_mfma_i8(bop[i], cop[j], acc[i][j]);
+      for (int j = 0; j < 4; ++j) acc[i][j] = lq_mfma_i8(bop[i], cop[n][j], acc[i][j]);
   }
 
-  const float inv_scb = (a_sc * b_sc) / cb_scale[g];
-  int8_t* op = out + ((((int64_t)b * nchunks + c) * G + g) * Q) * Q;
+  int8_t* op = out + ((((int64_t)b * nchunks + c) * G + g) * Q) * Q + (int64_t)(mt64 * 64) * Q + kt64 * 64;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int j = 0; j < 4; ++j) {
+    // accumulator rows = k (4 consecutive per lane: k = 16 i + 4 kg + r), column = m = 16 j + rl
+    uint32_t d[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // accumulator rows = k (4 consecutive per lane), column = m
-      const int m = mt64 * 64 + j * 16 + rl;
-      const int k = kt64 * 64 + i * 16 + 4 * kg;
-      int code[4];
+    for (int i = 0; i < 4; ++i) {
+      uint32_t cd[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) code[r] = lq_q_rint((float)acc[i][j][r] * inv_scb, -127, 127);
-      *(uint32_t*)(op + (int64_t)m * Q + k) = lq_pack4(code[0], code[1], code[2], code[3]);
+      for (int r = 0; r < 4; ++r) cd[r] = rint_code((float)acc[i][j][r] * inv_scb);
+      d[i] = pack_low_bytes(cd[0], cd[1], cd[2], cd[3]);
     }
+    // dword i of lane group kg covers k = 16 i + 4 kg ..: transposing register index with lane group leaves lane group
+    // kg with the four dwords of k = 16 kg .. 16 kg + 15
+    lq_v2u t;
+    t = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false), d[0] = t[0], d[2] = t[1];
+    t = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false), d[1] = t[0], d[3] = t[1];
+    t = __builtin_amdgcn_permlane16_swap(d[0], d[1], false, false), d[0] = t[0], d[1] = t[1];
+    t = __builtin_amdgcn_permlane16_swap(d[2], d[3], false, false), d[2] = t[0], d[3] = t[1];
+    *(lq_v4i*)(op + (uint32_t)((16 * j + rl) * Q + 16 * kg)) = lq_v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+  }
 }
 
 bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
@@ -94,22 +131,31 @@ extern "C" int lq_bmm_chunk(const lq_bmm_chunk_args* a, hipStream_t stream) {
   if (!a || !a->a || !a->b || !a->a_scale || !a->b_scale || !a->cb_scale || !a->out) return LQ_ERR_NULL;
   if (a->batch <= 0 || a->seqlen <= 0 || a->ngroups <= 0 || a->batch > 65535) return LQ_ERR_SHAPE;
   const int Q = a->chunk_size, N = a->dstate;
-  if (Q < 64 || Q % 64 != 0 || N < 64 || N % 64 != 0) return LQ_ERR_SHAPE;
+  if (Q < 64 || Q % 64 != 0 || Q > 4096 || N < 64 || N % 64 != 0 || N > 256) return LQ_ERR_SHAPE;
   if (a->a_stride_b % 16 || a->a_stride_l % 16 || a->a_stride_g % 16 || !al(a->a, 16)) return LQ_ERR_SHAPE;
   const int bal = 16;  // 16 int8 or 8 fp16 per vector load
   const int bmod = a->b_is_fp ? 8 : 16;
-  if (a->b_stride_b % bmod || a->b_stride_l % bmod || a->b_stride_g % bmod || !al(a->b, bal) || !al(a->out, 4))
+  if (a->b_stride_b % bmod || a->b_stride_l % bmod || a->b_stride_g % bmod || !al(a->b, bal) || !al(a->out, 16))
+    return LQ_ERR_SHAPE;
+  // 24-bit row * pitch products and 32-bit lane offsets inside a chunk
+  if (a->a_stride_l < 0 || a->b_stride_l < 0 || a->a_stride_l >= (1 << 23) || a->b_stride_l >= (1 << 22) ||
+      (int64_t)Q * a->a_stride_l >= (1ll << 31) || (int64_t)Q * a->b_stride_l * 2 >= (1ll << 31))
     return LQ_ERR_SHAPE;
   const int nchunks = (a->seqlen + Q - 1) / Q;
   if ((int64_t)nchunks * a->ngroups > 65535) return LQ_ERR_SHAPE;
+  const uint32_t shift = Q == 64 ? 0u : (uint32_t)(0x100000000ull / (uint32_t)(Q / 64)) + 1u;  // tiles per row, as a multiplier
+  const uint32_t g_magic = a->ngroups == 1 ? 0u : (uint32_t)(0x100000000ull / (uint32_t)a->ngroups) + 1u;
   dim3 grid((Q / 64) * (Q / 64), a->batch, nchunks * a->ngroups);
-  if (a->b_is_fp)
-    hipLaunchKernelGGL((bmm_chunk_kernel<true>), grid, dim3(64), 0, stream, a->a, a->a_stride_b, a->a_stride_l,
-                       a->a_stride_g, a->b, a->b_stride_b, a->b_stride_l, a->b_stride_g, a->a_scale, a->b_scale,
-                       a->cb_scale, a->out, a->seqlen, a->ngroups, N, Q, nchunks);
-  else
-    hipLaunchKernelGGL((bmm_chunk_kernel<false>), grid, dim3(64), 0, stream, a->a, a->a_stride_b, a->a_stride_l,
-                       a->a_stride_g, a->b, a->b_stride_b, a->b_stride_l, a->b_stride_g, a->a_scale, a->b_scale,
-                       a->cb_scale, a->out, a->seqlen, a->ngroups, N, Q, nchunks);
+#define LQ_BMM_LAUNCH(FP, NN)                                                                                              \
+  hipLaunchKernelGGL((bmm_chunk_kernel<FP, NN>), grid, dim3(64), 0, stream, a->a, a->a_stride_b, a->a_stride_l,            \
+                     a->a_stride_g, a->b, a->b_stride_b, a->b_stride_l, a->b_stride_g, a->a_scale, a->b_scale, a->cb_scale, \
+                     a->out, a->seqlen, a->ngroups, Q, nchunks, shift, g_magic)
+  switch (N / 64) {
+    case 1: if (a->b_is_fp) LQ_BMM_LAUNCH(true, 1); else LQ_BMM_LAUNCH(false, 1); break;
+    case 2: if (a->b_is_fp) LQ_BMM_LAUNCH(true, 2); else LQ_BMM_LAUNCH(false, 2); break;
+    case 3: if (a->b_is_fp) LQ_BMM_LAUNCH(true, 3); else LQ_BMM_LAUNCH(false, 3); break;
+    default: if (a->b_is_fp) LQ_BMM_LAUNCH(true, 4); else LQ_BMM_LAUNCH(false, 4); break;
+  }
+#undef LQ_BMM_LAUNCH
   return lq_check_launch();
 }
