@@ -107,6 +107,9 @@ typedef struct {
   int64_t bgs_stride_b, bgs_stride_c, bgs_stride_h, bgs_stride_n;
   int8_t* states;            /* (B,nc,H,P,N) int8 contiguous */
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+  float* b_rowmax;           /* NULL, or (B,L,G) fp32 scratch: the call first fills it with max_n |B[b,l,g,n]| and then leaves
+                                out every 64-token slab whose gated key codes are provably all zero (same result, bit for
+                                bit; see the kernel's header).  Contents undefined on entry. */
 } lq_chunk_state_key_args;
 int lq_chunk_state_key(const lq_chunk_state_key_args* args, hipStream_t stream);
 
@@ -544,6 +547,20 @@ typedef struct {
   int32_t mode;
 } lq_absmax_args;
 int lq_absmax(const lq_absmax_args* args, hipStream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference): a matrix-core-only launch whose rate is the MFMA issue peak of
+ * the machine, the denominator of the "fraction of INT8 MFMA peak" figures (the reference's metric is quoted against
+ * the chip's INT8 peak; this measures it instead of assuming it).  Work per launch: blocks * 4 waves * iters * 8
+ * instructions of 16x16x64 INT8 (32768 ops each) or 16x16x32 fp16 (16384 flops each), or blocks * 4 * iters * 4
+ * instructions of 32x32x32 INT8 (65536 ops each).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct {
+  int32_t kind;              /* 0: i32 16x16x64 i8;  1: f32 16x16x32 f16;  2: i32 32x32x32 i8 */
+  int32_t iters, blocks;
+  int32_t* sink;             /* one device int, never written in practice */
+} lq_probe_mfma_args;
+int lq_probe_mfma(const lq_probe_mfma_args* args, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 10; }
+extern "C" int lq_abi_version(void) { return 11; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)
@@ -33,5 +33,6 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_zoo_wy_prep_args);
   LQ_SIZE_OF(lq_zoo_rotate_qkv_args);
   LQ_SIZE_OF(lq_ssd_combined_args);
+  LQ_SIZE_OF(lq_probe_mfma_args);
   return LQ_ERR_SHAPE;
 }

@@ -306,19 +306,23 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       const lq_v2i cw = cwr[s & 3];
       if (s + 4 < NS) cwr[s & 3] = cb_slab(s + 4);
       const _Float16 sh = (_Float16)fexp2(aE - dA2_s[32 * J + 31]);
-      const lq_v2h s2 = {sh, sh};
-      lq_v4i xop[4];  // token pairs 16 J + 4 kg .. + 3 of channel 4 rl + j
+      // a slab whose factor underflows fp16 (more than 25 octaves of decay between it and the tile) would contribute
+      // fp16(code * 0) = 0 to every product: it is left out (wave-uniform; strongly decaying heads skip most slabs)
+      if (__builtin_amdgcn_readfirstlane((int)__builtin_bit_cast(uint16_t, sh)) != 0) {
+        const lq_v2h s2 = {sh, sh};
+        lq_v4i xop[4];  // token pairs 16 J + 4 kg .. + 3 of channel 4 rl + j
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xS + (4 * J + kg) * kQuad + (j * 16 + rl) * 4);
-      lq_v4i aw;
-      uint32_t lo, hi;
-      i8x4_to_f16x4((uint32_t)cw[0], s2, lo, hi);
-      aw[0] = (int)lo, aw[1] = (int)hi;
-      i8x4_to_f16x4((uint32_t)cw[1], s2, lo, hi);
-      aw[2] = (int)lo, aw[3] = (int)hi;
-      const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
+        for (int j = 0; j < 4; ++j) xop[j] = *(const lq_v4i*)(xS + (4 * J + kg) * kQuad + (j * 16 + rl) * 4);
+        lq_v4i aw;
+        uint32_t lo, hi;
+        i8x4_to_f16x4((uint32_t)cw[0], s2, lo, hi);
+        aw[0] = (int)lo, aw[1] = (int)hi;
+        i8x4_to_f16x4((uint32_t)cw[1], s2, lo, hi);
+        aw[2] = (int)lo, aw[3] = (int)hi;
+        const lq_v8h aop = __builtin_bit_cast(lq_v8h, aw);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) off[j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[j]);
+        for (int j = 0; j < 4; ++j) off[j] = lq_mfma_f16(aop, __builtin_bit_cast(lq_v8h, xop[j]), off[j]);
+      }
     }
     if (NS > 0) flush(1, aE1 - kf);
   }

@@ -20,6 +20,13 @@
 // stores them as one dword).  The gates of the whole chunk are evaluated once per workgroup.
 // Round-half-even + clamp + int conversion is one fp32 add of 1.5*2^23 after the clamp (the low byte of the
 // sum's bit pattern is the two's-complement code).
+// Key side, zero-slab elision: the gate exp(dA_last - dA_k) * dt_k decays towards the start of the chunk, and a gated key
+// code rint((B * gate) * 127 / b_gate) is exactly zero once gate_k * max_n |B[k, n]| * max_n (127 / b_gate[n]) < 0.5.  A
+// 64-token slab all of whose tokens satisfy that bound contributes nothing to the INT32 product, so neither its x rows nor
+// its B rows are fetched or quantized; the per-token max_n |B| comes from a small pre-pass over B (shared by all heads).
+// The result is bit-identical; the saving depends on the data (none for slowly decaying heads, three slabs of four for
+// per-token decays of 0.1 and more at chunk 256).  Slabs are walked from the end of the chunk backwards, so the last one
+// (live whenever anything is) can be requested before the gates are known.
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -45,6 +52,7 @@ struct Params {
   int64_t soq_h, soq_p;
   const float* bgs;
   int64_t sbg_b, sbg_c, sbg_h, sbg_n;
+  const float* rowmax;  // key side, optional: (B,L,G) max_n |B|, filled by row_absmax_kernel
   int8_t* states;
   int batch, seqlen, nheads, P, G, N, Q, nchunks, n_ntiles;
   // floor(2^32 / d) + 1 for d = heads per group, tiles per (batch, chunk, head), N tiles per P tile; 0 when d == 1:
@@ -127,6 +135,17 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   const int prow = p0 + (tid & 63);
   const float xs_t = p.xs[(int64_t)h * p.sxs_h + (int64_t)prow * p.sxs_p];
   const float so_t = p.oqs[(int64_t)h * p.soq_h + (int64_t)prow * p.soq_p];
+  // per-token max |B| of the first four slabs before the last (slabs further out, in chunks longer than 320 tokens, are
+  // fetched when they are tested); clamped rows, dead data when the elision is off
+  const bool elide = KEYSIDE && p.rowmax != nullptr;
+  const int nslab_all = Q >> 6;
+  float rmv[4];
+  {
+    const float* rmp = elide ? p.rowmax + ((int64_t)b * p.seqlen + (int64_t)c * Q) * p.G + g : p.dt + cs;
+    const int rstride = elide ? p.G : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rmv[i] = rmp[(int64_t)min(max(64 * (nslab_all - 2 - i), 0) + lane, limit - 1) * rstride];
+  }
   const float bs_t = KEYSIDE ? 0.0f : p.bscale_g[(int64_t)g * p.sbs_g];
 
   // fixed thread -> work mapping of the quantize phase: x slab = 16 token quads x 16 groups of 4 channels (all 256
@@ -174,7 +193,7 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
       }
     }
   };
-  load_slab(0, xrA, brA);
+  load_slab(NSLAB > 0 ? 0 : 64 * (nslab_all - 1), xrA, brA);  // the run-time loop starts at the last slab
 
   // ---- gates of the whole chunk, dequantization scales of B, reciprocal operand scales
   // (written by every thread, duplicates included: a store under `if (tid < Q)` lets the compiler sink the requests
@@ -213,10 +232,10 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   }
 
   const int nslab = Q >> 6;
-  auto slab = [&](int s, lq_v2i (&xr)[4], lq_v4i (&br)[4], auto post) {
+  auto slab = [&](int s, int par, lq_v2i (&xr)[4], lq_v4i (&br)[4], auto post) {
     const int k0 = s * 64;
-    uint32_t* xb = xq + (s & 1) * 16 * kXW;
-    uint32_t* bb = bq + (s & 1) * 16 * kBW;
+    uint32_t* xb = xq + (par & 1) * 16 * kXW;
+    uint32_t* bb = bq + (par & 1) * 16 * kBW;
     // ---- quantize this slab into LDS (codes of 4 consecutive tokens of one channel form one dword)
     {
       float gt[4];
@@ -295,16 +314,38 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
       if (s & 1) {
         if (s + 1 < NSLAB) load_slab(64 * (s + 1), xrA, brA);
         asm volatile("" ::: "memory");  // the requests stay ahead of the LDS traffic below
-        slab(s, xrB, brB, [] {});
+        slab(s, s, xrB, brB, [] {});
       } else {
         if (s + 1 < NSLAB) load_slab(64 * (s + 1), xrB, brB);
         asm volatile("" ::: "memory");
-        slab(s, xrA, brA, [] {});
+        slab(s, s, xrA, brA, [] {});
       }
     }
   } else {
-    for (int s = 0; s < nslab; ++s)
-      slab(s, xrA, brA, [&] { if (s + 1 < nslab) load_slab(64 * (s + 1), xrA, brA); });
+    // which slabs before the last can be left out (bit s of `live`; wave-uniform, every wave evaluates all of them)
+    uint64_t live = nslab >= 64 ? ~0ull : ((1ull << nslab) - 1);
+    if (elide) {
+      float bmax = 0.0f;
+      for (int n = lane; n < NT; n += 64) bmax = fmaxf(bmax, binv_s[n]);
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) bmax = fmaxf(bmax, __shfl_xor(bmax, o));
+      live = 1ull << (nslab - 1);
+      for (int i = 0; i < nslab - 1; ++i) {
+        const int sidx = nslab - 2 - i, k = 64 * sidx + lane;
+        float rm = rmv[i & 3];
+        if (i >= 4) rm = p.rowmax[((int64_t)b * p.seqlen + (int64_t)c * Q + min(k, limit - 1)) * p.G + g];
+        // not provably zero (NaN / Inf in B keep the slab)
+        const bool keep = !((gate_s[k] * rm) * bmax < 0.499f);
+        if (__ballot(keep)) live |= 1ull << sidx;
+      }
+    }
+    int cur = nslab - 1;
+    for (int it = 0; cur >= 0; ++it) {
+      const uint64_t below = live & ((1ull << cur) - 1);
+      const int next = below ? 63 - __builtin_clzll(below) : -1;
+      slab(cur, it, xrA, brA, [&] { if (next >= 0) load_slab(64 * next, xrA, brA); });
+      cur = next;
+    }
   }
 
   // ---- epilogue: lane holds N = n0 + 16q + 4kg + {0..3} of P row p0 + 16*wave + rl
@@ -343,6 +384,31 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   }
 }
 
+// max_n |B[b, l, g, n]| of the fp16 key tensor -> (B, L, G) fp32; N / 8 lanes per row, 16 bytes per lane
+template <int N>
+__global__ __launch_bounds__(256) void row_absmax_kernel(const _Float16* __restrict__ B, int64_t s_b, int64_t s_l, int64_t s_g,
+                                                         float* __restrict__ out, int L, int G, int64_t rows) {
+  constexpr int LPR = N / 8, RPB = 256 / LPR;
+  const int sub = threadIdx.x % LPR;
+  const int64_t row = min((int64_t)blockIdx.x * RPB + threadIdx.x / LPR, rows - 1);  // the tail repeats the last row
+  const int g = (int)(row % G);
+  const int64_t bl = row / G;
+  const int64_t bb = bl / L, l = bl % L;
+  const lq_v8h v = *(const lq_v8h*)(B + bb * s_b + l * s_l + (int64_t)g * s_g + 8 * sub);
+  float m = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float a = __builtin_fabsf((float)v[e]);
+    m = (a > m || a != a) ? a : m;  // NaN propagates, so a row holding one is never elided
+  }
+#pragma unroll
+  for (int o = 1; o < LPR; o <<= 1) {
+    const float t = __shfl_xor(m, o);
+    m = (t > m || t != t) ? t : m;
+  }
+  if (sub == 0) out[row] = m;
+}
+
 bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
 
 template <bool KEYSIDE>
@@ -359,6 +425,23 @@ int launch(const Params& p, hipStream_t stream) {
       (int64_t)p.Q * p.sB_l >= (1ll << 30))
     return LQ_ERR_SHAPE;  // 24-bit token * stride products in the slab loads
   Params q = p;
+  if (KEYSIDE && p.rowmax) {
+    if (p.N != 64 && p.N != 128 && p.N != 256) {
+      q.rowmax = nullptr;  // no pre-pass for this width: every slab is processed
+    } else {
+      const int64_t rows = (int64_t)p.batch * p.seqlen * p.G;
+      const int rpb = 256 / (p.N / 8);
+      const dim3 rgrid((unsigned)((rows + rpb - 1) / rpb));
+      float* out = const_cast<float*>(p.rowmax);
+      const _Float16* Bp = (const _Float16*)p.B;
+      if (p.N == 64)
+        hipLaunchKernelGGL((row_absmax_kernel<64>), rgrid, dim3(256), 0, stream, Bp, p.sB_b, p.sB_l, p.sB_g, out, p.seqlen, p.G, rows);
+      else if (p.N == 128)
+        hipLaunchKernelGGL((row_absmax_kernel<128>), rgrid, dim3(256), 0, stream, Bp, p.sB_b, p.sB_l, p.sB_g, out, p.seqlen, p.G, rows);
+      else
+        hipLaunchKernelGGL((row_absmax_kernel<256>), rgrid, dim3(256), 0, stream, Bp, p.sB_b, p.sB_l, p.sB_g, out, p.seqlen, p.G, rows);
+    }
+  }
   if (p.N % 128 == 0) {
     q.n_ntiles = p.N / 128;
     const size_t lds = (size_t)p.Q * 4 + (2 * 128 + 128) * 4 + (2 * 16 * kXW + 2 * 16 * (128 + kPad)) * 4;
@@ -423,6 +506,7 @@ extern "C" int lq_chunk_state_key(const lq_chunk_state_key_args* a, hipStream_t 
   p.xs = a->x_scale_hp, p.sxs_h = a->xs_stride_h, p.sxs_p = a->xs_stride_p;
   p.oqs = a->out_qscale, p.soq_h = a->oqs_stride_h, p.soq_p = a->oqs_stride_p;
   p.bgs = a->b_gate_scale;
+  p.rowmax = a->b_rowmax;
   p.sbg_b = a->bgs_stride_b, p.sbg_c = a->bgs_stride_c, p.sbg_h = a->bgs_stride_h, p.sbg_n = a->bgs_stride_n;
   p.states = a->states;
   p.batch = a->batch, p.seqlen = a->seqlen, p.nheads = a->nheads, p.P = a->headdim, p.G = a->ngroups, p.N = a->dstate;

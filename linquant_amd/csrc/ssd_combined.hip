@@ -13,7 +13,7 @@ constexpr int64_t kAlign = 256;
 int64_t up(int64_t n) { return (n + kAlign - 1) / kAlign * kAlign; }
 
 struct Layout {
-  int64_t dt, dA, states, passed, cb, total;
+  int64_t dt, dA, states, passed, cb, rowmax, total;
   int nchunks;
 };
 
@@ -31,7 +31,8 @@ int plan(const lq_ssd_combined_args* a, Layout* l) {
   l->states = l->dA + up(fl);
   l->passed = l->states + up(st);
   l->cb = l->passed + up(st);
-  l->total = l->cb + up(cb);
+  l->rowmax = l->cb + up(cb);
+  l->total = l->rowmax + up((int64_t)a->batch * a->seqlen * a->ngroups * 4);
   return LQ_OK;
 }
 
@@ -65,6 +66,7 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
     k.bgs_stride_b = a->bgs_stride_b, k.bgs_stride_c = a->bgs_stride_c, k.bgs_stride_h = a->bgs_stride_h,
     k.bgs_stride_n = a->bgs_stride_n;
     k.states = states;
+    k.b_rowmax = (float*)(ws + l.rowmax);
     k.batch = a->batch, k.seqlen = a->seqlen, k.nheads = a->nheads, k.headdim = a->headdim, k.ngroups = a->ngroups;
     k.dstate = a->dstate, k.chunk_size = Q;
     if ((rc = lq_chunk_state_key(&k, stream)) != LQ_OK) return rc;

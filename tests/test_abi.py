@@ -35,7 +35,8 @@ def test_struct_layouts_match_the_library():
 def test_every_declaration_cites_the_reference():
     header = (ROOT / "include" / "linquant_hip.h").read_text()
     for m in re.finditer(r"/\*((?:(?!\*/).)*?)\*/\s*typedef struct", header, flags=re.S):
-        assert re.search(r"linquant/[\w/]+\.py:\d+", m.group(1)), m.group(1)[:80]
+        text = m.group(1)
+        assert re.search(r"linquant/[\w/]+\.py:\d+", text) or "no counterpart in the reference" in text, text[:80]
 
 
 def test_null_and_shape_errors_without_launch():

@@ -163,6 +163,51 @@ def test_chunk_state(case, cuda, keyside):
     assert_same_codes(st, ref["states"], "states")
 
 
+@pytest.mark.parametrize("regime", ["strong", "weak"])
+def test_chunk_state_key_zero_slab_elision(cuda, regime):
+    """Leaving out the slabs whose gated key codes are provably zero changes nothing: same states with the elision on
+    and off, and against the oracle, also when the early tokens of every chunk carry keys large enough to saturate
+    their codes (slabs that a decay-only rule would have dropped), when a key is infinite, and on a ragged tail."""
+    from linquant_amd.kernels.mamba2.chunk_state_keyside import _chunk_state_keyside_fwd
+
+    s = Mamba2Shape(batch=2, seqlen=1024, nheads=4, headdim=64, dstate=128, ngroups=2, chunk=256)
+    say("zero-slab elision", regime, s)
+    c = build_case(s, regime=regime)
+    ref = oracle_pipeline(c, True)
+    sc = {k: v.to(cuda) for k, v in c["scales"].items()}
+    x = c["xBC"].to(cuda)[..., :s.d_ssm].view(s.batch, s.seqlen, s.nheads, s.headdim)
+    dt, dA = dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda)
+    variants = {"as drawn": ref["b_fp"].copy()}
+    big = ref["b_fp"].copy()
+    big.reshape(s.batch, 4, 256, s.ngroups, s.dstate)[:, :, :64] *= np.float16(3000.0)   # first slab of every chunk
+    variants["large early keys"] = big
+    inf = ref["b_fp"].copy()
+    inf[1, 300, 1, 7] = np.float16(np.inf)
+    variants["an infinite key"] = inf
+    for name, b_np in variants.items():
+        b_fp = dev(b_np, cuda)
+        on = _chunk_state_keyside_fwd(x, sc["x_scale_hp"], b_fp, dt, dA, sc["static_state_scale"], sc["b_gate_scale"])
+        off = _chunk_state_keyside_fwd(x, sc["x_scale_hp"], b_fp, dt, dA, sc["static_state_scale"], sc["b_gate_scale"],
+                                       elide_zero_slabs=False)
+        torch.cuda.synchronize()
+        assert torch.equal(on, off), f"{name}: the elision changed the states"
+        if name != "an infinite key":  # (inf * 0 is NaN on both sides; its integer conversion is not specified)
+            want = O.chunk_state_key(ref["x"], npy(sc["x_scale_hp"]), b_np, ref["dt"], ref["dA_cumsum"],
+                                     npy(sc["static_state_scale"]), npy(sc["b_gate_scale"]))
+            assert_same_codes(on, want, f"states ({name})")
+    # ragged: 1000 of the 1024 tokens
+    L = 1000
+    dAr, dtr = O.chunk_cumsum(npy(c["dt_raw"])[:, :L], 1.0, npy(c["params"]["A_log"]), float(c["params"]["A_log_scale"]), 256,
+                              None, True)
+    xr = c["xBC"][:, :L].to(cuda)[..., :s.d_ssm].view(s.batch, L, s.nheads, s.headdim)
+    on = _chunk_state_keyside_fwd(xr, sc["x_scale_hp"], dev(ref["b_fp"][:, :L], cuda), dev(dtr, cuda), dev(dAr, cuda),
+                                  sc["static_state_scale"], sc["b_gate_scale"])
+    want = O.chunk_state_key(ref["x"][:, :L], npy(sc["x_scale_hp"]), ref["b_fp"][:, :L], dtr, dAr,
+                             npy(sc["static_state_scale"]), npy(sc["b_gate_scale"]))
+    torch.cuda.synchronize()
+    assert_same_codes(on, want, "states (ragged)")
+
+
 def test_chunk_state_scalar_scales_and_ragged(cuda):
     """Per-head scalars passed as stride-0 (H,P) views, sequence length not a multiple of the chunk."""
     from linquant_amd.kernels.mamba2.chunk_state import _quant_chunk_state_fwd_xfp_static_int8
