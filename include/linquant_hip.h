@@ -84,8 +84,9 @@ typedef struct {
   int64_t bscale_stride_g;
   const float* out_qscale;   /* (H,P) view, stride_p may be 0 */
   int64_t oqs_stride_h, oqs_stride_p;
-  int8_t* states;            /* (B,nc,H,P,N) int8 contiguous */
+  int8_t* states;            /* (B,nc,H,P,N) int8, contiguous but for the batch stride */
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+  int64_t states_stride_b;   /* elements between batch rows of `states`; 0 = dense (nc*H*P*N) */
 } lq_chunk_state_value_args;
 int lq_chunk_state_value(const lq_chunk_state_value_args* args, hipStream_t stream);
 
@@ -105,8 +106,9 @@ typedef struct {
   int64_t oqs_stride_h, oqs_stride_p;
   const float* b_gate_scale; /* 4-D broadcastable (B,nc,H,N); size-1 dims carry stride 0 */
   int64_t bgs_stride_b, bgs_stride_c, bgs_stride_h, bgs_stride_n;
-  int8_t* states;            /* (B,nc,H,P,N) int8 contiguous */
+  int8_t* states;            /* (B,nc,H,P,N) int8, contiguous but for the batch stride */
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+  int64_t states_stride_b;   /* elements between batch rows of `states`; 0 = dense (nc*H*P*N) */
   float* b_rowmax;           /* NULL, or (B,L,G) fp32 scratch: the call first fills it with max_n |B[b,l,g,n]| and then leaves
                                 out every 64-token slab whose gated key codes are provably all zero (same result, bit for
                                 bit; see the kernel's header).  Contents undefined on entry. */
@@ -127,6 +129,11 @@ typedef struct {
   int32_t batch, nchunks, nheads, dim;
   int32_t gate_shift;        /* fractional bits of the fixed-point gate, 0..15 (reference: 7) */
   int32_t vec_hint;          /* 0 = auto; 4/8/16 = bytes per thread to try first */
+  int32_t in_place;          /* 0: `states` and `out` are distinct buffers.  1: they are one buffer of nc + 1 chunk slots per
+                                batch row, out = slot 0, states = slot 1 (same strides): slot c + 1 holds the local state of
+                                chunk c on entry and the state entering chunk c + 1 on return, slot 0 is zero-filled.  A
+                                (batch, head) all of whose gates quantize to zero then needs no pass at all: the state
+                                entering chunk c + 1 is the local state of chunk c, which is already in place. */
 } lq_state_passing_args;
 int lq_state_passing(const lq_state_passing_args* args, hipStream_t stream);
 
@@ -166,6 +173,7 @@ typedef struct {
   const float* cb_scale;     /* (G,) */
   void* out;                 /* (B,L,H,P) fp16 contiguous */
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+  int64_t states_stride_b;   /* elements between batch rows of `states`; 0 = dense (nc*H*P*N) */
 } lq_chunk_scan_args;
 int lq_chunk_scan(const lq_chunk_scan_args* args, hipStream_t stream);
 

@@ -44,6 +44,7 @@ struct ScanParams {
   int64_t sC_b, sC_l, sC_g;
   const float* C_scale;
   const int8_t* states;
+  int64_t sst_b;  // elements between batch rows of states
   const float* ss;
   int64_t sss_h, sss_p;
   const int8_t* D;
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   // round trip of the scalar cache before the next vector load can be issued.
   asm volatile("" ::"s"(p.cb), "s"(p.x), "s"(p.sx_b), "s"(p.sx_l), "s"(p.sx_h), "s"(p.dt), "s"(p.dA), "s"(p.C), "s"(p.sC_b),
                "s"(p.sC_l), "s"(p.sC_g), "s"(p.C_scale), "s"(p.states), "s"(p.ss), "s"(p.sss_h), "s"(p.sss_p));
-  asm volatile("" ::"s"(p.D), "s"(p.sD_h), "s"(p.D_has_hdim), "s"(p.D_scale), "s"(p.cb_scale), "s"(p.out), "s"(p.seqlen),
+  asm volatile("" ::"s"(p.sst_b), "s"(p.D), "s"(p.sD_h), "s"(p.D_has_hdim), "s"(p.D_scale), "s"(p.cb_scale), "s"(p.out), "s"(p.seqlen),
                "s"(p.nheads), "s"(p.P), "s"(p.G), "s"(p.Q), "s"(p.nchunks), "s"(p.hpg_magic), "s"(p.pt_magic));
   const int Q = p.Q;
   uint32_t* xP = (uint32_t*)lds_raw;          // [Q/8][kQuad]
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   // (one 16-byte piece per thread, shared through LDS by all waves), this wave's C rows, dA / dt, then the x tile.
   // Addresses are a wave-uniform 64-bit base plus a per-lane unsigned 32-bit byte offset (the launcher checks that every
   // tile fits 32 bits): per-lane 64-bit multiplies and adds ran at a quarter of the rate and made up a tenth of the kernel.
-  const int8_t* Sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + p0) * (int64_t)N;
+  const int8_t* Sp = p.states + (int64_t)b * p.sst_b + ((((int64_t)c * p.nheads + h) * p.P + p0) * (int64_t)N);
   lq_v4i spiece[kSPieces];
 #pragma unroll
   for (int k = 0; k < kSPieces; ++k) {
@@ -405,6 +406,8 @@ extern "C" int lq_chunk_scan(const lq_chunk_scan_args* a, hipStream_t stream) {
   if (p.sC_b % 16 || p.sC_l % 16 || p.sC_g % 16 || !al(p.C, 16) || !al(p.states, 16) || !al(p.cb, 8) || !al(p.out, 8))
     return LQ_ERR_SHAPE;
   p.nchunks = (p.seqlen + p.Q - 1) / p.Q;
+  p.sst_b = a->states_stride_b ? a->states_stride_b : (int64_t)p.nchunks * p.nheads * p.P * p.N;
+  if (p.sst_b % 16 != 0) return LQ_ERR_SHAPE;
   const int ptiles = p.P / 64;
   if ((int64_t)p.batch * ptiles > 65535 || p.nheads > 65535 || p.nchunks > 65535) return LQ_ERR_SHAPE;
   const uint32_t hpg = (uint32_t)(p.nheads / p.G);

@@ -54,6 +54,7 @@ struct Params {
   int64_t sbg_b, sbg_c, sbg_h, sbg_n;
   const float* rowmax;  // key side, optional: (B,L,G) max_n |B|, filled by row_absmax_kernel
   int8_t* states;
+  int64_t sst_b;        // elements between batch rows of states
   int batch, seqlen, nheads, P, G, N, Q, nchunks, n_ntiles;
   // floor(2^32 / d) + 1 for d = heads per group, tiles per (batch, chunk, head), N tiles per P tile; 0 when d == 1:
   // x / d == umulhi(x, magic) for x, d < 2^16
@@ -351,7 +352,7 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
   // ---- epilogue: lane holds N = n0 + 16q + 4kg + {0..3} of P row p0 + 16*wave + rl
   const float ratio = req_s[16 * wave + rl];  // key side: x_scale / S_out; value side: (alpha / S_out) * bscale
   const float req = ratio;
-  int8_t* sp = p.states + ((((int64_t)b * p.nchunks + c) * p.nheads + h) * p.P + pr) * p.N + n0;
+  int8_t* sp = p.states + (int64_t)b * p.sst_b + ((((int64_t)c * p.nheads + h) * p.P + pr) * p.N + n0);
   uint32_t dq[NT / 16];  // dword q of this lane: codes of N = n0 + 16 q + 4 kg + {0..3}
 #pragma unroll
   for (int q = 0; q < NT / 16; ++q) {
@@ -425,6 +426,8 @@ int launch(const Params& p, hipStream_t stream) {
       (int64_t)p.Q * p.sB_l >= (1ll << 30))
     return LQ_ERR_SHAPE;  // 24-bit token * stride products in the slab loads
   Params q = p;
+  if (q.sst_b == 0) q.sst_b = (int64_t)p.nchunks * p.nheads * p.P * p.N;
+  if (q.sst_b % 16 != 0) return LQ_ERR_SHAPE;
   if (KEYSIDE && p.rowmax) {
     if (p.N != 64 && p.N != 128 && p.N != 256) {
       q.rowmax = nullptr;  // no pre-pass for this width: every slab is processed
@@ -486,7 +489,7 @@ extern "C" int lq_chunk_state_value(const lq_chunk_state_value_args* a, hipStrea
   p.xs = a->alpha_hp, p.sxs_h = a->alpha_stride_h, p.sxs_p = a->alpha_stride_p;
   p.bscale_g = a->bscale_g, p.sbs_g = a->bscale_stride_g;
   p.oqs = a->out_qscale, p.soq_h = a->oqs_stride_h, p.soq_p = a->oqs_stride_p;
-  p.states = a->states;
+  p.states = a->states, p.sst_b = a->states_stride_b;
   p.batch = a->batch, p.seqlen = a->seqlen, p.nheads = a->nheads, p.P = a->headdim, p.G = a->ngroups, p.N = a->dstate;
   p.Q = a->chunk_size;
   if (p.Q <= 0) return LQ_ERR_SHAPE;
@@ -508,7 +511,7 @@ extern "C" int lq_chunk_state_key(const lq_chunk_state_key_args* a, hipStream_t 
   p.bgs = a->b_gate_scale;
   p.rowmax = a->b_rowmax;
   p.sbg_b = a->bgs_stride_b, p.sbg_c = a->bgs_stride_c, p.sbg_h = a->bgs_stride_h, p.sbg_n = a->bgs_stride_n;
-  p.states = a->states;
+  p.states = a->states, p.sst_b = a->states_stride_b;
   p.batch = a->batch, p.seqlen = a->seqlen, p.nheads = a->nheads, p.P = a->headdim, p.G = a->ngroups, p.N = a->dstate;
   p.Q = a->chunk_size;
   if (p.Q <= 0) return LQ_ERR_SHAPE;

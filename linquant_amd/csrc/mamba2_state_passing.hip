@@ -39,9 +39,14 @@ LQ_DEV uint32_t step_word(uint32_t w, int* s, int gate_q, int shift, int half) {
   return o;
 }
 
-template <int VEC, int DEPTH>
+// INPLACE: `states` and `out` are one buffer of nchunks + 1 slots (out = slot 0, states = slot 1): slot c + 1 is read as
+// the local state of chunk c and then overwritten, by the same thread, with the state entering chunk c + 1, so the two
+// pointers alias and carry no __restrict__.  A (batch, head) whose gates all quantize to zero is finished before it
+// starts: the state entering chunk c + 1 is then the local state of chunk c, which already sits in slot c + 1; only the
+// zero slot and the final state are written.  (Its states are requested after the gates are known, not before.)
+template <int VEC, int DEPTH, bool INPLACE>
 __global__ __launch_bounds__(256) void state_passing_kernel(
-    const int8_t* __restrict__ states, int64_t ss_b, int64_t ss_c, int64_t ss_h, int8_t* __restrict__ out,
+    const int8_t* states, int64_t ss_b, int64_t ss_c, int64_t ss_h, int8_t* out,
     int64_t so_b, int64_t so_c, int64_t so_h, int8_t* __restrict__ fin, int64_t sf_b, int64_t sf_h,
     const float* __restrict__ dA, int64_t sd_b, int64_t sd_h, int64_t sd_c, int dim, int nchunks, int shift) {
   typedef typename Vec<VEC>::T V;
@@ -65,16 +70,32 @@ __global__ __launch_bounds__(256) void state_passing_kernel(
   const int cg = min((int)threadIdx.x, nchunks - 1);
   const float dA0 = dA[(int64_t)b * sd_b + (int64_t)h * sd_h + (int64_t)cg * sd_c];
   V buf[DEPTH];
+  if (!INPLACE) {
 #pragma unroll
-  for (int j = 0; j < DEPTH; ++j) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)min(j, nchunks - 1) * ss_c));
+    for (int j = 0; j < DEPTH; ++j) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)min(j, nchunks - 1) * ss_c));
+  }
 
-  gate_lds[cg] = lq_q_rha(lq_expf(dA0) * fs, 127);  // surplus threads rewrite the last gate with the same value
+  const int gq0 = lq_q_rha(lq_expf(dA0) * fs, 127);
+  gate_lds[cg] = gq0;  // surplus threads rewrite the last gate with the same value
+  bool any_gate = gq0 != 0;
   for (int c = threadIdx.x + blockDim.x; c < nchunks; c += blockDim.x) {
     const float g = lq_expf(dA[(int64_t)b * sd_b + (int64_t)h * sd_h + (int64_t)c * sd_c]) * fs;
-    gate_lds[c] = lq_q_rha(g, 127);
+    const int gq = lq_q_rha(g, 127);
+    gate_lds[c] = gq;
+    any_gate = any_gate || gq != 0;
   }
-  __syncthreads();
+  const int some = __syncthreads_or((int)any_gate);  // also makes the gate table visible
   if (!live) return;
+  if (INPLACE) {
+    if (!some) {
+      V zero = {};
+      __builtin_nontemporal_store(zero, (V*)op);
+      if (fp) *(V*)fp = *(const V*)(sp + (int64_t)(nchunks - 1) * ss_c);  // codes of a chunk state lie within +-127 already
+      return;
+    }
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) buf[j] = __builtin_nontemporal_load((const V*)(sp + (int64_t)min(j, nchunks - 1) * ss_c));
+  }
 
   int s[VEC];
 #pragma unroll
@@ -159,14 +180,14 @@ __global__ __launch_bounds__(256) void state_passing_generic_kernel(
   }
 }
 
-template <int VEC, int DEPTH>
+template <int VEC, int DEPTH, bool INPLACE>
 void launch_vec(const lq_state_passing_args* a, hipStream_t stream) {
   // one wave per workgroup: the (batch, head, slice) count then divides evenly over the compute units (measured
   // 9 % faster than 256-thread groups at B4 H80 dim 8192, where 640 groups left some units with 3 and some with 2)
   const int threads = 64;
   const int per_block = threads * VEC;
   dim3 grid((a->dim + per_block - 1) / per_block, a->nheads, a->batch);
-  hipLaunchKernelGGL((state_passing_kernel<VEC, DEPTH>), grid, dim3(threads), (size_t)a->nchunks * sizeof(int), stream,
+  hipLaunchKernelGGL((state_passing_kernel<VEC, DEPTH, INPLACE>), grid, dim3(threads), (size_t)a->nchunks * sizeof(int), stream,
                      a->states, a->states_stride_b, a->states_stride_c, a->states_stride_h, a->out, a->out_stride_b,
                      a->out_stride_c, a->out_stride_h, a->final_states, a->final_stride_b, a->final_stride_h,
                      a->dA_chunk_cumsum, a->dA_stride_b, a->dA_stride_h, a->dA_stride_c, a->dim, a->nchunks,
@@ -198,12 +219,18 @@ extern "C" int lq_state_passing(const lq_state_passing_args* a, hipStream_t stre
            (!a->final_states || aligned(a->final_states, v));
   };
   while (vec >= 4 && !ok(vec)) vec >>= 1;
-  if (vec == 16) {
-    launch_vec<16, 8>(a, stream);
+  if (a->in_place) {
+    // one buffer of nchunks + 1 slots: out = slot 0, states = slot 1, same strides, 16-byte vectors only
+    if (a->in_place != 1 || vec != 16 || a->out_stride_b != a->states_stride_b || a->out_stride_c != a->states_stride_c ||
+        a->out_stride_h != a->states_stride_h || a->states != a->out + a->out_stride_c)
+      return LQ_ERR_SHAPE;
+    launch_vec<16, 8, true>(a, stream);
+  } else if (vec == 16) {
+    launch_vec<16, 8, false>(a, stream);
   } else if (vec == 8) {
-    launch_vec<8, 8>(a, stream);
+    launch_vec<8, 8, false>(a, stream);
   } else if (vec == 4) {
-    launch_vec<4, 8>(a, stream);
+    launch_vec<4, 8, false>(a, stream);
   } else {
     dim3 grid((a->dim + 255) / 256, a->nheads, a->batch);
     hipLaunchKernelGGL(state_passing_generic_kernel, grid, dim3(256), 0, stream, a->states, a->states_stride_b,

@@ -13,7 +13,7 @@ constexpr int64_t kAlign = 256;
 int64_t up(int64_t n) { return (n + kAlign - 1) / kAlign * kAlign; }
 
 struct Layout {
-  int64_t dt, dA, states, passed, cb, rowmax, total;
+  int64_t dt, dA, slots, cb, rowmax, total;  // slots: (B, nchunks + 1, H, P*N), slot c = state entering chunk c
   int nchunks;
 };
 
@@ -28,9 +28,8 @@ int plan(const lq_ssd_combined_args* a, Layout* l) {
   l->nchunks = (int)nc;
   l->dt = 0;
   l->dA = l->dt + up(fl);
-  l->states = l->dA + up(fl);
-  l->passed = l->states + up(st);
-  l->cb = l->passed + up(st);
+  l->slots = l->dA + up(fl);
+  l->cb = l->slots + up(st + (int64_t)a->batch * a->nheads * a->headdim * a->dstate);
   l->rowmax = l->cb + up(cb);
   l->total = l->rowmax + up((int64_t)a->batch * a->seqlen * a->ngroups * 4);
   return LQ_OK;
@@ -39,8 +38,13 @@ int plan(const lq_ssd_combined_args* a, Layout* l) {
 int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t stream) {
   float* dt = (float*)(ws + l.dt);
   float* dA = (float*)(ws + l.dA);
-  int8_t* states = (int8_t*)(ws + l.states);
-  int8_t* passed = (int8_t*)(ws + l.passed);
+  // chunk states and passed states share one buffer of nchunks + 1 slots per batch row: the chunk state kernel writes the
+  // local state of chunk c into slot c + 1, state passing turns it in place into the state entering chunk c + 1 (nothing
+  // to do where the gate quantizes to zero), the chunk scan reads slot c
+  const int64_t slot = (int64_t)a->nheads * a->headdim * a->dstate;
+  const int64_t slots_b = (int64_t)(l.nchunks + 1) * slot;
+  int8_t* passed = (int8_t*)(ws + l.slots);
+  int8_t* states = passed + slot;
   int8_t* cb = (int8_t*)(ws + l.cb);
   const int Q = a->chunk_size, nc = l.nchunks;
   int rc;
@@ -65,7 +69,7 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
     k.b_gate_scale = a->b_gate_scale;
     k.bgs_stride_b = a->bgs_stride_b, k.bgs_stride_c = a->bgs_stride_c, k.bgs_stride_h = a->bgs_stride_h,
     k.bgs_stride_n = a->bgs_stride_n;
-    k.states = states;
+    k.states = states, k.states_stride_b = slots_b;
     k.b_rowmax = (float*)(ws + l.rowmax);
     k.batch = a->batch, k.seqlen = a->seqlen, k.nheads = a->nheads, k.headdim = a->headdim, k.ngroups = a->ngroups;
     k.dstate = a->dstate, k.chunk_size = Q;
@@ -78,7 +82,7 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
     v.alpha_hp = a->alpha_hp, v.alpha_stride_h = a->alpha_stride_h, v.alpha_stride_p = a->alpha_stride_p;
     v.bscale_g = a->bscale_g, v.bscale_stride_g = a->bscale_stride_g;
     v.out_qscale = a->state_scale, v.oqs_stride_h = a->ss_stride_h, v.oqs_stride_p = a->ss_stride_p;
-    v.states = states;
+    v.states = states, v.states_stride_b = slots_b;
     v.batch = a->batch, v.seqlen = a->seqlen, v.nheads = a->nheads, v.headdim = a->headdim, v.ngroups = a->ngroups;
     v.dstate = a->dstate, v.chunk_size = Q;
     if ((rc = lq_chunk_state_value(&v, stream)) != LQ_OK) return rc;
@@ -87,7 +91,7 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
   const int64_t dim = (int64_t)a->headdim * a->dstate;
   lq_state_passing_args sp = {};
   sp.states = states;
-  sp.states_stride_b = (int64_t)nc * a->nheads * dim, sp.states_stride_c = (int64_t)a->nheads * dim, sp.states_stride_h = dim,
+  sp.states_stride_b = slots_b, sp.states_stride_c = (int64_t)a->nheads * dim, sp.states_stride_h = dim,
   sp.states_stride_d = 1;
   sp.dA_chunk_cumsum = dA + (Q - 1);  // last cumsum entry of every chunk: a (B,H,nc) view of (B,H,nc,Q)
   sp.dA_stride_b = (int64_t)a->nheads * nc * Q, sp.dA_stride_h = (int64_t)nc * Q, sp.dA_stride_c = Q;
@@ -96,7 +100,7 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
   sp.final_states = a->final_states;
   sp.final_stride_b = (int64_t)a->nheads * dim, sp.final_stride_h = dim, sp.final_stride_d = 1;
   sp.batch = a->batch, sp.nchunks = nc, sp.nheads = a->nheads, sp.dim = (int32_t)dim;
-  sp.gate_shift = a->gate_shift, sp.vec_hint = 0;
+  sp.gate_shift = a->gate_shift, sp.vec_hint = 0, sp.in_place = 1;
   if (dim > 0x7fffffffLL) return LQ_ERR_SHAPE;
   if ((rc = lq_state_passing(&sp, stream)) != LQ_OK) return rc;
 
@@ -119,7 +123,7 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
   sc.dt = dt, sc.dA_cumsum = dA;
   sc.C = a->qC, sc.C_stride_b = a->qC_stride_b, sc.C_stride_l = a->qC_stride_l, sc.C_stride_g = a->qC_stride_g;
   sc.C_scale = a->C_scale;
-  sc.states = passed;
+  sc.states = passed, sc.states_stride_b = slots_b;
   sc.states_scale = a->state_scale, sc.ss_stride_h = a->ss_stride_h, sc.ss_stride_p = a->ss_stride_p;
   sc.D = a->D, sc.D_stride_h = a->D_stride_h, sc.D_has_hdim = a->D_has_hdim, sc.D_scale = a->D_scale;
   sc.cb_scale = a->cb_scale;

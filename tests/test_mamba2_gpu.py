@@ -288,6 +288,38 @@ def test_state_passing(cuda, dim, shift, nc):
     assert_same_codes(fin, rfin, "final")
 
 
+@pytest.mark.parametrize("nc", [32, 5, 1])
+def test_state_passing_in_place(cuda, nc):
+    """The in-place form used by the one-call forward: one buffer of nc + 1 slots, slot c + 1 holding the local state
+    of chunk c on entry and the state entering chunk c + 1 on return; heads whose gates all quantize to zero are left
+    untouched (their slots are already right), heads with live gates run the full recurrence."""
+    from linquant_amd import _lib
+
+    say("state_passing in place", nc)
+    rng = np.random.default_rng(nc)
+    B, H, dim = 2, 4, 4096
+    states = rng.integers(-127, 128, size=(B, nc, H, dim)).astype(np.int8)
+    dA = -rng.random((B, H, nc)).astype(np.float32) * 3
+    dA[:, 0] = -200.0                      # every gate of head 0 is zero
+    dA[0, 1, : max(nc - 1, 1)] = -200.0    # all but the last gate of (0, 1) are zero
+    slots = torch.zeros(B, nc + 1, H, dim, dtype=torch.int8, device=cuda)
+    slots[:, 0] = 77                       # garbage in the zero slot on entry
+    slots[:, 1:] = dev(states, cuda)
+    fin = torch.empty(B, H, dim, dtype=torch.int8, device=cuda)
+    dAg = dev(dA, cuda)
+    st = slots[:, 1:]
+    _lib.call("lq_state_passing", slots.device, states=_lib.ptr(st), states_stride_b=st.stride(0), states_stride_c=st.stride(1),
+              states_stride_h=st.stride(2), states_stride_d=1, dA_chunk_cumsum=_lib.ptr(dAg), dA_stride_b=dAg.stride(0),
+              dA_stride_h=dAg.stride(1), dA_stride_c=dAg.stride(2), out=_lib.ptr(slots), out_stride_b=slots.stride(0),
+              out_stride_c=slots.stride(1), out_stride_h=slots.stride(2), out_stride_d=1, final_states=_lib.ptr(fin),
+              final_stride_b=fin.stride(0), final_stride_h=fin.stride(1), final_stride_d=1, batch=B, nchunks=nc, nheads=H,
+              dim=dim, gate_shift=7, vec_hint=0, in_place=1)
+    torch.cuda.synchronize()
+    rout, rfin = O.state_passing(states, dA, 7)
+    assert_same_codes(slots[:, :nc], rout, "passed (slots 0 .. nc-1)")
+    assert_same_codes(fin, rfin, "final")
+
+
 def test_state_passing_noncontiguous(cuda):
     from linquant_amd.kernels.mamba2.state_passing import _fixedpoint_state_passing_fwd
 
