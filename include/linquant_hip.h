@@ -174,6 +174,9 @@ typedef struct {
   void* out;                 /* (B,L,H,P) fp16 contiguous */
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
   int64_t states_stride_b;   /* elements between batch rows of `states`; 0 = dense (nc*H*P*N) */
+  int32_t heads_hint;        /* heads of one group that a workgroup walks one after the other (they share the C rows and CB
+                                codes it keeps in registers, and each head's loads overlap the previous head's arithmetic);
+                                0 = chosen from the grid size; clamped to heads per group.  Same bits for every value. */
 } lq_chunk_scan_args;
 int lq_chunk_scan(const lq_chunk_scan_args* args, hipStream_t stream);
 

@@ -8,10 +8,12 @@ from linquant_amd import _lib
 from .chunk_cumsum import _as_f32_scalar
 
 
-def _quant_chunk_scan_fwd(cb_i8, x_fp, dt, dA_cumsum, q_C, C_scale, states, q_D, D_scale, state_dequant_scale, cb_scale):
+def _quant_chunk_scan_fwd(cb_i8, x_fp, dt, dA_cumsum, q_C, C_scale, states, q_D, D_scale, state_dequant_scale, cb_scale,
+                          heads_per_workgroup=0):
     """cb_i8 (B,nc,G,Q,Q) int8, x_fp (B,L,H,P) fp16 view, dt / dA_cumsum (B,H,nc,Q), q_C (B,L,G,N) int8,
     states (B,nc,H,P,N) int8 (state entering each chunk), q_D (H,) or (H,P) int8 or None, D_scale scalar,
-    state_dequant_scale (H,P) fp32 view (P stride 0 allowed), cb_scale (G,). Returns fp16 (B,L,H,P)."""
+    state_dequant_scale (H,P) fp32 view (P stride 0 allowed), cb_scale (G,). Returns fp16 (B,L,H,P).
+    ``heads_per_workgroup`` (not in the reference) is a scheduling knob, 0 = automatic; the result does not depend on it."""
     _, _, nchunks, chunk_size = dt.shape
     _, _, ngroups, dstate = q_C.shape
     batch, seqlen, nheads, headdim = x_fp.shape
@@ -36,5 +38,5 @@ def _quant_chunk_scan_fwd(cb_i8, x_fp, dt, dA_cumsum, q_C, C_scale, states, q_D,
               D_has_hdim=int(q_D is not None and q_D.dim() == 2), D_scale=_lib.ptr(d_scale),
               cb_scale=_lib.ptr(cb_scale), out=_lib.ptr(out),
               batch=batch, seqlen=seqlen, nheads=nheads, headdim=headdim, ngroups=ngroups, dstate=dstate,
-              chunk_size=chunk_size)
+              chunk_size=chunk_size, heads_hint=int(heads_per_workgroup))
     return out

@@ -383,6 +383,12 @@ def test_chunk_scan(case, cuda, keyside):
     torch.cuda.synchronize()
     assert out.dtype == torch.float16 and out.is_contiguous()
     assert_close_out(out, ref["out"], "out")
+    # all heads of a group in one workgroup (small shapes default to one head per workgroup)
+    outg = _quant_chunk_scan_fwd(dev(ref["cb"], cuda), x, dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda),
+                                 dev(ref["q_C"], cuda), sc["C_scale"], dev(ref["passed"], cuda), p["D"], p["D_scale"],
+                                 sc["static_state_scale"], sc["static_cb_scale"], heads_per_workgroup=s.nheads // s.ngroups)
+    torch.cuda.synchronize()
+    assert torch.equal(outg, out)
     # without the D residual, with a per-(H,P) D and with a stride-0 state scale
     out2 = _quant_chunk_scan_fwd(dev(ref["cb"], cuda), x, dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda),
                                  dev(ref["q_C"], cuda), sc["C_scale"], dev(ref["passed"], cuda), None, None,
@@ -399,6 +405,41 @@ def test_chunk_scan(case, cuda, keyside):
     r3 = O.chunk_scan(ref["cb"], ref["x"], ref["dt"], ref["dA_cumsum"], ref["q_C"], npy(sc["C_scale"]),
                       np.zeros_like(ref["passed"]), None, None, npy(sc["static_state_scale"]), npy(small))
     assert_close_out(out3, r3, "out (small S_cb, causal path only)")
+
+
+@pytest.mark.parametrize("L,Q,H,G,P,N", [(600, 256, 16, 2, 64, 128), (200, 64, 12, 4, 128, 64), (1024, 128, 10, 1, 64, 64)])
+def test_chunk_scan_heads_per_workgroup(cuda, L, Q, H, G, P, N):
+    """A workgroup of the chunk scan walks several heads of one group; how many is a scheduling choice (made from the grid
+    size, so small shapes get one).  Every choice, including ones that leave a shorter last part, gives the same bits, on
+    ragged last chunks too; and the one-head form is what test_chunk_scan holds against the oracle."""
+    from linquant_amd.kernels.mamba2.chunk_scan_v2 import _quant_chunk_scan_fwd
+
+    say("chunk_scan heads per workgroup", L, Q, H, G, P, N)
+    g = torch.Generator().manual_seed(11)
+    B, nc = 2, (L + Q - 1) // Q
+    cb = torch.randint(-127, 128, (B, nc, G, Q, Q), generator=g, dtype=torch.int8).to(cuda)
+    x = torch.randn(B, L, H, P, generator=g).half().to(cuda)
+    dt = torch.rand(B, H, nc, Q, generator=g) * 0.05 + 0.001
+    pos = torch.arange(nc * Q).view(nc, Q)
+    dt = torch.where(pos < L, dt, torch.zeros(()))  # dt = 0 past the sequence end, as the cumsum stage writes it
+    a = -(torch.rand(H, generator=g) * 4 + 0.5)
+    dA = torch.cumsum(dt * a.view(1, H, 1, 1), dim=-1)
+    qC = torch.randint(-127, 128, (B, L, G, N), generator=g, dtype=torch.int8).to(cuda)
+    states = torch.randint(-127, 128, (B, nc, H, P, N), generator=g, dtype=torch.int8).to(cuda)
+    D = torch.randint(-127, 128, (H,), generator=g, dtype=torch.int8).to(cuda)
+    C_scale = (torch.rand(G, generator=g) * 0.01 + 0.01).to(cuda)
+    ss = (torch.rand(H, P, generator=g) * 0.01 + 0.01).to(cuda)
+    cbs = (torch.rand(G, generator=g) * 0.02 + 0.02).to(cuda)
+    args = (cb, x, dt.to(cuda), dA.to(cuda), qC, C_scale, states, D, torch.tensor(0.01, device=cuda), ss, cbs)
+    one = _quant_chunk_scan_fwd(*args, heads_per_workgroup=1)
+    torch.cuda.synchronize()
+    assert torch.isfinite(one).all()
+    hpg = H // G
+    for hint in sorted({0, 2, 3, hpg - 1, hpg, hpg + 5} - {1}):
+        say("  heads_per_workgroup", hint)
+        got = _quant_chunk_scan_fwd(*args, heads_per_workgroup=hint)
+        torch.cuda.synchronize()
+        assert torch.equal(got, one), f"heads_per_workgroup={hint}"
 
 
 @pytest.mark.parametrize("keyside", [False, True])
