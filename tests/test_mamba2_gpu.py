@@ -407,6 +407,43 @@ def test_chunk_scan(case, cuda, keyside):
     assert_close_out(out3, r3, "out (small S_cb, causal path only)")
 
 
+def _random_scan_case(L, Q, H, G, P, N, B=2, seed=11):
+    """Arbitrary codes and scales for the chunk scan alone (dt = 0 past the sequence end, as the cumsum stage writes it)."""
+    g = torch.Generator().manual_seed(seed)
+    nc = (L + Q - 1) // Q
+    cb = torch.randint(-127, 128, (B, nc, G, Q, Q), generator=g, dtype=torch.int8)
+    x = torch.randn(B, L, H, P, generator=g).half()
+    dt = torch.rand(B, H, nc, Q, generator=g) * 0.05 + 0.001
+    pos = torch.arange(nc * Q).view(nc, Q)
+    dt = torch.where(pos < L, dt, torch.zeros(()))
+    a = -(torch.rand(H, generator=g) * 4 + 0.5)
+    dA = torch.cumsum(dt * a.view(1, H, 1, 1), dim=-1)
+    qC = torch.randint(-127, 128, (B, L, G, N), generator=g, dtype=torch.int8)
+    states = torch.randint(-127, 128, (B, nc, H, P, N), generator=g, dtype=torch.int8)
+    D = torch.randint(-127, 128, (H,), generator=g, dtype=torch.int8)
+    C_scale = torch.rand(G, generator=g) * 0.01 + 0.01
+    ss = torch.rand(H, P, generator=g) * 0.01 + 0.01
+    cbs = torch.rand(G, generator=g) * 0.02 + 0.02
+    return (cb, x, dt, dA, qC, C_scale, states, D, torch.tensor(0.01), ss, cbs)
+
+
+@pytest.mark.parametrize("L,Q,H,G,P,N", [(700, 512, 4, 2, 64, 256), (200, 64, 6, 2, 64, 192), (300, 128, 4, 4, 128, 256)])
+def test_chunk_scan_wide_shapes(cuda, L, Q, H, G, P, N):
+    """Chunk 512 and state widths 192 / 256 against the oracle, one head per workgroup and all heads of a group."""
+    from linquant_amd.kernels.mamba2.chunk_scan_v2 import _quant_chunk_scan_fwd
+
+    say("chunk_scan wide", L, Q, H, G, P, N)
+    case = _random_scan_case(L, Q, H, G, P, N, B=1, seed=5)
+    cb, x, dt, dA, qC, C_scale, states, D, D_scale, ss, cbs = case
+    ref = O.chunk_scan(npy(cb), npy(x), npy(dt), npy(dA), npy(qC), npy(C_scale), npy(states), npy(D), np.float32(0.01), npy(ss), npy(cbs))
+    args = tuple(t.to(cuda) for t in case)
+    for hint in (1, H // G):
+        say("  heads_per_workgroup", hint)
+        got = _quant_chunk_scan_fwd(*args, heads_per_workgroup=hint)
+        torch.cuda.synchronize()
+        assert_close_out(got, ref, f"out (hint {hint})")
+
+
 @pytest.mark.parametrize("L,Q,H,G,P,N", [(600, 256, 16, 2, 64, 128), (200, 64, 12, 4, 128, 64), (1024, 128, 10, 1, 64, 64)])
 def test_chunk_scan_heads_per_workgroup(cuda, L, Q, H, G, P, N):
     """A workgroup of the chunk scan walks several heads of one group; how many is a scheduling choice (made from the grid
@@ -415,22 +452,7 @@ def test_chunk_scan_heads_per_workgroup(cuda, L, Q, H, G, P, N):
     from linquant_amd.kernels.mamba2.chunk_scan_v2 import _quant_chunk_scan_fwd
 
     say("chunk_scan heads per workgroup", L, Q, H, G, P, N)
-    g = torch.Generator().manual_seed(11)
-    B, nc = 2, (L + Q - 1) // Q
-    cb = torch.randint(-127, 128, (B, nc, G, Q, Q), generator=g, dtype=torch.int8).to(cuda)
-    x = torch.randn(B, L, H, P, generator=g).half().to(cuda)
-    dt = torch.rand(B, H, nc, Q, generator=g) * 0.05 + 0.001
-    pos = torch.arange(nc * Q).view(nc, Q)
-    dt = torch.where(pos < L, dt, torch.zeros(()))  # dt = 0 past the sequence end, as the cumsum stage writes it
-    a = -(torch.rand(H, generator=g) * 4 + 0.5)
-    dA = torch.cumsum(dt * a.view(1, H, 1, 1), dim=-1)
-    qC = torch.randint(-127, 128, (B, L, G, N), generator=g, dtype=torch.int8).to(cuda)
-    states = torch.randint(-127, 128, (B, nc, H, P, N), generator=g, dtype=torch.int8).to(cuda)
-    D = torch.randint(-127, 128, (H,), generator=g, dtype=torch.int8).to(cuda)
-    C_scale = (torch.rand(G, generator=g) * 0.01 + 0.01).to(cuda)
-    ss = (torch.rand(H, P, generator=g) * 0.01 + 0.01).to(cuda)
-    cbs = (torch.rand(G, generator=g) * 0.02 + 0.02).to(cuda)
-    args = (cb, x, dt.to(cuda), dA.to(cuda), qC, C_scale, states, D, torch.tensor(0.01, device=cuda), ss, cbs)
+    args = tuple(t.to(cuda) for t in _random_scan_case(L, Q, H, G, P, N))
     one = _quant_chunk_scan_fwd(*args, heads_per_workgroup=1)
     torch.cuda.synchronize()
     assert torch.isfinite(one).all()
