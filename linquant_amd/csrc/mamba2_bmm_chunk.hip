@@ -37,14 +37,30 @@ __global__ __launch_bounds__(64, 2) void bmm_chunk_kernel(const int8_t* __restri
                                                        const float* __restrict__ b_scale,
                                                        const float* __restrict__ cb_scale, int8_t* __restrict__ out,
                                                        int seqlen, int G, int Q, int nchunks, uint32_t tiles_magic,
-                                                       uint32_t g_magic) {
+                                                       uint32_t g_magic, uint32_t tpc, uint32_t tpc_magic, uint32_t ncg,
+                                                       uint32_t ncg_magic, int by_xcd) {
   const int lane = threadIdx.x, rl = lane & 15, kg = lane >> 4;
-  // floor(2^32 / d) + 1 multipliers (0 for d == 1) stand in for the run-time divisions by tiles per row and groups
-  const int mt64 = tiles_magic ? (int)__umulhi(blockIdx.x, tiles_magic) : (int)blockIdx.x;
-  const int kt64 = (int)blockIdx.x - mt64 * (Q >> 6);
-  const int b = blockIdx.y;
-  const int c = g_magic ? (int)__umulhi(blockIdx.z, g_magic) : (int)blockIdx.z;
-  const int g = (int)blockIdx.z - c * G;
+  // floor(2^32 / d) + 1 multipliers (0 for d == 1) stand in for the run-time divisions (exact while x * d < 2^32, which
+  // the launcher checks).
+  // Workgroups are dealt to the 8 XCDs round-robin in launch order, and the tpc tiles of one (batch, chunk, group) read
+  // the same C and B rows: with consecutive workgroups on consecutive tiles every XCD's L2 fetched those rows from HBM
+  // for itself (33.7 MB read for 12.6 MB of operands).  Workgroup 8 j + x takes tile j % tpc of unit 8 (j / tpc) + x, so
+  // a unit's tiles run on one XCD, one after the other.
+  uint32_t unit, tile;
+  if (by_xcd) {
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    const uint32_t uh = tpc_magic ? __umulhi(j, tpc_magic) : j;
+    tile = j - uh * tpc, unit = uh * 8u + x;
+  } else {
+    unit = tpc_magic ? __umulhi(blockIdx.x, tpc_magic) : blockIdx.x;
+    tile = blockIdx.x - unit * tpc;
+  }
+  const int mt64 = tiles_magic ? (int)__umulhi(tile, tiles_magic) : (int)tile;
+  const int kt64 = (int)tile - mt64 * (Q >> 6);
+  const int b = ncg_magic ? (int)__umulhi(unit, ncg_magic) : (int)unit;
+  const uint32_t cg = unit - (uint32_t)b * ncg;
+  const int c = g_magic ? (int)__umulhi(cg, g_magic) : (int)cg;
+  const int g = (int)cg - c * G;
   const int limit = min(Q, seqlen - c * Q);
   const float a_sc = a_scale[g], b_sc = b_scale[g], cb_sc = cb_scale[g];
 
@@ -145,11 +161,16 @@ extern "C" int lq_bmm_chunk(const lq_bmm_chunk_args* a, hipStream_t stream) {
   if ((int64_t)nchunks * a->ngroups > 65535) return LQ_ERR_SHAPE;
   const uint32_t shift = Q == 64 ? 0u : (uint32_t)(0x100000000ull / (uint32_t)(Q / 64)) + 1u;  // tiles per row, as a multiplier
   const uint32_t g_magic = a->ngroups == 1 ? 0u : (uint32_t)(0x100000000ull / (uint32_t)a->ngroups) + 1u;
-  dim3 grid((Q / 64) * (Q / 64), a->batch, nchunks * a->ngroups);
+  const uint32_t tpc = (uint32_t)((Q / 64) * (Q / 64)), ncg = (uint32_t)(nchunks * a->ngroups);
+  const uint64_t units = (uint64_t)a->batch * ncg, total = units * tpc;
+  if (total >= (1ull << 31) || total * tpc >= (1ull << 32) || units * ncg >= (1ull << 32)) return LQ_ERR_SHAPE;
+  auto magic = [](uint32_t d) { return d == 1 ? 0u : (uint32_t)(0x100000000ull / d) + 1u; };
+  const int by_xcd = units % 8 == 0;
+  dim3 grid((unsigned)total);
 #define LQ_BMM_LAUNCH(FP, NN)                                                                                              \
   hipLaunchKernelGGL((bmm_chunk_kernel<FP, NN>), grid, dim3(64), 0, stream, a->a, a->a_stride_b, a->a_stride_l,            \
                      a->a_stride_g, a->b, a->b_stride_b, a->b_stride_l, a->b_stride_g, a->a_scale, a->b_scale, a->cb_scale, \
-                     a->out, a->seqlen, a->ngroups, Q, nchunks, shift, g_magic)
+                     a->out, a->seqlen, a->ngroups, Q, nchunks, shift, g_magic, tpc, magic(tpc), ncg, magic(ncg), by_xcd)
   switch (N / 64) {
     case 1: if (a->b_is_fp) LQ_BMM_LAUNCH(true, 1); else LQ_BMM_LAUNCH(false, 1); break;
     case 2: if (a->b_is_fp) LQ_BMM_LAUNCH(true, 2); else LQ_BMM_LAUNCH(false, 2); break;

@@ -22,14 +22,36 @@ LQ_DEV float load_dt(const void* p, int64_t off, int dtype) {
 constexpr int kHG = 16;   // heads per workgroup: one token row of the tile is 16 adjacent heads (32 bytes of fp16 dt)
 constexpr int kWaves = 8;  // two heads per wave
 
+// Which (head group, chunk, batch) a workgroup of the flat grid works on.  Workgroups are dealt to the 8 XCDs round-robin
+// in launch order, and the head groups of one (chunk, batch) read the same 128-byte lines of dt (a token row of 80 heads
+// is 160 bytes): on consecutive workgroups every XCD's L2 fetched those lines from HBM for itself (21 MB read for 5 MB
+// of dt).  Workgroup 8 j + x takes head group j % hg of unit 8 (j / hg) + x, so a unit's head groups share one XCD.
+struct Where {
+  int h0, c, b;
+};
+LQ_DEV Where where(int hg, int nchunks, int by_xcd) {
+  uint32_t unit, grp;
+  if (by_xcd) {
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    const uint32_t uh = j / (uint32_t)hg;
+    grp = j - uh * (uint32_t)hg, unit = uh * 8u + x;
+  } else {
+    unit = blockIdx.x / (uint32_t)hg, grp = blockIdx.x - unit * (uint32_t)hg;
+  }
+  Where w;
+  w.b = (int)(unit / (uint32_t)nchunks), w.c = (int)(unit - (uint32_t)w.b * (uint32_t)nchunks), w.h0 = (int)grp * kHG;
+  return w;
+}
+
 __global__ __launch_bounds__(kWaves * 64) void chunk_cumsum_kernel(
     const void* __restrict__ dt_in, int dt_dtype, int64_t sdt_b, int64_t sdt_l, int64_t sdt_h,
     const float* __restrict__ dt_scale_p, const int8_t* __restrict__ a_log, int64_t sa_h,
     const float* __restrict__ a_log_scale_p, const float* __restrict__ dt_bias, int64_t sbias_h,
     float* __restrict__ dt_out, float* __restrict__ dA_cs, int seqlen, int nheads, int nchunks, int Q,
-    int softplus, float dt_min, float dt_max) {
+    int softplus, float dt_min, float dt_max, int hg, int by_xcd) {
   extern __shared__ float tile[];  // [Q][kHG + 1] raw dt as float
-  const int h0 = blockIdx.x * kHG, c = blockIdx.y, b = blockIdx.z;
+  const Where wh = where(hg, nchunks, by_xcd);
+  const int h0 = wh.h0, c = wh.c, b = wh.b;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int E = Q >> 6;
   const int limit = min(Q, seqlen - c * Q);
@@ -99,10 +121,11 @@ __global__ __launch_bounds__(kWaves * 64) void chunk_cumsum_fixed_kernel(
     const float* __restrict__ dt_scale_p, const int8_t* __restrict__ a_log, int64_t sa_h,
     const float* __restrict__ a_log_scale_p, const float* __restrict__ dt_bias, int64_t sbias_h,
     float* __restrict__ dt_out, float* __restrict__ dA_cs, int seqlen, int nheads, int nchunks,
-    int softplus, float dt_min, float dt_max) {
+    int softplus, float dt_min, float dt_max, int hg, int by_xcd) {
   constexpr int Q = 64 * E, NIT = Q * kHG / (kWaves * 64);
   extern __shared__ float tile[];  // [Q][kHG + 1] raw dt as float
-  const int h0 = blockIdx.x * kHG, c = blockIdx.y, b = blockIdx.z;
+  const Where wh = where(hg, nchunks, by_xcd);
+  const int h0 = wh.h0, c = wh.c, b = wh.b;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int limit = min(Q, seqlen - c * Q);
   // ---- requests: the (token, head) tile (consecutive lanes read consecutive heads of one token; positions past the
@@ -201,7 +224,11 @@ extern "C" int lq_chunk_cumsum(const lq_chunk_cumsum_args* a, hipStream_t stream
   if (a->dt_dtype != LQ_DT_F16 && a->dt_dtype != LQ_DT_F32 && a->dt_dtype != LQ_DT_I8) return LQ_ERR_SHAPE;
   const int nchunks = (a->seqlen + Q - 1) / Q;
   if (nchunks > 65535) return LQ_ERR_SHAPE;
-  dim3 grid((a->nheads + kHG - 1) / kHG, nchunks, a->batch);
+  const int hg = (a->nheads + kHG - 1) / kHG;
+  const int64_t units = (int64_t)nchunks * a->batch;
+  if (units * hg >= (1ll << 31)) return LQ_ERR_SHAPE;
+  const int by_xcd = units % 8 == 0;
+  dim3 grid((unsigned)(units * hg));
   const size_t lds = (size_t)Q * (kHG + 1) * sizeof(float);
   if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&chunk_cumsum_kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -211,7 +238,7 @@ extern "C" int lq_chunk_cumsum(const lq_chunk_cumsum_args* a, hipStream_t stream
   hipLaunchKernelGGL(chunk_cumsum_fixed_kernel<EE>, grid, dim3(kWaves * 64), lds, stream, a->dt, a->dt_dtype,             \
                      a->dt_stride_b, a->dt_stride_l, a->dt_stride_h, a->dt_scale, a->A_log, a->A_log_stride_h,            \
                      a->A_log_scale, a->dt_bias, a->dt_bias_stride_h, a->dt_out, a->dA_cumsum, a->seqlen, a->nheads,      \
-                     nchunks, a->dt_softplus, a->dt_min, a->dt_max)
+                     nchunks, a->dt_softplus, a->dt_min, a->dt_max, hg, by_xcd)
   if (Q == 64)
     LQ_CUMSUM_FIXED(1);
   else if (Q == 128)
@@ -224,7 +251,7 @@ extern "C" int lq_chunk_cumsum(const lq_chunk_cumsum_args* a, hipStream_t stream
     hipLaunchKernelGGL(chunk_cumsum_kernel, grid, dim3(kWaves * 64), lds, stream, a->dt, a->dt_dtype, a->dt_stride_b,
                        a->dt_stride_l, a->dt_stride_h, a->dt_scale, a->A_log, a->A_log_stride_h, a->A_log_scale,
                        a->dt_bias, a->dt_bias_stride_h, a->dt_out, a->dA_cumsum, a->seqlen, a->nheads, nchunks, Q,
-                       a->dt_softplus, a->dt_min, a->dt_max);
+                       a->dt_softplus, a->dt_min, a->dt_max, hg, by_xcd);
 #undef LQ_CUMSUM_FIXED
   return lq_check_launch();
 }
