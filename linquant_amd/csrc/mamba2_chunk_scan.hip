@@ -126,12 +126,15 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // known to be wave-uniform: everything derived from it is scalar
   const int rl = lane & 15, kg = lane >> 4;
-  // grid = (groups x head parts) x chunks x (batch * P tiles): no integer division on the way to the first load
-  const int c = blockIdx.y;
+  // grid = chunks x (groups x head parts) x (batch * P tiles): no integer division on the way to the first load.  Chunks
+  // vary fastest across consecutive workgroups, which are dealt to the 8 XCDs round-robin: the head parts of one (batch,
+  // chunk), which read the same C rows and CB codes, then share an XCD's L2 whenever the chunk count is a multiple of 8
+  // (with the parts fastest every XCD fetched them from HBM for itself: 75 MB of 527 read).
+  const int c = blockIdx.x;
   const int b = p.pt_magic ? (int)__umulhi(blockIdx.z, p.pt_magic) : (int)blockIdx.z;
   const int p0 = ((int)blockIdx.z - b * (p.P >> 6)) * 64;
-  const int g = p.hs_magic ? (int)__umulhi(blockIdx.x, p.hs_magic) : (int)blockIdx.x;
-  const int part = (int)blockIdx.x - g * p.hsplit;
+  const int g = p.hs_magic ? (int)__umulhi(blockIdx.y, p.hs_magic) : (int)blockIdx.y;
+  const int part = (int)blockIdx.y - g * p.hsplit;
   const int h0 = g * p.hpg + part * p.hpw;            // this workgroup's heads: h0 .. h0 + nh - 1, all of group g
   const int nh = min(p.hpw, p.hpg - part * p.hpw);
   const int limit = min(Q, p.seqlen - c * Q);
@@ -491,7 +494,7 @@ extern "C" int lq_chunk_scan(const lq_chunk_scan_args* a, hipStream_t stream) {
   if ((int64_t)p.nheads * p.P * 2 >= (1 << 24) || (int64_t)p.Q * p.nheads * p.P * 2 >= (1ll << 31)) return LQ_ERR_SHAPE;
   if (p.sss_p < 0 || p.sss_p >= (1 << 24)) return LQ_ERR_SHAPE;
   const size_t lds = (size_t)2 * (p.Q / 8) * kQuad * 4 + 2 * ((size_t)p.Q * 8 + 512) + (size_t)64 * (p.N + 32);  // x tiles, two sets of dA2 / akw / per-channel tables, states
-  dim3 grid(p.G * p.hsplit, p.nchunks, p.batch * ptiles);
+  dim3 grid(p.nchunks, p.G * p.hsplit, p.batch * ptiles);
   // more than 64 KB of dynamic LDS has to be opted into per kernel
 #define LQ_SCAN_LAUNCH(W, NN)                                                                                   \
   do {                                                                                                          \

@@ -105,10 +105,11 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  // heads vary fastest across consecutive workgroups: the B tile of a (batch, chunk) is shared by the heads of
-  // a group and stays in L2 while they are swept
-  // (grid = heads x chunks x (batch * tiles): no run-time integer division in front of the first request)
-  const int h = blockIdx.x, c = blockIdx.y;
+  // grid = chunks x heads x (batch * tiles): no run-time integer division in front of the first request.  Chunks vary
+  // fastest across consecutive workgroups, which are dealt to the 8 XCDs round-robin: the heads of one (batch, chunk),
+  // which share its B tile, then meet in one XCD's L2 whenever the chunk count is a multiple of 8 (with the heads fastest
+  // every XCD fetched the tile from HBM for itself)
+  const int h = blockIdx.y, c = blockIdx.x;
   const int b = div_magic(blockIdx.z, p.tiles_magic);
   const int tile = (int)blockIdx.z - b * (p.P >> 6) * p.n_ntiles;
   const int ptile = div_magic((uint32_t)tile, p.nt_magic), ntile = tile - ptile * p.n_ntiles;
@@ -451,7 +452,7 @@ int launch(const Params& p, hipStream_t stream) {
     const int tiles = (p.P / 64) * q.n_ntiles;
     if ((int64_t)p.batch * tiles > 65535) return LQ_ERR_SHAPE;
     q.hpg_magic = magic((uint32_t)(p.nheads / p.G)), q.tiles_magic = magic((uint32_t)tiles), q.nt_magic = magic((uint32_t)q.n_ntiles);
-    dim3 grid(p.nheads, p.nchunks, p.batch * tiles);
+    dim3 grid(p.nchunks, p.nheads, p.batch * tiles);
     if (!KEYSIDE && p.Q == 256)
       hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 128, 4>), grid, dim3(256), lds, stream, q);
     else if (!KEYSIDE && p.Q == 128)
@@ -464,7 +465,7 @@ int launch(const Params& p, hipStream_t stream) {
     const int tiles = (p.P / 64) * q.n_ntiles;
     if ((int64_t)p.batch * tiles > 65535) return LQ_ERR_SHAPE;
     q.hpg_magic = magic((uint32_t)(p.nheads / p.G)), q.tiles_magic = magic((uint32_t)tiles), q.nt_magic = magic((uint32_t)q.n_ntiles);
-    dim3 grid(p.nheads, p.nchunks, p.batch * tiles);
+    dim3 grid(p.nchunks, p.nheads, p.batch * tiles);
     if (!KEYSIDE && p.Q == 256)
       hipLaunchKernelGGL((chunk_state_kernel<KEYSIDE, 64, 4>), grid, dim3(256), lds, stream, q);
     else if (!KEYSIDE && p.Q == 128)
