@@ -31,84 +31,109 @@ LQ_DEV uint16_t f_to_bf16(float x) {  // round to nearest even (finite inputs)
   return (uint16_t)(u >> 16);
 }
 
-template <int D, bool BF16>
+// R rows per thread (R * 256 / (D / 8) rows per workgroup): all R requests of a thread are issued before the first row is
+// transformed, so a workgroup has R times the bytes in flight of the one-row form (a thread that moves 16 bytes in and
+// 16 bytes out and exits spends most of its life on the way in and out of the machine).
+template <int D, bool BF16, int R>
 __global__ __launch_bounds__(256) void zoo_rotate_kernel(RotParams p) {
   constexpr int LPR = D / 8;      // lanes per row
-  constexpr int RPB = 256 / LPR;  // rows per block
+  constexpr int RPB = 256 / LPR;  // rows per pass of the workgroup
   const int which = blockIdx.y;
   const uint16_t* src = p.src[which];
   if (!src) return;  // block-uniform: this tensor is not part of the call
   const float* diag = p.diag[which];
   const float* signs = p.signs[which];
   const int sub = threadIdx.x % LPR;
-  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
-  const bool live = row < p.rows;
-  const int64_t rr = live ? row : p.rows - 1;  // surplus rows still take part in the shuffles
-  const int h = (int)(rr % p.nheads);
-  const lq_v4i raw = *(const lq_v4i*)(src + rr * D + sub * 8);
+  const int64_t row0 = (int64_t)blockIdx.x * (R * RPB) + threadIdx.x / LPR;
+  lq_v4i raw[R];
+  int hh[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t rr = min(row0 + r * RPB, p.rows - 1);  // surplus rows still take part in the shuffles
+    hh[r] = (int)(rr % p.nheads);
+    raw[r] = *(const lq_v4i*)(src + rr * D + sub * 8);
+  }
   // operands that are absent are read from a valid address and ignored: every request is issued before the first use
-  const float* dp = diag ? diag + (int64_t)h * D + sub * 8 : p.signs[which] ? p.signs[which] : (const float*)src;
   const float* sp = signs ? signs + sub * 8 : (const float*)src;
-  const lq_v4f d0 = *(const lq_v4f*)dp, d1 = *(const lq_v4f*)(diag ? dp + 4 : dp);
   const lq_v4f s0 = *(const lq_v4f*)sp, s1 = *(const lq_v4f*)(signs ? sp + 4 : sp);
-  float v[8];
+  lq_v4f d0[R], d1[R];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint16_t u = (uint16_t)((uint32_t)raw[i >> 1] >> (16 * (i & 1)));
-    v[i] = BF16 ? bf16_to_f(u) : (float)__builtin_bit_cast(_Float16, u);
+  for (int r = 0; r < R; ++r) {
+    const float* dp = diag ? diag + (int64_t)hh[r] * D + sub * 8 : sp;
+    d0[r] = *(const lq_v4f*)dp, d1[r] = *(const lq_v4f*)(diag ? dp + 4 : dp);
   }
-  if (diag) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = v[i] * (i < 4 ? d0[i & 3] : d1[i & 3]);
-  }
-  if (signs) {
+  for (int r = 0; r < R; ++r) {
+    const int64_t row = row0 + r * RPB;
+    float v[8];
 #pragma unroll
-    for (int hh = 1; hh < 8; hh <<= 1)
+    for (int i = 0; i < 8; ++i) {
+      const uint16_t u = (uint16_t)((uint32_t)raw[r][i >> 1] >> (16 * (i & 1)));
+      v[i] = BF16 ? bf16_to_f(u) : (float)__builtin_bit_cast(_Float16, u);
+    }
+    if (diag) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if ((i & hh) == 0) {
-          const float a = v[i], b = v[i + hh];
-          v[i] = a + b;
-          v[i + hh] = a - b;
+      for (int i = 0; i < 8; ++i) v[i] = v[i] * (i < 4 ? d0[r][i & 3] : d1[r][i & 3]);
+    }
+    if (signs) {
+#pragma unroll
+      for (int h2 = 1; h2 < 8; h2 <<= 1)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if ((i & h2) == 0) {
+            const float a = v[i], b = v[i + h2];
+            v[i] = a + b;
+            v[i + h2] = a - b;
+          }
+#pragma unroll
+      for (int m = 1; m < LPR; m <<= 1)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float o = __shfl_xor(v[i], m, 64);
+          v[i] = (sub & m) ? (o - v[i]) : (v[i] + o);
         }
 #pragma unroll
-    for (int m = 1; m < LPR; m <<= 1)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float o = __shfl_xor(v[i], m, 64);
-        v[i] = (sub & m) ? (o - v[i]) : (v[i] + o);
-      }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (v[i] * p.rsqrt_n) * (i < 4 ? s0[i & 3] : s1[i & 3]);
-  }
-  if (!live) return;
-  lq_v4i out;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    uint16_t lo, hi;
-    if (BF16) {
-      lo = f_to_bf16(v[2 * i]), hi = f_to_bf16(v[2 * i + 1]);
-    } else {
-      lo = __builtin_bit_cast(uint16_t, (_Float16)v[2 * i]), hi = __builtin_bit_cast(uint16_t, (_Float16)v[2 * i + 1]);
+      for (int i = 0; i < 8; ++i) v[i] = (v[i] * p.rsqrt_n) * (i < 4 ? s0[i & 3] : s1[i & 3]);
     }
-    out[i] = (int)((uint32_t)lo | ((uint32_t)hi << 16));
+    if (row < p.rows) {
+      lq_v4i out;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint16_t lo, hi;
+        if (BF16) {
+          lo = f_to_bf16(v[2 * i]), hi = f_to_bf16(v[2 * i + 1]);
+        } else {
+          lo = __builtin_bit_cast(uint16_t, (_Float16)v[2 * i]), hi = __builtin_bit_cast(uint16_t, (_Float16)v[2 * i + 1]);
+        }
+        out[i] = (int)((uint32_t)lo | ((uint32_t)hi << 16));
+      }
+      *(lq_v4i*)(p.dst[which] + row * D + sub * 8) = out;
+    }
   }
-  *(lq_v4i*)(p.dst[which] + row * D + sub * 8) = out;
 }
 
 bool al16(const void* q) { return ((uintptr_t)q % 16) == 0; }
 
-template <int D>
-int launch(const RotParams& p, bool bf16, int64_t rows, hipStream_t stream) {
-  constexpr int RPB = 256 / (D / 8);
+// Rows per thread: four for the pure rescaling (a copy with one multiply: 537 MB in 117 -> 104 us at B2 T8192 H32 K128),
+// two with the butterflies (their lane exchanges keep the vector ALU busy; one, two and four rows measured 56.6, 55.7
+// and 61 us for 268 MB).
+template <int D, int R>
+int launch_r(const RotParams& p, bool bf16, int64_t rows, hipStream_t stream) {
+  constexpr int RPB = R * 256 / (D / 8);
   const int64_t gx = (rows + RPB - 1) / RPB;
   if (gx > 0x7fffffffLL) return LQ_ERR_SHAPE;
   dim3 grid((unsigned)gx, 3);
   if (bf16)
-    hipLaunchKernelGGL((zoo_rotate_kernel<D, true>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_rotate_kernel<D, true, R>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_rotate_kernel<D, false>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_rotate_kernel<D, false, R>), grid, dim3(256), 0, stream, p);
   return lq_check_launch();
+}
+
+template <int D>
+int launch(const RotParams& p, bool bf16, int64_t rows, hipStream_t stream) {
+  const bool rotates = p.signs[0] || p.signs[1] || p.signs[2];
+  return rotates ? launch_r<D, 2>(p, bf16, rows, stream) : launch_r<D, 4>(p, bf16, rows, stream);
 }
 
 }  // namespace
