@@ -367,3 +367,46 @@ def test_reference_mamba2_cell_config(cuda):
     out, _ = zoo.chunk_simple_gla_int8(q.cuda(), k.cuda(), v.cuda(), g.cuda(), sc, eta=1.0, scale=1.0, chunk_size=64)
     torch.cuda.synchronize()
     zc.check(out, run, qz, "Mamba-2 cell at the c1 shape")
+
+
+@pytest.mark.parametrize("cell", ["linear_none", "gla", "gated_deltanet", "kda"])
+def test_hip_graph_capture_and_replay(cuda, cell):
+    """A whole zoo call (its three to six launches, no synchronisation inside the library) captured once in a HIP graph and
+    replayed: every replay equals the eager result bit for bit, with eager work and synchronisations between the replays
+    and with new input values written into the captured buffers."""
+    tensors = zc.cut(zc.inputs(cell), 256)
+    qz, _ = zc.calibrated(cell, tensors, policy="kernel_static", bits=8, eta=DEFAULT_ETA[cell], rho=1.0, tau=1.0)
+    B, T, H, K = tensors[0].shape
+    V = tensors[2].shape[-1]
+    scales = {n: t.to(cuda) for n, t in qz.kernel_scales(0, H, K, V, delta=zc.CELLS[cell][0] == "delta").items()}
+    dev_tensors = tuple(t.to(cuda) if t is not None else None for t in tensors)
+
+    def call():  # everything already on the device: no copy inside the capture
+        return zc.run_kernel(cell, dev_tensors, scales, eta=DEFAULT_ETA[cell], device=cuda)[0]
+
+    eager = call().clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = call()
+    torch.cuda.synchronize()
+    for i in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured, eager), f"{cell}: replay {i} differs from the eager result"
+        again = call()
+        torch.cuda.synchronize()
+        assert torch.equal(again, eager)
+    # new values in the captured input buffers
+    for t in dev_tensors[:3]:
+        t.mul_(0.5)
+    eager2 = call().clone()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(captured, eager2), f"{cell}: replay on new inputs differs from the eager result"
