@@ -427,9 +427,11 @@ def _random_scan_case(L, Q, H, G, P, N, B=2, seed=11):
     return (cb, x, dt, dA, qC, C_scale, states, D, torch.tensor(0.01), ss, cbs)
 
 
-@pytest.mark.parametrize("L,Q,H,G,P,N", [(700, 512, 4, 2, 64, 256), (200, 64, 6, 2, 64, 192), (300, 128, 4, 4, 128, 256)])
+@pytest.mark.parametrize("L,Q,H,G,P,N", [(700, 512, 4, 2, 64, 256), (200, 64, 6, 2, 64, 192), (300, 128, 4, 4, 128, 256),
+                                         (40, 64, 2, 1, 64, 64), (17, 256, 3, 3, 64, 128)])
 def test_chunk_scan_wide_shapes(cuda, L, Q, H, G, P, N):
-    """Chunk 512 and state widths 192 / 256 against the oracle, one head per workgroup and all heads of a group."""
+    """Chunk 512, state widths 192 / 256 and sequences shorter than one chunk against the oracle, one head per workgroup
+    and all heads of a group."""
     from linquant_amd.kernels.mamba2.chunk_scan_v2 import _quant_chunk_scan_fwd
 
     say("chunk_scan wide", L, Q, H, G, P, N)
