@@ -368,6 +368,29 @@ def test_bmm_chunk(case, cuda, keyside):
     assert_same_codes(cb, ref["cb"], "cb")
 
 
+@pytest.mark.parametrize("L,Q,G,N,fp", [(2000, 256, 64, 64, True), (2048, 256, 64, 128, False), (300, 128, 3, 192, True),
+                                        (1000, 64, 5, 256, False)])
+def test_bmm_chunk_shapes(cuda, L, Q, G, N, fp):
+    """C.B^T with many and with few groups (both workgroup orders), ragged last chunks, both B dtypes and every state
+    width, against the oracle's exact integer product."""
+    from linquant_amd.kernels.mamba2.bmm_chunk import _quant_bmm_chunk_fwd
+
+    say("bmm_chunk shapes", L, Q, G, N, fp)
+    g = torch.Generator().manual_seed(3)
+    qC = torch.randint(-127, 128, (1, L, G, N), generator=g, dtype=torch.int8)
+    C_scale = torch.rand(G, generator=g) * 0.01 + 0.01
+    B_scale = torch.rand(G, generator=g) * 0.01 + 0.01
+    cb_scale = torch.rand(G, generator=g) * 0.5 + 0.5
+    if fp:
+        b = (torch.randn(1, L, G, N, generator=g) * B_scale.view(1, 1, G, 1) * 50).half()
+    else:
+        b = torch.randint(-127, 128, (1, L, G, N), generator=g, dtype=torch.int8)
+    cb = _quant_bmm_chunk_fwd(qC.to(cuda), C_scale.to(cuda), b.to(cuda), B_scale.to(cuda), Q, cb_scale.to(cuda), b_is_fp=fp)
+    torch.cuda.synchronize()
+    ref = O.bmm_chunk(npy(qC), npy(C_scale), npy(b), npy(B_scale), Q, npy(cb_scale), b_is_fp=fp)
+    assert_same_codes(cb, ref, "cb")
+
+
 @pytest.mark.parametrize("keyside", [False, True])
 def test_chunk_scan(case, cuda, keyside):
     from linquant_amd.kernels.mamba2.chunk_scan_v2 import _quant_chunk_scan_fwd
