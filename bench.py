@@ -629,9 +629,11 @@ def main():
     def step():
         kw = {}
         if keyside:  # one prologue launch also stores the rotated fp16 B of the key-side chunk state
-            x, qB, qC, b_fp = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
-                                                           sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True)
-            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"])
+            # (and its per-token maxima, which the chunk state needs to leave out all-zero slabs)
+            x, qB, qC, b_fp, b_rmax = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                                   sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True,
+                                                                   return_b_rowmax=True)
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"], b_rowmax=b_rmax)
         else:
             x, qB, qC = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
                                                      sc["B_inv_scale"], sc["C_inv_scale"])
@@ -680,9 +682,9 @@ def main():
     def step_staged():
         kw = {}
         if keyside:
-            x, qB, qC, b_fp = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"],
-                                      sc["C_inv_scale"], return_b_fp=True)
-            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"])
+            x, qB, qC, b_fp, b_rmax = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"],
+                                              sc["C_inv_scale"], return_b_fp=True, return_b_rowmax=True)
+            kw = dict(keyside=True, x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"], b_rowmax=b_rmax)
         else:
             x, qB, qC = fused_t(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim, sc["B_inv_scale"],
                                 sc["C_inv_scale"])

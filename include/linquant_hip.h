@@ -112,6 +112,8 @@ typedef struct {
   float* b_rowmax;           /* NULL, or (B,L,G) fp32 scratch: the call first fills it with max_n |B[b,l,g,n]| and then leaves
                                 out every 64-token slab whose gated key codes are provably all zero (same result, bit for
                                 bit; see the kernel's header).  Contents undefined on entry. */
+  int32_t b_rowmax_ready;    /* 1: b_rowmax already holds the row maxima (lq_split_rotate_quant_xBC wrote them beside b_fp):
+                                the pre-pass over B is left out */
 } lq_chunk_state_key_args;
 int lq_chunk_state_key(const lq_chunk_state_key_args* args, hipStream_t stream);
 
@@ -230,6 +232,8 @@ typedef struct {
                                 on entry and on return (ignored by lq_ssd_combined_static) */
   int64_t workspace_bytes;
   int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size;
+  const float* b_rowmax;     /* key side, optional: (B,L,G) fp32 max_n |b_fp| per token row as lq_split_rotate_quant_xBC
+                                writes it beside b_fp; NULL: the call computes it into the workspace */
 } lq_ssd_combined_args;
 int lq_ssd_combined(const lq_ssd_combined_args* args, hipStream_t stream);
 /* workspace size for the dims in `args` (pointers are not read), written to *bytes */
@@ -266,6 +270,8 @@ typedef struct {
   const float* dqk_b;        /* (G*N,) fp32 holding fp16-rounded values, or NULL */
   const float* dqk_c;
   int32_t batch, seqlen, d_ssm, ngroups, dstate;
+  float* b_rowmax;           /* NULL, or (B,T,G) fp32: max_n |b_fp[b,t,g,n]| per token row (needs b_fp), the table the
+                                key-side chunk state uses to leave out all-zero slabs (its b_rowmax with b_rowmax_ready) */
 } lq_split_rotate_quant_xBC_args;
 int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* args, hipStream_t stream);
 

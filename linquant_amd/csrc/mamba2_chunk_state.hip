@@ -53,6 +53,7 @@ struct Params {
   const float* bgs;
   int64_t sbg_b, sbg_c, sbg_h, sbg_n;
   const float* rowmax;  // key side, optional: (B,L,G) max_n |B|, filled by row_absmax_kernel
+  int rowmax_ready;     // the table is already filled (by the prologue that produced B)
   int8_t* states;
   int64_t sst_b;        // elements between batch rows of states
   int batch, seqlen, nheads, P, G, N, Q, nchunks, n_ntiles;
@@ -430,7 +431,9 @@ int launch(const Params& p, hipStream_t stream) {
   if (q.sst_b == 0) q.sst_b = (int64_t)p.nchunks * p.nheads * p.P * p.N;
   if (q.sst_b % 16 != 0) return LQ_ERR_SHAPE;
   if (KEYSIDE && p.rowmax) {
-    if (p.N != 64 && p.N != 128 && p.N != 256) {
+    if (p.rowmax_ready) {
+      // nothing to do: the caller's table is used as it is
+    } else if (p.N != 64 && p.N != 128 && p.N != 256) {
       q.rowmax = nullptr;  // no pre-pass for this width: every slab is processed
     } else {
       const int64_t rows = (int64_t)p.batch * p.seqlen * p.G;
@@ -511,6 +514,8 @@ extern "C" int lq_chunk_state_key(const lq_chunk_state_key_args* a, hipStream_t 
   p.oqs = a->out_qscale, p.soq_h = a->oqs_stride_h, p.soq_p = a->oqs_stride_p;
   p.bgs = a->b_gate_scale;
   p.rowmax = a->b_rowmax;
+  p.rowmax_ready = a->b_rowmax_ready;
+  if (p.rowmax_ready != 0 && p.rowmax_ready != 1) return LQ_ERR_SHAPE;
   p.sbg_b = a->bgs_stride_b, p.sbg_c = a->bgs_stride_c, p.sbg_h = a->bgs_stride_h, p.sbg_n = a->bgs_stride_n;
   p.states = a->states, p.sst_b = a->states_stride_b;
   p.batch = a->batch, p.seqlen = a->seqlen, p.nheads = a->nheads, p.P = a->headdim, p.G = a->ngroups, p.N = a->dstate;

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
                                                      const void* __restrict__ signs, int signs_dtype,
                                                      const float* __restrict__ inv0, const float* __restrict__ inv1,
                                                      const float* __restrict__ dqk0, const float* __restrict__ dqk1,
-                                                     int T, float hb, float kron) {
+                                                     int T, float hb, float kron, float* __restrict__ rowmax) {
   constexpr int LPR = N / 8;       // lanes per row
   constexpr int LPH = LPR / 2;     // lanes per half
   constexpr int RPB = 256 / LPR;   // rows per block
@@ -128,6 +128,21 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
       fwht_row<LPH>(v, sub, hb, kron);
     }
   }
+  // max |fp16 value| of the rotated B row, for the key-side chunk state's zero-slab test: the same comparison sequence as
+  // its own pre-pass (a NaN wins, so a row holding one is never left out)
+  float rmax = 0.0f;
+  if (QUANT && rowmax && side == 0) {  // uniform over the block
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float a = __builtin_fabsf((float)(_Float16)v[i]);
+      rmax = (a > rmax || a != a) ? a : rmax;
+    }
+#pragma unroll
+    for (int o = 1; o < LPR; o <<= 1) {
+      const float t2 = __shfl_xor(rmax, o, 64);
+      rmax = (t2 > rmax || t2 != t2) ? t2 : rmax;
+    }
+  }
   if (!live) return;
   if (QUANT) {
     const float inv = (side ? inv1 : inv0)[seg];
@@ -144,6 +159,7 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
 #pragma unroll
       for (int i = 0; i < 8; ++i) f[i] = (_Float16)v[i];
       *(lq_v8h*)(fp0 + (((int64_t)b * T + t) * nseg_per_side + seg) * N + sub * 8) = f;
+      if (rowmax && sub == 0) rowmax[((int64_t)b * T + t) * nseg_per_side + seg] = rmax;
     }
   } else {
     _Float16* dp = (_Float16*)dst0 + (((int64_t)b * T + t) * nseg_per_side + seg) * N + sub * 8;
@@ -179,6 +195,7 @@ extern "C" int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* a
     return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * 2 * G > 65535) return LQ_ERR_SHAPE;
   if (a->b_fp && !al(a->b_fp, 16)) return LQ_ERR_SHAPE;
+  if (a->b_rowmax && !a->b_fp) return LQ_ERR_NULL;
   const _Float16* src = (const _Float16*)a->xBC + a->d_ssm;
   const float hb = hblock_value(N / 2);
   const float kron = (float)(1.0 / sqrt(2.0));
@@ -188,7 +205,7 @@ extern "C" int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* a
 #define LQ_ROT_LAUNCH(NN, VV)                                                                                          \
   hipLaunchKernelGGL((rotate_kernel<NN, true, VV>), grid, dim3(256), 0, stream, src, a->xBC_stride_b, a->xBC_stride_t, \
                      (int64_t)N, G, (int64_t)G * N, a->qB, a->qC, (_Float16*)a->b_fp, a->signs, a->signs_dtype,         \
-                     a->B_inv_scale, a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron)
+                     a->B_inv_scale, a->C_inv_scale, a->dqk_b, a->dqk_c, a->seqlen, hb, kron, a->b_fp ? a->b_rowmax : nullptr)
   if (N == 128) {
     if (vec) LQ_ROT_LAUNCH(128, true); else LQ_ROT_LAUNCH(128, false);
   } else {
@@ -214,21 +231,21 @@ extern "C" int lq_kron_hadamard(const lq_kron_hadamard_args* a, hipStream_t stre
     hipLaunchKernelGGL((rotate_kernel<128, false, true>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
                        a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron);
+                       a->seqlen, hb, kron, (float*)nullptr);
   else if (vec)
     hipLaunchKernelGGL((rotate_kernel<64, false, true>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
                        a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron);
+                       a->seqlen, hb, kron, (float*)nullptr);
   else if (D == 128)
     hipLaunchKernelGGL((rotate_kernel<128, false, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
                        a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron);
+                       a->seqlen, hb, kron, (float*)nullptr);
   else
     hipLaunchKernelGGL((rotate_kernel<64, false, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
                        a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
                        (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron);
+                       a->seqlen, hb, kron, (float*)nullptr);
   return lq_check_launch();
 }

@@ -70,7 +70,10 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
     k.bgs_stride_b = a->bgs_stride_b, k.bgs_stride_c = a->bgs_stride_c, k.bgs_stride_h = a->bgs_stride_h,
     k.bgs_stride_n = a->bgs_stride_n;
     k.states = states, k.states_stride_b = slots_b;
-    k.b_rowmax = (float*)(ws + l.rowmax);
+    // the table of per-token max |B| for the zero-slab test: the caller's (the prologue writes it beside b_fp) or this
+    // call's own pre-pass into the workspace
+    k.b_rowmax = a->b_rowmax ? const_cast<float*>(a->b_rowmax) : (float*)(ws + l.rowmax);
+    k.b_rowmax_ready = a->b_rowmax ? 1 : 0;
     k.batch = a->batch, k.seqlen = a->seqlen, k.nheads = a->nheads, k.headdim = a->headdim, k.ngroups = a->ngroups;
     k.dstate = a->dstate, k.chunk_size = Q;
     if ((rc = lq_chunk_state_key(&k, stream)) != LQ_OK) return rc;

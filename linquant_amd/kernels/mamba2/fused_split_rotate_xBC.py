@@ -24,12 +24,14 @@ def _signs_arg(signs):
 
 
 def fused_split_rotate_quant_xBC(xBC, r_signs, nheads, ngroups, d_state, headdim, B_inv_scale, C_inv_scale,
-                                 dqk_b=None, dqk_c=None, return_b_fp=False):
+                                 dqk_b=None, dqk_c=None, return_b_fp=False, return_b_rowmax=False):
     """xBC (B,T,d_ssm+2*G*N) fp16; r_signs (G,N) +-1 or None (split + INT8 only); B/C_inv_scale (G,) fp32;
     dqk_b/dqk_c (G*N,) or (G,N) diagonal key scalings applied (fp16-rounded) before the rotation, or None.
     Returns (x view (B,T,H,P), q_B (B,T,G,N) int8, q_C (B,T,G,N) int8).  With ``return_b_fp`` (an extension of the
     reference signature) a fourth value follows: the rotated fp16 B that q_B is quantized from, identical to
-    ``kronecker_hadamard_fwd`` of the [dqk-scaled] B lanes, so a key-side caller saves that second launch."""
+    ``kronecker_hadamard_fwd`` of the [dqk-scaled] B lanes, so a key-side caller saves that second launch.  With
+    ``return_b_rowmax`` as well a fifth: max_n |b_fp| per (batch, token, group), fp32, the table the key-side chunk state
+    uses to leave out all-zero slabs (its ``b_rowmax``), which saves that stage's pre-pass over B."""
     batch, seq_len, xBC_dim = xBC.shape
     d_ssm = nheads * headdim
     g_n = ngroups * d_state
@@ -47,13 +49,17 @@ def fused_split_rotate_quant_xBC(xBC, r_signs, nheads, ngroups, d_state, headdim
     q_B = torch.empty(batch, seq_len, ngroups, d_state, device=xBC.device, dtype=torch.int8)
     q_C = torch.empty(batch, seq_len, ngroups, d_state, device=xBC.device, dtype=torch.int8)
     b_fp = torch.empty(batch, seq_len, ngroups, d_state, device=xBC.device, dtype=torch.float16) if return_b_fp else None
+    assert return_b_fp or not return_b_rowmax, "the row maxima are a by-product of b_fp"
+    b_rowmax = torch.empty(batch, seq_len, ngroups, device=xBC.device, dtype=torch.float32) if return_b_rowmax else None
     _lib.call("lq_split_rotate_quant_xBC", xBC.device,
               xBC=_lib.ptr(xBC), xBC_stride_b=xBC.stride(0), xBC_stride_t=xBC.stride(1),
               qB=_lib.ptr(q_B), qC=_lib.ptr(q_C), b_fp=_lib.ptr(b_fp), signs=_lib.ptr(signs),
               signs_dtype=0 if signs is None else _SIGN_CODES[signs.dtype],
               B_inv_scale=_lib.ptr(_lib.f32(B_inv_scale)), C_inv_scale=_lib.ptr(_lib.f32(C_inv_scale)),
               dqk_b=_lib.ptr(dqk_b) if has_dqk else None, dqk_c=_lib.ptr(dqk_c) if has_dqk else None,
-              batch=batch, seqlen=seq_len, d_ssm=d_ssm, ngroups=ngroups, dstate=d_state)
+              batch=batch, seqlen=seq_len, d_ssm=d_ssm, ngroups=ngroups, dstate=d_state, b_rowmax=_lib.ptr(b_rowmax))
+    if return_b_rowmax:
+        return x_out, q_B, q_C, b_fp, b_rowmax
     if return_b_fp:
         return x_out, q_B, q_C, b_fp
     return x_out, q_B, q_C

@@ -27,22 +27,25 @@ def _quant_mamba_chunk_scan_combined_fwd(x_fp, q_dt, dt_scale, q_A_log, A_log_sc
                                          chunk_size, q_D, D_scale, dt_bias=None, dt_softplus=True,
                                          dt_limit=(0.0, float("inf")), static_state_scale=None, static_cb_scale=None,
                                          alpha_hp=None, bscale_g=None, keyside=False, x_scale_hp=None, b_fp=None,
-                                         b_gate_scale=None):
+                                         b_gate_scale=None, b_rowmax=None):
     """fp16 x in, INT8 chunk states (value side: x quantized per tile with ``alpha_hp`` against INT8 ``q_B``; key
     side: x quantized with ``x_scale_hp`` against gated fp16 ``b_fp`` quantized with ``b_gate_scale``), INT8
-    fixed-point recurrence, INT8 CB on ``static_cb_scale``, INT8 chunk scan. Returns (out fp16 (B,L,H,P), None)."""
+    fixed-point recurrence, INT8 CB on ``static_cb_scale``, INT8 chunk scan. Returns (out fp16 (B,L,H,P), None).
+    ``b_rowmax`` (not in the reference; key side, optional): the per-token max |b_fp| that the prologue can return beside
+    ``b_fp``; without it the chunk state stage computes the table itself.  Same result either way."""
     batch, seqlen, nheads, headdim = x_fp.shape
     _, _, ngroups, dstate = q_B.shape
 
     if not _stages_rebound():
         return _one_call(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale, chunk_size, q_D, D_scale,
                          dt_bias, dt_softplus, dt_limit, static_state_scale, static_cb_scale, alpha_hp, bscale_g, keyside,
-                         x_scale_hp, b_fp, b_gate_scale), None
+                         x_scale_hp, b_fp, b_gate_scale, b_rowmax=b_rowmax), None
 
     dA_cumsum, dt = _quant_chunk_cumsum_fwd(q_dt, dt_scale, q_A_log, A_log_scale, chunk_size, dt_bias=dt_bias,
                                             dt_softplus=dt_softplus, dt_limit=dt_limit)
     if keyside:
-        states_i8 = _chunk_state_keyside_fwd(x_fp, x_scale_hp, b_fp, dt, dA_cumsum, static_state_scale, b_gate_scale)
+        kw = {} if b_rowmax is None else {"b_rowmax": b_rowmax}
+        states_i8 = _chunk_state_keyside_fwd(x_fp, x_scale_hp, b_fp, dt, dA_cumsum, static_state_scale, b_gate_scale, **kw)
     else:
         states_i8 = _quant_chunk_state_fwd_xfp_static_int8(x_fp, q_B, dt, dA_cumsum, alpha_hp, bscale_g,
                                                            static_state_scale)
@@ -68,7 +71,7 @@ def _stages_rebound():
 
 def combined_args(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale, chunk_size, q_D, D_scale, dt_bias,
                   dt_softplus, dt_limit, static_state_scale, static_cb_scale, alpha_hp, bscale_g, keyside, x_scale_hp, b_fp,
-                  b_gate_scale, out, workspace=None, final_states=None):
+                  b_gate_scale, out, workspace=None, final_states=None, b_rowmax=None):
     """(lq_ssd_combined_args, keep-alive list) for one forward; the host-side checks of the stage wrappers apply."""
     from .chunk_cumsum import _DT_CODES, _as_f32_scalar
     from .chunk_state_keyside import _bgs_strides
@@ -109,6 +112,9 @@ def combined_args(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C,
         f.update(b_fp=_lib.ptr(b_fp), bfp_stride_b=b_fp.stride(0), bfp_stride_l=b_fp.stride(1), bfp_stride_g=b_fp.stride(2),
                  x_scale_hp=_lib.ptr(xs), xs_stride_h=xs.stride(0), xs_stride_p=xs.stride(1), b_gate_scale=_lib.ptr(bgs),
                  bgs_stride_b=sb[0], bgs_stride_c=sb[1], bgs_stride_h=sb[2], bgs_stride_n=sb[3])
+        if b_rowmax is not None:
+            assert b_rowmax.dtype == torch.float32 and b_rowmax.is_contiguous() and b_rowmax.shape == (batch, seqlen, ngroups)
+            f.update(b_rowmax=_lib.ptr(b_rowmax))
     else:
         assert q_B.dtype == torch.int8 and q_B.stride(3) == 1
         f.update(qB=_lib.ptr(q_B), qB_stride_b=q_B.stride(0), qB_stride_l=q_B.stride(1), qB_stride_g=q_B.stride(2),
@@ -130,7 +136,7 @@ def workspace_bytes(batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size)
 
 def _one_call(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale, chunk_size, q_D, D_scale, dt_bias,
               dt_softplus, dt_limit, static_state_scale, static_cb_scale, alpha_hp, bscale_g, keyside, x_scale_hp, b_fp,
-              b_gate_scale, static=False):
+              b_gate_scale, static=False, b_rowmax=None):
     batch, seqlen, nheads, headdim = x_fp.shape
     _, _, ngroups, dstate = q_C.shape
     out = torch.empty(batch, seqlen, nheads, headdim, device=x_fp.device, dtype=torch.float16)
@@ -140,7 +146,7 @@ def _one_call(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_s
                          device=x_fp.device)
     st, keep = combined_args(x_fp, q_dt, dt_scale, q_A_log, A_log_scale, q_B, B_scale, q_C, C_scale, chunk_size, q_D, D_scale,
                              dt_bias, dt_softplus, dt_limit, static_state_scale, static_cb_scale, alpha_hp, bscale_g, keyside,
-                             x_scale_hp, b_fp, b_gate_scale, out, ws)
+                             x_scale_hp, b_fp, b_gate_scale, out, ws, b_rowmax=b_rowmax)
     _lib.launch("lq_ssd_combined_static" if static else "lq_ssd_combined", x_fp.device, st)
     del keep
     return out

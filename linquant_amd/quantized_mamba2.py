@@ -149,11 +149,13 @@ class QuantizedMamba2(nn.Module):
         keyside = getattr(self, "keyside", False)
         keyside_kwargs = {}
         if keyside:  # the fp B of the key-side chunk state carries D_qk and the rotation q_B was quantized under: the
-            # prologue kernel stores it next to the codes (one launch instead of the reference's two)
-            x_fp, q_B, q_C, b_fp = fused_split_rotate_quant_xBC(
+            # prologue kernel stores it next to the codes (one launch instead of the reference's two), with its per-token
+            # maxima, which the chunk state stage would otherwise compute in a pass of its own
+            x_fp, q_B, q_C, b_fp, b_rowmax = fused_split_rotate_quant_xBC(
                 xBC, r_signs, self.nheads, self.ngroups, self.d_state, self.headdim, self.B_inv_scale, self.C_inv_scale,
-                dqk_b=dqk_b, dqk_c=dqk_c, return_b_fp=True)
-            keyside_kwargs = dict(keyside=True, x_scale_hp=self.x_quant_scale_hp, b_fp=b_fp, b_gate_scale=self.b_gate_scale)
+                dqk_b=dqk_b, dqk_c=dqk_c, return_b_fp=True, return_b_rowmax=True)
+            keyside_kwargs = dict(keyside=True, x_scale_hp=self.x_quant_scale_hp, b_fp=b_fp, b_gate_scale=self.b_gate_scale,
+                                  b_rowmax=b_rowmax)
         else:
             x_fp, q_B, q_C = fused_split_rotate_quant_xBC(xBC, r_signs, self.nheads, self.ngroups, self.d_state,
                                                           self.headdim, self.B_inv_scale, self.C_inv_scale,

@@ -368,6 +368,40 @@ def test_bmm_chunk(case, cuda, keyside):
     assert_same_codes(cb, ref["cb"], "cb")
 
 
+@pytest.mark.parametrize("keyside_rowmax", [True])
+def test_prologue_row_maxima_feed_the_chunk_state(case, cuda, keyside_rowmax):
+    """The prologue's fifth output, max_n |b_fp| per token row, is exactly that maximum; handed to the key-side chunk state
+    (alone or through the combined forward) it replaces the stage's own pre-pass: same states, same output, bit for bit."""
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.chunk_state_keyside import _chunk_state_keyside_fwd
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    s = case["shape"]
+    say("prologue row maxima", s)
+    xBC, dt_raw, p, sc = gpu_inputs(case, cuda)
+    x, qB, qC, b_fp, rmax = fused_split_rotate_quant_xBC(xBC, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                         sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True,
+                                                         return_b_rowmax=True)
+    torch.cuda.synchronize()
+    assert rmax.shape == (s.batch, s.seqlen, s.ngroups) and rmax.dtype == torch.float32
+    assert torch.equal(rmax, b_fp.float().abs().amax(dim=-1))
+    ref = case["oracle"][True]
+    dt, dA = dev(ref["dt"], cuda), dev(ref["dA_cumsum"], cuda)
+    st0 = _chunk_state_keyside_fwd(x, sc["x_scale_hp"], b_fp, dt, dA, sc["static_state_scale"], sc["b_gate_scale"])
+    st1 = _chunk_state_keyside_fwd(x, sc["x_scale_hp"], b_fp, dt, dA, sc["static_state_scale"], sc["b_gate_scale"], b_rowmax=rmax)
+    torch.cuda.synchronize()
+    assert torch.equal(st0, st1)
+    assert_same_codes(st1, ref["states"], "states")
+    kw = dict(dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+              static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], keyside=True,
+              x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"])
+    args = (x, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk, p["D"], p["D_scale"])
+    o0 = M._quant_mamba_chunk_scan_combined_fwd(*args, **kw)[0]
+    o1 = M._quant_mamba_chunk_scan_combined_fwd(*args, b_rowmax=rmax, **kw)[0]
+    torch.cuda.synchronize()
+    assert torch.equal(o0, o1)
+
+
 @pytest.mark.parametrize("L,Q,G,N,fp", [(2000, 256, 64, 64, True), (2048, 256, 64, 128, False), (300, 128, 3, 192, True),
                                         (1000, 64, 5, 256, False)])
 def test_bmm_chunk_shapes(cuda, L, Q, G, N, fp):
