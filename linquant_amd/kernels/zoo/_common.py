@@ -11,13 +11,45 @@ DECAY_NONE, DECAY_SCALAR, DECAY_DIAGONAL = 0, 1, 2
 CHUNK = 64
 
 
+def pad_keys(q, k, g, scales, rot=None):
+    """Key widths other than 64 and 128 run as the next of the two (the reference pads to the next power of two inside its
+    kernels, linquant/kernels/zoo/gla.py:253, kda.py:176, gated_delta_rule.py:182).  q and k gain zero channels: their
+    codes are zero, so every dot product, the Gram matrix and the state rows of the real channels keep their values.  A
+    per-channel decay repeats its first channel there (the envelope, a maximum over channels, is unchanged; a zero decay
+    would raise it to one), the per-channel key scale is one and a local rotation is extended by the identity.
+    Returns (q, k, g, scales, rot, K) with K the caller's key width (final states are cut back to it)."""
+    K = q.shape[-1]
+    assert 1 <= K <= 128, f"K={K}: the state kernels hold the whole key axis (K <= 128)"
+    Kp = 64 if K <= 64 else 128
+    if K == Kp:
+        return q, k, g, scales, rot, K
+    pad = Kp - K
+    q, k = torch.nn.functional.pad(q, (0, pad)), torch.nn.functional.pad(k, (0, pad))
+    if g is not None and g.dim() == 4:
+        g = torch.cat([g, g[..., :1].expand(*g.shape[:3], pad)], dim=-1)
+    scales = dict(scales)
+    kw = f32(scales["kw"])
+    assert kw.shape[-1] == K, f"scales['kw']: (H, {K}) per key channel"
+    scales["kw"] = torch.nn.functional.pad(kw, (0, pad), value=1.0)
+    if rot is not None:
+        assert tuple(rot.shape) == (K, K), "rot: (K, K) R_QK"
+        ext = torch.eye(Kp, dtype=rot.dtype, device=rot.device)
+        ext[:K, :K] = rot
+        rot = ext
+    return q, k, g, scales, rot, K
+
+
+def cut_keys(ht, K):
+    """Final state of the caller's key channels (the padded rows hold zeros)."""
+    return ht if ht is None or ht.shape[2] == K else ht[:, :, :K].contiguous()
+
+
 def check_shapes(q, k, v, chunk_size):
     B, T, H, K = q.shape
     V = v.shape[-1]
     assert T % chunk_size == 0, f"T={T} must be a multiple of the chunk size {chunk_size}"
-    assert K <= 128, f"K={K}: the state kernels hold the whole key axis (K <= 128)"
     assert chunk_size == CHUNK, f"chunk_size={chunk_size}: the HIP kernels are built for 64-token chunks"
-    assert K in (64, 128), f"K={K}: built for key dims 64 and 128"
+    assert K in (64, 128), f"K={K}: the kernels take 64 or 128 key channels (pad_keys widens anything else)"
     assert V % 64 == 0, f"V={V}: value dim must be a multiple of 64"
     assert q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype, \
         "q, k, v: one 16-bit activation dtype (fp16 or bf16)"

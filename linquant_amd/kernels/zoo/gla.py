@@ -17,13 +17,15 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
                    rot=None, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
     Returns (o, final fp32 state or None)."""
+    assert g.shape == q.shape
+    q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
-    assert chunk_size % BC == 0 and g.shape == (B, T, H, K)
+    assert chunk_size % BC == 0
     Ru = C.unrot_matrix(unrot, V)
     R = None if rot is None else rot.to(torch.float16).contiguous()
-    scale = K ** -0.5 if scale is None else scale
+    scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     gc, logenv = C.cumsum(g, B, T, H, K)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
@@ -37,4 +39,4 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     C.run_output(None, None, v, h_i8, None, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, g=gc, logenv=logenv)
-    return o, ht
+    return o, C.cut_keys(ht, K0)

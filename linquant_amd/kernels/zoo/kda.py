@@ -16,13 +16,15 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
                    output_final_state=False, unrot=None, rot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay, beta [B,T,H].
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
+    assert g.shape == q.shape
+    q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
-    assert chunk_size % BC == 0 and g.shape == (B, T, H, K) and beta.shape == (B, T, H)
+    assert chunk_size % BC == 0 and beta.shape == (B, T, H)
     Ru = C.unrot_matrix(unrot, V)
     R = None if rot is None else rot.to(torch.float16).contiguous()
-    scale = K ** -0.5 if scale is None else scale
+    scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     gc, logenv = C.cumsum(g, B, T, H, K)
     Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL)
@@ -38,4 +40,4 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     C.run_output(None, None, e_out, h_i8, None, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
-    return o, ht
+    return o, C.cut_keys(ht, K0)

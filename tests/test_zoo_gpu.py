@@ -214,6 +214,32 @@ def test_stored_state_codes_and_final_state(cuda, cell, seed):
     assert (last - codes[-1]).abs().max().item() <= limit
 
 
+@pytest.mark.parametrize("K", [16, 32, 48, 96])
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+def test_key_widths_between_the_built_ones(cuda, cell, K):
+    """Any K <= 128 as the reference takes it (/root/reference linquant/kernels/zoo/gla.py:246-253: K <= 128, tiles of
+    next_power_of_2(K) with masked channels): outputs by the reference's criterion, stored state codes of the caller's
+    K channels within one step of the oracle's (two for DeltaNet), final state of shape (B, H, K, V); the diagonal-decay
+    cells also with a local R_QK of that width where one exists (powers of two)."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell, K=K, H=2, seed=5), 256)
+    dbg = {}
+    out, ht, qz, run = _go(cell, tensors, debug=dbg, final_state=True)
+    zc.check(out, run, qz, f"{cell} K={K}")
+    assert ht.shape == (2, 2, K, 128)
+    codes = zc.state_codes(qz, run)                      # (NT, B, H, K, V)
+    got = dbg["h_i8"].cpu()                              # (B, NT, H, Kp, V)
+    assert (got[..., K:, :] == 0).all(), "state rows of the padded key channels must stay zero"
+    NT = codes.shape[0]
+    diff = (got[:, 1:, :, :K].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
+    assert diff.max().item() <= (2 if cell == "deltanet" else 1)
+    assert (diff != 0).float().mean().item() < 1e-3
+    if zc.CELLS[cell][1] == "diagonal" and K & (K - 1) == 0:
+        out, _, qz, run = _go(cell, tensors, rot=signed_hadamard(K, 3))
+        zc.check(out, run, qz, f"{cell} K={K} local R_QK")
+
+
 # Measured on MI355X (T = 256, B2, H4 / H2, 131072 .. 262144 codes per role): no code of any role differs from the
 # oracle's, in any of the six cells, at K = 64 and K = 128.  A tie between the fp32 and the float64 evaluation of an
 # exponentially weighted operand is possible in principle (about 1e-5 per code), so the bound is not zero.
