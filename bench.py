@@ -724,6 +724,12 @@ def main():
             st["int8_TOPS"] = round(int8_ops[label] / 1e12 / (st["ms"] * 1e-3), 1)
             st["int8_peak_frac"] = round(st["int8_TOPS"] / INT8_PEAK_TOPS, 4)
         st.update({k: v for k, v in counters.get(label, {}).items() if k in ("traffic_MB", "mfma_busy_frac")})
+        if "traffic_MB" in st and st["traffic_MB"] < 0.9 * st["MB"]:
+            # a data-dependent shortcut (all-zero slabs of the key-side chunk state left out) moved fewer bytes than the
+            # dense count: the fraction that describes the kernel is the one on the bytes it moved
+            st["hbm_frac_dense_bytes"] = st.pop("hbm_frac")
+            st["hbm_frac"] = round(st["traffic_MB"] / st["ms"] / HBM_PEAK_GBS, 4)
+            st["note"] = "fewer bytes moved than the dense count (zero slabs left out): hbm_frac is on the measured traffic"
     if "traffic_MB" in counters.get(dom, {}):
         roofline["traffic"] = int(counters[dom]["traffic_MB"] * 1e6)
     graph = None
