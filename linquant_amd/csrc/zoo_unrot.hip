@@ -17,8 +17,9 @@ namespace {
 
 // out[v'][c] = sum_v Rs[v'][v] * x[v][c] for one 16-column tile c: x arrives as accumulator fragments
 // d[vt][r] (rows v = 16vt + 4kg + r); slot e of step sg is channel 16*(2sg + (e >> 2)) + 4kg + (e & 3).
-template <int V>
-LQ_DEV void rotate_tile(const _Float16* Rs, const float (&d)[V / 16][4], lq_v4f (&out)[V / 16], int rl, int kg) {
+// VO output rows v' (the rows Rs holds): all V of them, or the slice a workgroup owns.
+template <int V, int VO = V>
+LQ_DEV void rotate_tile(const _Float16* Rs, const float (&d)[V / 16][4], lq_v4f (&out)[VO / 16], int rl, int kg) {
   constexpr int RS = V + 8;
   lq_v8h bop[V / 32];
 #pragma unroll
@@ -26,7 +27,7 @@ LQ_DEV void rotate_tile(const _Float16* Rs, const float (&d)[V / 16][4], lq_v4f 
 #pragma unroll
     for (int e = 0; e < 8; ++e) bop[sg][e] = (_Float16)d[2 * sg + (e >> 2)][e & 3];
 #pragma unroll
-  for (int vt = 0; vt < V / 16; ++vt) {
+  for (int vt = 0; vt < VO / 16; ++vt) {
     lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sg = 0; sg < V / 32; ++sg) {
@@ -44,16 +45,17 @@ LQ_DEV void rotate_tile(const _Float16* Rs, const float (&d)[V / 16][4], lq_v4f 
   }
 }
 
-// Rs[m][n] = R[n][m] (transposed copy, lanes walk m) or Rs[m][n] = R[m][n]
-template <int V, bool TRANSPOSE>
-LQ_DEV void stage_rotation(_Float16* Rs, const _Float16* R, int tid) {
+// Rs[m][n] = R[n][m0 + m] (transposed copy, lanes walk m) or Rs[m][n] = R[m][n]; VO rows m (a slice starting at row m0
+// in the transposed form)
+template <int V, bool TRANSPOSE, int VO = V>
+LQ_DEV void stage_rotation(_Float16* Rs, const _Float16* R, int tid, int m0 = 0) {
   constexpr int RS = V + 8;
-  for (int it = tid; it < V * (V / 8); it += 256) {
+  for (int it = tid; it < VO * (V / 8); it += 256) {
     if (TRANSPOSE) {
-      const int m = it % V, n8 = it / V;
+      const int m = it % VO, n8 = it / VO;
       lq_v8h rv;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) rv[e] = R[(8 * n8 + e) * V + m];
+      for (int e = 0; e < 8; ++e) rv[e] = R[(8 * n8 + e) * V + m0 + m];
       *(lq_v8h*)(Rs + m * RS + 8 * n8) = rv;
     } else {
       const int m = it / (V / 8), n8 = it % (V / 8);
@@ -74,15 +76,24 @@ struct UStepOps {
 
 // KP: workgroups per (batch, head) along K.  The key rows of the linear family are independent recurrences, so a
 // workgroup may own K / KP of them (the delta family reads the whole state per step: KP = 1).
-template <bool DELTA, int K, int V, int KP>
+// VS: workgroups per (batch, head, key part) along the canonical value axis, linear family only.  The un-rotation mixes
+// all rotated value channels into every canonical one, but the canonical channels are independent of each other: a
+// workgroup forms the whole rotated product of its key rows (eight INT8 products, repeated by its VS - 1 siblings) and
+// un-rotates it into its own V / VS canonical columns only, which is where the step's time goes (a quarter of the fp16
+// products and of the carry at VS = 4).  The delta family rotates the state read back into the basis of U, which needs
+// every canonical column: VS = 1.
+template <bool DELTA, int K, int V, int KP, int VS = 1>
 __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) {
   static_assert(KP == 1 || !DELTA, "the delta family needs all of K in one workgroup");
+  static_assert(VS == 1 || !DELTA, "the delta family needs all of V in one workgroup");
   constexpr int KW = K / KP, KR = KW / 4, KT = KR / 16, VT = V / 16;
+  constexpr int VO = V / VS, VOT = VO / 16;  // canonical value channels (and 16-row tiles of them) of this workgroup
   static_assert(KT >= 1, "a wave owns at least one 16-row tile");
+  static_assert(VOT >= 1, "a workgroup owns at least one 16-channel tile");
   constexpr int HS = KW + 16, ES = 64 + 16, RS = V + 8;
-  __shared__ __align__(16) unsigned char hT[V * HS];
+  __shared__ __align__(16) unsigned char hT[VO * HS];
   __shared__ __align__(16) unsigned char eT[DELTA ? V * ES : 16];
-  __shared__ __align__(16) _Float16 RuT_s[V * RS];          // RuT_s[v'][v] = Ru[v][v']: x . Ru
+  __shared__ __align__(16) _Float16 RuT_s[VO * RS];         // RuT_s[v'][v] = Ru[v][v0 + v']: x . Ru
   __shared__ __align__(16) _Float16 Ru_s[DELTA ? V * RS : 8];  // Ru_s[v'][v] = Ru[v'][v]: x . Ru^T
   __shared__ __align__(16) float ss_s[V], inv_ss_s[V], svw_s[V], inv_svw_s[V];
 
@@ -90,11 +101,12 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
   const int rl = lane & 15, kg = lane >> 4;
   const int b = blockIdx.x / p.H, h = blockIdx.x % p.H;
   const int kb = blockIdx.y * KW;  // first key row of this workgroup
+  const int v0 = VS == 1 ? 0 : (int)blockIdx.z * VO;  // first canonical value channel of this workgroup
   const int H = p.H, T = p.T, NT = p.NT;
   const int qmax = p.qmax;
   const bool bf = p.bf != 0;
 
-  stage_rotation<V, true>(RuT_s, p.unrot, tid);
+  stage_rotation<V, true, VO>(RuT_s, p.unrot, tid, v0);
   if (DELTA) stage_rotation<V, false>(Ru_s, p.unrot, tid);
   if (tid < V) {
     const float s = p.ss[h * V + tid], w = p.svw[h * V + tid];
@@ -127,10 +139,10 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
     }
   };
 
-  // carry, transposed: rows v = 16vt + 4kg + r, column k = KR*wave + 16kt + rl
-  float hc[VT][KT][4];
+  // carry, transposed: rows v = v0 + 16vt + 4kg + r, column k = KR*wave + 16kt + rl
+  float hc[VOT][KT][4];
 #pragma unroll
-  for (int vt = 0; vt < VT; ++vt)
+  for (int vt = 0; vt < VOT; ++vt)
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -143,22 +155,24 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
 
   for (int ct = 0; ct < NT; ++ct) {
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
+    // the next step's operands are requested first and without a condition (the last step asks for its own again): a
+    // request inside a branch is waited for where the paths join, in front of the products below
+    load_step(min(ct + 1, NT - 1), nxt);
     // ---- stored copy of the incoming state -> LDS (V-major), one byte per (v, k)
 #pragma unroll
-    for (int vt = 0; vt < VT; ++vt) {
-      const lq_v4f is4 = *(const lq_v4f*)(inv_ss_s + 16 * vt + 4 * kg);
+    for (int vt = 0; vt < VOT; ++vt) {
+      const lq_v4f is4 = *(const lq_v4f*)(inv_ss_s + v0 + 16 * vt + 4 * kg);
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           hT[(16 * vt + 4 * kg + r) * HS + KR * wave + 16 * kt + rl] = (unsigned char)zoo_q8(hc[vt][kt][r], is4[r], 127);
     }
-    if (ct + 1 < NT) load_step(ct + 1, nxt);
     __syncthreads();
     {
-      int8_t* dst = p.h_i8 + (((int64_t)b * NT + ct) * H + h) * V * K + kb;
+      int8_t* dst = p.h_i8 + ((((int64_t)b * NT + ct) * H + h) * V + v0) * K + kb;
       constexpr int SEG = KW / 16;
-      for (int it = tid; it < V * SEG; it += 256) {
+      for (int it = tid; it < VO * SEG; it += 256) {
         const int vr = it / SEG, sg = it % SEG;
         *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hT + vr * HS + sg * 16);
       }
@@ -220,10 +234,10 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
           d[vt][r] = x * w4[r];
         }
       }
-      lq_v4f rot[VT];
-      rotate_tile<V>(RuT_s, d, rot, rl, kg);
+      lq_v4f rot[VOT];
+      rotate_tile<V, VO>(RuT_s, d, rot, rl, kg);
 #pragma unroll
-      for (int vt = 0; vt < VT; ++vt)
+      for (int vt = 0; vt < VOT; ++vt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) hc[vt][kt][r] = hc[vt][kt][r] * cur.gam[kt] + rot[vt][r];
     }
@@ -232,10 +246,10 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
 
   if (p.ht) {
 #pragma unroll
-    for (int vt = 0; vt < VT; ++vt)
+    for (int vt = 0; vt < VOT; ++vt)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
-        *(lq_v4f*)(p.ht + (((int64_t)b * H + h) * K + kb + KR * wave + 16 * kt + rl) * V + 16 * vt + 4 * kg) =
+        *(lq_v4f*)(p.ht + (((int64_t)b * H + h) * K + kb + KR * wave + 16 * kt + rl) * V + v0 + 16 * vt + 4 * kg) =
             lq_v4f{hc[vt][kt][0], hc[vt][kt][1], hc[vt][kt][2], hc[vt][kt][3]};
   }
 }
@@ -430,11 +444,14 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
 template <bool DELTA, int K>
 int launch_state(const ZooStateParams& p, int batch, hipStream_t stream) {
   constexpr int KP = (!DELTA && K == 128) ? 2 : 1;
-  dim3 grid(batch * p.H, KP);
+  // canonical value slices of 32 (V = 128) or 16 (V = 64) channels; measured at B4 T4096 H16 K = V = 128, no decay: one
+  // slice 158 us, two 107, four 101, eight 167 (the rotated product every sibling repeats starts to dominate)
+  constexpr int VS = DELTA ? 1 : 4;
+  dim3 grid(batch * p.H, KP, VS);
   if (p.V == 128)
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP, VS>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP, VS>), grid, dim3(256), 0, stream, p);
   return lq_check_launch();
 }
 
