@@ -47,10 +47,10 @@ LQ_DEV void rotate_tile(const _Float16* Rs, const float (&d)[V / 16][4], lq_v4f 
 
 // Rs[m][n] = R[n][m0 + m] (transposed copy, lanes walk m) or Rs[m][n] = R[m][n]; VO rows m (a slice starting at row m0
 // in the transposed form)
-template <int V, bool TRANSPOSE, int VO = V>
+template <int V, bool TRANSPOSE, int VO = V, int NTHR = 256>
 LQ_DEV void stage_rotation(_Float16* Rs, const _Float16* R, int tid, int m0 = 0) {
   constexpr int RS = V + 8;
-  for (int it = tid; it < VO * (V / 8); it += 256) {
+  for (int it = tid; it < VO * (V / 8); it += NTHR) {
     if (TRANSPOSE) {
       const int m = it % VO, n8 = it / VO;
       lq_v8h rv;
@@ -82,11 +82,20 @@ struct UStepOps {
 // un-rotates it into its own V / VS canonical columns only, which is where the step's time goes (a quarter of the fp16
 // products and of the carry at VS = 4).  The delta family rotates the state read back into the basis of U, which needs
 // every canonical column: VS = 1.
-template <bool DELTA, int K, int V, int KP, int VS = 1>
-__global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) {
+// NW: wavefronts per workgroup, 4 or 8.  Each owns KW / NW key rows of the carry.  The state read and E are per token
+// tile (four of them per chunk): with eight waves, two share a token tile, both form its whole state read (the rotation
+// back into the basis of U contracts over all canonical channels) and each rotates it into, and finishes E for, one half
+// of the value channels.  The delta family's single workgroup per (batch, head) runs one dependent chain of chunk steps,
+// so halving what a wave does per step is what shortens it.
+template <bool DELTA, int K, int V, int KP, int VS = 1, int NW = 4>
+__global__ __launch_bounds__(NW * 64) void zoo_state_unrot_kernel(ZooStateParams p) {
   static_assert(KP == 1 || !DELTA, "the delta family needs all of K in one workgroup");
   static_assert(VS == 1 || !DELTA, "the delta family needs all of V in one workgroup");
-  constexpr int KW = K / KP, KR = KW / 4, KT = KR / 16, VT = V / 16;
+  static_assert(NW == 4 || (NW == 8 && DELTA), "eight waves: delta family only");
+  constexpr int NTHR = NW * 64;
+  constexpr int VH = NW / 4;               // waves per token tile = parts of the value axis of E
+  constexpr int VE = V / VH, VET = VE / 16;  // value channels (and tiles) of E one wave finishes
+  constexpr int KW = K / KP, KR = KW / NW, KT = KR / 16, VT = V / 16;
   constexpr int VO = V / VS, VOT = VO / 16;  // canonical value channels (and 16-row tiles of them) of this workgroup
   static_assert(KT >= 1, "a wave owns at least one 16-row tile");
   static_assert(VOT >= 1, "a workgroup owns at least one 16-channel tile");
@@ -98,6 +107,8 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
   __shared__ __align__(16) float ss_s[V], inv_ss_s[V], svw_s[V], inv_svw_s[V];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tt = wave & 3;                 // token tile of the state read / E
+  const int ve0 = (wave >> 2) * VE;        // first value channel of the part of E this wave finishes
   const int rl = lane & 15, kg = lane >> 4;
   const int b = blockIdx.x / p.H, h = blockIdx.x % p.H;
   const int kb = blockIdx.y * KW;  // first key row of this workgroup
@@ -106,8 +117,8 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
   const int qmax = p.qmax;
   const bool bf = p.bf != 0;
 
-  stage_rotation<V, true, VO>(RuT_s, p.unrot, tid, v0);
-  if (DELTA) stage_rotation<V, false>(Ru_s, p.unrot, tid);
+  stage_rotation<V, true, VO, NTHR>(RuT_s, p.unrot, tid, v0);
+  if (DELTA) stage_rotation<V, false, V, NTHR>(Ru_s, p.unrot, tid);
   if (tid < V) {
     const float s = p.ss[h * V + tid], w = p.svw[h * V + tid];
     ss_s[tid] = s, inv_ss_s[tid] = 1.0f / s, svw_s[tid] = w, inv_svw_s[tid] = 1.0f / w;
@@ -129,11 +140,11 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
 #pragma unroll
       for (int vt = 0; vt < VT; ++vt) o.vop[vt] = *(const lq_v4i*)(p.vqT + (cb * V + 16 * vt + rl) * 64 + 16 * kg);
     } else {
-      const int64_t tr = (t0 + 16 * wave + rl) * H + h;
+      const int64_t tr = (t0 + 16 * tt + rl) * H + h;
 #pragma unroll
       for (int ks = 0; ks < K / 64; ++ks) o.wop[ks] = *(const lq_v4i*)(p.wq + tr * K + 64 * ks + 16 * kg);
 #pragma unroll
-      for (int vt = 0; vt < VT; ++vt) o.u[vt] = *(const lq_v2i*)(p.u + tr * V + 16 * vt + 4 * kg);
+      for (int vt = 0; vt < VET; ++vt) o.u[vt] = *(const lq_v2i*)(p.u + tr * V + ve0 + 16 * vt + 4 * kg);
       o.fw = p.fw[tr];
       o.ev = p.ev[tr];
     }
@@ -172,7 +183,7 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
     {
       int8_t* dst = p.h_i8 + ((((int64_t)b * NT + ct) * H + h) * V + v0) * K + kb;
       constexpr int SEG = KW / 16;
-      for (int it = tid; it < VO * SEG; it += 256) {
+      for (int it = tid; it < VO * SEG; it += NTHR) {
         const int vr = it / SEG, sg = it % SEG;
         *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hT + vr * HS + sg * 16);
       }
@@ -194,18 +205,18 @@ __global__ __launch_bounds__(256) void zoo_state_unrot_kernel(ZooStateParams p) 
           ws[vt][r] = x * s4[r];
         }
       }
-      lq_v4f wsr[VT];
-      rotate_tile<V>(Ru_s, ws, wsr, rl, kg);
-      const int64_t eoff = ((t0 + 16 * wave + rl) * H + h) * V;
+      lq_v4f wsr[VET];
+      rotate_tile<V, VE>(Ru_s + ve0 * RS, ws, wsr, rl, kg);
+      const int64_t eoff = ((t0 + 16 * tt + rl) * H + h) * V + ve0;
 #pragma unroll
-      for (int vt = 0; vt < VT; ++vt) {
-        const lq_v4f iw4 = *(const lq_v4f*)(inv_svw_s + 16 * vt + 4 * kg);
+      for (int vt = 0; vt < VET; ++vt) {
+        const lq_v4f iw4 = *(const lq_v4f*)(inv_svw_s + ve0 + 16 * vt + 4 * kg);
         float ef[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float u = zoo_dec1(((uint32_t)cur.u[vt][r >> 1] >> (16 * (r & 1))) & 0xffffu, bf);
           ef[r] = (u - wsr[vt][r]) * cur.fw;
-          eT[(16 * vt + 4 * kg + r) * ES + 16 * wave + rl] = (unsigned char)zoo_q8(ef[r] * cur.ev, iw4[r], qmax);
+          eT[(ve0 + 16 * vt + 4 * kg + r) * ES + 16 * tt + rl] = (unsigned char)zoo_q8(ef[r] * cur.ev, iw4[r], qmax);
         }
         lq_v2i eo;
         eo[0] = (int)zoo_enc2(ef[0], ef[1], bf);
@@ -447,11 +458,13 @@ int launch_state(const ZooStateParams& p, int batch, hipStream_t stream) {
   // canonical value slices of 32 (V = 128) or 16 (V = 64) channels; measured at B4 T4096 H16 K = V = 128, no decay: one
   // slice 158 us, two 107, four 101, eight 167 (the rotated product every sibling repeats starts to dominate)
   constexpr int VS = DELTA ? 1 : 4;
+  // delta family at K = 128: eight waves, one 16-row key tile each (four waves carry two)
+  constexpr int NW = (DELTA && K == 128) ? 8 : 4;
   dim3 grid(batch * p.H, KP, VS);
   if (p.V == 128)
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP, VS>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP, VS, NW>), grid, dim3(NW * 64), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP, VS>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP, VS, NW>), grid, dim3(NW * 64), 0, stream, p);
   return lq_check_launch();
 }
 
