@@ -1,0 +1,97 @@
+"""Tensors with more than 2^31 elements (and more than 2^32 bytes): every (batch row, head) is an independent recurrence
+in both lineages, so a launch over many batch rows must reproduce, bit for bit, a launch on one batch row cut out of
+the same inputs.  The rows compared sit below 2^31 elements, across that boundary and at the far end of the tensors,
+where a 32-bit element or byte offset anywhere in a kernel would read or write the wrong place.  Inputs are drawn on
+the device (the host generator would take minutes at these sizes); no oracle is involved, the small launch is the
+reference and is itself covered by the oracle tests at the same per-row shape."""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _rows(batch):
+    return sorted({0, batch // 2 - 1, batch // 2, batch - 1})
+
+
+def test_mamba2_ssd_beyond_2_31_elements(cuda):
+    from linquant_amd.calibration import Mamba2Shape, calibrate_mamba2, mamba2_params, mamba2_synthetic
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    B, L = 52, 8192                                            # x and out: 52 * 8192 * 80 * 64 = 2.18e9 elements
+    s = Mamba2Shape(batch=B, seqlen=L, nheads=80, headdim=64, dstate=128, ngroups=1, chunk=256)
+    assert B * L * s.nheads * s.headdim > 2 ** 31
+    p = mamba2_params(s, 42, cuda)
+    cal = Mamba2Shape(batch=1, seqlen=2048, nheads=s.nheads, headdim=s.headdim, dstate=s.dstate, ngroups=1, chunk=256)
+    cx, cdt = mamba2_synthetic(cal, 1, cuda)
+    sc = calibrate_mamba2(cal, cx, cdt, p)
+    gen = torch.Generator(device=cuda).manual_seed(0)
+    xBC = torch.randn(B, L, s.xbc_dim, generator=gen, device=cuda, dtype=torch.float16)
+    dt_raw = (torch.randn(B, L, s.nheads, generator=gen, device=cuda) * 0.5 - 2.0).half()
+
+    def forward(xb, dtb):
+        x, qB, qC, b_fp, b_rmax = fused_split_rotate_quant_xBC(xb, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                               sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True,
+                                                               return_b_rowmax=True)
+        out, _ = M._quant_mamba_chunk_scan_combined_fwd(
+            x, dtb, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], keyside=True,
+            x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"], b_rowmax=b_rmax)
+        return out
+
+    print("mamba2 large: full launch", flush=True)
+    full = forward(xBC, dt_raw)
+    torch.cuda.synchronize()
+    assert full.numel() > 2 ** 31 and torch.isfinite(full[-1]).all()
+    for b in _rows(B):
+        print("mamba2 large: row", b, flush=True)
+        one = forward(xBC[b:b + 1], dt_raw[b:b + 1])
+        assert torch.equal(full[b:b + 1], one), f"batch row {b} of the {B}-row launch differs from its own launch"
+
+
+@pytest.mark.parametrize("cell", ["linear_none", "gla", "gated_deltanet", "kda"])
+def test_zoo_beyond_2_31_elements(cuda, cell):
+    from linquant_amd.kernels import zoo
+
+    B, T, H, K, V = 34, 8192, 64, 128, 128                     # q, k, v: 34 * 8192 * 64 * 128 = 2.28e9 elements each
+    assert B * T * H * K > 2 ** 31
+    gen = torch.Generator(device=cuda).manual_seed(0)
+    q = torch.randn(B, T, H, K, generator=gen, device=cuda, dtype=torch.float16)
+    k = torch.randn(B, T, H, K, generator=gen, device=cuda, dtype=torch.float16)
+    k = k / k.float().norm(dim=-1, keepdim=True).clamp_min(1e-6).half()
+    v = torch.randn(B, T, H, V, generator=gen, device=cuda, dtype=torch.float16)
+    full = lambda shape, val: torch.full(shape, val, device=cuda, dtype=torch.float32)  # noqa: E731
+    sc = {"q": full((H,), 4.0 / 127 * K ** -0.5), "k": full((H,), 0.4 / 127), "w": full((H,), 0.8 / 127),
+          "kw": full((H, K), 0.4 / 127), "vw": full((H, V), 4.0 / 127), "vl": full((H, V), 4.0 / 127),
+          "el": full((H, V), 8.0 / 127), "ew": full((H, V), 8.0 / 127), "state": full((H, V), 0.05)}
+    if cell in ("kda", "gla"):
+        g = torch.nn.functional.logsigmoid(torch.randn(B, T, H, K, generator=gen, device=cuda) + 1.0)
+    if cell in ("kda", "gated_deltanet"):
+        beta = torch.sigmoid(torch.randn(B, T, H, generator=gen, device=cuda))
+    if cell == "kda":
+        def forward(sl):
+            return zoo.chunk_kda_int8(q[sl], k[sl], v[sl], g[sl], beta[sl], sc, sigma=0.5, eta=0.0, output_final_state=True)
+    elif cell == "gla":
+        def forward(sl):
+            return zoo.chunk_gla_int8(q[sl], k[sl], v[sl], g[sl], sc, eta=0.0, output_final_state=True)
+    elif cell == "gated_deltanet":
+        gs = torch.nn.functional.logsigmoid(torch.randn(B, T, H, generator=gen, device=cuda) + 2.0)
+
+        def forward(sl):
+            return zoo.chunk_delta_int8(q[sl], k[sl], v[sl], gs[sl], beta[sl], sc, sigma=0.5, eta=1.0, output_final_state=True)
+    else:
+        def forward(sl):
+            return zoo.chunk_simple_gla_int8(q[sl], k[sl], v[sl], None, sc, eta=1.0, output_final_state=True)
+
+    print("zoo large", cell, ": full launch", flush=True)
+    o_full, ht_full = forward(slice(0, B))
+    torch.cuda.synchronize()
+    assert o_full.numel() > 2 ** 31 and torch.isfinite(o_full[-1]).all()
+    for b in _rows(B):
+        print("zoo large", cell, ": row", b, flush=True)
+        o_one, ht_one = forward(slice(b, b + 1))
+        assert torch.equal(o_full[b:b + 1], o_one), f"{cell}: batch row {b} of the {B}-row launch differs from its own launch"
+        assert torch.equal(ht_full[b:b + 1], ht_one), f"{cell}: final state of batch row {b} differs"
