@@ -95,3 +95,52 @@ def test_zoo_beyond_2_31_elements(cuda, cell):
         o_one, ht_one = forward(slice(b, b + 1))
         assert torch.equal(o_full[b:b + 1], o_one), f"{cell}: batch row {b} of the {B}-row launch differs from its own launch"
         assert torch.equal(ht_full[b:b + 1], ht_one), f"{cell}: final state of batch row {b} differs"
+
+
+def test_front_and_epilogue_stages_beyond_2_31_elements(cuda):
+    """Activation quantizer, causal conv1d + SiLU and the fused gated RMSNorm + Hadamard + INT8 stage on tensors of more
+    than 2^31 elements: slices at the start, across the 2^31-element mark and at the end equal the launch on the slice."""
+    from linquant_amd import hadamard_utils as HU
+    from linquant_amd.kernels.mamba2.causal_conv1d import causal_conv1d_fn
+    from linquant_amd.norm import rmsnorm_gated_qhad
+    from linquant_amd.w4a8_linear import _fused_fp16_to_int8
+
+    gen = torch.Generator(device=cuda).manual_seed(0)
+    # ---- activation quantizer: 900 000 rows x 2560
+    M, N = 900_000, 2560
+    assert M * N > 2 ** 31
+    x = torch.randn(M, N, generator=gen, device=cuda, dtype=torch.float16)
+    scale = torch.tensor(4.0 / 127, device=cuda)
+    print("large: fp16_to_int8", flush=True)
+    q = _fused_fp16_to_int8(x, scale)
+    mark = 2 ** 31 // N
+    for r0 in (0, mark - 8, M - 1000):
+        assert torch.equal(q[r0:r0 + 1000], _fused_fp16_to_int8(x[r0:r0 + 1000], scale)), f"rows from {r0}"
+    del x, q
+    # ---- conv1d + SiLU: 52 batch rows of the c5 layer's xBC slice inside the in_proj output
+    B, L, D = 52, 8192, 5376
+    assert B * L * D > 2 ** 31
+    proj = torch.randn(B, L, D + 80, generator=gen, device=cuda, dtype=torch.float16)
+    xin = proj[..., :D].transpose(1, 2)                        # (B, D, L) channel-last view with a padded row stride
+    w = (torch.randn(D, 4, generator=gen, device=cuda) * 0.5).half()
+    bias = (torch.randn(D, generator=gen, device=cuda) * 0.1).half()
+    print("large: conv1d", flush=True)
+    y = causal_conv1d_fn(xin, w, bias, activation="silu")
+    for b in _rows(B):
+        assert torch.equal(y[b:b + 1], causal_conv1d_fn(xin[b:b + 1], w, bias, activation="silu")), f"conv batch row {b}"
+    del proj, xin, y
+    # ---- gated RMSNorm + Hadamard + INT8: 450 000 rows x 5120
+    R, d_ssm = 450_000, 5120
+    assert R * d_ssm > 2 ** 31
+    HU.register_hadamard(40, HU.hadamard_matrix(40))
+    yv = torch.randn(R, d_ssm, generator=gen, device=cuda, dtype=torch.float16)
+    zv = torch.randn(R, d_ssm, generator=gen, device=cuda, dtype=torch.float16)
+    wn = (1 + 0.1 * torch.randn(d_ssm, generator=gen, device=cuda)).half()
+    print("large: norm + hadamard", flush=True)
+    qo = rmsnorm_gated_qhad(yv, zv, wn, 4.0 / 127, 1e-5, d_ssm)
+    codes = qo[0] if isinstance(qo, tuple) else qo
+    mark = 2 ** 31 // d_ssm
+    for r0 in (0, mark - 8, R - 512):
+        part = rmsnorm_gated_qhad(yv[r0:r0 + 512], zv[r0:r0 + 512], wn, 4.0 / 127, 1e-5, d_ssm)
+        part = part[0] if isinstance(part, tuple) else part
+        assert torch.equal(codes[r0:r0 + 512], part), f"norm rows from {r0}"
