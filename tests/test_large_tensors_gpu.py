@@ -144,3 +144,65 @@ def test_front_and_epilogue_stages_beyond_2_31_elements(cuda):
         part = rmsnorm_gated_qhad(yv[r0:r0 + 512], zv[r0:r0 + 512], wn, 4.0 / 127, 1e-5, d_ssm)
         part = part[0] if isinstance(part, tuple) else part
         assert torch.equal(codes[r0:r0 + 512], part), f"norm rows from {r0}"
+
+
+def test_long_sequences(cuda):
+    """262 144 tokens per sequence (1024 Mamba-2 chunks, 4096 zoo chunks): two batch rows holding the same data give the
+    same bits although the second lies beyond 2^31 elements, and the causal prefix equals a launch on the prefix alone."""
+    from linquant_amd.calibration import Mamba2Shape, calibrate_mamba2, mamba2_params, mamba2_synthetic
+    from linquant_amd.kernels import zoo
+    from linquant_amd.kernels.mamba2 import ssd_combined as M
+    from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
+
+    L = 262_144
+    s = Mamba2Shape(batch=2, seqlen=L, nheads=80, headdim=64, dstate=128, ngroups=1, chunk=256)
+    p = mamba2_params(s, 42, cuda, a_max=1.3)                  # weak decay: the state carries across many chunks
+    cal = Mamba2Shape(batch=1, seqlen=2048, nheads=s.nheads, headdim=s.headdim, dstate=s.dstate, ngroups=1, chunk=256)
+    cx, cdt = mamba2_synthetic(cal, 1, cuda, dt_mean=-4.5)
+    sc = calibrate_mamba2(cal, cx, cdt, p)
+    gen = torch.Generator(device=cuda).manual_seed(0)
+    row = torch.randn(1, L, s.xbc_dim, generator=gen, device=cuda, dtype=torch.float16)
+    dt_row = (torch.randn(1, L, s.nheads, generator=gen, device=cuda) * 0.5 - 4.5).half()
+    xBC, dt_raw = row.repeat(2, 1, 1), dt_row.repeat(2, 1, 1)
+    assert xBC.numel() > 2 ** 31
+    del row
+
+    def forward(xb, dtb):
+        x, qB, qC, b_fp, b_rmax = fused_split_rotate_quant_xBC(xb, p["r_signs"], s.nheads, s.ngroups, s.dstate, s.headdim,
+                                                               sc["B_inv_scale"], sc["C_inv_scale"], return_b_fp=True,
+                                                               return_b_rowmax=True)
+        out, _ = M._quant_mamba_chunk_scan_combined_fwd(
+            x, dtb, p["dt_scale"], p["A_log"], p["A_log_scale"], qB, sc["B_scale"], qC, sc["C_scale"], s.chunk,
+            p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+            static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], keyside=True,
+            x_scale_hp=sc["x_scale_hp"], b_fp=b_fp, b_gate_scale=sc["b_gate_scale"], b_rowmax=b_rmax)
+        return out
+
+    print("long: mamba2", flush=True)
+    out = forward(xBC, dt_raw)
+    assert torch.isfinite(out[1, -256:]).all()
+    assert torch.equal(out[0], out[1]), "two batch rows with the same data differ"
+    short = forward(xBC[:1, :8192], dt_raw[:1, :8192])
+    assert torch.equal(out[:1, :8192], short), "causal prefix differs from the launch on the prefix"
+    del out, short, xBC, dt_raw
+
+    B, T, H, K, V = 3, L, 24, 128, 128
+    assert B * T * H * K > 2 ** 31
+    q1 = torch.randn(1, T, H, K, generator=gen, device=cuda, dtype=torch.float16)
+    k1 = torch.randn(1, T, H, K, generator=gen, device=cuda, dtype=torch.float16)
+    k1 = k1 / k1.float().norm(dim=-1, keepdim=True).clamp_min(1e-6).half()
+    v1 = torch.randn(1, T, H, V, generator=gen, device=cuda, dtype=torch.float16)
+    g1 = torch.nn.functional.logsigmoid(torch.randn(1, T, H, K, generator=gen, device=cuda) + 1.0)
+    b1 = torch.sigmoid(torch.randn(1, T, H, generator=gen, device=cuda))
+    q, k, v, g, beta = (t.repeat(B, *([1] * (t.dim() - 1))) for t in (q1, k1, v1, g1, b1))
+    del q1, k1, v1, g1, b1
+    full = lambda shape, val: torch.full(shape, val, device=cuda, dtype=torch.float32)  # noqa: E731
+    zs = {"q": full((H,), 4.0 / 127 * K ** -0.5), "k": full((H,), 0.4 / 127), "w": full((H,), 0.8 / 127),
+          "kw": full((H, K), 0.4 / 127), "el": full((H, V), 8.0 / 127), "ew": full((H, V), 8.0 / 127),
+          "state": full((H, V), 0.05)}
+    print("long: kda", flush=True)
+    o, ht = zoo.chunk_kda_int8(q, k, v, g, beta, zs, sigma=0.5, eta=0.0, output_final_state=True)
+    assert torch.isfinite(o[-1, -64:]).all() and torch.isfinite(ht).all()
+    assert torch.equal(o[0], o[2]) and torch.equal(ht[0], ht[2]), "batch rows with the same data differ"
+    o_s, _ = zoo.chunk_kda_int8(q[:1, :4096], k[:1, :4096], v[:1, :4096], g[:1, :4096], beta[:1, :4096], zs, sigma=0.5, eta=0.0)
+    assert torch.equal(o[:1, :4096], o_s), "causal prefix differs from the launch on the prefix"
