@@ -53,6 +53,25 @@ def test_null_and_shape_errors_without_launch():
     assert lib.lq_chunk_cumsum(ctypes.byref(st2), None) == -22
 
 
+def test_every_entry_point_rejects_an_empty_argument_struct():
+    """A zeroed argument struct (every pointer NULL, every size 0) and a NULL struct pointer come back as an error code
+    from every entry point: nothing is launched and no device is touched."""
+    lib = _lib.load()
+    checked = 0
+    for fn in _lib.FUNCTIONS:
+        sname = _lib._SHARED_ARGS.get(fn, fn + "_args")
+        if sname not in _lib.STRUCTS:
+            continue
+        f = getattr(lib, fn)
+        if fn == "lq_ssd_combined_workspace_bytes":   # (args, int64_t* bytes)
+            f.argtypes = [ctypes.POINTER(_lib.STRUCTS[sname]), ctypes.c_void_p]
+        st = _lib.STRUCTS[sname]()
+        assert f(ctypes.byref(st), None) in (-14, -22), fn
+        assert f(None, None) in (-14, -22), fn
+        checked += 1
+    assert checked >= 20
+
+
 def test_wrapper_contracts_raise_assertion_errors():
     from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
     from linquant_amd.kernels.mamba2.bmm_chunk import _quant_bmm_chunk_fwd
