@@ -120,7 +120,7 @@ def stage_bytes(s, keyside):
 
 
 ZOO_WORKLOADS = {
-    # name: (cell, B, T, H, K, V, description) -- shapes of BASELINE.json configs[0..3]
+    # name: (cell, B, T, H, K, V, description) -- shapes of the first four benchmark configurations
     "c1": ("mamba2", 1, 2048, 8, 64, 64, "configs[0]: Mamba-2 cell (linear family, scalar decay) B=1 T=2048 H=8 K=V=64 chunk 64"),
     "c2_la": ("linear_none", 4, 4096, 16, 128, 128, "configs[1]: linear attention B=4 T=4096 H=16 K=V=128 chunk 64, q,k pre-rotated"),
     "c2_gla": ("gla", 4, 4096, 16, 128, 128, "configs[1]: GLA B=4 T=4096 H=16 K=V=128 chunk 64, local R_QK in the A kernel"),
