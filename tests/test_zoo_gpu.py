@@ -104,6 +104,35 @@ def test_beta_placement(cuda, cell, rho, tau):
     zc.check(out, run, qz, f"{cell} sigma={rho} tau={tau}")
 
 
+@pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet"])
+@pytest.mark.parametrize("sigma,tau,eta", [(1.0, 1.0, 1.0), (0.0, 1.0, 1.0), (0.5, 0.5, 1.0), (1.0, 1.0, 0.0), (0.0, 1.0, 0.5)])
+def test_delta_placement_and_eta_grid_of_the_reference(cuda, cell, sigma, tau, eta):
+    """The (sigma, tau, eta) combinations of /root/reference tests/test_kernel_delta.py:36-54, with and without decay."""
+    tensors = zc.inputs(cell)
+    out, _, qz, run = _go(cell, tensors, eta=eta, rho=sigma, tau=tau)
+    zc.check(out, run, qz, f"{cell} sigma={sigma} tau={tau} eta={eta}")
+
+
+@pytest.mark.parametrize("sigma,tau,eta", [(1.0, 1.0, 0.0), (0.0, 1.0, 0.5), (0.5, 0.5, 1.0)])
+def test_kda_placement_and_eta_grid_of_the_reference(cuda, sigma, tau, eta):
+    """/root/reference tests/test_kernel_kda.py:24-37."""
+    tensors = zc.inputs("kda")
+    out, _, qz, run = _go("kda", tensors, eta=eta, rho=sigma, tau=tau)
+    zc.check(out, run, qz, f"kda sigma={sigma} tau={tau} eta={eta}")
+
+
+@pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet"])
+@pytest.mark.parametrize("n", [128, 512])
+def test_delta_canonical_storage_with_the_write_gate_on_the_value_side(cuda, cell, n):
+    """Canonical R_V storage at sigma = 0 (/root/reference tests/test_kernel_delta.py:57-80; sigma = 1 is covered by
+    test_canonical_storage_rv)."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell), n)
+    out, _, qz, run = _go(cell, tensors, eta=1.0, rho=0.0, tau=1.0, rot_v=signed_hadamard(128, 7))
+    zc.check(out, run, qz, f"{cell} canonical R_V sigma=0 T={n}")
+
+
 @pytest.mark.parametrize("cell", list(zc.CELLS))
 @pytest.mark.parametrize("policy", ["kernel_pt", "kernel_ptk"])
 def test_policies(cuda, cell, policy):
@@ -164,6 +193,39 @@ def test_canonical_storage_rv(cuda, cell, n, K, V):
     tensors = zc.cut(zc.inputs(cell, K=K, V=V, H=2 if K == 128 else 4), n)
     out, _, qz, run = _go(cell, tensors, eta=1.0, rot_v=signed_hadamard(V, 7))
     zc.check(out, run, qz, f"{cell} canonical R_V T={n} K={K} V={V}")
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+@pytest.mark.parametrize("storage", ["canonical", "rotated"])
+def test_rv_storage_per_tensor_policy(cuda, cell, storage):
+    """R_V under the per-tensor policy with the state stored canonically (in-kernel un-rotation) or rotated (fp32 output
+    in the rotated basis, un-rotated by the caller at the exit): /root/reference tests/test_kernel_regimes.py:80-128."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.inputs(cell)
+    q, k, v, g, beta = tensors
+    R = signed_hadamard(v.shape[-1], 2)
+    eta = DEFAULT_ETA[cell]
+    qz, run = zc.calibrated(cell, tensors, policy="kernel_pt", eta=eta, rot_v=R, storage=storage)
+    B, T, H, K = q.shape
+    scales = qz.kernel_scales(0, H, K, v.shape[-1], delta=zc.CELLS[cell][0] == "delta")
+    vr = (v.double() @ R).to(v.dtype)
+    if storage == "canonical":
+        out, _ = zc.run_kernel(cell, (q, k, vr, g, beta), scales, eta=eta, unrot=R.T.contiguous())
+    else:
+        out, _ = zc.run_kernel(cell, (q, k, vr, g, beta), scales, eta=eta, out_dtype=torch.float32)
+        assert out.dtype == torch.float32
+        out = (out.float() @ R.T.float().to(out.device)).to(v.dtype)
+    torch.cuda.synchronize()
+    zc.check(out, run, qz, f"{cell} R_V {storage} kernel_pt")
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+def test_per_tensor_policy_with_six_bit_codes(cuda, cell):
+    """kernel_pt with INT6 codes in INT8 containers (/root/reference tests/test_kernel_regimes.py:31-34)."""
+    tensors = zc.cut(zc.inputs(cell, seed=2), 256)
+    out, _, qz, run = _go(cell, tensors, policy="kernel_pt", bits=6)
+    zc.check(out, run, qz, f"{cell} kernel_pt bits=6")
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))

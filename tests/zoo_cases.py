@@ -67,7 +67,7 @@ def cut(tensors, n):
 
 
 def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None, out_dtype=None,
-               calib_tensors=None):
+               calib_tensors=None, storage=None):
     """Returns (qz, run): the oracle's quantizer with scales calibrated on these inputs (or on ``calib_tensors``, a
     separate batch), and a closure that evaluates the oracle on ``tensors`` under the quantizer's current arithmetic
     mode; like the kernels, the oracle materializes its output in the activation dtype unless ``out_dtype`` says
@@ -80,7 +80,7 @@ def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.
         q, k, v, g, beta = t
         return Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=qz, eta=eta, rho=rho,
                                tau=tau, read_post=True, C=64, out_dtype=out_dtype, rot_qk=rot_qk, rot_v=rot_v,
-                               storage="canonical" if rot_v is not None else "rotated")
+                               storage=storage or ("canonical" if rot_v is not None else "rotated"))
 
     qz.calibrating = True
     forward(tensors if calib_tensors is None else calib_tensors)
