@@ -565,6 +565,41 @@ typedef struct {
 } lq_absmax_args;
 int lq_absmax(const lq_absmax_args* args, hipStream_t stream);
 
+/* replaces the chunk-state observer of scripts/nemotron_h_calibration.py:602-651, which wraps the unquantized
+ * _chunk_state_fwd and keeps amax over (batch, chunk, N) of its fp32 result per (H, P):
+ *   S[b,c,h][p][n] = sum_{k in chunk c} x[b,k,h,p] * gate[b,k,h] * B[b,k,h / heads_per_group,n]
+ *   out[h][p] = max(out[h][p], max_{b,c,n} |S|)      (fp32 products and sums; the caller zero-fills `out` once)
+ * gate = exp(dA_last - dA_k) * dt_k, fp32. */
+typedef struct {
+  const void* x;             /* (B,L,H,P) view, unit P stride */
+  int32_t x_dtype;           /* LQ_DT_F16 / LQ_DT_BF16 / LQ_DT_F32 */
+  int64_t x_stride_b, x_stride_l, x_stride_h;
+  const void* B;             /* (B,L,G,N) view, unit N stride, 16-byte aligned rows */
+  int32_t B_dtype;
+  int64_t B_stride_b, B_stride_l, B_stride_g;
+  const float* gate;         /* (B,L,H) fp32 view */
+  int64_t gate_stride_b, gate_stride_l, gate_stride_h;
+  float* out;                /* (H,P) fp32, updated in place */
+  int32_t batch, seqlen, nheads, headdim, ngroups, dstate, chunk_size; /* P a multiple of 64; N 64, 128 or 256 */
+} lq_absmax_chunk_state_args;
+int lq_absmax_chunk_state(const lq_absmax_chunk_state_args* args, hipStream_t stream);
+
+/* replaces the C.B^T observer of scripts/nemotron_h_w4a8.py:126-169, which wraps the unquantized _bmm_chunk_fwd and
+ * keeps amax over (batch, chunk, Q, Q) of its result per group:
+ *   CB[b,c,g][m][k] = sum_n C[b,c*Q+m,g,n] * B[b,c*Q+k,g,n]     (every (m, k) pair of a chunk, not only k <= m)
+ *   out[g] = max(out[g], max |CB|) */
+typedef struct {
+  const void* C;             /* (B,L,G,N) view, unit N stride, 16-byte aligned rows */
+  int32_t C_dtype;
+  int64_t C_stride_b, C_stride_l, C_stride_g;
+  const void* B;
+  int32_t B_dtype;
+  int64_t B_stride_b, B_stride_l, B_stride_g;
+  float* out;                /* (G,) fp32, updated in place */
+  int32_t batch, seqlen, ngroups, dstate, chunk_size; /* N a multiple of 8 */
+} lq_absmax_cb_args;
+int lq_absmax_cb(const lq_absmax_cb_args* args, hipStream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Measurement aid (no counterpart in the reference): a matrix-core-only launch whose rate is the MFMA issue peak of
  * the machine, the denominator of the "fraction of INT8 MFMA peak" figures (the reference's metric is quoted against

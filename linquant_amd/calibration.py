@@ -96,37 +96,44 @@ def calibrate_mamba2(shape: Mamba2Shape, xBC, dt_raw, params, head_block: int = 
     A = -torch.exp(params["A_log_scale"] * params["A_log"].float())  # (H,)
     dA = (dt * A).view(B, nc, Q, H).cumsum(dim=2)
     gate = (torch.exp(dA[:, :, -1:, :] - dA) * dt.view(B, nc, Q, H))  # (B,nc,Q,H)
-    cb = torch.einsum("bcqgn,bckgn->bcgqk", Crot.view(B, nc, Q, G, N), Brot.view(B, nc, Q, G, N))
-    static_cb_scale = (cb.abs().amax(dim=(0, 1, 3, 4)) / 127.0).clamp_min(1e-8)
-    del cb
+    on_gpu = xBC.is_cuda
+    if on_gpu:  # the C.B^T observer as a device reduction: the products are never stored
+        cb_amax = torch.zeros(G, device=dev)
+        absmax_cb_update(cb_amax, Crot.contiguous(), Brot.contiguous(), Q)
+        static_cb_scale = (cb_amax / 127.0).clamp_min(1e-8)
+    else:
+        cb = torch.einsum("bcqgn,bckgn->bcgqk", Crot.view(B, nc, Q, G, N), Brot.view(B, nc, Q, G, N))
+        static_cb_scale = (cb.abs().amax(dim=(0, 1, 3, 4)) / 127.0).clamp_min(1e-8)
+        del cb
     alpha = torch.empty(H, P, device=dev)
     x_scale = torch.empty(H, P, device=dev)
     b_gate = torch.empty(H, N, device=dev)
     state_scale = torch.empty(H, P, device=dev)
     rep = H // G
-    on_gpu = xBC.is_cuda
-    if on_gpu:  # the three element-wise observers as device reductions straight from the fp16 view (no fp32 copy of x)
+    if on_gpu:  # every observer as a device reduction straight from the fp16 view (no fp32 copy of x, no stored states)
         gate_blh = gate.reshape(B, L, H)
-        xs_hp, x_hp, bg_hn = (torch.zeros(n, device=dev) for n in (H * P, H * P, H * N))
+        xs_hp, x_hp, bg_hn, st_hp = (torch.zeros(n, device=dev) for n in (H * P, H * P, H * N, H * P))
         x_view = xBC[..., :d_ssm].view(B, L, H, P)
+        Bc = Brot.contiguous()
         absmax_update(xs_hp, x_view, "pc_static", gate=gate_blh)
         absmax_update(x_hp, x_view, "pc_static")
-        absmax_update(bg_hn, Brot.contiguous(), "pc_static", gate=gate_blh, heads_per_group=rep)
-    for h0 in range(0, H, head_block):
-        h1 = min(H, h0 + head_block)
-        xh = xBC[..., h0 * P:h1 * P].float().view(B, nc, Q, h1 - h0, P)
-        gh = gate[..., h0:h1]
-        xg = xh * gh[..., None]
-        gidx = torch.arange(h0, h1, device=dev) // rep
-        Bh = Brot.view(B, nc, Q, G, N)[:, :, :, gidx]  # (B,nc,Q,hb,N)
-        if not on_gpu:
+        absmax_update(bg_hn, Bc, "pc_static", gate=gate_blh, heads_per_group=rep)
+        absmax_chunk_state_update(st_hp, x_view, Bc, gate_blh, Q)
+        state_scale = st_hp.view(H, P) / 127.0
+        alpha, x_scale, b_gate = xs_hp.view(H, P) / 127.0, x_hp.view(H, P) / 127.0, bg_hn.view(H, N)
+    else:  # the same observers as torch expressions (CPU tensors: the checker's side of the CPU tests)
+        for h0 in range(0, H, head_block):
+            h1 = min(H, h0 + head_block)
+            xh = xBC[..., h0 * P:h1 * P].float().view(B, nc, Q, h1 - h0, P)
+            gh = gate[..., h0:h1]
+            xg = xh * gh[..., None]
+            gidx = torch.arange(h0, h1, device=dev) // rep
+            Bh = Brot.view(B, nc, Q, G, N)[:, :, :, gidx]  # (B,nc,Q,hb,N)
             alpha[h0:h1] = xg.abs().amax(dim=(0, 1, 2)) / 127.0
             x_scale[h0:h1] = xh.abs().amax(dim=(0, 1, 2)) / 127.0
             b_gate[h0:h1] = (Bh * gh[..., None]).abs().amax(dim=(0, 1, 2))
-        st = torch.einsum("bcqhp,bcqhn->bchpn", xg, Bh)
-        state_scale[h0:h1] = st.abs().amax(dim=(0, 1, 4)) / 127.0
-    if on_gpu:
-        alpha, x_scale, b_gate = xs_hp.view(H, P) / 127.0, x_hp.view(H, P) / 127.0, bg_hn.view(H, N)
+            st = torch.einsum("bcqhp,bcqhn->bchpn", xg, Bh)
+            state_scale[h0:h1] = st.abs().amax(dim=(0, 1, 4)) / 127.0
     tiny = 1e-8
     return dict(
         B_scale=B_scale.float().contiguous(), C_scale=C_scale.float().contiguous(),
@@ -165,6 +172,47 @@ def absmax_update(out: torch.Tensor, x: torch.Tensor, scheme: str, gate: torch.T
               x_stride_h=x.stride(2), gate=_lib.ptr(gate), gate_stride_b=0 if gate is None else gate.stride(0),
               gate_stride_t=0 if gate is None else gate.stride(1), gate_stride_h=0 if gate is None else gate.stride(2),
               out=_lib.ptr(out), batch=B, rows=T, nheads=H, dim=D, heads_per_group=heads_per_group, mode=mode)
+    return out
+
+
+def _dt_code(t):
+    from linquant_amd import _lib
+
+    return {torch.float16: _lib.LQ_DT_F16, torch.bfloat16: _lib.LQ_DT_BF16, torch.float32: _lib.LQ_DT_F32}[t.dtype]
+
+
+def absmax_chunk_state_update(out: torch.Tensor, x: torch.Tensor, B: torch.Tensor, gate: torch.Tensor, chunk_size: int) -> torch.Tensor:
+    """``out[h, p] = max(out[h, p], max_{b, chunk, n} |sum_k x[b,k,h,p] gate[b,k,h] B[b,k,g,n]|)`` on the device, in place:
+    the chunk-state observer of the reference's calibration script (scripts/nemotron_h_calibration.py:602-651) without
+    materializing the fp32 states.  x (B,L,H,P) and B (B,L,G,N) views with unit last stride, gate (B,L,H) fp32, out (H,P)
+    fp32 zero-filled before the first batch."""
+    from linquant_amd import _lib
+
+    Bn, L, H, P = x.shape
+    G, N = B.shape[2], B.shape[3]
+    assert x.stride(3) == 1 and B.stride(3) == 1 and B.shape[:2] == (Bn, L) and H % G == 0
+    assert gate.dtype == torch.float32 and gate.shape == (Bn, L, H)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.numel() == H * P
+    _lib.call("lq_absmax_chunk_state", x.device, x=_lib.ptr(x), x_dtype=_dt_code(x), x_stride_b=x.stride(0),
+              x_stride_l=x.stride(1), x_stride_h=x.stride(2), B=_lib.ptr(B), B_dtype=_dt_code(B), B_stride_b=B.stride(0),
+              B_stride_l=B.stride(1), B_stride_g=B.stride(2), gate=_lib.ptr(gate), gate_stride_b=gate.stride(0),
+              gate_stride_l=gate.stride(1), gate_stride_h=gate.stride(2), out=_lib.ptr(out), batch=Bn, seqlen=L, nheads=H,
+              headdim=P, ngroups=G, dstate=N, chunk_size=chunk_size)
+    return out
+
+
+def absmax_cb_update(out: torch.Tensor, C: torch.Tensor, B: torch.Tensor, chunk_size: int) -> torch.Tensor:
+    """``out[g] = max(out[g], max |C . B^T|)`` over every (m, k) pair of every chunk, on the device, in place: the C.B^T
+    observer of scripts/nemotron_h_w4a8.py:126-169 without materializing the products.  C, B (B,L,G,N) views with unit last
+    stride, out (G,) fp32 zero-filled before the first batch."""
+    from linquant_amd import _lib
+
+    Bn, L, G, N = C.shape
+    assert B.shape == C.shape and C.stride(3) == 1 and B.stride(3) == 1
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.numel() == G
+    _lib.call("lq_absmax_cb", C.device, C=_lib.ptr(C), C_dtype=_dt_code(C), C_stride_b=C.stride(0), C_stride_l=C.stride(1),
+              C_stride_g=C.stride(2), B=_lib.ptr(B), B_dtype=_dt_code(B), B_stride_b=B.stride(0), B_stride_l=B.stride(1),
+              B_stride_g=B.stride(2), out=_lib.ptr(out), batch=Bn, seqlen=L, ngroups=G, dstate=N, chunk_size=chunk_size)
     return out
 
 

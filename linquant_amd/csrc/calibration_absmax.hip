@@ -4,6 +4,9 @@
 // (H, P)).  Pure HBM streaming: a workgroup owns a slab of rows and all H * D channels, a lane 8 adjacent channels (16
 // bytes of fp16 / bf16, 32 of fp32); maxima live in registers and leave through one atomic maximum per lane and slab.
 // |v| is never negative, so the fp32 bit pattern orders like an unsigned integer and atomicMax on the bits is exact.
+// The two observers that reduce a product rather than a tensor (the chunk states of scripts/nemotron_h_calibration.py:
+// 602-651 and C.B^T of scripts/nemotron_h_w4a8.py:126-169) form the product in fp32 on the vector ALU, tile by tile in
+// registers, and keep only its running maximum: calibration-time code, a few GFLOP per batch, nothing is stored.
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
@@ -68,7 +71,130 @@ __global__ __launch_bounds__(256) void absmax_kernel(lq_absmax_args a) {
 
 bool al(const void* q, int n) { return ((uintptr_t)q % n) == 0; }
 
+LQ_DEV float load1(const void* x, int dtype, int64_t off) {
+  if (dtype == LQ_DT_F32) return ((const float*)x)[off];
+  const uint32_t w = ((const uint16_t*)x)[off];
+  return dtype == LQ_DT_BF16 ? __uint_as_float(w << 16) : (float)__builtin_bit_cast(_Float16, (uint16_t)w);
+}
+
+LQ_DEV float nanmax(float m, float a) { return (a > m || a != a) ? a : m; }
+
+// Chunk-state observer: one workgroup per (64 value channels, chunk, head, batch).  Thread (p = tid & 63, quarter =
+// tid >> 6) keeps the N / 4 sums of its channel against one quarter of the state columns; a token's B row is the same
+// for every lane of a wavefront (one broadcast request), its gated x value differs per lane (128 contiguous bytes).
+// fp32 products and sums in token order: what an fp32 einsum of the same operands computes, in a fixed order.
+template <int NPT>
+__global__ __launch_bounds__(256) void chunk_state_absmax_kernel(lq_absmax_chunk_state_args a) {
+  const int tid = threadIdx.x, p = (int)blockIdx.x * 64 + (tid & 63), quarter = tid >> 6;
+  const int c = blockIdx.y;
+  const int h = (int)blockIdx.z % a.nheads, b = (int)blockIdx.z / a.nheads;
+  const int g = h / (a.nheads / a.ngroups);
+  const int k0 = c * a.chunk_size, k1 = min(a.seqlen, k0 + a.chunk_size);
+  float acc[NPT];
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) acc[i] = 0.0f;
+  const int64_t xb = (int64_t)b * a.x_stride_b + (int64_t)h * a.x_stride_h + p;
+  const int64_t bb = (int64_t)b * a.B_stride_b + (int64_t)g * a.B_stride_g + quarter * NPT;
+  const int64_t gb = (int64_t)b * a.gate_stride_b + (int64_t)h * a.gate_stride_h;
+  for (int k = k0; k < k1; ++k) {
+    const float xg = load1(a.x, a.x_dtype, xb + (int64_t)k * a.x_stride_l) * a.gate[gb + (int64_t)k * a.gate_stride_l];
+#pragma unroll
+    for (int i8 = 0; i8 < NPT; i8 += 8) {
+      float bv[8];
+      load8(a.B, a.B_dtype, bb + (int64_t)k * a.B_stride_l + i8, bv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[i8 + e] = acc[i8 + e] + xg * bv[e];
+    }
+  }
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) m = nanmax(m, __builtin_fabsf(acc[i]));
+  atomicMax((uint32_t*)a.out + (int64_t)h * a.headdim + p, __float_as_uint(m));
+}
+
+// C.B^T observer: one workgroup per (64 rows m, chunk, group, batch); thread (m = tid & 63, quarter = tid >> 6) meets
+// its C row with the tokens k of one quarter of the chunk, sixteen at a time; B rows are broadcast
+// requests, the C row piece is re-read per block of sixteen tokens (it stays in the first-level cache).
+__global__ __launch_bounds__(256) void cb_absmax_kernel(lq_absmax_cb_args a) {
+  const int tid = threadIdx.x, quarter = tid >> 6;
+  const int Q = a.chunk_size;
+  const int mtiles = (Q + 63) / 64;
+  const int c = (int)blockIdx.x / mtiles, m = ((int)blockIdx.x % mtiles) * 64 + (tid & 63);
+  const int g = blockIdx.y, b = blockIdx.z;
+  const int t0 = c * Q, limit = min(Q, a.seqlen - t0);
+  const int kq = (Q + 3) / 4;  // tokens per quarter
+  const int kbeg = quarter * kq, kend = min(limit, kbeg + kq);
+  const int mrow = min(m, limit - 1);  // rows past the end repeat the last one (a maximum does not mind)
+  const int64_t cbase = (int64_t)b * a.C_stride_b + (int64_t)(t0 + mrow) * a.C_stride_l + (int64_t)g * a.C_stride_g;
+  const int64_t bbase = (int64_t)b * a.B_stride_b + (int64_t)t0 * a.B_stride_l + (int64_t)g * a.B_stride_g;
+  float best = 0.0f;
+  for (int kb = kbeg; kb < kend; kb += 16) {
+    float acc[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = 0.0f;
+    for (int n = 0; n < a.dstate; n += 8) {
+      float cv[8];
+      load8(a.C, a.C_dtype, cbase + n, cv);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int k = min(kb + j, limit - 1);
+        float bv[8];
+        load8(a.B, a.B_dtype, bbase + (int64_t)k * a.B_stride_l + n, bv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j] = acc[j] + cv[e] * bv[e];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+      if (kb + j < kend) best = nanmax(best, __builtin_fabsf(acc[j]));
+  }
+  atomicMax((uint32_t*)a.out + g, __float_as_uint(best));
+}
+
+bool dtype_ok(int d) { return d == LQ_DT_F16 || d == LQ_DT_BF16 || d == LQ_DT_F32; }
+
+// rows read as 16-byte (two-byte types) or 2 x 16-byte (fp32) pieces of eight elements
+bool rows_ok(const void* p, int dtype, int64_t s0, int64_t s1, int64_t s2) {
+  const int esz = dtype == LQ_DT_F32 ? 4 : 2;
+  return al(p, 16) && (s0 * esz) % 16 == 0 && (s1 * esz) % 16 == 0 && (s2 * esz) % 16 == 0;
+}
+
 }  // namespace
+
+extern "C" int lq_absmax_chunk_state(const lq_absmax_chunk_state_args* a, hipStream_t stream) {
+  if (!a || !a->x || !a->B || !a->gate || !a->out) return LQ_ERR_NULL;
+  if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0 || a->ngroups <= 0 || a->nheads % a->ngroups != 0) return LQ_ERR_SHAPE;
+  if (a->headdim <= 0 || a->headdim % 64 != 0 || a->chunk_size <= 0) return LQ_ERR_SHAPE;
+  if (a->dstate != 64 && a->dstate != 128 && a->dstate != 256) return LQ_ERR_SHAPE;
+  if (!dtype_ok(a->x_dtype) || !dtype_ok(a->B_dtype)) return LQ_ERR_SHAPE;
+  if (!rows_ok(a->B, a->B_dtype, a->B_stride_b, a->B_stride_l, a->B_stride_g)) return LQ_ERR_SHAPE;
+  const int64_t nchunks = ((int64_t)a->seqlen + a->chunk_size - 1) / a->chunk_size;
+  if (nchunks > 65535 || (int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
+  dim3 grid((unsigned)(a->headdim / 64), (unsigned)nchunks, (unsigned)(a->batch * a->nheads));
+  if (a->dstate == 64)
+    hipLaunchKernelGGL(chunk_state_absmax_kernel<16>, grid, dim3(256), 0, stream, *a);
+  else if (a->dstate == 128)
+    hipLaunchKernelGGL(chunk_state_absmax_kernel<32>, grid, dim3(256), 0, stream, *a);
+  else
+    hipLaunchKernelGGL(chunk_state_absmax_kernel<64>, grid, dim3(256), 0, stream, *a);
+  return lq_check_launch();
+}
+
+extern "C" int lq_absmax_cb(const lq_absmax_cb_args* a, hipStream_t stream) {
+  if (!a || !a->C || !a->B || !a->out) return LQ_ERR_NULL;
+  if (a->batch <= 0 || a->seqlen <= 0 || a->ngroups <= 0 || a->chunk_size <= 0) return LQ_ERR_SHAPE;
+  if (a->dstate <= 0 || a->dstate % 8 != 0) return LQ_ERR_SHAPE;
+  if (!dtype_ok(a->C_dtype) || !dtype_ok(a->B_dtype)) return LQ_ERR_SHAPE;
+  if (!rows_ok(a->C, a->C_dtype, a->C_stride_b, a->C_stride_l, a->C_stride_g) ||
+      !rows_ok(a->B, a->B_dtype, a->B_stride_b, a->B_stride_l, a->B_stride_g))
+    return LQ_ERR_SHAPE;
+  const int64_t nchunks = ((int64_t)a->seqlen + a->chunk_size - 1) / a->chunk_size;
+  const int64_t mtiles = ((int64_t)a->chunk_size + 63) / 64;
+  if (nchunks * mtiles >= (1ll << 31) || a->ngroups > 65535 || a->batch > 65535) return LQ_ERR_SHAPE;
+  dim3 grid((unsigned)(nchunks * mtiles), (unsigned)a->ngroups, (unsigned)a->batch);
+  hipLaunchKernelGGL(cb_absmax_kernel, grid, dim3(256), 0, stream, *a);
+  return lq_check_launch();
+}
 
 extern "C" int lq_absmax(const lq_absmax_args* a, hipStream_t stream) {
   if (!a || !a->x || !a->out) return LQ_ERR_NULL;

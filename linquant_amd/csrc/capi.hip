@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 12; }
+extern "C" int lq_abi_version(void) { return 13; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)
@@ -23,6 +23,8 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_causal_conv1d_args);
   LQ_SIZE_OF(lq_rmsnorm_gated_args);
   LQ_SIZE_OF(lq_absmax_args);
+  LQ_SIZE_OF(lq_absmax_chunk_state_args);
+  LQ_SIZE_OF(lq_absmax_cb_args);
   LQ_SIZE_OF(lq_qhad_transform_args);
   LQ_SIZE_OF(lq_rmsnorm_gated_qhad_args);
   LQ_SIZE_OF(lq_zoo_cumsum_args);

@@ -36,7 +36,7 @@ def test_every_declaration_cites_the_reference():
     header = (ROOT / "include" / "linquant_hip.h").read_text()
     for m in re.finditer(r"/\*((?:(?!\*/).)*?)\*/\s*typedef struct", header, flags=re.S):
         text = m.group(1)
-        assert re.search(r"linquant/[\w/]+\.py:\d+", text) or "no counterpart in the reference" in text, text[:80]
+        assert re.search(r"(linquant|scripts|bench)/[\w/]+\.py:\d+", text) or "no counterpart in the reference" in text, text[:80]
 
 
 def test_null_and_shape_errors_without_launch():

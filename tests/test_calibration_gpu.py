@@ -75,3 +75,75 @@ def test_absmax_rejections(cuda):
     x = torch.zeros(1, 4, 2, 24, dtype=torch.float16, device="cuda")[..., 4:20]  # misaligned view
     with pytest.raises(_lib.LinQuantHipError):
         absmax_update(torch.zeros(32, device="cuda"), x, "pc_static")
+
+
+@pytest.mark.parametrize("b_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("N", [64, 128, 256])
+def test_chunk_state_observer(cuda, b_dtype, N):
+    """The chunk-state observer (scripts/nemotron_h_calibration.py:602-651: amax over (batch, chunk, N) of the unquantized
+    chunk states per (H, P)) against a float64 einsum of the same operands, over two calibration batches, with a ragged
+    last chunk, x as a strided view, B shared by the heads of a group.  fp32 sums of up to 128 terms: 1e-5 relative."""
+    from linquant_amd.calibration import absmax_chunk_state_update
+
+    gen = torch.Generator().manual_seed(0)
+    Bn, L, H, G, P, Q = 2, 450, 8, 2, 128, 128
+    out = torch.zeros(H * P, device=cuda)
+    ref = torch.zeros(H, P, dtype=torch.float64)
+    for batch in range(2):
+        big = (torch.randn(Bn, L, H * P + 64, generator=gen) * (1 + batch)).half()
+        x = big[..., 32:32 + H * P].view(Bn, L, H, P)
+        Bt = torch.randn(Bn, L, G, N, generator=gen).to(b_dtype)
+        gate = torch.rand(Bn, L, H, generator=gen) * 0.3
+        absmax_chunk_state_update(out, x.cuda(), Bt.cuda(), gate.cuda(), Q)
+        nc = (L + Q - 1) // Q
+        pad = nc * Q - L
+        xg = torch.nn.functional.pad((x.double() * gate.double()[..., None]), (0, 0, 0, 0, 0, pad)).view(Bn, nc, Q, H, P)
+        Bh = torch.nn.functional.pad(Bt.double(), (0, 0, 0, 0, 0, pad)).view(Bn, nc, Q, G, N).repeat_interleave(H // G, dim=3)
+        st = torch.einsum("bcqhp,bcqhn->bchpn", xg, Bh)
+        ref = torch.maximum(ref, st.abs().amax(dim=(0, 1, 4)))
+    torch.cuda.synchronize()
+    got = out.view(H, P).cpu().double()
+    assert ((got - ref).abs() / ref).max().item() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Q", [64, 256])
+def test_cb_observer(cuda, dtype, Q):
+    """The C.B^T observer (scripts/nemotron_h_w4a8.py:126-169: amax over (batch, chunk, Q, Q) per group, every (m, k)
+    pair of a chunk) against a float64 einsum; ragged last chunk, two batches."""
+    from linquant_amd.calibration import absmax_cb_update
+
+    gen = torch.Generator().manual_seed(1)
+    Bn, L, G, N = 2, 600, 3, 128
+    out = torch.zeros(G, device=cuda)
+    ref = torch.zeros(G, dtype=torch.float64)
+    for batch in range(2):
+        C = (torch.randn(Bn, L, G, N, generator=gen) * (1 + batch)).to(dtype)
+        Bt = torch.randn(Bn, L, G, N, generator=gen).to(dtype)
+        absmax_cb_update(out, C.cuda(), Bt.cuda(), Q)
+        nc = (L + Q - 1) // Q
+        for c in range(nc):
+            cc, bb = C[:, c * Q:(c + 1) * Q].double(), Bt[:, c * Q:(c + 1) * Q].double()
+            cb = torch.einsum("bmgn,bkgn->bgmk", cc, bb)
+            ref = torch.maximum(ref, cb.abs().amax(dim=(0, 2, 3)))
+    torch.cuda.synchronize()
+    got = out.cpu().double()
+    assert ((got - ref).abs() / ref).max().item() < 1e-5
+
+
+def test_calibrate_mamba2_on_the_device_matches_the_torch_expressions(cuda):
+    """calibrate_mamba2 runs its observers as device reductions on GPU tensors and as torch expressions on CPU tensors:
+    the two give the same scales up to what torch's own CPU and GPU evaluations of the gate differ by (the chunk-local
+    cumulative sum of dt * A is an fp32 sum of 256 terms in a different order on each: about 1e-5 of the exponent)."""
+    from linquant_amd.calibration import Mamba2Shape, calibrate_mamba2, mamba2_params, mamba2_synthetic
+
+    s = Mamba2Shape(batch=1, seqlen=1024, nheads=8, headdim=64, dstate=128, ngroups=2, chunk=256)
+    p_cpu = mamba2_params(s, 42, "cpu")
+    x, dt = mamba2_synthetic(s, 1, "cpu")
+    ref = calibrate_mamba2(s, x, dt, p_cpu)
+    p_gpu = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in p_cpu.items()}
+    got = calibrate_mamba2(s, x.cuda(), dt.cuda(), p_gpu)
+    for name, r in ref.items():
+        g = got[name].cpu()
+        assert g.shape == r.shape, name
+        assert ((g - r).abs() / r.abs().clamp_min(1e-12)).max().item() < 2e-4, name
