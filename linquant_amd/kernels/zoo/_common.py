@@ -39,6 +39,37 @@ def pad_keys(q, k, g, scales, rot=None):
     return q, k, g, scales, rot, K
 
 
+_VALUE_SCALES = ("vw", "vl", "state", "el", "ew")
+
+
+def pad_values(v, scales, unrot=None):
+    """Value widths that are not a multiple of 64 run as the next one (the reference masks the surplus channels of its
+    64- or 128-wide tiles, linquant/kernels/zoo/simple_gla.py:40-55): v gains zero channels, whose codes, pseudo-values,
+    state columns and outputs stay zero; the per-channel value / state scales there are one.  Canonical storage keeps
+    the reference's own restriction to V = 64 or 128.  Returns (v, scales, V) with V the caller's value width."""
+    V = v.shape[-1]
+    Vp = (V + 63) // 64 * 64
+    if V == Vp or unrot is not None:
+        return v, scales, V
+    pad = Vp - V
+    v = torch.nn.functional.pad(v, (0, pad))
+    scales = dict(scales)
+    for name in _VALUE_SCALES:
+        if name in scales:
+            s = f32(scales[name])
+            assert s.shape[-1] == V, f"scales['{name}']: (H, {V}) per value channel"
+            scales[name] = torch.nn.functional.pad(s, (0, pad), value=1.0)
+    return v, scales, V
+
+
+def cut_values(o, ht, V):
+    """Outputs and final state of the caller's value channels."""
+    if o.shape[-1] != V:
+        o = o[..., :V].contiguous()
+        ht = None if ht is None else ht[..., :V].contiguous()
+    return o, ht
+
+
 def cut_keys(ht, K):
     """Final state of the caller's key channels (the padded rows hold zeros)."""
     return ht if ht is None or ht.shape[2] == K else ht[:, :, :K].contiguous()

@@ -19,6 +19,7 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     Returns (o, final fp32 state or None)."""
     assert g.shape == q.shape
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
+    v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
@@ -39,4 +40,4 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     C.run_output(None, None, v, h_i8, None, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, g=gc, logenv=logenv)
-    return o, C.cut_keys(ht, K0)
+    return C.cut_values(o, C.cut_keys(ht, K0), V0)

@@ -18,6 +18,7 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
     assert g.shape == q.shape
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
+    v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
@@ -40,4 +41,4 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     C.run_output(None, None, e_out, h_i8, None, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
-    return o, C.cut_keys(ht, K0)
+    return C.cut_values(o, C.cut_keys(ht, K0), V0)

@@ -17,6 +17,7 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None. scales: 'q','k' (H,), 'kw' (H,K),
     'vw','vl','state' (H,V) fp32. Returns (o [B,T,H,V] in v.dtype or out_dtype, final fp32 state [B,H,K,V] or None)."""
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
+    v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     dims = C.check_shapes(q, k, v, chunk_size)
     B, T, H, K, V = dims
@@ -36,4 +37,4 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     codes = C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru)
     C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
     C.export_debug(_debug, h_i8, codes, g=gg)
-    return o, C.cut_keys(ht, K0)
+    return C.cut_values(o, C.cut_keys(ht, K0), V0)

@@ -302,6 +302,26 @@ def test_key_widths_between_the_built_ones(cuda, cell, K):
         zc.check(out, run, qz, f"{cell} K={K} local R_QK")
 
 
+@pytest.mark.parametrize("V", [16, 48, 96, 160])
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+def test_value_widths_between_the_built_ones(cuda, cell, V):
+    """Any V as the reference takes it (masked surplus channels of its value tiles, /root/reference
+    linquant/kernels/zoo/simple_gla.py:40-55): outputs by the reference's criterion, output and final state of the
+    caller's shape, stored state codes of the caller's channels within one step of the oracle's (two for DeltaNet)."""
+    tensors = zc.cut(zc.inputs(cell, K=64, V=V, H=2, seed=6), 256)
+    dbg = {}
+    out, ht, qz, run = _go(cell, tensors, debug=dbg, final_state=True)
+    assert out.shape[-1] == V and ht.shape == (2, 2, 64, V)
+    zc.check(out, run, qz, f"{cell} V={V}")
+    codes = zc.state_codes(qz, run)                      # (NT, B, H, K, V)
+    got = dbg["h_i8"].cpu()                              # (B, NT, H, K, Vp)
+    assert (got[..., V:] == 0).all(), "state columns of the padded value channels must stay zero"
+    NT = codes.shape[0]
+    diff = (got[:, 1:, ..., :V].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
+    assert diff.max().item() <= (2 if cell == "deltanet" else 1)
+    assert (diff != 0).float().mean().item() < 1e-3
+
+
 # Measured on MI355X (T = 256, B2, H4 / H2, 131072 .. 262144 codes per role): no code of any role differs from the
 # oracle's, in any of the six cells, at K = 64 and K = 128.  A tie between the fp32 and the float64 evaluation of an
 # exponentially weighted operand is possible in principle (about 1e-5 per code), so the bound is not zero.
