@@ -1,12 +1,14 @@
 """Benchmark of the INT8 chunkwise linear-recurrence prefill on one MI355X.
 
-Workload (the configuration the metric is quoted on): Mamba-2 2.7B-shape SSD layer, INT8 prefill, batch 4,
+Headline workload (the configuration the metric is quoted on): Mamba-2 2.7B-shape SSD layer, INT8 prefill, batch 4,
 seqlen 8192, 80 heads x headdim 64, d_state 128, 1 group, chunk 256, key-side absorption. One step = the whole
 hot path over one batch resident in HBM: split/rotate/quantize prologue of B and C, rotation of the fp16 B
 used by the key-side chunk state, then cumsum -> chunk state -> INT8 state passing -> C.B^T -> chunk scan.
 
 Prints ONE JSON line: the whole-step throughput, a per-stage breakdown measured with HIP events on the
-launch stream, the roofline of the dominant kernel, and the CPU oracle timed on a bounded sample.
+launch stream, the roofline of the dominant kernel, and the CPU oracle timed on a bounded sample.  The default run
+also measures every other benchmark configuration (the six zoo cells of the first four configurations and the
+headline shape under weak decay) under the same protocol and reports them in the line's "configs" object.
 """
 
 from __future__ import annotations
@@ -19,6 +21,7 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0
+RAMP_MS = 50.0           # untimed back-to-back launches in front of the warm-up steps
 INT8_PEAK_TOPS = 5000.0  # published dense INT8 MFMA rate of MI355X; the measured issue peak is reported next to it
 
 # source file of each stage's kernel: a counter figure from profiles/ is attached to a stage only while that file (and the
@@ -174,8 +177,24 @@ def hadamard_signed(n, seed, device):
     return (Hm / n ** 0.5 * signs).to(device)
 
 
-def bench_zoo(args):
-    """One step = one chunk-forward call (cumsum, WY prep, A, state, output kernels) over inputs resident in HBM."""
+def ramp(step, min_ms=RAMP_MS):
+    """Runs ``step`` back to back for at least ``min_ms`` of wall time, untimed: the GPU's clocks rise under sustained
+    load, and a timed region of a few milliseconds right after an idle period would measure that rise, not the kernels.
+    Returns the number of steps it ran."""
+    import torch
+
+    n, t0 = 0, time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        for _ in range(4):
+            step()
+        n += 4
+        torch.cuda.synchronize()
+    return n
+
+
+def measure_zoo(args, workload, cpu_baseline):
+    """One step = the operand prologue + one chunk-forward call (cumsum, WY prep, A, state, output kernels) over inputs
+    resident in HBM.  Returns the JSON line as a dict."""
     import torch
 
     from linquant_amd import _lib
@@ -184,7 +203,7 @@ def bench_zoo(args):
 
     _lib.load()
     dev = torch.device("cuda:0")
-    cell, B, T, H, K, V, desc = ZOO_WORKLOADS[args.workload]
+    cell, B, T, H, K, V, desc = ZOO_WORKLOADS[workload]
     fam, dec = ZOO_CELLS[cell]
     from linquant_amd.calibration import dqk_from_absmax, zoo_synthetic
 
@@ -196,10 +215,10 @@ def bench_zoo(args):
     g = g.to(dev) if g is not None else None
     # operand prologue, part of the timed step: persistent R_QK on q, k (no / scalar decay; the diagonal-decay cells rotate
     # locally inside the A kernel) and, for the KDA configuration, D_QK (alpha = 0.5) from a seed-1 calibration batch
-    persistent = dec != "diagonal" and args.workload != "c1"
+    persistent = dec != "diagonal" and workload != "c1"
     sq = zoo.rotation_signs(R) if persistent else None
     dqk = None
-    if args.workload == "c4_kda":
+    if workload == "c4_kda":
         cq, ck, *_ = zoo_synthetic(cell, 1, 2048, H, K, V, seed=1)
         dqk = dqk_from_absmax(cq.half().float(), ck.half().float(), 0.5).to(dev)
     has_prologue = persistent or dqk is not None
@@ -212,8 +231,8 @@ def bench_zoo(args):
         return q0, k0
 
     q, k = prologue()
-    scale = 1.0 if args.workload == "c1" else K ** -0.5
-    sigma = 0.5 if args.workload.startswith("c3") else 1.0
+    scale = 1.0 if workload == "c1" else K ** -0.5
+    sigma = 0.5 if workload.startswith("c3") else 1.0
     eta = 0.0 if dec == "diagonal" else 1.0
 
     def kernels(sc, **kw):
@@ -247,6 +266,7 @@ def bench_zoo(args):
 
     if args.copy_probe:
         copy_probe(dev)
+    ramp_steps = 0 if args.no_ramp else ramp(lambda: call(sc))
     for _ in range(args.warmup):
         call(sc)
     torch.cuda.synchronize()
@@ -299,7 +319,7 @@ def bench_zoo(args):
     roofline = {"kernel": "zoo_" + dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "avg_ms": round(avg_dom, 4),
                 "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
-    counters, mfma_peak = measured_counters(args.workload, "zoo")
+    counters, mfma_peak = measured_counters(workload, "zoo")
     for label, rec in counters.items():
         if label in stages:
             stages[label].update({k: v for k, v in rec.items() if k in ("traffic_MB", "mfma_busy_frac")})
@@ -307,7 +327,7 @@ def bench_zoo(args):
         roofline["traffic"] = int(counters[dom]["traffic_MB"] * 1e6)
 
     cpu = None
-    if not args.no_cpu_baseline:
+    if cpu_baseline:
         from oracle import zoo_reference as Z
 
         threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
@@ -333,14 +353,23 @@ def bench_zoo(args):
         "metric": f"prefill tokens/s per layer at T={T}", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"{args.workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
-                   "tokens_per_step": tokens,
+        "config": {"workload": f"{workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
+                   "tokens_per_step": tokens, "ramp": ramp_note(ramp_steps),
                    "prologue": ("in the timed step: " + ("R_QK on q, k" if persistent else "") +
                                 (" D_QK (alpha 0.5) on q, k" if dqk is not None else "")) if has_prologue else
                                "none (local R_QK inside the A kernel)" if rot is not None else "none"},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
     }
-    print(json.dumps(line), flush=True)
+    return line
+
+
+def bench_zoo(args):
+    print(json.dumps(measure_zoo(args, args.workload, not args.no_cpu_baseline)), flush=True)
+
+
+def ramp_note(n):
+    return (f"{n} untimed steps (at least {RAMP_MS:.0f} ms of back-to-back launches) ran before the --warmup steps, so that the "
+            "timed steps do not measure the clocks rising from idle") if n else "none"
 
 
 def bench_front(args):
@@ -565,38 +594,8 @@ def _stage_bench(args, stages, step_names, tokens, dtype, cpu_sample, workload):
         "roofline": roofline, "cpu_baseline": cpu, "stages": out}), flush=True)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--workload", default="c5", choices=["c5", "c5_front", "c5_epilogue", "c5_layer", "mfma_peak"] + list(ZOO_WORKLOADS),
-                    help="c5 (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on; others: zoo kernels")
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--value-side", action="store_true", help="value-side absorption instead of key-side")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run one plain device copy of 256 MiB (reference point for HBM byte counters)")
-    ap.add_argument("--regime", default="strong", choices=["strong", "weak"],
-                    help="c5: decay regime of the synthetic dt / A (strong = the stated recipe)")
-    ap.add_argument("--graph", action="store_true", help="c5: also time the step replayed from one captured HIP graph")
-    ap.add_argument("--cpu-heads", type=int, default=8, help="heads per slice of the CPU-oracle sample")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="stop the CPU-oracle sample after about this long")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards over batch x head "
-              "with no communication); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-
-    if args.workload != "c5":
-        from linquant_amd import _lib as _l
-
-        if not _l.LIB_PATH.exists():
-            from linquant_amd.build import build
-
-            build()
-        return {"c5_front": bench_front, "c5_epilogue": bench_epilogue, "c5_layer": bench_layer,
-                "mfma_peak": bench_mfma_peak}.get(args.workload, bench_zoo)(args)
-
+def measure_c5(args, regime, keyside, cpu_baseline, with_graph=False):
+    """The Mamba-2 2.7B-shape SSD step (prologue + one-call forward) under one decay regime; returns the JSON line."""
     import torch
 
     from linquant_amd import _lib
@@ -605,18 +604,13 @@ def main():
     from linquant_amd.kernels.mamba2 import ssd_combined as M
     from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC
 
-    if not _lib.LIB_PATH.exists():
-        from linquant_amd.build import build
-
-        build()
     _lib.load()
     dev = torch.device("cuda:0")
-    keyside = not args.value_side
     s = Mamba2Shape(batch=4, seqlen=8192, nheads=80, headdim=64, dstate=128, ngroups=1, chunk=256)
     # decay regime of the synthetic inputs: "strong" is the recipe the metric is quoted on (dt = softplus(N(-2, 0.5)) ~ 0.13,
     # A = -exp(U(log 1, log 16))); "weak" (dt ~ 0.011, A in [-1.3, -1]) is what slowly forgetting trained layers look like:
     # there the chunk state kernel finds no all-zero slab to leave out and the chunk scan no underflowing slab factor
-    dt_mean, a_max = (-2.0, 16.0) if args.regime == "strong" else (-4.5, 1.3)
+    dt_mean, a_max = (-2.0, 16.0) if regime == "strong" else (-4.5, 1.3)
     p = mamba2_params(s, 42, dev, a_max=a_max)
     cal = Mamba2Shape(batch=1, seqlen=2048, nheads=s.nheads, headdim=s.headdim, dstate=s.dstate, ngroups=s.ngroups, chunk=s.chunk)
     cx, cdt = mamba2_synthetic(cal, 1, dev, dt_mean=dt_mean)
@@ -645,6 +639,7 @@ def main():
 
     if args.copy_probe:
         copy_probe(dev)
+    ramp_steps = 0 if args.no_ramp else ramp(step)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -719,12 +714,20 @@ def main():
     # summary, attached only while the kernel's source is unchanged since they were collected)
     int8_ops = stage_int8_ops(s)
     counters, mfma_peak = measured_counters("c5_keyside" if keyside else "c5_valueside", "c5")
-    if args.regime != "strong":  # the committed counters were collected on the stated recipe's data
+    if regime != "strong":  # the committed counters were collected on the stated recipe's data
         counters = {}
     for label, st in stages.items():
         if label in int8_ops:
-            st["int8_TOPS"] = round(int8_ops[label] / 1e12 / (st["ms"] * 1e-3), 1)
-            st["int8_peak_frac"] = round(st["int8_TOPS"] / INT8_PEAK_TOPS, 4)
+            # dense-equivalent: the operations of the full contraction over the stage's time, whether or not a data-dependent
+            # shortcut (all-zero slabs left out) skipped part of them; "issued" counts the INT8 MFMA instructions the
+            # counters saw (32 768 operations per 16x16x64 instruction and wave), over the live time
+            st["int8_TOPS_dense_equivalent"] = round(int8_ops[label] / 1e12 / (st["ms"] * 1e-3), 1)
+            issued = counters.get(label, {}).get("mfma_i8_insts")
+            if issued is not None:
+                st["int8_TOPS_issued"] = round(issued * 32768 / 1e12 / (st["ms"] * 1e-3), 1)
+                st["int8_peak_frac"] = round(st["int8_TOPS_issued"] / INT8_PEAK_TOPS, 4)
+            else:
+                st["int8_peak_frac_dense_equivalent"] = round(st["int8_TOPS_dense_equivalent"] / INT8_PEAK_TOPS, 4)
         st.update({k: v for k, v in counters.get(label, {}).items() if k in ("traffic_MB", "mfma_busy_frac")})
         if "traffic_MB" in st and st["traffic_MB"] < 0.9 * st["MB"]:
             # a data-dependent shortcut (all-zero slabs of the key-side chunk state left out) moved fewer bytes than the
@@ -735,7 +738,7 @@ def main():
     if "traffic_MB" in counters.get(dom, {}):
         roofline["traffic"] = int(counters[dom]["traffic_MB"] * 1e6)
     graph = None
-    if args.graph:  # the same step captured once in a HIP graph and replayed: no host work between the launches
+    if with_graph:  # the same step captured once in a HIP graph and replayed: no host work between the launches
         g = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -757,7 +760,7 @@ def main():
 
     # ---- CPU baseline: the CPU oracle on a bounded sample (batch 1 x a few heads x full length), same seeds
     cpu = None
-    if not args.no_cpu_baseline:
+    if cpu_baseline:
         import numpy as np
 
         from oracle import mamba2_ssd as O
@@ -805,14 +808,91 @@ def main():
         "config": {"workload": "mamba2-2.7b-shape SSD layer INT8 prefill (BASELINE.json configs[4]): B=4 L=8192 H=80 P=64 "
                                "N=128 G=1 chunk=256, " + ("key-side" if keyside else "value-side") + " absorption, "
                                "prologue + 5 SSD stages", "tokens_per_step": tokens,
-                   "decay_regime": args.regime + (" (the stated recipe: dt ~ 0.13, A in [-16, -1])" if args.regime == "strong"
+                   "ramp": ramp_note(ramp_steps),
+                   "decay_regime": regime + (" (the stated recipe: dt ~ 0.13, A in [-16, -1])" if regime == "strong"
                                                   else " (dt ~ 0.011, A in [-1.3, -1]: no zero slab to leave out)")},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
-        "mfma": {"int8_peak_TOPS_published": INT8_PEAK_TOPS, "measured_issue_peak": mfma_peak or None,
-                 "note": "every stage is HBM-bound (26-100 op/B against a ridge of about 630): int8_peak_frac is achieved "
-                         "INT8 ops over stage time, mfma_busy_frac the matrix pipeline's busy share of the kernel from counters"},
+        "mfma": {"int8_peak_TOPS_published": INT8_PEAK_TOPS, "issue_peak_from_committed_profile": mfma_peak or None,
+                 "note": "every stage is HBM-bound (26-100 op/B against a ridge of about 630). traffic_MB, mfma_busy_frac, "
+                         "int8_TOPS_issued and the issue peak are not measured in this run: they come from the committed "
+                         "counter summary (profiles/hbm_traffic_and_mfma_counters.md) and are attached only while the "
+                         "kernel's source hashes to what the counters were taken on; times are live"},
         "hip_graph": graph,
     }
+    return line
+
+
+
+def compact(line, keep_cpu):
+    """What a configuration contributes to the 'configs' object of the default run."""
+    rec = {"workload": line["config"]["workload"], "ms": line["ms_per_step"], "tokens_per_s": line["value"],
+           "stages": {n: {k: v for k, v in st.items() if k in ("ms", "MB", "hbm_frac", "traffic_MB", "note")}
+                      for n, st in line["stages"].items()},
+           "roofline": line["roofline"]}
+    if keep_cpu:
+        rec["cpu_baseline"] = line["cpu_baseline"]
+    return rec
+
+
+def other_configs(args, keyside):
+    """Every benchmark configuration other than the headline, measured in the same run under the same protocol (ramp,
+    --warmup untimed steps, --steps timed steps): the six zoo cells of configs[0..3] and the headline's shape under weak
+    decay, where its data-dependent shortcuts find nothing to leave out.  The first configuration, which the CPU oracle
+    finishes in seconds, carries its CPU baseline."""
+    import gc
+
+    import torch
+
+    out = {}
+    for w in ZOO_WORKLOADS:
+        out[w] = compact(measure_zoo(args, w, cpu_baseline=(w == "c1" and not args.no_cpu_baseline)), keep_cpu=(w == "c1"))
+        gc.collect()
+        torch.cuda.empty_cache()
+    other = "weak" if args.regime == "strong" else "strong"
+    out["c5_" + other] = compact(measure_c5(args, other, keyside, cpu_baseline=False), keep_cpu=False)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "c5", "c5_front", "c5_epilogue", "c5_layer", "mfma_peak"] + list(ZOO_WORKLOADS),
+                    help="all (default): the Mamba-2 2.7B-shape SSD layer the metric is quoted on as the headline, and every "
+                         "other benchmark configuration beside it under 'configs'; c5: the headline alone; others: one "
+                         "zoo configuration, the stages around the SSD, the whole mixer, the MFMA issue peak")
+    ap.add_argument("--no-ramp", action="store_true",
+                    help="skip the untimed back-to-back launches that bring the clocks up before the warm-up steps")
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--value-side", action="store_true", help="value-side absorption instead of key-side")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain device copy of 256 MiB (reference point for HBM byte counters)")
+    ap.add_argument("--regime", default="strong", choices=["strong", "weak"],
+                    help="c5: decay regime of the synthetic dt / A (strong = the stated recipe)")
+    ap.add_argument("--graph", action="store_true", help="c5: also time the step replayed from one captured HIP graph")
+    ap.add_argument("--cpu-heads", type=int, default=8, help="heads per slice of the CPU-oracle sample")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="stop the CPU-oracle sample after about this long")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the hot path shards over batch x head "
+              "with no communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from linquant_amd import _lib as _l
+
+    if not _l.LIB_PATH.exists():
+        from linquant_amd.build import build
+
+        build()
+    if args.workload not in ("c5", "all"):
+        return {"c5_front": bench_front, "c5_epilogue": bench_epilogue, "c5_layer": bench_layer,
+                "mfma_peak": bench_mfma_peak}.get(args.workload, bench_zoo)(args)
+    keyside = not args.value_side
+    line = measure_c5(args, args.regime, keyside, not args.no_cpu_baseline, args.graph)
+    if args.workload == "all":
+        line["configs"] = other_configs(args, keyside)
     print(json.dumps(line), flush=True)
 
 

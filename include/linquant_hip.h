@@ -5,6 +5,7 @@
  *   LQ_E_NULL  (-14) a required pointer is missing
  *   LQ_E_SHAPE (-22) unsupported size / stride / alignment / flag
  *   LQ_E_LAUNCH (-5) hipGetLastError() reported a launch failure
+ *   LQ_E_STATE (-11) the call needs set-up that cannot run now (stream under graph capture)
  * Entry points never allocate, never synchronise, never throw and keep no mutable global state:
  * the caller owns every buffer (inputs, outputs, intermediates) and may call concurrently on
  * different streams.  All strides are in elements of the tensor's dtype.  "device float*" scalars
@@ -31,6 +32,7 @@ typedef struct ihipStream_t* hipStream_t;
 #define LQ_E_NULL (-14)
 #define LQ_E_SHAPE (-22)
 #define LQ_E_LAUNCH (-5)
+#define LQ_E_STATE (-11)
 
 /* element types accepted for the raw dt input */
 #define LQ_DT_F16 0
@@ -245,9 +247,15 @@ int lq_ssd_combined_workspace_bytes(const lq_ssd_combined_args* args, int64_t* b
  * call takes inputs and outputs only (`workspace` is ignored) and allocates nothing.  Returns LQ_E_SHAPE when the dims
  * need more than that.  Every call on one GPU shares the array: calls that overlap on one GPU race (serialize them on
  * one stream or with events); nothing in it needs clearing between calls, every byte a stage reads was written by an
- * earlier stage of the same call. */
+ * earlier stage of the same call.  A graph that captured this call replays into the same array: replays race with any
+ * other call of this entry on that GPU unless the caller orders them.
+ * The array's device address is looked up once per GPU, by lq_ssd_static_init() or by the first call on that GPU; the
+ * look-up never runs on a stream that is being captured: such a call returns LQ_E_STATE when no earlier eager call or
+ * lq_ssd_static_init() (with that device current) has done it. */
 #define LQ_SSD_STATIC_WORKSPACE_BYTES (64ll << 20)
 int lq_ssd_combined_static(const lq_ssd_combined_args* args, hipStream_t stream);
+/* No counterpart in the reference.  Set-up of lq_ssd_combined_static for the current device (idempotent, launches nothing). */
+int lq_ssd_static_init(void);
 
 /* ------------------------------------------------------------------------------------------
  * Rotation + quantize prologue.

@@ -13,14 +13,15 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 HEADER = ROOT.parent / "include" / "linquant_hip.h"
 LIB_PATH = ROOT / "csrc" / "liblinquant_hip.so"
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 LQ_DT_F16, LQ_DT_F32, LQ_DT_I8, LQ_DT_BF16 = 0, 1, 2, 3
 
 _CTYPES = {"int64_t": ctypes.c_int64, "int32_t": ctypes.c_int32, "float": ctypes.c_float, "int": ctypes.c_int}
 _ERRORS = {-14: "a required pointer is missing (LQ_E_NULL)",
            -22: "unsupported size / stride / alignment / flag (LQ_E_SHAPE)",
-           -5: "kernel launch failed (LQ_E_LAUNCH)"}
+           -5: "kernel launch failed (LQ_E_LAUNCH)",
+           -11: "set-up needed that cannot run now: stream under graph capture (LQ_E_STATE)"}
 
 
 class LinQuantHipError(RuntimeError):

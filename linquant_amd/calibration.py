@@ -96,7 +96,10 @@ def calibrate_mamba2(shape: Mamba2Shape, xBC, dt_raw, params, head_block: int = 
     A = -torch.exp(params["A_log_scale"] * params["A_log"].float())  # (H,)
     dA = (dt * A).view(B, nc, Q, H).cumsum(dim=2)
     gate = (torch.exp(dA[:, :, -1:, :] - dA) * dt.view(B, nc, Q, H))  # (B,nc,Q,H)
-    on_gpu = xBC.is_cuda
+    # the device reductions cover the shapes the SSD kernels themselves take; any other shape (small debug sizes, N = 16
+    # or 32, rows that are not 16-byte multiples) goes through the torch expressions below, which run on any device
+    on_gpu = (xBC.is_cuda and N in (64, 128, 256) and P % 64 == 0 and (xBC.stride(1) * xBC.element_size()) % 16 == 0
+              and (xBC.stride(0) * xBC.element_size()) % 16 == 0 and xBC.data_ptr() % 16 == 0 and B * H <= 65535)
     if on_gpu:  # the C.B^T observer as a device reduction: the products are never stored
         cb_amax = torch.zeros(G, device=dev)
         absmax_cb_update(cb_amax, Crot.contiguous(), Brot.contiguous(), Q)

@@ -15,6 +15,7 @@
 #define LQ_ERR_SHAPE (-22)      // bad / unsupported shape, stride or flag
 #define LQ_ERR_LAUNCH (-5)      // hipGetLastError() reported a launch failure
 #define LQ_ERR_NULL (-14)       // required pointer missing
+#define LQ_ERR_STATE (-11)      // set-up needed that cannot run now (stream under graph capture)
 
 typedef int lq_v4i __attribute__((ext_vector_type(4)));
 typedef int lq_v2i __attribute__((ext_vector_type(2)));

@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
     uint64_t live = nslab >= 64 ? ~0ull : ((1ull << nslab) - 1);
     if (elide) {
       float bmax = 0.0f;
-      for (int n = lane; n < NT; n += 64) bmax = fmaxf(bmax, binv_s[n]);
+      for (int n = lane; n < NT; n += 64) bmax = fmaxf(bmax, fabsf(binv_s[n]));
 #pragma unroll
       for (int o = 32; o >= 1; o >>= 1) bmax = fmaxf(bmax, __shfl_xor(bmax, o));
       live = 1ull << (nslab - 1);
@@ -337,8 +337,9 @@ __global__ __launch_bounds__(256, 2) void chunk_state_kernel(Params p) {
         const int sidx = nslab - 2 - i, k = 64 * sidx + lane;
         float rm = rmv[i & 3];
         if (i >= 4) rm = p.rowmax[((int64_t)b * p.seqlen + (int64_t)c * Q + min(k, limit - 1)) * p.G + g];
-        // not provably zero (NaN / Inf in B keep the slab)
-        const bool keep = !((gate_s[k] * rm) * bmax < 0.499f);
+        // not provably zero (NaN / Inf in B keep the slab); magnitudes, so that a negative gate (dt_min < 0 without
+        // softplus) or a negative gate scale cannot make the bound negative
+        const bool keep = !((fabsf(gate_s[k]) * rm) * bmax < 0.499f);
         if (__ballot(keep)) live |= 1ull << sidx;
       }
     }

@@ -136,9 +136,24 @@ int run(const lq_ssd_combined_args* a, char* ws, const Layout& l, hipStream_t st
   return lq_chunk_scan(&sc, stream);
 }
 
+// Everything the five stages would reject, checked before the first launch (the intersection of their limits), so that a
+// bad call returns without having queued a kernel or written into the workspace.
 int check(const lq_ssd_combined_args* a) {
   if (!a || !a->x || !a->dt || !a->qC || !a->out) return LQ_ERR_NULL;
-  if (a->keyside ? !a->b_fp : !a->qB) return LQ_ERR_NULL;
+  if (!a->dt_scale || !a->A_log || !a->A_log_scale) return LQ_ERR_NULL;
+  if (!a->state_scale || !a->cb_scale || !a->C_scale || !a->B_scale) return LQ_ERR_NULL;
+  if (a->D && !a->D_scale) return LQ_ERR_NULL;
+  if (a->keyside ? (!a->b_fp || !a->x_scale_hp || !a->b_gate_scale) : (!a->qB || !a->alpha_hp || !a->bscale_g))
+    return LQ_ERR_NULL;
+  if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0 || a->headdim <= 0 || a->ngroups <= 0 || a->dstate <= 0 ||
+      a->chunk_size <= 0)
+    return LQ_ERR_SHAPE;
+  const int Q = a->chunk_size;
+  if (Q != 64 && Q != 128 && Q != 256 && Q != 512) return LQ_ERR_SHAPE;  // the chunk scan's sizes
+  if (a->dstate % 64 != 0 || a->dstate > 256 || a->headdim % 64 != 0) return LQ_ERR_SHAPE;
+  if (a->nheads % a->ngroups != 0) return LQ_ERR_SHAPE;
+  if ((int64_t)a->headdim * a->dstate > 0x7fffffffLL) return LQ_ERR_SHAPE;
+  if (a->gate_shift < 0 || a->gate_shift > 15) return LQ_ERR_SHAPE;
   return LQ_OK;
 }
 
@@ -155,11 +170,19 @@ constexpr int kMaxDevices = 64;
 std::mutex scratch_mutex;
 char* scratch_ptr[kMaxDevices];  // by device ordinal; nullptr until resolved
 
-int static_workspace(char** out) {
+// Address of the current device's copy of `scratch`.  The look-up (which may load the code object) runs once per
+// device and never while `stream` is being captured into a graph: a call under capture on a device whose address is not
+// known yet is refused, so set-up work cannot land inside a capture (lq_ssd_static_init or one eager call comes first).
+int static_workspace(char** out, hipStream_t stream, bool may_be_capturing) {
   int dev = -1;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return LQ_ERR_LAUNCH;
   std::lock_guard<std::mutex> lock(scratch_mutex);
   if (!scratch_ptr[dev]) {
+    if (may_be_capturing) {
+      hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(stream, &st) != hipSuccess) return LQ_ERR_LAUNCH;
+      if (st != hipStreamCaptureStatusNone) return LQ_ERR_STATE;
+    }
     void* p = nullptr;
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return LQ_ERR_LAUNCH;
     scratch_ptr[dev] = (char*)p;
@@ -196,6 +219,11 @@ extern "C" int lq_ssd_combined_static(const lq_ssd_combined_args* a, hipStream_t
   if ((rc = plan(a, &l)) != LQ_OK) return rc;
   if (l.total > LQ_SSD_STATIC_WORKSPACE_BYTES) return LQ_ERR_SHAPE;  // larger than the built-in scratch: use lq_ssd_combined
   char* ws = nullptr;
-  if ((rc = static_workspace(&ws)) != LQ_OK) return rc;
+  if ((rc = static_workspace(&ws, stream, true)) != LQ_OK) return rc;
   return run(a, ws, l, stream);
+}
+
+extern "C" int lq_ssd_static_init(void) {
+  char* ws = nullptr;
+  return static_workspace(&ws, nullptr, false);
 }

@@ -53,6 +53,38 @@ def test_null_and_shape_errors_without_launch():
     assert lib.lq_chunk_cumsum(ctypes.byref(st2), None) == -22
 
 
+def test_one_call_forward_validates_every_stage_limit_before_the_first_launch():
+    """lq_ssd_combined / lq_ssd_combined_static check the intersection of their five stages' limits up front: a call
+    that one of the later stages would refuse returns its code without having queued a kernel (no device is touched
+    here: the buffers are host memory, and a launch on them would fail differently)."""
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    ptrs = ("x", "dt", "qC", "out", "b_fp", "qB", "dt_scale", "A_log", "A_log_scale", "state_scale", "cb_scale", "C_scale",
+            "B_scale", "alpha_hp", "bscale_g", "x_scale_hp", "b_gate_scale", "workspace")
+
+    def args(**kw):
+        st = _lib.fill("lq_ssd_combined_args", batch=1, seqlen=512, nheads=4, headdim=64, ngroups=1, dstate=128,
+                       chunk_size=256, gate_shift=7, workspace_bytes=1 << 40)
+        for f in ptrs:
+            setattr(st, f, ctypes.addressof(buf))
+        for k, v in kw.items():
+            setattr(st, k, v)
+        return st
+
+    for entry in (lib.lq_ssd_combined, lib.lq_ssd_combined_static):
+        assert entry(ctypes.byref(args(chunk_size=1024)), None) == -22     # only the chunk scan refuses it
+        assert entry(ctypes.byref(args(chunk_size=192)), None) == -22
+        assert entry(ctypes.byref(args(dstate=320)), None) == -22
+        assert entry(ctypes.byref(args(headdim=48)), None) == -22
+        assert entry(ctypes.byref(args(nheads=3, ngroups=2)), None) == -22
+        assert entry(ctypes.byref(args(gate_shift=16)), None) == -22
+        for missing in ("state_scale", "cb_scale", "C_scale", "B_scale", "dt_scale", "A_log"):
+            assert entry(ctypes.byref(args(**{missing: None})), None) == -14, missing
+        assert entry(ctypes.byref(args(keyside=1, x_scale_hp=None)), None) == -14
+        assert entry(ctypes.byref(args(keyside=0, alpha_hp=None)), None) == -14
+        assert entry(ctypes.byref(args(D=ctypes.addressof(buf), D_scale=None)), None) == -14
+
+
 def test_every_entry_point_rejects_an_empty_argument_struct():
     """A zeroed argument struct (every pointer NULL, every size 0) and a NULL struct pointer come back as an error code
     from every entry point: nothing is launched and no device is touched."""

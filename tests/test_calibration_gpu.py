@@ -147,3 +147,20 @@ def test_calibrate_mamba2_on_the_device_matches_the_torch_expressions(cuda):
         g = got[name].cpu()
         assert g.shape == r.shape, name
         assert ((g - r).abs() / r.abs().clamp_min(1e-12)).max().item() < 2e-4, name
+
+
+def test_calibrate_mamba2_on_the_device_at_a_shape_the_reductions_do_not_take(cuda):
+    """A state width the device observers are not built for (N = 32) and a head width of 32: calibrate_mamba2 on GPU
+    tensors evaluates its torch expressions there instead of raising, and agrees with the CPU evaluation."""
+    from linquant_amd.calibration import Mamba2Shape, calibrate_mamba2, mamba2_params, mamba2_synthetic
+
+    s = Mamba2Shape(batch=1, seqlen=256, nheads=4, headdim=32, dstate=32, ngroups=1, chunk=64)
+    p_cpu = mamba2_params(s, 42, "cpu")
+    x, dt = mamba2_synthetic(s, 1, "cpu")
+    ref = calibrate_mamba2(s, x, dt, p_cpu)
+    p_gpu = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in p_cpu.items()}
+    got = calibrate_mamba2(s, x.cuda(), dt.cuda(), p_gpu)
+    for name, r in ref.items():
+        g = got[name].cpu()
+        assert g.shape == r.shape, name
+        assert ((g - r).abs() / r.abs().clamp_min(1e-12)).max().item() < 2e-4, name

@@ -706,6 +706,21 @@ def test_full_size_config5_slices(cuda):
             outs[keyside] = (out, seen["states"], seen["passed"])
     finally:
         M._fixedpoint_state_passing_fwd = orig_sp
+    # the route the benchmark times, exactly as bench.py's step() calls it: nothing re-bound (one C call, state passing in
+    # place with its zero-gate early exit), rotated fp16 B and its per-token maxima from the prologue's own launch.  It
+    # must equal, bit for bit, the stage-by-stage key-side output that is checked against the oracle below.
+    say("full size, one-call route as benchmarked")
+    x1, qB1, qC1, b_fp1, b_rmax = fused_split_rotate_quant_xBC(xBC, p["r_signs"], 80, 1, 128, 64, sc["B_inv_scale"],
+                                                               sc["C_inv_scale"], return_b_fp=True, return_b_rowmax=True)
+    assert torch.equal(qB1, qB) and torch.equal(qC1, qC) and torch.equal(b_fp1, b_fp)
+    out1, _ = M._quant_mamba_chunk_scan_combined_fwd(
+        x1, dt_raw, p["dt_scale"], p["A_log"], p["A_log_scale"], qB1, sc["B_scale"], qC1, sc["C_scale"], s.chunk,
+        p["D"], p["D_scale"], dt_bias=p["dt_bias"], dt_softplus=True, static_state_scale=sc["static_state_scale"],
+        static_cb_scale=sc["static_cb_scale"], alpha_hp=sc["alpha_hp"], bscale_g=sc["bscale_g"], keyside=True,
+        x_scale_hp=sc["x_scale_hp"], b_fp=b_fp1, b_gate_scale=sc["b_gate_scale"], b_rowmax=b_rmax)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, outs[True][0]), "one-call route differs from the stage-by-stage route at full size"
+    del x1, qB1, qC1, b_fp1, b_rmax, out1
     # oracle on slices: batch b, heads hs
     for keyside, b, hs in ((False, 0, [0, 79]), (True, 3, [17, 42])):
         say("full size slice check", keyside, b, hs)
