@@ -432,13 +432,26 @@ typedef struct {
   const float* beta;         /* (B,T,H) fp32 */
   const float* g;            /* cumulative log decay (B,T,H) / (B,T,H,K) or NULL */
   void* Hw;                  /* (B,T,H,K) fp16/bf16 */
-  void* W;                   /* (B,T,H,K) fp16/bf16 */
+  void* W;                   /* (B,T,H,K) fp16/bf16; may be NULL when the codes below are requested */
   void* U;                   /* (B,T,H,V) fp16/bf16 */
   float* fw;                 /* (B,T,H) fp32 */
   float sigma, tau;
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
   int32_t decay;
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
+  /* Optional (all of them when kqT is set): the write-operand codes lq_zoo_write_codes would make from the stored Hw
+   * and W, made here from the same rounded values (same bits), so that the state kernel needs no pre-pass of its own
+   * and W need not be stored: operand preparation inside _delta_state_body (gated_delta_rule.py:85-105) and
+   * _kda_state_body (kda.py:100-124). */
+  int8_t* kqT;               /* (B,NT,H,K,C) int8 key write codes, channel-major inside the chunk */
+  int8_t* wq;                /* (B,T,H,K) int8 state-read codes of W */
+  float* ev;                 /* (B,T,H) per-token value factor */
+  float* gam;                /* (B,NT,H,K) per-channel chunk decay */
+  const float* logenv;       /* (B,T,H) log envelope (per-channel decay) */
+  const float* skw;          /* (H,K) key write scales */
+  const float* sw;           /* (H,) state-read scale of W */
+  float eta;
+  int32_t qmax;
 } lq_zoo_wy_prep_args;
 int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
 

@@ -34,6 +34,18 @@ struct WyParams {
   float sigma, tau;
   int bf;
   int B, T, H, V;
+  // write-operand codes of the state kernel, made here when kqT is set (otherwise lq_zoo_write_codes makes them from the
+  // stored Hw and W)
+  int8_t* kqT;
+  int8_t* wq;
+  float* ev;
+  float* gam;
+  const float* logenv;
+  const float* skw;
+  const float* sw;
+  float eta;
+  int qmax;
+  int NT;
 };
 
 LQ_DEV float powb(float b, float e) {
@@ -238,7 +250,10 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
     }
 }
 
-template <int DECAY, int K, bool BF>
+// CODES: the kernel also emits what lq_zoo_write_codes would make from the stored Hw and W (same arithmetic on the same
+// rounded values, so the same bits): channel-major key write codes, token-major state-read codes of W, the per-token
+// value factor and the per-channel chunk decay.  W itself is then stored only when p.W is set.
+template <int DECAY, int K, bool BF, bool CODES>
 __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   constexpr int LS = 64 + 16;  // floats per row of the buffer that holds the Gram tile and then the X tiles
   static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
@@ -253,6 +268,7 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   float* Lg_s = lds_f;
   float* Hg_s = lds_f + 64 * kOP;
   __shared__ float gs_s[64], bs_s[64], bh_s[64];
+  __shared__ float iskw_s[CODES ? K : 1], glast_s[CODES ? K : 1], bw_s[CODES ? 64 : 1], el_s[CODES ? 64 : 1];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -270,6 +286,36 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
     bh_s[tid] = powb(bt, 1.0f - sigma);
     p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
     if (DECAY == LQ_DECAY_SCALAR) gs_s[tid] = p.g[(t0 + tid) * H + h];
+  }
+  if constexpr (CODES) {
+    // per-token value factor and per-channel chunk decay, as lq_zoo_write_codes writes them
+    if (tid < 64) {
+      float evv = 1.0f;
+      if (DECAY == LQ_DECAY_SCALAR) evv = zoo_exp(p.eta * (p.g[(t0 + 63) * H + h] - p.g[(t0 + tid) * H + h]));
+      if (DECAY == LQ_DECAY_DIAGONAL) evv = zoo_exp(p.eta * p.logenv[(t0 + tid) * H + h]);
+      p.ev[(t0 + tid) * H + h] = evv;
+    }
+    if (tid < K) {
+      float gm = 1.0f, gl = 0.0f;
+      if (DECAY == LQ_DECAY_SCALAR) gm = zoo_exp(p.g[(t0 + 63) * H + h]);
+      if (DECAY == LQ_DECAY_DIAGONAL) {
+        gl = p.g[((t0 + 63) * H + h) * K + tid];
+        gm = zoo_exp(gl);
+      }
+      p.gam[(((int64_t)b * p.NT + ct) * H + h) * K + tid] = gm;
+      glast_s[tid] = gl;
+      iskw_s[tid] = 1.0f / p.skw[h * K + tid];
+    }
+    if (tid >= 128 && tid < 192) {
+      // per token: the factor of Hw and the key-side factor of the write codes (scalar decay: exp((1-eta)(g_last - g_t));
+      // per-channel decay: eta * log envelope, subtracted in the exponent per element)
+      const int t = tid - 128;
+      bw_s[t] = powb(p.beta[(t0 + t) * H + h], (1.0f - sigma) * tau);
+      float e = 1.0f;
+      if (DECAY == LQ_DECAY_SCALAR) e = zoo_exp((1.0f - p.eta) * (p.g[(t0 + 63) * H + h] - p.g[(t0 + t) * H + h]));
+      if (DECAY == LQ_DECAY_DIAGONAL) e = p.eta * p.logenv[(t0 + t) * H + h];
+      el_s[t] = e;
+    }
   }
   __syncthreads();
 
@@ -291,17 +337,20 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
 #pragma unroll 1
     for (int ps = 0; ps < K / 64; ++ps) {
       if (ps > 0) __syncthreads();
+      uint32_t c03[2], c47[2];  // CODES: the thread's write codes, channels 0..3 / 4..7 of its eight, per token
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
         const int it = tid + 256 * q;
-        const int r = it >> 3, c8 = it & 7;
+        // with CODES a thread takes two adjacent tokens, so that a token quad of a channel sits in two lanes
+        const int r = CODES ? 2 * (tid >> 3) + q : it >> 3, c8 = it & 7;
         const int64_t off = ((t0 + r) * H + h) * K + 64 * ps + 8 * c8;
         float kv[8];
         zoo_ld8(p.k + off, bf, kv);
         const float bs = bs_s[r], bh = bh_s[r];
         lq_v4f l0, l1, h0, h1;
+        lq_v4f g0 = {0.f, 0.f, 0.f, 0.f}, g1 = g0;
         if (DECAY == LQ_DECAY_DIAGONAL) {
-          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
+          g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
           const lq_v4f a0 = *(const lq_v4f*)(p.g + arow + 64 * ps + 8 * c8), a1 = *(const lq_v4f*)(p.g + arow + 64 * ps + 8 * c8 + 4);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -325,6 +374,55 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
         *(lq_v4f*)(Lg_s + r * kOP + 8 * c8 + 4) = l1;
         *(lq_v4f*)(Hg_s + r * kOP + 8 * c8) = h0;
         *(lq_v4f*)(Hg_s + r * kOP + 8 * c8 + 4) = h1;
+        if constexpr (CODES) {
+          // Hw = beta^((1-sigma) tau) k rounded to the activation dtype, stored; its write codes
+          // q8(Hw * fk, 1 / skw), fk = 1 | exp((1-eta)(g_last - g_t)) | exp(gk_last - gk_t - eta * le_t), go out
+          // channel-major: the four lanes that hold tokens 4Q .. 4Q+3 of these eight channels (eight lanes apart)
+          // exchange codes so that lane j of them owns channels 2j, 2j+1 of all four tokens, one dword each
+          const float bw = bw_s[r], el = el_s[r];
+          lq_v4i o;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(bw * kv[2 * d], bw * kv[2 * d + 1], bf);
+          *(lq_v4i*)(p.Hw + off) = o;
+          const int n8 = 64 * ps + 8 * c8;
+          const lq_v4f is0 = *(const lq_v4f*)(iskw_s + n8), is1 = *(const lq_v4f*)(iskw_s + n8 + 4);
+          lq_v4f gl0 = {0.f, 0.f, 0.f, 0.f}, gl1 = gl0;
+          if (DECAY == LQ_DECAY_DIAGONAL) gl0 = *(const lq_v4f*)(glast_s + n8), gl1 = *(const lq_v4f*)(glast_s + n8 + 4);
+          int kc8[8];
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            float x0, x1;
+            zoo_dec2((uint32_t)o[d], bf, x0, x1);
+            if (DECAY == LQ_DECAY_SCALAR) x0 = x0 * el, x1 = x1 * el;
+            if (DECAY == LQ_DECAY_DIAGONAL) {
+              const float ga = d < 2 ? g0[(2 * d) & 3] : g1[(2 * d) & 3], gb = d < 2 ? g0[(2 * d + 1) & 3] : g1[(2 * d + 1) & 3];
+              const float la = d < 2 ? gl0[(2 * d) & 3] : gl1[(2 * d) & 3], lb = d < 2 ? gl0[(2 * d + 1) & 3] : gl1[(2 * d + 1) & 3];
+              x0 = x0 * zoo_exp(la - ga - el);
+              x1 = x1 * zoo_exp(lb - gb - el);
+            }
+            const float ia = d < 2 ? is0[(2 * d) & 3] : is1[(2 * d) & 3], ib = d < 2 ? is0[(2 * d + 1) & 3] : is1[(2 * d + 1) & 3];
+            kc8[2 * d] = zoo_q8(x0, ia, p.qmax), kc8[2 * d + 1] = zoo_q8(x1, ib, p.qmax);
+          }
+          c03[q] = zoo_pack_codes(kc8[0], kc8[1], kc8[2], kc8[3]), c47[q] = zoo_pack_codes(kc8[4], kc8[5], kc8[6], kc8[7]);
+        }
+      }
+      if constexpr (CODES) {
+        // the thread eight lanes away holds the other token pair of the quad (same channels): the even pair assembles
+        // channels 0..3, the odd pair channels 4..7; four tokens x four channels are transposed bytewise in registers
+        const int rr = tid >> 3, c8 = tid & 7;
+        const bool odd = rr & 1;
+        const uint32_t m0 = odd ? c47[0] : c03[0], m1 = odd ? c47[1] : c03[1];
+        const uint32_t r0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? c03[0] : c47[0]), 0x128, 0xf, 0xf, false);  // row_ror:8
+        const uint32_t r1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? c03[1] : c47[1]), 0x128, 0xf, 0xf, false);
+        const uint32_t t0_ = odd ? r0 : m0, t1_ = odd ? r1 : m1, t2_ = odd ? m0 : r0, t3_ = odd ? m1 : r1;
+        const uint32_t a01 = __builtin_amdgcn_perm(t1_, t0_, 0x05010400u), b01 = __builtin_amdgcn_perm(t3_, t2_, 0x05010400u);
+        const uint32_t a23 = __builtin_amdgcn_perm(t1_, t0_, 0x07030602u), b23 = __builtin_amdgcn_perm(t3_, t2_, 0x07030602u);
+        uint32_t ch[4];
+        ch[0] = __builtin_amdgcn_perm(b01, a01, 0x05040100u), ch[1] = __builtin_amdgcn_perm(b01, a01, 0x07060302u);
+        ch[2] = __builtin_amdgcn_perm(b23, a23, 0x05040100u), ch[3] = __builtin_amdgcn_perm(b23, a23, 0x07060302u);
+        int8_t* kq = p.kqT + ((((int64_t)b * p.NT + ct) * H + h) * K + 64 * ps + 8 * c8 + 4 * (rr & 1)) * 64 + 4 * (rr >> 1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) *(uint32_t*)(kq + 64 * e) = ch[e];
       }
       __syncthreads();
 #pragma unroll
@@ -448,6 +546,8 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   // across the products spilled: 272 -> 316 us; it requests at the point of use)
   constexpr bool kAhead = DECAY != LQ_DECAY_DIAGONAL;
   if (kAhead) request_k(0);
+  float inv_sw = 0.0f;
+  if constexpr (CODES) inv_sw = 1.0f / p.sw[h];
 
   // Hw is written straight out; X = beta^sigma k exp(g) is staged (over the dead Gram tile)
 #pragma unroll
@@ -475,10 +575,12 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
           xr[u][2 * d] = x0, xr[u][2 * d + 1] = x1;
           hw[2 * d] = bw * k0, hw[2 * d + 1] = bw * k1;
         }
-        lq_v4i o;
+        if constexpr (!CODES) {  // with CODES, Hw and its codes were written while the Gram operands were staged
+          lq_v4i o;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
-        *(lq_v4i*)(p.Hw + off) = o;
+          for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+          *(lq_v4i*)(p.Hw + off) = o;
+        }
       }
       stage(xr[0], xr[1]);
     }
@@ -497,7 +599,15 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
       lq_v2i o;
       o[0] = (int)zoo_enc2(a[0], a[1], bf);
       o[1] = (int)zoo_enc2(a[2], a[3], bf);
-      *(lq_v2i*)(p.W + ((t0 + 16 * I + rl) * H + h) * K + kc + 16 * nt + 4 * kg) = o;
+      const int64_t woff = ((t0 + 16 * I + rl) * H + h) * K + kc + 16 * nt + 4 * kg;
+      if (!CODES || p.W) *(lq_v2i*)(p.W + woff) = o;
+      if constexpr (CODES) {  // state-read codes of the rounded W
+        float w0, w1, w2, w3;
+        zoo_dec2((uint32_t)o[0], bf, w0, w1);
+        zoo_dec2((uint32_t)o[1], bf, w2, w3);
+        *(uint32_t*)(p.wq + woff) = zoo_pack_codes(zoo_q8(w0, inv_sw, p.qmax), zoo_q8(w1, inv_sw, p.qmax),
+                                                    zoo_q8(w2, inv_sw, p.qmax), zoo_q8(w3, inv_sw, p.qmax));
+      }
     }
   }
 
@@ -534,13 +644,18 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   }
 }
 
+template <int DECAY, int K, bool CODES>
+int launch_c(const WyParams& p, dim3 grid, hipStream_t stream) {
+  if (p.bf)
+    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, true, CODES>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, false, CODES>), grid, dim3(256), 0, stream, p);
+  return lq_check_launch();
+}
+
 template <int DECAY, int K>
 int launch(const WyParams& p, dim3 grid, hipStream_t stream) {
-  if (p.bf)
-    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, true>), grid, dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, false>), grid, dim3(256), 0, stream, p);
-  return lq_check_launch();
+  return p.kqT ? launch_c<DECAY, K, true>(p, grid, stream) : launch_c<DECAY, K, false>(p, grid, stream);
 }
 
 template <int K>
@@ -556,8 +671,14 @@ int launch_decay(const WyParams& p, int decay, dim3 grid, hipStream_t stream) {
 }  // namespace
 
 extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) {
-  if (!a || !a->k || !a->v || !a->beta || !a->Hw || !a->W || !a->U || !a->fw) return LQ_ERR_NULL;
+  if (!a || !a->k || !a->v || !a->beta || !a->Hw || !a->U || !a->fw) return LQ_ERR_NULL;
   if (a->decay != LQ_DECAY_NONE && !a->g) return LQ_ERR_NULL;
+  const bool codes = a->kqT != nullptr;
+  if (!codes && !a->W) return LQ_ERR_NULL;
+  if (codes && (!a->wq || !a->ev || !a->gam || !a->skw || !a->sw)) return LQ_ERR_NULL;
+  if (codes && a->decay == LQ_DECAY_DIAGONAL && !a->logenv) return LQ_ERR_NULL;
+  if (codes && (a->qmax < 1 || a->qmax > 127)) return LQ_ERR_SHAPE;
+  if (codes && (!zoo_al(a->kqT, 16) || !zoo_al(a->wq, 4) || !zoo_al(a->skw, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
@@ -569,6 +690,8 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   p.Hw = (_Float16*)a->Hw, p.W = (_Float16*)a->W, p.U = (_Float16*)a->U, p.fw = a->fw;
   p.sigma = a->sigma, p.tau = a->tau, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim;
+  p.kqT = a->kqT, p.wq = a->wq, p.ev = a->ev, p.gam = a->gam, p.logenv = a->logenv, p.skw = a->skw, p.sw = a->sw;
+  p.eta = a->eta, p.qmax = a->qmax, p.NT = a->seqlen / 64;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);
   return a->kdim == 128 ? launch_decay<128>(p, a->decay, grid, stream) : launch_decay<64>(p, a->decay, grid, stream);
 }

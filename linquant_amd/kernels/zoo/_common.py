@@ -146,9 +146,10 @@ def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, fa
 
 
 def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
-              sw=None, vtile=0, unrot=None):
-    """``value`` is v (linear family) or U (delta family)."""
-    c = write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay)
+              sw=None, vtile=0, unrot=None, codes=None):
+    """``value`` is v (linear family) or U (delta family); ``codes``: write-operand codes that ``run_wy_prep`` already made
+    (no pre-pass then)."""
+    c = codes if codes is not None else write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay)
     state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile, unrot)
     return c
 
@@ -176,16 +177,31 @@ def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None):
     return A, qg
 
 
-def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay):
-    """Returns (Hw, W, U, fw): fp16 operands of the delta state kernel and the value-side share of beta."""
+def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True):
+    """Returns (Hw, W, U, fw, codes): operands of the delta state kernel in the activation dtype and the value-side share
+    of beta.  ``write`` = dict(logenv, skw, sw, eta, qmax): the launch also makes the state kernel's write-operand codes
+    (what ``write_codes`` would make from the stored Hw and W, same bits) and returns them as ``codes``; W itself is
+    then stored only when ``keep_W``."""
     B, T, H, K, V = dims
-    Hw, W = torch.empty_like(k), torch.empty_like(k)
+    dev, NT = k.device, T // CHUNK
+    Hw = torch.empty_like(k)
+    W = torch.empty_like(k) if (keep_W or write is None) else None
     U = torch.empty_like(v)
-    fw = torch.empty(B, T, H, dtype=torch.float32, device=k.device)
-    _lib.call("lq_zoo_wy_prep", k.device, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
+    fw = torch.empty(B, T, H, dtype=torch.float32, device=dev)
+    extra, c = {}, None
+    if write is not None:
+        c = {"kqT": torch.empty(B, NT, H, K, CHUNK, dtype=torch.int8, device=dev), "vqT": None,
+             "wq": torch.empty(B, T, H, K, dtype=torch.int8, device=dev),
+             "ev": torch.empty(B, T, H, dtype=torch.float32, device=dev),
+             "gam": torch.empty(B, NT, H, K, dtype=torch.float32, device=dev)}
+        skw = _lib.aligned(write["skw"])
+        extra = dict(kqT=_lib.ptr(c["kqT"]), wq=_lib.ptr(c["wq"]), ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]),
+                     logenv=_lib.ptr(write["logenv"]), skw=_lib.ptr(skw), sw=_lib.ptr(write["sw"]), eta=float(write["eta"]),
+                     qmax=int(write["qmax"]))
+    _lib.call("lq_zoo_wy_prep", dev, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
               Hw=_lib.ptr(Hw), W=_lib.ptr(W), U=_lib.ptr(U), fw=_lib.ptr(fw), sigma=float(sigma), tau=float(tau),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(k))
-    return Hw, W, U, fw
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(k), **extra)
+    return Hw, W, U, fw, c
 
 
 def out_buffer(v, out_dtype):

@@ -30,15 +30,18 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     if g is not None:
         assert g.shape == (B, T, H)
         gg, _ = C.cumsum(g, B, T, H, 0)
-    Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
+    # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
+    Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay,
+                                        write=dict(logenv=None, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
+                                        keep_W=_debug is not None)
     NT = T // chunk_size
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    codes = C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
-                w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru)
+    C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
+                w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes)
     C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
     C.export_debug(_debug, h_i8, codes, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return C.cut_values(o, C.cut_keys(ht, K0), V0)

@@ -28,16 +28,19 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     gc, logenv = C.cumsum(g, B, T, H, K)
-    Hw, W, U, fw = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
+    # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
+    Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL,
+                                        write=dict(logenv=logenv, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
+                                        keep_W=_debug is not None)
     A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R)
     NT = T // chunk_size
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    codes = C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
-                C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru)
+    C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
+                C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes)
     C.run_output(None, None, e_out, h_i8, None, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)

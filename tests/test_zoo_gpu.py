@@ -442,13 +442,50 @@ def test_wy_prep_kernel(cuda, cell, sigma, tau, K, gscale):
     if g is not None:
         gc = g.double().reshape(B, T // 64, 64, H, -1).cumsum(2).reshape(g.shape).float()
     code = {"none": C.DECAY_NONE, "scalar": C.DECAY_SCALAR, "diagonal": C.DECAY_DIAGONAL}[decay]
-    Hw, W, U, fw = C.run_wy_prep(k.cuda(), v.cuda(), beta.cuda(), None if gc is None else gc.cuda(), sigma, tau,
-                                 (B, T, H, K, V), code)
+    Hw, W, U, fw, _ = C.run_wy_prep(k.cuda(), v.cuda(), beta.cuda(), None if gc is None else gc.cuda(), sigma, tau,
+                                    (B, T, H, K, V), code)
     torch.cuda.synchronize()
     rHw, rW, rU, rfw = _wy_reference(k, v, beta, gc, decay, sigma, tau)
     for name, got, ref in (("Hw", Hw, rHw), ("W", W, rW), ("U", U, rU), ("fw", fw, rfw)):
         err = (got.double().cpu() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
         assert err <= 1e-3, f"{cell} {name}: rel max {err:.2e}"  # half-precision storage: 2^-11 per element
+
+
+@pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet", "kda"])
+@pytest.mark.parametrize("K,dtype,eta,bits", [(64, torch.float16, 1.0, 8), (128, torch.float16, 0.5, 8),
+                                              (128, torch.bfloat16, 0.0, 6), (64, torch.bfloat16, 0.3, 8)])
+def test_wy_prep_also_makes_the_write_codes(cuda, cell, K, dtype, eta, bits):
+    """The WY prep launch that also emits the state kernel's write operands (key write codes, state-read codes of W,
+    value factor, chunk decay) gives, bit for bit, what the stand-alone pre-pass makes from the stored Hw and W; Hw, U
+    and fw are the same with and without the codes, and W may be left unstored."""
+    from linquant_amd.kernels.zoo import _common as C
+
+    decay = zc.CELLS[cell][1]
+    q, k, v, g, beta = zc.cut(zc.inputs(cell, B=2, H=3, K=K, V=64, seed=21), 192)
+    B, T, H, V = 2, 192, 3, 64
+    dims = (B, T, H, K, V)
+    code = {"none": C.DECAY_NONE, "scalar": C.DECAY_SCALAR, "diagonal": C.DECAY_DIAGONAL}[decay]
+    k, v, beta = k.to(dtype).cuda(), v.to(dtype).cuda(), beta.cuda()
+    gc = logenv = None
+    if g is not None:
+        gc, logenv = C.cumsum(g.cuda(), B, T, H, K if decay == "diagonal" else 0)
+    gen = torch.Generator().manual_seed(3)
+    skw = (torch.rand(H, K, generator=gen) * 0.02 + 0.002).cuda()
+    sw = (torch.rand(H, generator=gen) * 0.02 + 0.004).cuda()
+    qmax = 2 ** (bits - 1) - 1
+    Hw0, W0, U0, fw0, none = C.run_wy_prep(k, v, beta, gc, 0.5, 0.5, dims, code)
+    ref = C.write_codes(Hw0, None, W0, gc, logenv, skw, None, sw, eta, qmax, dims, C.FAMILY_DELTA, code)
+    write = dict(logenv=logenv, skw=skw, sw=sw, eta=eta, qmax=qmax)
+    Hw1, W1, U1, fw1, got = C.run_wy_prep(k, v, beta, gc, 0.5, 0.5, dims, code, write=write, keep_W=True)
+    Hw2, W2, U2, fw2, got2 = C.run_wy_prep(k, v, beta, gc, 0.5, 0.5, dims, code, write=write, keep_W=False)
+    torch.cuda.synchronize()
+    assert none is None and W2 is None
+    for name, a, b_ in (("Hw", Hw1, Hw0), ("W", W1, W0), ("U", U1, U0), ("fw", fw1, fw0), ("Hw", Hw2, Hw0), ("U", U2, U0)):
+        assert torch.equal(a, b_), f"{cell} {name} changes when the codes are made in the same launch"
+    for name in ("kqT", "wq", "ev", "gam"):
+        assert torch.equal(got[name], ref[name]), f"{cell} {name}: differs from the stand-alone pre-pass"
+        assert torch.equal(got2[name], ref[name]), f"{cell} {name} (W not stored): differs from the stand-alone pre-pass"
+    assert int(ref["kqT"].abs().max()) > qmax // 2 and int(ref["wq"].abs().max()) > 0  # the comparison is not vacuous
 
 
 def test_reference_mamba2_cell_config(cuda):
