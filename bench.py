@@ -223,12 +223,12 @@ def measure_zoo(args, workload, cpu_baseline):
     if workload == "c4_kda":
         cq, ck, *_ = zoo_synthetic(cell, 1, 2048, H, K, V, seed=1)
         dqk = dqk_from_absmax(cq.half().float(), ck.half().float(), 0.5).to(dev)
-    has_prologue = persistent or dqk is not None
-    qr, kr = torch.empty_like(q0), torch.empty_like(k0)
+    has_prologue = persistent  # D_QK is applied inside the KDA kernels as they load q and k: no launch of its own
+    qr, kr = (torch.empty_like(q0), torch.empty_like(k0)) if has_prologue else (None, None)
 
     def prologue():
         if has_prologue:
-            zoo.rotate_qkv(q0, k0, None, signs_qk=sq, dqk=dqk, out=(qr, kr, None))
+            zoo.rotate_qkv(q0, k0, None, signs_qk=sq, out=(qr, kr, None))
             return qr, kr
         return q0, k0
 
@@ -243,7 +243,7 @@ def measure_zoo(args, workload, cpu_baseline):
         if fam == "linear":
             return zoo.chunk_simple_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, **kw)
         if dec == "diagonal":
-            return zoo.chunk_kda_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, rot=rot, **kw)
+            return zoo.chunk_kda_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, rot=rot, dqk=dqk, **kw)
         return zoo.chunk_delta_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, **kw)
 
     def call(sc, **kw):
@@ -254,7 +254,8 @@ def measure_zoo(args, workload, cpu_baseline):
     # pilot run of the kernels themselves with a coarse state grid
     ph = lambda t: (t.float().abs().amax(dim=(0, 1, 3)) / 127).clamp_min(1e-6)  # noqa: E731
     pc = lambda t: (t.float().abs().amax(dim=(0, 1)) / 127).clamp_min(1e-6)  # noqa: E731
-    sc = {"q": ph(q) * scale, "k": ph(k), "w": ph(k) * 2, "kw": pc(k), "vw": pc(v), "vl": pc(v),
+    qs, ks = (q, k) if dqk is None else zoo.rotate_qkv(q0, k0, None, dqk=dqk)[:2]  # the operands the kernels will see
+    sc = {"q": ph(qs) * scale, "k": ph(ks), "w": ph(ks) * 2, "kw": pc(ks), "vw": pc(v), "vl": pc(v),
           "el": pc(v) * 2, "ew": pc(v) * 2, "state": torch.full((H, V), 1.0, device=dev)}
     sc = {n: t.contiguous() for n, t in sc.items()}
     dbg = {}
@@ -308,6 +309,7 @@ def measure_zoo(args, workload, cpu_baseline):
             setattr(C, n, f)
     nbytes = zoo_stage_bytes(fam, dec, B, T, H, K, V)
     nbytes["prologue"] = 2 * (B * T * H * K * 2) * 2  # q and k, read and written once
+    del qs, ks
     stages = {}
     for label, evs in records.items():
         ts = sorted(a.elapsed_time(b) for a, b in evs)
@@ -357,9 +359,10 @@ def measure_zoo(args, workload, cpu_baseline):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
                    "tokens_per_step": tokens, "ramp": ramp_note(ramp_steps),
-                   "prologue": ("in the timed step: " + ("R_QK on q, k" if persistent else "") +
-                                (" D_QK (alpha 0.5) on q, k" if dqk is not None else "")) if has_prologue else
-                               "none (local R_QK inside the A kernel)" if rot is not None else "none"},
+                   "prologue": "in the timed step: R_QK on q, k" if has_prologue else
+                               ("none (local R_QK inside the A kernel" +
+                                ("; D_QK (alpha 0.5) applied inside the WY prep and A kernels as they load k and q)"
+                                 if dqk is not None else ")")) if rot is not None else "none"},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
     }
     return line

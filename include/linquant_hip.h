@@ -419,6 +419,8 @@ typedef struct {
   int32_t qmax;
   int32_t batch, seqlen, nheads, kdim, chunk_size;
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
+  const float* dq;           /* optional (H,K) fp32 D_QK (linquant/harness.py:68-88) applied to q as it is loaded:
+                                q' = act(q * dq), exactly what lq_zoo_rotate_qkv would have stored; NULL: q as it is */
 } lq_zoo_gla_A_args;
 int lq_zoo_gla_A(const lq_zoo_gla_A_args* args, hipStream_t stream);
 
@@ -452,13 +454,18 @@ typedef struct {
   const float* sw;           /* (H,) state-read scale of W */
   float eta;
   int32_t qmax;
+  /* Optional D_QK (linquant/harness.py:68-88) applied to k as it is loaded: k' = act(k / dk_div), the quotient rounded
+   * once, exactly what lq_zoo_rotate_qkv would have stored; both NULL: k is used as it is.  Taken only together with the
+   * write-operand codes above (kqT set). */
+  const float* dk_div;       /* (H,K) fp32 D_QK, finite and positive */
+  const float* dk_rcp;       /* (H,K) fp32 RN(1 / dk_div) */
 } lq_zoo_wy_prep_args;
 int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
 
 /* replaces the operand rotations in front of a zoo call: the three GEMMs q @ R_QK, k @ R_QK, v @ R_V of
  * bench/zoo_kernels.py:135-140 (the oracle's entry rotation, linquant/reference.py:42-46) and the diagonal q / k
  * rescaling D_QK of linquant/harness.py:68-88, in one launch:
- *   q_out = act((q * dq) . H_K / sqrt(K) * signs_qk),  k_out likewise with dk (= 1 / dq),  v_out = act(v . H_V / sqrt(V) * signs_v)
+ *   q_out = act((q * dq) . H_K / sqrt(K) * signs_qk),  k_out likewise with k / dq,  v_out = act(v . H_V / sqrt(V) * signs_v)
  * with the Sylvester Hadamard matrix H_n (linquant/reference.py:232-239: R = H_n / sqrt(n) . diag(signs)), evaluated as a
  * fast Walsh-Hadamard transform in fp32 and rounded once to the activation dtype.  A tensor whose input pointer is NULL
  * is skipped; NULL signs leave out the rotation (diagonal-decay cells rotate locally inside lq_zoo_gla_A); NULL dq / dk
@@ -470,8 +477,9 @@ typedef struct {
   void* q_out;               /* same shape and dtype as the input */
   void* k_out;
   void* v_out;
-  const float* dq;           /* (H,K) fp32 factor on q (D_QK), or NULL */
-  const float* dk;           /* (H,K) fp32 factor on k (1 / D_QK), or NULL */
+  const float* dq;           /* (H,K) fp32 D_QK, finite and positive: q is multiplied by it, k divided (the quotient is
+                                rounded once to fp32, as the float64 division of harness.py:86 rounds); or NULL */
+  const float* dk;           /* (H,K) fp32 RN(1 / dq), set exactly when k is to be rescaled (needs dq), or NULL */
   const float* signs_qk;     /* (K,) fp32 +-1 column signs of R_QK, or NULL */
   const float* signs_v;      /* (V,) fp32 +-1 column signs of R_V, or NULL */
   int32_t batch, seqlen, nheads, kdim, vdim; /* kdim, vdim in {64, 128} */

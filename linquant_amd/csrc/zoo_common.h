@@ -78,3 +78,18 @@ LQ_DEV uint32_t zoo_enc2(float a, float b, bool bf) {
 LQ_DEV uint16_t zoo_enc1(float a, bool bf) {
   return bf ? (uint16_t)zoo_bf16_bits(a) : __builtin_bit_cast(uint16_t, (_Float16)a);
 }
+// x rounded to the activation dtype and back: what a consumer reads when a producer stored x there
+LQ_DEV float zoo_round_act(float x, bool bf) { return zoo_dec1((uint32_t)zoo_enc1(x, bf), bf); }
+
+// x / d rounded once to fp32 (the IEEE quotient) from r = RN(1 / d): q0 = RN(x r), rem = x - q0 d (exact in the fused
+// multiply-add), q = RN(q0 + rem r).  Correct for finite d > 0 and half-precision x (checked over every fp16 and bf16
+// value on the CPU); three instructions instead of the division sequence.
+LQ_DEV float zoo_div_rn(float x, float d, float r) {
+  const float q0 = x * r;
+  const float rem = __builtin_fmaf(-q0, d, x);
+  float q = __builtin_fmaf(rem, r, q0);
+  // the quotient exists as an fp32 value before anything narrows it: without this the compiler folds a following
+  // conversion to half precision into the multiply-add (one rounding instead of two)
+  asm volatile("" : "+v"(q));
+  return q;
+}

@@ -35,6 +35,7 @@ struct AParams {
   const float* sq;
   const float* sk;
   const _Float16* rot;
+  const float* dq;  // (H,K) D_QK applied to q at load (q' = act(q * dq)), or nullptr
   float scale;
   int qmax;
   int bf;
@@ -59,6 +60,10 @@ LQ_DEV void diag_exact(const AParams& p, float sq, float sk, float inv_sq, float
   for (int n8 = 0; n8 < K; n8 += 8) {
     float qv[8];
     zoo_ld8(p.q + irow + n8, bf, qv);
+    if (p.dq) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qv[e] = zoo_round_act(qv[e] * p.dq[h * K + n8 + e], bf);
+    }
     const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
@@ -90,12 +95,14 @@ LQ_DEV void diag_exact(const AParams& p, float sq, float sk, float inv_sq, float
 
 // QG: the state-read codes are wanted (p.qg is set); a compile-time flag keeps the own-rows loop
 // one basic block.
-template <int K, bool ROT, bool BF, bool QG>
+// DQ: q is rescaled per (head, channel) as it is loaded (a compile-time flag: the kernel sits at its register limit).
+template <int K, bool ROT, bool BF, bool QG, bool DQ>
 __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   constexpr int RS = K + 8;  // halves per row of the transposed rotation
   __shared__ __align__(16) _Float16 RT[ROT ? K * RS : 8];  // RT[m][n] = R[n][m]
   // rotated query codes of sub-blocks 1..3 of both chunks: [pass][I - 1][lane][dword]
   __shared__ __align__(16) uint32_t QC[2 * 3 * 64 * (K / 16)];
+  __shared__ __align__(16) float DQs[DQ ? K : 4];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -107,6 +114,10 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   constexpr bool bf = BF;
   const int nchunks = p.T / 64;
 
+  if constexpr (DQ) {
+    if (tid < K) DQs[tid] = p.dq[h * K + tid];
+    if constexpr (!ROT) __syncthreads();
+  }
   if constexpr (ROT) {
     // lanes walk m (coalesced rows of R), each thread gathers 8 consecutive n and writes one 16-byte piece of a row
     for (int it = tid; it < K * (K / 8); it += 256) {
@@ -246,6 +257,11 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
       float qf[8], kf[8];
       unpack(r.q, qf);
       unpack(r.k, kf);
+      if constexpr (DQ) {  // D_QK at load: q' = act(q * D), what the stand-alone rescaling launch would have stored
+        const lq_v4f d0 = *(const lq_v4f*)(DQs + 32 * ks + 8 * kg), d1 = *(const lq_v4f*)(DQs + 32 * ks + 8 * kg + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[e] = zoo_round_act(qf[e] * (e < 4 ? d0[e & 3] : d1[e & 3]), bf);
+      }
       int cs[8], iq[8], ik[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -311,7 +327,7 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
       for (int r = 0; r < 4; ++r)
         p.A[((t0 + i0 + 4 * kg + r) * H + h) * 64 + i0 + rl] = (_Float16)((rl <= 4 * kg + r) ? dacc[r] : 0.0f);
     } else {
-      diag_exact<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);
+      diag_exact<K, BF>(p, sq, sk, inv_sq, inv_sk, rl, kg, t0 + i0, h, i0);  // (applies p.dq itself)
     }
   }
   // zero blocks above the diagonal
@@ -333,18 +349,27 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   if (!zoo_al(a->q, 16) || !zoo_al(a->k, 16) || !zoo_al(a->g, 16) || !zoo_al(a->A, 16) || (a->qg && !zoo_al(a->qg, 8)))
     return LQ_ERR_SHAPE;
   if (a->rot && !zoo_al(a->rot, 16)) return LQ_ERR_SHAPE;
+  if (a->dq && !zoo_al(a->dq, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   AParams p = {};
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.g = a->g, p.A = (_Float16*)a->A, p.qg = a->qg;
+  p.dq = a->dq;
   p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
   dim3 grid((a->seqlen / 64 + 1) / 2, a->batch * a->nheads);
+#define LQ_A_LAUNCH3(KV, ROTV, BFV, QGV)                                                                   \
+  do {                                                                                                     \
+    if (p.dq)                                                                                              \
+      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, BFV, QGV, true>), grid, dim3(256), 0, stream, p);     \
+    else                                                                                                   \
+      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, BFV, QGV, false>), grid, dim3(256), 0, stream, p);    \
+  } while (0)
 #define LQ_A_LAUNCH2(KV, ROTV, QGV)                                                                        \
   do {                                                                                                     \
     if (p.bf)                                                                                              \
-      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, true, QGV>), grid, dim3(256), 0, stream, p);          \
+      LQ_A_LAUNCH3(KV, ROTV, true, QGV);                                                                   \
     else                                                                                                   \
-      hipLaunchKernelGGL((zoo_gla_A_kernel<KV, ROTV, false, QGV>), grid, dim3(256), 0, stream, p);         \
+      LQ_A_LAUNCH3(KV, ROTV, false, QGV);                                                                  \
   } while (0)
 #define LQ_A_LAUNCH(KV)                 \
   do {                                  \
@@ -361,6 +386,7 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
     LQ_A_LAUNCH(128);
   else
     LQ_A_LAUNCH(64);
+#undef LQ_A_LAUNCH3
 #undef LQ_A_LAUNCH2
 #undef LQ_A_LAUNCH
   return lq_check_launch();

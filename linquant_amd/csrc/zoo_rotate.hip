@@ -2,14 +2,15 @@
 // one launch for all three tensors.
 // Replaces the three bf16 GEMMs q @ R, k @ R, v @ R_V of the reference's timing script (bench/zoo_kernels.py:135-140,
 // "not fused yet"), the rotation the oracle applies on entry (linquant/reference.py:42-46: mat(q @ rot_qk),
-// mat(k @ rot_qk), mat(v @ rot_v)) and the D_QK input transform (linquant/harness.py:68-88: q' = q D, k' = k / D).
+// mat(k @ rot_qk), mat(v @ rot_v)) and the D_QK input transform (linquant/harness.py:68-88: q' = q D, k' = k / D, the
+// quotient rounded once as the division there rounds it).
 //
 // R = H_n / sqrt(n) . diag(signs) with the Sylvester H_n (linquant/reference.py:232-239), so a row is rotated by a fast
 // Walsh-Hadamard transform instead of a GEMM: y_j = signs_j / sqrt(n) * sum_i (x_i d_i) H_ij.  HBM-bound byte work:
 // a row of n channels is spread over n / 8 lanes, 16 bytes per lane in and out; butterfly stages 1, 2, 4 run in
 // registers, the rest through wave shuffles.  fp32 sums of at most 128 half-precision values, one multiply, one
 // rounding to the activation dtype.
-#include "lq_common.h"
+#include "zoo_common.h"
 #include "../../include/linquant_hip.h"
 
 namespace {
@@ -17,7 +18,8 @@ namespace {
 struct RotParams {
   const uint16_t* src[3];
   uint16_t* dst[3];
-  const float* diag[3];   // (H, D) or nullptr
+  const float* diag[3];   // (H, D) multiplier, or nullptr
+  const float* divd[3];   // (H, D) divisor whose reciprocal diag holds (the row is divided, rounded once), or nullptr
   const float* signs[3];  // (D,) or nullptr: no rotation
   int64_t rows;           // B * T * H
   int nheads;
@@ -42,6 +44,7 @@ __global__ __launch_bounds__(256) void zoo_rotate_kernel(RotParams p) {
   const uint16_t* src = p.src[which];
   if (!src) return;  // block-uniform: this tensor is not part of the call
   const float* diag = p.diag[which];
+  const float* divd = p.divd[which];
   const float* signs = p.signs[which];
   const int sub = threadIdx.x % LPR;
   const int64_t row0 = (int64_t)blockIdx.x * (R * RPB) + threadIdx.x / LPR;
@@ -56,11 +59,13 @@ __global__ __launch_bounds__(256) void zoo_rotate_kernel(RotParams p) {
   // operands that are absent are read from a valid address and ignored: every request is issued before the first use
   const float* sp = signs ? signs + sub * 8 : (const float*)src;
   const lq_v4f s0 = *(const lq_v4f*)sp, s1 = *(const lq_v4f*)(signs ? sp + 4 : sp);
-  lq_v4f d0[R], d1[R];
+  lq_v4f d0[R], d1[R], e0[R], e1[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const float* dp = diag ? diag + (int64_t)hh[r] * D + sub * 8 : sp;
     d0[r] = *(const lq_v4f*)dp, d1[r] = *(const lq_v4f*)(diag ? dp + 4 : dp);
+    const float* ep = divd ? divd + (int64_t)hh[r] * D + sub * 8 : sp;
+    e0[r] = *(const lq_v4f*)ep, e1[r] = *(const lq_v4f*)(divd ? ep + 4 : ep);
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -71,7 +76,10 @@ __global__ __launch_bounds__(256) void zoo_rotate_kernel(RotParams p) {
       const uint16_t u = (uint16_t)((uint32_t)raw[r][i >> 1] >> (16 * (i & 1)));
       v[i] = BF16 ? bf16_to_f(u) : (float)__builtin_bit_cast(_Float16, u);
     }
-    if (diag) {
+    if (divd) {  // the quotient rounded once, as a division would give it
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = zoo_div_rn(v[i], i < 4 ? e0[r][i & 3] : e1[r][i & 3], i < 4 ? d0[r][i & 3] : d1[r][i & 3]);
+    } else if (diag) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = v[i] * (i < 4 ? d0[r][i & 3] : d1[r][i & 3]);
     }
@@ -142,6 +150,7 @@ extern "C" int lq_zoo_rotate_qkv(const lq_zoo_rotate_qkv_args* a, hipStream_t st
   if (!a) return LQ_ERR_NULL;
   if ((a->q && !a->q_out) || (a->k && !a->k_out) || (a->v && !a->v_out)) return LQ_ERR_NULL;
   if (!a->q && !a->k && !a->v) return LQ_ERR_NULL;
+  if (a->k && a->dk && !a->dq) return LQ_ERR_NULL;  // k is divided by dq; dk is its reciprocal
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   const int K = a->kdim, V = a->vdim;
@@ -162,6 +171,7 @@ extern "C" int lq_zoo_rotate_qkv(const lq_zoo_rotate_qkv_args* a, hipStream_t st
     if (qk) {
       p.src[0] = (const uint16_t*)a->q, p.dst[0] = (uint16_t*)a->q_out, p.diag[0] = a->dq, p.signs[0] = a->signs_qk;
       p.src[1] = (const uint16_t*)a->k, p.dst[1] = (uint16_t*)a->k_out, p.diag[1] = a->dk, p.signs[1] = a->signs_qk;
+      p.divd[1] = a->dk ? a->dq : nullptr;
       if (a->v && V == K) p.src[2] = (const uint16_t*)a->v, p.dst[2] = (uint16_t*)a->v_out, p.signs[2] = a->signs_v;
       if (!a->q && !a->k && !(a->v && V == K)) continue;
     } else {

@@ -46,12 +46,32 @@ struct WyParams {
   float eta;
   int qmax;
   int NT;
+  const float* dk_div;  // (H,K) D_QK applied to k at load (k' = act(k / D)), with its reciprocal; or nullptr
+  const float* dk_rcp;
 };
 
 LQ_DEV float powb(float b, float e) {
   if (e == 0.0f) return 1.0f;
   if (e == 1.0f) return b;
   return __builtin_amdgcn_exp2f(e * __builtin_amdgcn_logf(b));
+}
+
+typedef float wy_v2f __attribute__((ext_vector_type(2)));
+
+// D_QK at load: k' = act(k / D) for the eight adjacent channels n .. n + 7 (the quotient rounded once to fp32, then to
+// the activation dtype: what the stand-alone rescaling launch would have stored).  tab: D at [n], RN(1 / D) at [128 + n],
+// staged per head in LDS.  DK is a compile-time flag: the kernels sit at their register limit, and a run-time test
+// around this arithmetic spilled dozens of registers in the variants that never rescale.
+template <bool BF, bool DK>
+LQ_DEV void wy_dk8(const float* tab, int n, float (&kv)[8]) {
+  if constexpr (DK) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {  // two channels at a time: the table entries are short-lived
+      const wy_v2f dd = *(const wy_v2f*)(tab + n + 2 * d), rr = *(const wy_v2f*)(tab + 128 + n + 2 * d);
+      kv[2 * d] = zoo_round_act(zoo_div_rn(kv[2 * d], dd[0], rr[0]), BF);
+      kv[2 * d + 1] = zoo_round_act(zoo_div_rn(kv[2 * d + 1], dd[1], rr[1]), BF);
+    }
+  }
 }
 
 LQ_DEV lq_v4f mfma_f32(float a, float b, lq_v4f c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
@@ -69,7 +89,6 @@ constexpr int kGS = 70;  // floats per row of the G / T tiles: measured, an A-op
 // leading one (hi.hi, hi.mid, mid.hi, mid.mid, hi.lo, lo.hi) reproduce the fp32 product to about 2^-23 at 3/8 of the
 // fp32 MFMA's issue time.  (Two pieces per factor, 2^-16, moved stored state codes by two steps in places.)
 typedef __bf16 wy_v8bf __attribute__((ext_vector_type(8)));
-typedef float wy_v2f __attribute__((ext_vector_type(2)));
 
 LQ_DEV lq_v4f mfma_bf16(lq_v4i a, lq_v4i b, lq_v4f c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(wy_v8bf, a), __builtin_bit_cast(wy_v8bf, b), c, 0, 0, 0);
@@ -132,9 +151,9 @@ LQ_DEV lq_v4f tx_tile(const uint32_t* Xt, const lq_v4i (&th)[2], const lq_v4i (&
 // the decay spread over the whole chunk is too large for one anchor): operands straight from global memory, lane
 // (rl, kg) supplies 16 contiguous channels of token rl per 64-channel pass; off-diagonal blocks: both factors <= 1;
 // diagonal block: only when the spread inside the block is small, otherwise one exponential per (i, j, channel).
-template <int DECAY, int K, bool BF>
+template <int DECAY, int K, bool BF, bool DK>
 LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, const float* bh_s, const float* gs_s, int wave,
-                          int rl, int kg, int64_t t0, int h) {
+                          int rl, int kg, int64_t t0, int h, const float* dk_s) {
   const int H = p.H;
   constexpr bool bf = BF;
     const int I = wave;
@@ -165,6 +184,8 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
         zoo_ld8(p.k + irow + c0, bf, k0);
         float k1[8];
         zoo_ld8(p.k + irow + c0 + 8, bf, k1);
+        wy_dk8<BF, DK>(dk_s, c0, k0);
+        wy_dk8<BF, DK>(dk_s, c0 + 8, k1);
 #pragma unroll
         for (int e = 0; e < 16; ++e) Lr[e] = bs_i * (float)(e < 8 ? k0[e & 7] : k1[e & 7]);
         if (DECAY == LQ_DECAY_DIAGONAL) {
@@ -191,6 +212,8 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
         zoo_ld8(p.k + jrow + c0, bf, k0);
         float k1[8];
         zoo_ld8(p.k + jrow + c0 + 8, bf, k1);
+        wy_dk8<BF, DK>(dk_s, c0, k0);
+        wy_dk8<BF, DK>(dk_s, c0 + 8, k1);
         float Hr[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) Hr[e] = bh_j * (float)(e < 8 ? k0[e & 7] : k1[e & 7]);
@@ -228,6 +251,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
       for (int n8 = 0; n8 < K; n8 += 8) {
         float ki[8];
         zoo_ld8(p.k + irow + n8, bf, ki);
+        wy_dk8<BF, DK>(dk_s, n8, ki);
         const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
@@ -235,6 +259,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
           const int64_t jrow = ((t0 + 16 * I + j) * H + h) * K;
           float kj[8];
           zoo_ld8(p.k + jrow + n8, bf, kj);
+          wy_dk8<BF, DK>(dk_s, n8, kj);
           const lq_v4f gj0 = *(const lq_v4f*)(p.g + jrow + n8), gj1 = *(const lq_v4f*)(p.g + jrow + n8 + 4);
           const float bh_j = bh_s[16 * I + j];
 #pragma unroll
@@ -253,7 +278,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
 // CODES: the kernel also emits what lq_zoo_write_codes would make from the stored Hw and W (same arithmetic on the same
 // rounded values, so the same bits): channel-major key write codes, token-major state-read codes of W, the per-token
 // value factor and the per-channel chunk decay.  W itself is then stored only when p.W is set.
-template <int DECAY, int K, bool BF, bool CODES>
+template <int DECAY, int K, bool BF, bool CODES, bool DK>
 __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   constexpr int LS = 64 + 16;  // floats per row of the buffer that holds the Gram tile and then the X tiles
   static_assert(LS >= kGS, "the Gram tile lives in the X buffer until the inverse is done");
@@ -267,8 +292,14 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   static_assert(2 * 64 * kOP <= 64 * kGS + 64 * LS, "the Gram operands live in the T / X buffers until G is written");
   float* Lg_s = lds_f;
   float* Hg_s = lds_f + 64 * kOP;
-  __shared__ float gs_s[64], bs_s[64], bh_s[64];
-  __shared__ float iskw_s[CODES ? K : 1], glast_s[CODES ? K : 1], bw_s[CODES ? 64 : 1], el_s[CODES ? 64 : 1];
+  __shared__ float gs_s[DECAY == LQ_DECAY_SCALAR ? 64 : 1], bs_s[64], bh_s[64];
+  __shared__ float iskw_s[CODES ? K : 1], bw_s[CODES ? 64 : 1], el_s[CODES ? 64 : 1];
+  // the last 1.5 KB of the big buffer lie beyond the Gram operands, the G / T tiles and the X tiles alike: the per-head
+  // tables live there for the whole kernel (D_QK and its reciprocal, 128 floats each; the chunk's last decay row)
+  static_assert(2 * 64 * kOP + 384 <= 64 * kGS + 64 * LS && 2 * 64 * kGS + 384 <= 64 * kGS + 64 * LS &&
+                3 * kXT + 384 <= 64 * kGS + 64 * LS, "table space behind every overlay");
+  float* dk_s = lds_f + 64 * kGS + 64 * LS - 384;
+  float* glast_s = dk_s + 256;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -279,6 +310,10 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   const float sigma = p.sigma, tau = p.tau;
   constexpr bool bf = BF;
 
+  if (DK && tid < K) {
+    dk_s[tid] = p.dk_div[blockIdx.y % p.H * K + tid];
+    dk_s[128 + tid] = p.dk_rcp[blockIdx.y % p.H * K + tid];
+  }
   // ---- per-token factors; fw is written straight out
   if (tid < 64) {
     const float bt = p.beta[(t0 + tid) * H + h];
@@ -303,7 +338,7 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
         gm = zoo_exp(gl);
       }
       p.gam[(((int64_t)b * p.NT + ct) * H + h) * K + tid] = gm;
-      glast_s[tid] = gl;
+      if (DECAY == LQ_DECAY_DIAGONAL) glast_s[tid] = gl;
       iskw_s[tid] = 1.0f / p.skw[h * K + tid];
     }
     if (tid >= 128 && tid < 192) {
@@ -346,6 +381,7 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
         const int64_t off = ((t0 + r) * H + h) * K + 64 * ps + 8 * c8;
         float kv[8];
         zoo_ld8(p.k + off, bf, kv);
+        wy_dk8<BF, DK>(dk_s, 64 * ps + 8 * c8, kv);
         const float bs = bs_s[r], bh = bh_s[r];
         lq_v4f l0, l1, h0, h1;
         lq_v4f g0 = {0.f, 0.f, 0.f, 0.f}, g1 = g0;
@@ -459,7 +495,7 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
         }
       }
     } else {
-      gram_rowblock<DECAY, K, BF>(p, G_s, bs_s, bh_s, gs_s, wave, rl, kg, t0, h);
+      gram_rowblock<DECAY, K, BF, DK>(p, G_s, bs_s, bh_s, gs_s, wave, rl, kg, t0, h, dk_s);
     }
   }
   __syncthreads();
@@ -554,6 +590,44 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   for (int kc = 0; kc < K; kc += 64) {
     if (kc > 0) __syncthreads();
     if (!kAhead) request_k(kc);
+    if constexpr (CODES) {
+      // Hw and its codes were written while the Gram operands were staged: only X is formed here, two channels at a time
+      // for both tokens of the thread (a token pair is one dword of the transposed tile), so that few values are live
+      float bl[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        bl[u] = bs_s[2 * rp + u];
+        if (DECAY == LQ_DECAY_SCALAR) bl[u] = bl[u] * zoo_exp(gs_s[2 * rp + u]);
+      }
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        float x[2][2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          float k0, k1;
+          zoo_dec2((uint32_t)kraw[u][d], bf, k0, k1);
+          if constexpr (DK) {
+            const int n = kc + 8 * c8 + 2 * d;
+            const wy_v2f dd = *(const wy_v2f*)(dk_s + n), rr = *(const wy_v2f*)(dk_s + 128 + n);
+            k0 = zoo_round_act(zoo_div_rn(k0, dd[0], rr[0]), BF);
+            k1 = zoo_round_act(zoo_div_rn(k1, dd[1], rr[1]), BF);
+          }
+          float x0 = bl[u] * k0, x1 = bl[u] * k1;
+          if (DECAY == LQ_DECAY_DIAGONAL) {
+            x0 = x0 * zoo_exp(graw[u][d >> 1][(2 * d) & 3]);
+            x1 = x1 * zoo_exp(graw[u][d >> 1][(2 * d + 1) & 3]);
+          }
+          x[u][0] = x0, x[u][1] = x1;
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          uint32_t hi, mid, lo;
+          split3(x[0][j], x[1][j], hi, mid, lo);
+          const int at = xt_index(8 * c8 + 2 * d + j, rp);
+          Xt[at] = hi, Xt[kXT + at] = mid, Xt[2 * kXT + at] = lo;
+        }
+      }
+    } else
     {
       float xr[2][8];
 #pragma unroll
@@ -562,11 +636,12 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
         const float bw = powb(btr[u], (1.0f - sigma) * tau);
         float bl = bs_s[2 * rp + u];
         if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(gs_s[2 * rp + u]);
-        float hw[8];
+        float hw[8], kk[8];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) zoo_dec2((uint32_t)kraw[u][d], bf, kk[2 * d], kk[2 * d + 1]);
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          float k0, k1;
-          zoo_dec2((uint32_t)kraw[u][d], bf, k0, k1);
+          const float k0 = kk[2 * d], k1 = kk[2 * d + 1];
           float x0 = bl * k0, x1 = bl * k1;
           if (DECAY == LQ_DECAY_DIAGONAL) {
             x0 = x0 * zoo_exp(graw[u][d >> 1][(2 * d) & 3]);
@@ -575,12 +650,10 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
           xr[u][2 * d] = x0, xr[u][2 * d + 1] = x1;
           hw[2 * d] = bw * k0, hw[2 * d + 1] = bw * k1;
         }
-        if constexpr (!CODES) {  // with CODES, Hw and its codes were written while the Gram operands were staged
-          lq_v4i o;
+        lq_v4i o;
 #pragma unroll
-          for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
-          *(lq_v4i*)(p.Hw + off) = o;
-        }
+        for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+        *(lq_v4i*)(p.Hw + off) = o;
       }
       stage(xr[0], xr[1]);
     }
@@ -644,18 +717,19 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   }
 }
 
-template <int DECAY, int K, bool CODES>
+template <int DECAY, int K, bool CODES, bool DK>
 int launch_c(const WyParams& p, dim3 grid, hipStream_t stream) {
   if (p.bf)
-    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, true, CODES>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, true, CODES, DK>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, false, CODES>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_wy_prep_kernel<DECAY, K, false, CODES, DK>), grid, dim3(256), 0, stream, p);
   return lq_check_launch();
 }
 
 template <int DECAY, int K>
 int launch(const WyParams& p, dim3 grid, hipStream_t stream) {
-  return p.kqT ? launch_c<DECAY, K, true>(p, grid, stream) : launch_c<DECAY, K, false>(p, grid, stream);
+  if (p.dk_div) return launch_c<DECAY, K, true, true>(p, grid, stream);  // the rescaling comes with the codes (checked)
+  return p.kqT ? launch_c<DECAY, K, true, false>(p, grid, stream) : launch_c<DECAY, K, false, false>(p, grid, stream);
 }
 
 template <int K>
@@ -679,6 +753,9 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   if (codes && a->decay == LQ_DECAY_DIAGONAL && !a->logenv) return LQ_ERR_NULL;
   if (codes && (a->qmax < 1 || a->qmax > 127)) return LQ_ERR_SHAPE;
   if (codes && (!zoo_al(a->kqT, 16) || !zoo_al(a->wq, 4) || !zoo_al(a->skw, 16))) return LQ_ERR_SHAPE;
+  if ((a->dk_div != nullptr) != (a->dk_rcp != nullptr)) return LQ_ERR_NULL;
+  if (a->dk_div && !codes) return LQ_ERR_SHAPE;  // built for the launch that also makes the write operands
+  if (a->dk_div && (!zoo_al(a->dk_div, 16) || !zoo_al(a->dk_rcp, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
   if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
@@ -692,6 +769,7 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim;
   p.kqT = a->kqT, p.wq = a->wq, p.ev = a->ev, p.gam = a->gam, p.logenv = a->logenv, p.skw = a->skw, p.sw = a->sw;
   p.eta = a->eta, p.qmax = a->qmax, p.NT = a->seqlen / 64;
+  p.dk_div = a->dk_div, p.dk_rcp = a->dk_rcp;
   dim3 grid(a->seqlen / 64, a->batch * a->nheads);
   return a->kdim == 128 ? launch_decay<128>(p, a->decay, grid, stream) : launch_decay<64>(p, a->decay, grid, stream);
 }

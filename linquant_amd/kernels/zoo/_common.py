@@ -165,23 +165,35 @@ def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims,
               batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(value))
 
 
-def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None):
-    """Returns (A fp16 (B,T,H,64), qg int8 (B,T,H,K)): the intra-chunk product and the codes of q*exp(g)*scale."""
+def dqk_tables(dqk, H, K):
+    """(D, RN(1 / D)) as aligned fp32 (H,K) tables for the kernels that apply D_QK while they load q / k (None, None
+    without one)."""
+    if dqk is None:
+        return None, None
+    d = _lib.aligned(f32(dqk))
+    assert tuple(d.shape) == (H, K), f"dqk: (H, K) = ({H}, {K}) positive factors"
+    return d, _lib.aligned((1.0 / d).contiguous())
+
+
+def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None, dq=None):
+    """Returns (A fp16 (B,T,H,64), qg int8 (B,T,H,K)): the intra-chunk product and the codes of q*exp(g)*scale.
+    ``dq`` (H,K): q is multiplied by it (and rounded to the activation dtype) as it is loaded."""
     B, T, H, K, _ = dims
     A = torch.empty(B, T, H, CHUNK, dtype=torch.float16, device=q.device)
     qg = torch.empty(B, T, H, K, dtype=torch.int8, device=q.device)
     assert rot is None or tuple(rot.shape) == (K, K), "rot: (K, K) R_QK"
     _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), qg=_lib.ptr(qg), rot=_lib.ptr(rot),
               sq=_lib.ptr(sq), sk=_lib.ptr(sk), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K,
-              chunk_size=CHUNK, act_dtype=act_code(q))
+              chunk_size=CHUNK, act_dtype=act_code(q), dq=_lib.ptr(dq))
     return A, qg
 
 
-def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True):
+def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True, dk=(None, None)):
     """Returns (Hw, W, U, fw, codes): operands of the delta state kernel in the activation dtype and the value-side share
     of beta.  ``write`` = dict(logenv, skw, sw, eta, qmax): the launch also makes the state kernel's write-operand codes
     (what ``write_codes`` would make from the stored Hw and W, same bits) and returns them as ``codes``; W itself is
-    then stored only when ``keep_W``."""
+    then stored only when ``keep_W``.  ``dk`` = (D, 1 / D) from ``dqk_tables``: k is divided by D (and rounded to the
+    activation dtype) as it is loaded; needs ``write``."""
     B, T, H, K, V = dims
     dev, NT = k.device, T // CHUNK
     Hw = torch.empty_like(k)
@@ -200,7 +212,8 @@ def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True
                      qmax=int(write["qmax"]))
     _lib.call("lq_zoo_wy_prep", dev, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
               Hw=_lib.ptr(Hw), W=_lib.ptr(W), U=_lib.ptr(U), fw=_lib.ptr(fw), sigma=float(sigma), tau=float(tau),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(k), **extra)
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(k),
+              dk_div=_lib.ptr(dk[0]), dk_rcp=_lib.ptr(dk[1]), **extra)
     return Hw, W, U, fw, c
 
 

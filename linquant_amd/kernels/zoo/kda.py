@@ -13,10 +13,19 @@ from .gla import BC
 
 
 def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, scale=None, chunk_size=64,
-                   output_final_state=False, unrot=None, rot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
+                   output_final_state=False, unrot=None, rot=None, fla_prep=True, bits=8, out_dtype=None, dqk=None,
+                   _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay, beta [B,T,H].
-    scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
+    scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None).
+    ``dqk`` (H,K) fp32, not in the reference's signature: the diagonal rescaling D_QK of linquant/harness.py:68-88
+    (q' = q D, k' = k / D, rounded to the activation dtype) applied inside the kernels as they load q and k, with the
+    result of calling ``rotate_qkv(q, k, None, dqk=dqk)`` first, bit for bit, and without that launch."""
     assert g.shape == q.shape
+    if dqk is not None and q.shape[-1] not in (64, 128):
+        # widths the kernels widen with zero channels: rescale up front (same roundings: one fp32 product, one quotient)
+        d = dqk.to(q.device)
+        q, k = (q.float() * d.float()).to(q.dtype), (k.double() / d.double()).float().to(k.dtype)
+        dqk = None
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
@@ -30,10 +39,11 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     gc, logenv = C.cumsum(g, B, T, H, K)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
     # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
+    dq, dq_rcp = C.dqk_tables(dqk, H, K)
     Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL,
                                         write=dict(logenv=logenv, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
-                                        keep_W=_debug is not None)
-    A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R)
+                                        keep_W=_debug is not None, dk=(dq, dq_rcp))
+    A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R, dq=dq)
     NT = T // chunk_size
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)

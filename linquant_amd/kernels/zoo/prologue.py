@@ -29,8 +29,8 @@ def rotation_signs(R: torch.Tensor) -> torch.Tensor:
 
 def rotate_qkv(q=None, k=None, v=None, *, signs_qk=None, signs_v=None, dqk=None, out=None):
     """q, k [B,T,H,K], v [B,T,H,V] fp16 / bf16 (any may be None).  ``signs_qk`` (K,), ``signs_v`` (V,): +-1 column signs
-    of R_QK / R_V (``rotation_signs``), None = that rotation is left out.  ``dqk`` (H,K) fp32: q is multiplied by it and
-    k divided (the reciprocal is formed once, in fp32).  Returns the tuple (q', k', v') of new tensors (None where the
+    of R_QK / R_V (``rotation_signs``), None = that rotation is left out.  ``dqk`` (H,K) fp32, finite and positive: q is
+    multiplied by it and k divided (the quotient rounded once, as the division of linquant/harness.py:86 rounds it).  Returns the tuple (q', k', v') of new tensors (None where the
     input was None); ``out=(q_out, k_out, v_out)`` supplies the destinations (an input itself for in-place)."""
     ref = next(t for t in (q, k, v) if t is not None)
     B, T, H = ref.shape[:3]

@@ -165,15 +165,15 @@ def signed_hadamard(n, seed, device=None):
 def rotate_operands(q, k, v, rot_qk=None, rot_v=None, dqk=None):
     """The operand prologue in front of a kernel call: q' = mat((q D) @ R_QK), k' = mat((k / D) @ R_QK),
     v' = mat(v @ R_V) with mat = float64 -> fp32 -> activation dtype (linquant/reference.py:40-46; D_QK as
-    linquant/harness.py:84-87 applies it, the reciprocal formed in fp32 as the kernels receive it).  Any of rot_qk,
-    rot_v, dqk (H,K) may be None.  Returns tensors in the inputs' dtype."""
+    linquant/harness.py:84-87 applies it: a float64 product for q, a float64 division for k).  Any of rot_qk, rot_v,
+    dqk (H,K) may be None.  Returns tensors in the inputs' dtype."""
     def mat(t, like):
         return t.float().to(like.dtype)
 
     qq, kk = q.double(), k.double()
     if dqk is not None:
-        d = dqk.float()
-        qq, kk = qq * d.double()[None, None], kk * (1.0 / d).double()[None, None]
+        d = dqk.double()
+        qq, kk = qq * d[None, None], kk / d[None, None]
     if rot_qk is not None:
         qq, kk = qq @ rot_qk.double(), kk @ rot_qk.double()
     vv = v.double() if rot_v is None else v.double() @ rot_v.double()

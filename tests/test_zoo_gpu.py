@@ -488,6 +488,38 @@ def test_wy_prep_also_makes_the_write_codes(cuda, cell, K, dtype, eta, bits):
     assert int(ref["kqT"].abs().max()) > qmax // 2 and int(ref["wq"].abs().max()) > 0  # the comparison is not vacuous
 
 
+@pytest.mark.parametrize("K,dtype,rot", [(128, torch.float16, True), (64, torch.float16, False), (128, torch.bfloat16, False),
+                                         (48, torch.float16, False)])
+def test_kda_applies_dqk_inside_its_kernels(cuda, K, dtype, rot):
+    """chunk_kda_int8(..., dqk=D) gives, bit for bit, what the stand-alone rescaling launch followed by the plain call
+    gives: outputs, final state, stored state codes, Hw / U, the A tile and the decayed-query codes."""
+    from linquant_amd.kernels import zoo
+    from oracle import zoo_reference as Z
+
+    q, k, v, g, beta = zc.cut(zc.inputs("kda", B=2, H=3, K=K, V=64, seed=31, dtype=dtype), 192)
+    gen = torch.Generator().manual_seed(4)
+    D = (torch.rand(3, K, generator=gen) * 1.5 + 0.25)
+    R = Z.signed_hadamard(K, 2).float() if rot else None
+    sc = {"q": torch.full((3,), 0.004), "k": torch.full((3,), 0.02), "w": torch.full((3,), 0.03),
+          "kw": torch.rand(3, K, generator=gen) * 0.01 + 0.005, "el": torch.full((3, 64), 0.05),
+          "ew": torch.full((3, 64), 0.05), "state": torch.full((3, 64), 0.02)}
+    sc = {n: t.to(cuda) for n, t in sc.items()}
+    dev = lambda t: t.to(cuda)  # noqa: E731
+    kw = dict(sigma=0.5, tau=0.5, eta=0.25, rot=None if R is None else dev(R), output_final_state=True)
+    if K in (64, 128):
+        qd, kd, _ = zoo.rotate_qkv(dev(q), dev(k), None, dqk=dev(D))
+    else:  # a width the rescaling launch is not built for: the oracle's form of it
+        qd, kd = (dev(t) for t in Z.rotate_operands(q, k, v, None, None, D)[:2])
+    d0, d1 = {}, {}
+    o0, h0 = zoo.chunk_kda_int8(qd, kd, dev(v), dev(g), dev(beta), sc, _debug=d0, **kw)
+    o1, h1 = zoo.chunk_kda_int8(dev(q), dev(k), dev(v), dev(g), dev(beta), sc, dqk=dev(D), _debug=d1, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(o0, o1) and torch.equal(h0, h1)
+    for name in ("h_i8", "Hw", "U", "W", "A", "qg", "kq", "wq", "e_out"):
+        assert torch.equal(d0[name], d1[name]), name
+    assert float(o0.float().abs().max()) > 0
+
+
 def test_reference_mamba2_cell_config(cuda):
     """The benchmark's first configuration (the CPU-runnable one): the Mamba-2 cell through chunk_simple_gla (q = C, k = B broadcast to heads, v = x*dt,
     g = dt*A, scale = 1), B1 T2048 H8 K = V = 64, per-head / per-channel static scales."""

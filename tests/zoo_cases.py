@@ -57,9 +57,12 @@ def config_inputs(name, seed, K=128, V=128, heads=None, batch_row=None):
 
 
 def apply_dqk(tensors, D):
-    """q' = fp16(q * D), k' = fp16(k / D) with D (H, K) fp32: products formed in fp32, rounded once to fp16."""
+    """q' = fp16(q * D), k' = fp16(k / D) with D (H, K) fp32: the oracle's operand prologue without a rotation."""
+    from oracle import zoo_reference as Z
+
     q, k, v, g, beta = tensors
-    return ((q.float() * D[None, None]).half(), (k.float() * (1.0 / D)[None, None]).half(), v, g, beta)
+    qd, kd, _ = Z.rotate_operands(q, k, v, None, None, D)
+    return (qd, kd, v, g, beta)
 
 
 def cut(tensors, n):
