@@ -223,7 +223,10 @@ def measure_zoo(args, workload, cpu_baseline):
     if workload == "c4_kda":
         cq, ck, *_ = zoo_synthetic(cell, 1, 2048, H, K, V, seed=1)
         dqk = dqk_from_absmax(cq.half().float(), ck.half().float(), 0.5).to(dev)
-    has_prologue = persistent  # D_QK is applied inside the KDA kernels as they load q and k: no launch of its own
+    # linear family: the rotation is part of the call's own operand launch (prologue=...); delta family: a launch of its own.
+    # D_QK is applied inside the KDA kernels as they load q and k
+    fused = persistent and fam == "linear"
+    has_prologue = persistent and not fused
     qr, kr = (torch.empty_like(q0), torch.empty_like(k0)) if has_prologue else (None, None)
 
     def prologue():
@@ -241,7 +244,8 @@ def measure_zoo(args, workload, cpu_baseline):
         if fam == "linear" and dec == "diagonal":
             return zoo.chunk_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, rot=rot, **kw)
         if fam == "linear":
-            return zoo.chunk_simple_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, **kw)
+            return zoo.chunk_simple_gla_int8(q, k, v, g, sc, eta=eta, scale=scale,
+                                             prologue=dict(signs_qk=sq) if fused else None, **kw)
         if dec == "diagonal":
             return zoo.chunk_kda_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, rot=rot, dqk=dqk, **kw)
         return zoo.chunk_delta_int8(q, k, v, g, beta, sc, sigma=sigma, eta=eta, scale=scale, **kw)
@@ -254,7 +258,8 @@ def measure_zoo(args, workload, cpu_baseline):
     # pilot run of the kernels themselves with a coarse state grid
     ph = lambda t: (t.float().abs().amax(dim=(0, 1, 3)) / 127).clamp_min(1e-6)  # noqa: E731
     pc = lambda t: (t.float().abs().amax(dim=(0, 1)) / 127).clamp_min(1e-6)  # noqa: E731
-    qs, ks = (q, k) if dqk is None else zoo.rotate_qkv(q0, k0, None, dqk=dqk)[:2]  # the operands the kernels will see
+    # the operands the kernels will see (for the scales only)
+    qs, ks = zoo.rotate_qkv(q0, k0, None, signs_qk=sq if fused else None, dqk=dqk)[:2] if (dqk is not None or fused) else (q, k)
     sc = {"q": ph(qs) * scale, "k": ph(ks), "w": ph(ks) * 2, "kw": pc(ks), "vw": pc(v), "vl": pc(v),
           "el": pc(v) * 2, "ew": pc(v) * 2, "state": torch.full((H, V), 1.0, device=dev)}
     sc = {n: t.contiguous() for n, t in sc.items()}
@@ -282,7 +287,7 @@ def measure_zoo(args, workload, cpu_baseline):
 
     records = {}
     names = {"cumsum": "cumsum", "run_wy_prep": "wy_prep", "run_gla_A": "gla_A", "write_codes": "write_codes",
-             "state_kernel": "state", "run_output": "output"}
+             "rotate_quant": "rotate_quant", "state_kernel": "state", "run_output": "output"}
     saved = {n: getattr(C, n) for n in names}
 
     def timed(fn, label):
@@ -309,6 +314,11 @@ def measure_zoo(args, workload, cpu_baseline):
             setattr(C, n, f)
     nbytes = zoo_stage_bytes(fam, dec, B, T, H, K, V)
     nbytes["prologue"] = 2 * (B * T * H * K * 2) * 2  # q and k, read and written once
+    if fused:  # q, k, v read once; five code tensors written; the output kernel reads codes
+        qk_b, vv_b = B * T * H * K * 2, B * T * H * V * 2
+        nbytes["rotate_quant"] = 2 * qk_b + vv_b + 3 * (qk_b // 2) + 2 * (vv_b // 2)
+        nbytes["output"] = 2 * (qk_b // 2) + vv_b // 2 + B * (T // 64) * H * K * V + vv_b
+        nbytes.pop("write_codes", None)
     del qs, ks
     stages = {}
     for label, evs in records.items():
@@ -360,6 +370,7 @@ def measure_zoo(args, workload, cpu_baseline):
         "config": {"workload": f"{workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
                    "tokens_per_step": tokens, "ramp": ramp_note(ramp_steps),
                    "prologue": "in the timed step: R_QK on q, k" if has_prologue else
+                               "R_QK on q, k inside the call's operand launch (rotate + quantize in one)" if fused else
                                ("none (local R_QK inside the A kernel" +
                                 ("; D_QK (alpha 0.5) applied inside the WY prep and A kernels as they load k and q)"
                                  if dqk is not None else ")")) if rot is not None else "none"},

@@ -399,6 +399,11 @@ typedef struct {
   int32_t batch, seqlen, nheads, kdim, vdim, chunk_size;
   int32_t decay;
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
+  /* Optional (no / scalar decay, rotated storage): the local codes of q, k and v ready-made by lq_zoo_rotate_quant;
+   * q, k, v are then not read (may be NULL) and nothing is quantized here. */
+  const int8_t* qc;          /* (B,T,H,K) int8 q8(q*scale, 1/sq) */
+  const int8_t* kc;          /* (B,T,H,K) int8 q8(k, 1/sk) */
+  const int8_t* vc;          /* (B,T,H,V) int8 q8(v, 1/svl) */
 } lq_zoo_output_args;
 int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
 
@@ -486,6 +491,43 @@ typedef struct {
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16 */
 } lq_zoo_rotate_qkv_args;
 int lq_zoo_rotate_qkv(const lq_zoo_rotate_qkv_args* args, hipStream_t stream);
+
+/* replaces, for the linear family under no / scalar decay, the same operand prologue (bench/zoo_kernels.py:135-140, "not
+ * fused yet"; linquant/harness.py:68-88) TOGETHER WITH the operand quantization it feeds: the write-operand preparation
+ * inside _state_body (linquant/kernels/zoo/simple_gla.py:55-66) and the code loop at the top of _output_body
+ * (simple_gla.py:125-140).  One launch reads q, k, v once and emits every INT8 operand of lq_zoo_state and lq_zoo_output;
+ * each code equals what lq_zoo_rotate_qkv -> lq_zoo_write_codes / lq_zoo_output would have made from the rotated
+ * activations stored in between (same arithmetic on the same rounded values).  q_out / k_out / v_out are optional. */
+typedef struct {
+  const void* q;             /* (B,T,H,K) fp16/bf16 contiguous */
+  const void* k;             /* (B,T,H,K) */
+  const void* v;             /* (B,T,H,V) */
+  void* q_out;               /* rotated / rescaled activations, same shape and dtype; NULL: not stored */
+  void* k_out;
+  void* v_out;
+  int8_t* qc;                /* (B,T,H,K) local codes q8(q'*scale, 1/sq) */
+  int8_t* kc;                /* (B,T,H,K) local codes q8(k', 1/sk) */
+  int8_t* vc;                /* (B,T,H,V) local codes q8(v', 1/svl) */
+  int8_t* kqT;               /* (B,NT,H,K,C) key write codes q8(k'*fk, 1/skw), channel-major inside the chunk */
+  int8_t* vqT;               /* (B,NT,H,V,C) value write codes q8(v'*fv, 1/svw) */
+  float* ev;                 /* (B,T,H) per-token value factor fv */
+  float* gam;                /* (B,NT,H,K) chunk decay */
+  const float* dq;           /* (H,K) D_QK or NULL (see lq_zoo_rotate_qkv) */
+  const float* dk;           /* (H,K) RN(1 / dq), set exactly when k is to be rescaled, or NULL */
+  const float* signs_qk;     /* (K,) +-1 column signs of R_QK, or NULL */
+  const float* signs_v;      /* (V,) +-1 column signs of R_V, or NULL */
+  const float* g;            /* (B,T,H) chunk-local cumulative log decay (scalar decay), or NULL */
+  const float* sq;           /* (H,) */
+  const float* sk;           /* (H,) */
+  const float* svl;          /* (H,V) */
+  const float* skw;          /* (H,K) */
+  const float* svw;          /* (H,V) */
+  float eta, scale;
+  int32_t qmax;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size; /* kdim, vdim in {64, 128}; chunk 64 */
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16 */
+} lq_zoo_rotate_quant_args;
+int lq_zoo_rotate_quant(const lq_zoo_rotate_quant_args* args, hipStream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Element-wise stages in front of the Mamba-2 SSD prologue.

@@ -34,6 +34,7 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_zoo_gla_A_args);
   LQ_SIZE_OF(lq_zoo_wy_prep_args);
   LQ_SIZE_OF(lq_zoo_rotate_qkv_args);
+  LQ_SIZE_OF(lq_zoo_rotate_quant_args);
   LQ_SIZE_OF(lq_ssd_combined_args);
   LQ_SIZE_OF(lq_probe_mfma_args);
   return LQ_ERR_SHAPE;

@@ -81,6 +81,14 @@ LQ_DEV uint16_t zoo_enc1(float a, bool bf) {
 // x rounded to the activation dtype and back: what a consumer reads when a producer stored x there
 LQ_DEV float zoo_round_act(float x, bool bf) { return zoo_dec1((uint32_t)zoo_enc1(x, bf), bf); }
 
+// a * b as an fp32 value of its own: a conversion to half precision that follows is a second rounding (left to the
+// compiler, it is folded into the multiply: one rounding of the exact product)
+LQ_DEV float zoo_mul_rn(float a, float b) {
+  float p = a * b;
+  asm volatile("" : "+v"(p));
+  return p;
+}
+
 // x / d rounded once to fp32 (the IEEE quotient) from r = RN(1 / d): q0 = RN(x r), rem = x - q0 d (exact in the fused
 // multiply-add), q = RN(q0 + rem r).  Correct for finite d > 0 and half-precision x (checked over every fp16 and bf16
 // value on the CPU); three instructions instead of the division sequence.
@@ -92,4 +100,46 @@ LQ_DEV float zoo_div_rn(float x, float d, float r) {
   // conversion to half precision into the multiply-add (one rounding instead of two)
   asm volatile("" : "+v"(q));
   return q;
+}
+
+// ---- fast Walsh-Hadamard transform of a row spread over LPR adjacent lanes (LPR = 8 or 16, rows aligned to LPR lanes),
+// eight adjacent channels per lane: butterflies 1, 2, 4 inside the lane, then across lanes l ^ 1, l ^ 2, l ^ 4 (, l ^ 8)
+// through DPP lane permutations (no LDS traffic).  fp32 sums in a fixed order: y = sum_i x_i H_ij, unnormalized.
+template <int M>
+LQ_DEV float zoo_lane_xor(float v) {
+  int x = __float_as_int(v);
+  // every lane has a source, so nothing depends on the "old" operand
+  if constexpr (M == 1) x = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+  if constexpr (M == 2) x = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+  if constexpr (M == 4) {  // l ^ 7 (mirror of each half row) followed by l ^ 3 (mirror of each quad)
+    x = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xf, 0xf, true);  // row_half_mirror
+    x = __builtin_amdgcn_update_dpp(x, x, 0x1B, 0xf, 0xf, true);   // quad_perm [3,2,1,0]
+  }
+  if constexpr (M == 8) x = __builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, true);  // row_ror:8
+  return __int_as_float(x);
+}
+
+template <int M>
+LQ_DEV void zoo_fwht_stage(float (&v)[8], int sub) {
+  // lanes whose bit M is set hold the difference o - v = (-v) + o, the others the sum v + o
+  const uint32_t neg = (sub & M) ? 0x80000000u : 0u;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = __uint_as_float(__float_as_uint(v[e]) ^ neg) + zoo_lane_xor<M>(v[e]);
+}
+
+template <int LPR>
+LQ_DEV void zoo_fwht(float (&v)[8], int sub) {
+#pragma unroll
+  for (int h2 = 1; h2 < 8; h2 <<= 1)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if ((e & h2) == 0) {
+        const float a = v[e], c = v[e + h2];
+        v[e] = a + c;
+        v[e + h2] = a - c;
+      }
+  zoo_fwht_stage<1>(v, sub);
+  zoo_fwht_stage<2>(v, sub);
+  zoo_fwht_stage<4>(v, sub);
+  if constexpr (LPR == 16) zoo_fwht_stage<8>(v, sub);
 }

@@ -62,7 +62,7 @@ LQ_DEV void diag_exact(const AParams& p, float sq, float sk, float inv_sq, float
     zoo_ld8(p.q + irow + n8, bf, qv);
     if (p.dq) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qv[e] = zoo_round_act(qv[e] * p.dq[h * K + n8 + e], bf);
+      for (int e = 0; e < 8; ++e) qv[e] = zoo_round_act(zoo_mul_rn(qv[e], p.dq[h * K + n8 + e]), bf);
     }
     const lq_v4f gi0 = *(const lq_v4f*)(p.g + irow + n8), gi1 = *(const lq_v4f*)(p.g + irow + n8 + 4);
 #pragma unroll
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
       if constexpr (DQ) {  // D_QK at load: q' = act(q * D), what the stand-alone rescaling launch would have stored
         const lq_v4f d0 = *(const lq_v4f*)(DQs + 32 * ks + 8 * kg), d1 = *(const lq_v4f*)(DQs + 32 * ks + 8 * kg + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qf[e] = zoo_round_act(qf[e] * (e < 4 ? d0[e & 3] : d1[e & 3]), bf);
+        for (int e = 0; e < 8; ++e) qf[e] = zoo_round_act(zoo_mul_rn(qf[e], e < 4 ? d0[e & 3] : d1[e & 3]), bf);
       }
       int cs[8], iq[8], ik[8];
 #pragma unroll

@@ -27,7 +27,9 @@ using OutParams = ZooOutParams;
 
 // NV: 64-column V tiles per workgroup (2 when V is a multiple of 128: the q / k codes and the A tile are then made once
 // for both tiles)
-template <bool GLA, bool USE_G, int K, bool BF, int NV>
+// CIN: the local codes of q, k, v arrive ready-made (lq_zoo_rotate_quant made them): they are copied into the same LDS
+// tiles instead of being quantized here.
+template <bool GLA, bool USE_G, int K, bool BF, int NV, bool CIN>
 __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   constexpr int QS = K + 16;  // byte stride of a code row
   __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   // iteration of the code loop, one for v, one per contraction step of the state read, one per scale vector.)
   constexpr int NQ = K / 32;  // 16-byte pieces of q (and of k) per thread: 64 tokens x K / 8 pieces over 256 threads
   lq_v4i qraw[GLA ? 1 : NQ], kraw[GLA ? 1 : NQ];
-  if constexpr (!GLA) {
+  if constexpr (!GLA && !CIN) {
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
       const int it = tid + 256 * i;
@@ -77,14 +79,29 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       kraw[i] = *(const lq_v4i*)(p.k + off);
     }
   }
+  if constexpr (!GLA && CIN) {  // 16 codes per piece: half as many pieces
+#pragma unroll
+    for (int i = 0; i < NQ / 2; ++i) {
+      const int it = tid + 256 * i;
+      const int t = it / (K / 16), c16 = it % (K / 16);
+      const int64_t off = ((t0 + t) * H + h) * K + 16 * c16;
+      qraw[i] = *(const lq_v4i*)(p.qc + off);
+      kraw[i] = *(const lq_v4i*)(p.kc + off);
+    }
+  }
   const int tp = tid >> 3, c8v = tid & 7;  // value tile: 32 token pairs x 8 groups of 8 channels
   const int64_t voff = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8v;
   lq_v4i va_raw[NV], vb_raw[NV];
   lq_v4f sv0[NV], sv1[NV];
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
-    va_raw[n] = *(const lq_v4i*)(p.v + voff + BV * n), vb_raw[n] = *(const lq_v4i*)(p.v + voff + BV * n + (int64_t)H * V);
-    sv0[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 8 * c8v), sv1[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 8 * c8v + 4);
+    if constexpr (CIN) {  // eight codes per token: the low two dwords of the raw registers
+      const lq_v2i ca = *(const lq_v2i*)(p.vc + voff + BV * n), cb2 = *(const lq_v2i*)(p.vc + voff + BV * n + (int64_t)H * V);
+      va_raw[n] = lq_v4i{ca[0], ca[1], 0, 0}, vb_raw[n] = lq_v4i{cb2[0], cb2[1], 0, 0};
+    } else {
+      va_raw[n] = *(const lq_v4i*)(p.v + voff + BV * n), vb_raw[n] = *(const lq_v4i*)(p.v + voff + BV * n + (int64_t)H * V);
+      sv0[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 8 * c8v), sv1[n] = *(const lq_v4f*)(p.svl + h * V + v0 + BV * n + 8 * c8v + 4);
+    }
   }
   const float g_raw = (USE_G && !GLA) ? p.g[(t0 + (tid & 63)) * H + h] : 0.0f;
   const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
@@ -106,7 +123,16 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
 
   // ---- phase 1: q (and k) codes -> LDS, value codes -> LDS (fp16, token-pair interleaved)
-  if constexpr (!GLA) {
+  if constexpr (!GLA && CIN) {
+#pragma unroll
+    for (int i = 0; i < NQ / 2; ++i) {
+      const int it = tid + 256 * i;
+      const int t = it / (K / 16), c16 = it % (K / 16);
+      *(lq_v4i*)(qc + t * QS + 16 * c16) = qraw[i];
+      *(lq_v4i*)(kc + t * QS + 16 * c16) = kraw[i];
+    }
+  }
+  if constexpr (!GLA && !CIN) {
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
       const int it = tid + 256 * i;
@@ -133,6 +159,14 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
 #pragma unroll
   for (int n = 0; n < NV; ++n) {
     lq_v4i o0, o1;
+    if constexpr (CIN) {  // codes -> exact fp16, token pair per dword
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int ca = lq_sbyte((uint32_t)va_raw[n][e >> 2], e & 3), cb2 = lq_sbyte((uint32_t)vb_raw[n][e >> 2], e & 3);
+        const int w = (int)zoo_pack_h2((float)ca, (float)cb2);
+        if (e < 4) o0[e] = w; else o1[e - 4] = w;
+      }
+    } else {
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       float a0, a1, b0, b1;
@@ -143,6 +177,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       const int w0 = (int)zoo_pack_h2((float)zoo_q8(a0, i0, qmax), (float)zoo_q8(b0, i0, qmax));
       const int w1 = (int)zoo_pack_h2((float)zoo_q8(a1, i1, qmax), (float)zoo_q8(b1, i1, qmax));
       if (d < 2) o0[2 * d] = w0, o0[2 * d + 1] = w1; else o1[2 * d - 4] = w0, o1[2 * d - 3] = w1;
+    }
     }
     *(lq_v4i*)(vP + (32 * n + tp) * kVW + 8 * c8v) = o0;
     *(lq_v4i*)(vP + (32 * n + tp) * kVW + 8 * c8v + 4) = o1;
@@ -262,10 +297,19 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
 
 template <bool GLA, bool USE_G, int K, int NV>
 void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
+  if constexpr (!GLA) {
+    if (p.qc) {  // ready-made codes: the activation dtype only matters for a 16-bit output
+      if (p.bf)
+        hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true, NV, true>), grid, dim3(256), 0, stream, p);
+      else
+        hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false, NV, true>), grid, dim3(256), 0, stream, p);
+      return;
+    }
+  }
   if (p.bf)
-    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true, NV>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true, NV, false>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false, NV>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false, NV, false>), grid, dim3(256), 0, stream, p);
 }
 
 template <bool GLA, bool USE_G>
@@ -289,10 +333,13 @@ int launch(const OutParams& p, int K, hipStream_t stream) {
 }  // namespace
 
 extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
-  if (!a || !a->v || !a->h_i8 || !a->o || !a->sq || !a->svl || !a->ss) return LQ_ERR_NULL;
+  if (!a || !a->h_i8 || !a->o || !a->sq || !a->svl || !a->ss) return LQ_ERR_NULL;
   const bool gla = a->decay == LQ_DECAY_DIAGONAL;
+  const bool cin = a->qc != nullptr;  // ready-made local codes of q, k, v (no / scalar decay, rotated storage)
+  if (cin && (gla || a->unrot || !a->kc || !a->vc || !a->sk)) return LQ_ERR_NULL;
+  if (!cin && !a->v) return LQ_ERR_NULL;
   if (gla && (!a->A || !a->qg)) return LQ_ERR_NULL;
-  if (!gla && (!a->q || !a->k || !a->sk)) return LQ_ERR_NULL;
+  if (!gla && !cin && (!a->q || !a->k || !a->sk)) return LQ_ERR_NULL;
   if (a->decay == LQ_DECAY_SCALAR && !a->g) return LQ_ERR_NULL;
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
@@ -301,8 +348,9 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
-  if ((a->q && !zoo_al(a->q, 16)) || (a->qg && !zoo_al(a->qg, 16)) || (a->A && !zoo_al(a->A, 16)) || (a->k && !zoo_al(a->k, 16)) || !zoo_al(a->v, 16) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16) || !zoo_al(a->ss, 16) || !zoo_al(a->svl, 16))
+  if ((a->q && !zoo_al(a->q, 16)) || (a->qg && !zoo_al(a->qg, 16)) || (a->A && !zoo_al(a->A, 16)) || (a->k && !zoo_al(a->k, 16)) || (a->v && !zoo_al(a->v, 16)) || !zoo_al(a->h_i8, 16) || !zoo_al(a->o, 16) || !zoo_al(a->ss, 16) || !zoo_al(a->svl, 16))
     return LQ_ERR_SHAPE;
+  if (cin && (!zoo_al(a->qc, 16) || !zoo_al(a->kc, 16) || !zoo_al(a->vc, 8))) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535 || a->seqlen / 64 > 65535) return LQ_ERR_SHAPE;
   OutParams p = {};
   p.q = (const _Float16*)a->q, p.k = (const _Float16*)a->k, p.v = (const _Float16*)a->v;
@@ -310,6 +358,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.sq = a->sq, p.sk = a->sk, p.svl = a->svl, p.ss = a->ss, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   p.unrot = (const _Float16*)a->unrot;
+  p.qc = a->qc, p.kc = a->kc, p.vc = a->vc;
   if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
   if (gla) return launch<true, true>(p, a->kdim, stream);
   if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, stream);

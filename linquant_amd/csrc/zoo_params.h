@@ -33,6 +33,9 @@ struct ZooOutParams {
   const float* g;
   const _Float16* A;
   const int8_t* qg;
+  const int8_t* qc;  // ready-made local codes of q, k (B,T,H,K) and v (B,T,H,V): q, k, v are then not read
+  const int8_t* kc;
+  const int8_t* vc;
   void* o;
   int o_is_f32;
   const float* sq;

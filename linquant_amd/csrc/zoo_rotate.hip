@@ -8,7 +8,7 @@
 // R = H_n / sqrt(n) . diag(signs) with the Sylvester H_n (linquant/reference.py:232-239), so a row is rotated by a fast
 // Walsh-Hadamard transform instead of a GEMM: y_j = signs_j / sqrt(n) * sum_i (x_i d_i) H_ij.  HBM-bound byte work:
 // a row of n channels is spread over n / 8 lanes, 16 bytes per lane in and out; butterfly stages 1, 2, 4 run in
-// registers, the rest through wave shuffles.  fp32 sums of at most 128 half-precision values, one multiply, one
+// registers, the rest through DPP lane permutations.  fp32 sums of at most 128 half-precision values, one multiply, one
 // rounding to the activation dtype.
 #include "zoo_common.h"
 #include "../../include/linquant_hip.h"
@@ -81,25 +81,10 @@ __global__ __launch_bounds__(256) void zoo_rotate_kernel(RotParams p) {
       for (int i = 0; i < 8; ++i) v[i] = zoo_div_rn(v[i], i < 4 ? e0[r][i & 3] : e1[r][i & 3], i < 4 ? d0[r][i & 3] : d1[r][i & 3]);
     } else if (diag) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) v[i] = v[i] * (i < 4 ? d0[r][i & 3] : d1[r][i & 3]);
+      for (int i = 0; i < 8; ++i) v[i] = zoo_mul_rn(v[i], i < 4 ? d0[r][i & 3] : d1[r][i & 3]);
     }
     if (signs) {
-#pragma unroll
-      for (int h2 = 1; h2 < 8; h2 <<= 1)
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if ((i & h2) == 0) {
-            const float a = v[i], b = v[i + h2];
-            v[i] = a + b;
-            v[i + h2] = a - b;
-          }
-#pragma unroll
-      for (int m = 1; m < LPR; m <<= 1)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float o = __shfl_xor(v[i], m, 64);
-          v[i] = (sub & m) ? (o - v[i]) : (v[i] + o);
-        }
+      zoo_fwht<LPR>(v, sub);
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = (v[i] * p.rsqrt_n) * (i < 4 ? s0[i & 3] : s1[i & 3]);
     }

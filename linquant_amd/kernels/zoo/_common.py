@@ -154,15 +154,46 @@ def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, fa
     return c
 
 
-def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None, qg=None):
+def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None, qg=None, local=None,
+               act=None):
     """``A`` (fp16) and ``qg`` (INT8 codes of the decayed query) come from run_gla_A under per-channel decay; q and key
-    are only read under no / scalar decay."""
+    are only read under no / scalar decay.  ``local`` = (qc, kc, vc): ready-made local codes from ``rotate_quant`` (q,
+    key and value are then not read; ``act`` names the activation dtype code)."""
     B, T, H, K, V = dims
     svl, ss = _lib.aligned(svl), _lib.aligned(ss)
-    _lib.call("lq_zoo_output", value.device, q=_lib.ptr(q), qg=_lib.ptr(qg), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
+    qc, kc, vc = local if local is not None else (None, None, None)
+    _lib.call("lq_zoo_output", h_i8.device, q=_lib.ptr(q), qg=_lib.ptr(qg), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
               g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
               sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(value))
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay,
+              act_dtype=act if act is not None else act_code(value), qc=_lib.ptr(qc), kc=_lib.ptr(kc), vc=_lib.ptr(vc))
+
+
+def rotate_quant(q, k, v, g, sq, sk, svl, skw, svw, eta, scale, qmax, dims, signs_qk=None, signs_v=None, dqk=None,
+                 keep=False):
+    """The fused operand prologue of the linear family (no / scalar decay): one launch rotates / rescales q, k, v and
+    emits every INT8 operand of the state and output kernels.  Returns (codes for ``state_kernel``, (qc, kc, vc) for
+    ``run_output``, (q', k', v') or None): the rotated activations are stored only when ``keep``."""
+    B, T, H, K, V = dims
+    dev, NT = q.device, T // CHUNK
+    i8 = lambda *shape: torch.empty(*shape, dtype=torch.int8, device=dev)  # noqa: E731
+    c = {"kqT": i8(B, NT, H, K, CHUNK), "vqT": i8(B, NT, H, V, CHUNK), "wq": None,
+         "ev": torch.empty(B, T, H, dtype=torch.float32, device=dev),
+         "gam": torch.empty(B, NT, H, K, dtype=torch.float32, device=dev)}
+    local = (i8(B, T, H, K), i8(B, T, H, K), i8(B, T, H, V))
+    outs = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)) if keep else (None, None, None)
+    dq, dk = dqk_tables(dqk, H, K)
+    al = _lib.aligned
+    sg = lambda t, n: None if t is None else al(f32(t).reshape(n))  # noqa: E731
+    svl, skw, svw = al(svl), al(skw), al(svw)
+    _lib.call("lq_zoo_rotate_quant", dev, q=_lib.ptr(q), k=_lib.ptr(k), v=_lib.ptr(v), q_out=_lib.ptr(outs[0]),
+              k_out=_lib.ptr(outs[1]), v_out=_lib.ptr(outs[2]), qc=_lib.ptr(local[0]), kc=_lib.ptr(local[1]),
+              vc=_lib.ptr(local[2]), kqT=_lib.ptr(c["kqT"]), vqT=_lib.ptr(c["vqT"]), ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]),
+              dq=_lib.ptr(dq), dk=_lib.ptr(dk), signs_qk=_lib.ptr(sg(signs_qk, K)), signs_v=_lib.ptr(sg(signs_v, V)),
+              g=_lib.ptr(g), sq=_lib.ptr(sq), sk=_lib.ptr(sk), svl=_lib.ptr(svl), skw=_lib.ptr(skw), svw=_lib.ptr(svw),
+              eta=float(eta), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K, vdim=V,
+              chunk_size=CHUNK, act_dtype=act_code(q))
+    return c, local, (outs if keep else None)
 
 
 def dqk_tables(dqk, H, K):

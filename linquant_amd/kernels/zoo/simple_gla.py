@@ -13,9 +13,28 @@ from . import _common as C
 
 
 def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size=64, output_final_state=False,
-                          unrot=None, bits=8, out_dtype=None, _debug=None):
+                          unrot=None, bits=8, out_dtype=None, prologue=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None. scales: 'q','k' (H,), 'kw' (H,K),
-    'vw','vl','state' (H,V) fp32. Returns (o [B,T,H,V] in v.dtype or out_dtype, final fp32 state [B,H,K,V] or None)."""
+    'vw','vl','state' (H,V) fp32. Returns (o [B,T,H,V] in v.dtype or out_dtype, final fp32 state [B,H,K,V] or None).
+    ``prologue`` (not in the reference's signature) = dict(signs_qk=, signs_v=, dqk=), each optional: q, k, v arrive as
+    the model produced them, and the persistent rotations R_QK / R_V (``rotation_signs`` of a signed Hadamard matrix) and
+    the D_QK rescaling are applied in the launch that also quantizes the operands: the result of calling
+    ``rotate_qkv(q, k, v, ...)`` first and this function on its outputs, bit for bit, in one launch fewer and without the
+    rotated activations ever reaching memory (K, V in {64, 128}, rotated storage)."""
+    if prologue is not None and (q.shape[-1] not in (64, 128) or v.shape[-1] not in (64, 128) or unrot is not None):
+        from .prologue import rotate_qkv  # shapes the fused launch is not built for: rotate up front
+
+        K, V = q.shape[-1], v.shape[-1]
+        assert (K in (64, 128) or not (prologue.get("signs_qk") is not None or prologue.get("dqk") is not None)) and \
+            (V in (64, 128) or prologue.get("signs_v") is None), "rotations are built for row widths 64 and 128"
+        do_qk, do_v = K in (64, 128), V in (64, 128)
+        rq, rk, rv = rotate_qkv(q.contiguous() if do_qk else None, k.contiguous() if do_qk else None,
+                                v.contiguous() if do_v else None, **prologue)
+        if do_qk:
+            q, k = rq, rk
+        if do_v:
+            v = rv
+        prologue = None
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
@@ -34,6 +53,15 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
+    if prologue is not None:
+        # one launch: rotation / rescaling + every INT8 operand of the two kernels below
+        codes, local, rotated = C.rotate_quant(q, k, v, gg, sc["q"], sc["k"], sc["vl"], sc["kw"], sc["vw"], eta, scale, qmax, dims,
+                                               keep=_debug is not None, **prologue)
+        C.state_kernel(codes, v, None, h_i8, None, ht, sc["kw"], sc["vw"], None, sc["state"], qmax, dims, C.FAMILY_LINEAR)
+        C.run_output(None, None, None, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay,
+                     local=local, act=C.act_code(v))
+        C.export_debug(_debug, h_i8, codes, g=gg, local=local, rotated=rotated)
+        return C.cut_values(o, C.cut_keys(ht, K0), V0)
     codes = C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru)
     C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
     C.export_debug(_debug, h_i8, codes, g=gg)

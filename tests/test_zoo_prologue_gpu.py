@@ -86,3 +86,67 @@ def test_rotate_qkv_rejections(cuda):
         rotate_qkv(q, q, None)
     with pytest.raises(_lib.LinQuantHipError):
         _lib.call("lq_zoo_rotate_qkv", q.device, batch=1, seqlen=1, nheads=1, kdim=64, vdim=64)
+
+
+@pytest.mark.parametrize("cell", ["linear_none", "mamba2"])
+@pytest.mark.parametrize("K,V,dtype,use_dqk,rot_v,eta,bits", [
+    (128, 128, torch.float16, False, False, 1.0, 8),   # the benchmark's linear-attention call: R_QK on q, k only
+    (128, 128, torch.float16, True, True, 0.5, 8),
+    (64, 128, torch.bfloat16, False, True, 1.0, 8),
+    (128, 64, torch.float16, True, False, 0.0, 6),
+    (64, 64, torch.bfloat16, True, True, 0.25, 8),
+])
+def test_fused_prologue_equals_rotation_then_call(cuda, cell, K, V, dtype, use_dqk, rot_v, eta, bits):
+    """chunk_simple_gla_int8(..., prologue=...) (one launch rotates, rescales and quantizes every operand; the output
+    kernel reads codes) against rotate_qkv followed by the plain call: outputs, final state, stored state codes and the
+    write codes are the same bits; the rotated activations it can export equal rotate_qkv's."""
+    from linquant_amd.kernels import zoo
+
+    print("[case] fused prologue", cell, K, V, dtype, use_dqk, rot_v, eta, bits, flush=True)
+    H = 3
+    q, k, v, g, _ = zc.cut(zc.inputs(cell, B=2, H=H, K=K, V=V, seed=17, dtype=dtype), 192)
+    gen = torch.Generator().manual_seed(6)
+    D = (torch.rand(H, K, generator=gen) + 0.5).to(cuda) if use_dqk else None
+    sq = zoo.rotation_signs(Z.signed_hadamard(K, 1).to(cuda))
+    sv = zoo.rotation_signs(Z.signed_hadamard(V, 2).to(cuda)) if rot_v else None
+    sc = {"q": torch.rand(H, generator=gen) * 0.002 + 0.001, "k": torch.rand(H, generator=gen) * 0.01 + 0.005,
+          "kw": torch.rand(H, K, generator=gen) * 0.01 + 0.004, "vw": torch.rand(H, V, generator=gen) * 0.02 + 0.02,
+          "vl": torch.rand(H, V, generator=gen) * 0.02 + 0.02, "state": torch.rand(H, V, generator=gen) * 0.05 + 0.02}
+    sc = {n: t.to(cuda) for n, t in sc.items()}
+    dev = lambda t: None if t is None else t.to(cuda)  # noqa: E731
+    kw = dict(eta=eta, scale=K ** -0.5, bits=bits, output_final_state=True)
+    qr, kr, vr = zoo.rotate_qkv(dev(q), dev(k), dev(v), signs_qk=sq, signs_v=sv, dqk=D)
+    d0, d1 = {}, {}
+    o0, h0 = zoo.chunk_simple_gla_int8(qr, kr, vr, dev(g), sc, _debug=d0, **kw)
+    o1, h1 = zoo.chunk_simple_gla_int8(dev(q), dev(k), dev(v), dev(g), sc, prologue=dict(signs_qk=sq, signs_v=sv, dqk=D),
+                                       _debug=d1, **kw)
+    o2, h2 = zoo.chunk_simple_gla_int8(dev(q), dev(k), dev(v), dev(g), sc, prologue=dict(signs_qk=sq, signs_v=sv, dqk=D), **kw)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o0.float()).all() and float(o0.float().abs().max()) > 0
+    assert torch.equal(o0, o1) and torch.equal(h0, h1), "fused prologue differs from rotation followed by the call"
+    assert torch.equal(o0, o2) and torch.equal(h0, h2), "fused prologue without the exported activations differs"
+    for name in ("h_i8", "kq", "vq"):
+        assert torch.equal(d0[name], d1[name]), name
+    for got, ref in zip(d1["rotated"], (qr, kr, vr)):
+        assert torch.equal(got, ref)
+    qmax = 2 ** (bits - 1) - 1
+    assert all(int(c.abs().max()) <= qmax for c in d1["local"]) and int(d1["local"][1].abs().max()) > qmax // 4
+
+
+def test_fused_prologue_falls_back_for_widths_it_is_not_built_for(cuda):
+    """A key width of 48 (widened by the wrappers) with a persistent rotation of the value axis only: the call rotates
+    up front and gives what the two-step route gives."""
+    from linquant_amd.kernels import zoo
+
+    q, k, v, g, _ = zc.cut(zc.inputs("mamba2", B=1, H=2, K=48, V=64, seed=5), 128)
+    sv = zoo.rotation_signs(Z.signed_hadamard(64, 2).to(cuda))
+    gen = torch.Generator().manual_seed(2)
+    sc = {"q": torch.full((2,), 0.002), "k": torch.full((2,), 0.01), "kw": torch.full((2, 48), 0.01),
+          "vw": torch.full((2, 64), 0.03), "vl": torch.full((2, 64), 0.03), "state": torch.full((2, 64), 0.05)}
+    sc = {n: t.to(cuda) for n, t in sc.items()}
+    dev = lambda t: t.to(cuda)  # noqa: E731
+    _, _, vr = zoo.rotate_qkv(None, None, dev(v), signs_v=sv)
+    o0, _ = zoo.chunk_simple_gla_int8(dev(q), dev(k), vr, dev(g), sc)
+    o1, _ = zoo.chunk_simple_gla_int8(dev(q), dev(k), dev(v), dev(g), sc, prologue=dict(signs_v=sv))
+    torch.cuda.synchronize()
+    assert torch.equal(o0, o1)
