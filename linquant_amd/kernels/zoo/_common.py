@@ -39,6 +39,35 @@ def pad_keys(q, k, g, scales, rot=None):
     return q, k, g, scales, rot, K
 
 
+def pad_chunks(chunk_size, q, k, v, g=None, beta=None):
+    """Chunk sizes below 64 run on the 64-token kernels: every chunk of C tokens is followed by 64 - C padding tokens with
+    q = k = v = 0, log decay 0 and beta = 1.  Padding tokens add nothing to any product (their codes are zero), leave the
+    decay accumulated over the chunk and hence the carried state unchanged, their Gram rows and columns are zero (the
+    triangular inverse is the identity there), and the sub-block anchoring of the per-channel decay (16-token sub-blocks
+    from the start of the chunk) is the reference's own for C a multiple of 16; the state is quantized at every chunk
+    boundary as before, i.e. every C real tokens.  Returns (q, k, v, g, beta, restore) with ``restore`` cutting an
+    output back to the caller's tokens.  Chunk sizes above 64 are not built."""
+    T = q.shape[1]
+    assert T % chunk_size == 0, f"T={T} must be a multiple of the chunk size {chunk_size}"
+    assert 1 <= chunk_size <= CHUNK, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {CHUNK} tokens"
+    if chunk_size == CHUNK:
+        return q, k, v, g, beta, lambda o: o
+    NT, pad = T // chunk_size, CHUNK - chunk_size
+
+    def widen(t, value=0.0):
+        if t is None:
+            return None
+        x = t.reshape(t.shape[0], NT, chunk_size, *t.shape[2:])
+        x = torch.nn.functional.pad(x, (0, 0) * (x.dim() - 3) + (0, pad), value=value)
+        return x.reshape(t.shape[0], NT * CHUNK, *t.shape[2:])
+
+    def restore(o):
+        x = o.reshape(o.shape[0], NT, CHUNK, *o.shape[2:])[:, :, :chunk_size]
+        return x.reshape(o.shape[0], T, *o.shape[2:]).contiguous()
+
+    return widen(q), widen(k), widen(v), widen(g), widen(beta, 1.0), restore
+
+
 _VALUE_SCALES = ("vw", "vl", "state", "el", "ew")
 
 
@@ -79,7 +108,7 @@ def check_shapes(q, k, v, chunk_size):
     B, T, H, K = q.shape
     V = v.shape[-1]
     assert T % chunk_size == 0, f"T={T} must be a multiple of the chunk size {chunk_size}"
-    assert chunk_size == CHUNK, f"chunk_size={chunk_size}: the HIP kernels are built for 64-token chunks"
+    assert chunk_size == CHUNK, f"chunk_size={chunk_size}: the HIP kernels are built for 64-token chunks (pad_chunks widens smaller ones)"
     assert K in (64, 128), f"K={K}: the kernels take 64 or 128 key channels (pad_keys widens anything else)"
     assert V % 64 == 0, f"V={V}: value dim must be a multiple of 64"
     assert q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype, \

@@ -16,10 +16,11 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
                      output_final_state=False, unrot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None (DeltaNet), beta [B,T,H].
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
+    q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta)
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
-    dims = C.check_shapes(q, k, v, chunk_size)
+    dims = C.check_shapes(q, k, v, C.CHUNK)
     B, T, H, K, V = dims
     assert beta.shape == (B, T, H)
     Ru = C.unrot_matrix(unrot, V)
@@ -35,7 +36,7 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay,
                                         write=dict(logenv=None, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
                                         keep_W=_debug is not None)
-    NT = T // chunk_size
+    NT = T // C.CHUNK
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
@@ -44,4 +45,4 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
                 w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes)
     C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
     C.export_debug(_debug, h_i8, codes, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
-    return C.cut_values(o, C.cut_keys(ht, K0), V0)
+    return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -18,10 +18,11 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
     Returns (o, final fp32 state or None)."""
     assert g.shape == q.shape
+    q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g)
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    dims = C.check_shapes(q, k, v, chunk_size)
+    dims = C.check_shapes(q, k, v, C.CHUNK)
     B, T, H, K, V = dims
     assert chunk_size % BC == 0
     Ru = C.unrot_matrix(unrot, V)
@@ -31,7 +32,7 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     gc, logenv = C.cumsum(g, B, T, H, K)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
     A, qg = C.run_gla_A(q, k, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R)
-    NT = T // chunk_size
+    NT = T // C.CHUNK
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
@@ -40,4 +41,4 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     C.run_output(None, None, v, h_i8, None, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, g=gc, logenv=logenv)
-    return C.cut_values(o, C.cut_keys(ht, K0), V0)
+    return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

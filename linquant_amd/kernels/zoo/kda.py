@@ -26,10 +26,11 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
         d = dqk.to(q.device)
         q, k = (q.float() * d.float()).to(q.dtype), (k.double() / d.double()).float().to(k.dtype)
         dqk = None
+    q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta)
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
-    dims = C.check_shapes(q, k, v, chunk_size)
+    dims = C.check_shapes(q, k, v, C.CHUNK)
     B, T, H, K, V = dims
     assert chunk_size % BC == 0 and beta.shape == (B, T, H)
     Ru = C.unrot_matrix(unrot, V)
@@ -44,7 +45,7 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
                                         write=dict(logenv=logenv, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
                                         keep_W=_debug is not None, dk=(dq, dq_rcp))
     A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R, dq=dq)
-    NT = T // chunk_size
+    NT = T // C.CHUNK
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
@@ -54,4 +55,4 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     C.run_output(None, None, e_out, h_i8, None, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
-    return C.cut_values(o, C.cut_keys(ht, K0), V0)
+    return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -35,10 +35,11 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
         if do_v:
             v = rv
         prologue = None
+    q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g)
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    dims = C.check_shapes(q, k, v, chunk_size)
+    dims = C.check_shapes(q, k, v, C.CHUNK)
     B, T, H, K, V = dims
     Ru = C.unrot_matrix(unrot, V)
     scale = K0 ** -0.5 if scale is None else scale
@@ -48,7 +49,7 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     if g is not None:
         assert g.shape == (B, T, H)
         gg, _ = C.cumsum(g, B, T, H, 0)
-    NT = T // chunk_size
+    NT = T // C.CHUNK
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
@@ -61,8 +62,8 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
         C.run_output(None, None, None, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay,
                      local=local, act=C.act_code(v))
         C.export_debug(_debug, h_i8, codes, g=gg, local=local, rotated=rotated)
-        return C.cut_values(o, C.cut_keys(ht, K0), V0)
+        return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
     codes = C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru)
     C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
     C.export_debug(_debug, h_i8, codes, g=gg)
-    return C.cut_values(o, C.cut_keys(ht, K0), V0)
+    return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

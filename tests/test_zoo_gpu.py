@@ -48,6 +48,34 @@ def test_cell_matches_oracle(cuda, cell, n):
         assert err_max <= max(1e-3, noise_max), f"{cell}: two-chunk horizon rel max {err_max:.2e} (noise {noise_max:.2e})"
 
 
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+@pytest.mark.parametrize("chunk", [16, 32, 48])
+def test_chunk_sizes_below_64(cuda, cell, chunk):
+    """Chunk sizes the reference accepts besides its default (multiples of 16, linquant/kernels/zoo/gla.py:244-246,
+    kda.py:163-165; any divisor of T for the scalar-decay kernels): outputs by the reference's criterion against the
+    oracle run with the same chunk size, stored state codes (one per C tokens) within one step of the oracle's and the
+    final state close to its carry."""
+    tensors = zc.cut(zc.inputs(cell, B=1, H=2, K=64, V=64, seed=23), 192)
+    eta = DEFAULT_ETA[cell]
+    qz, run = zc.calibrated(cell, tensors, eta=eta, rho=0.5, tau=0.5, chunk=chunk)
+    scales = qz.kernel_scales(0, 2, 64, 64, delta=zc.CELLS[cell][0] == "delta")
+    dbg = {}
+    out, ht = zc.run_kernel(cell, tensors, scales, eta=eta, rho=0.5, tau=0.5, chunk=chunk, final_state=True, debug=dbg)
+    torch.cuda.synchronize()
+    assert out.shape == tensors[2].shape and dbg["h_i8"].shape[1] == 192 // chunk
+    zc.check(out, run, qz, f"{cell} chunk {chunk}")
+    codes = zc.state_codes(qz, run)                      # (NT, B, H, K, V): state after each chunk
+    got = dbg["h_i8"].cpu()                              # (B, NT, H, K, V): state entering each chunk
+    NT = codes.shape[0]
+    assert NT == 192 // chunk and (got[:, 0] == 0).all()
+    d = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
+    assert int(d.max()) <= (2 if cell == "deltanet" else 1) and (d != 0).float().mean().item() < 2e-3, \
+        (int(d.max()), (d != 0).float().mean().item())
+    sc = qz.kernel_scales(0, 2, 64, 64)["state"]
+    last = torch.round(ht.cpu() / sc[None, :, None, :]).clamp(-127, 127)
+    assert (last - codes[-1]).abs().max().item() <= (2 if cell == "deltanet" else 1)
+
+
 @pytest.mark.parametrize("cell,eta", [("mamba2", 0.0), ("mamba2", 0.5), ("gla", 0.5), ("gla", 1.0),
                                       ("gated_deltanet", 0.0), ("gated_deltanet", 0.5), ("kda", 0.5), ("kda", 1.0)])
 def test_eta_split(cuda, cell, eta):

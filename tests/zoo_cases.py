@@ -70,7 +70,7 @@ def cut(tensors, n):
 
 
 def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.0, tau=1.0, rot_qk=None, rot_v=None, out_dtype=None,
-               calib_tensors=None, storage=None):
+               calib_tensors=None, storage=None, chunk=64):
     """Returns (qz, run): the oracle's quantizer with scales calibrated on these inputs (or on ``calib_tensors``, a
     separate batch), and a closure that evaluates the oracle on ``tensors`` under the quantizer's current arithmetic
     mode; like the kernels, the oracle materializes its output in the activation dtype unless ``out_dtype`` says
@@ -82,7 +82,7 @@ def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.
     def forward(t):
         q, k, v, g, beta = t
         return Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=qz, eta=eta, rho=rho,
-                               tau=tau, read_post=True, C=64, out_dtype=out_dtype, rot_qk=rot_qk, rot_v=rot_v,
+                               tau=tau, read_post=True, C=chunk, out_dtype=out_dtype, rot_qk=rot_qk, rot_v=rot_v,
                                storage=storage or ("canonical" if rot_v is not None else "rotated"))
 
     qz.calibrating = True
@@ -92,14 +92,14 @@ def calibrated(cell, tensors, *, policy="kernel_static", bits=8, eta=1.0, rho=1.
 
 
 def run_kernel(cell, tensors, scales, *, eta=1.0, rho=1.0, tau=1.0, bits=8, out_dtype=None, final_state=False,
-               debug=None, device="cuda", rot=None, unrot=None):
+               debug=None, device="cuda", rot=None, unrot=None, chunk=64):
     from linquant_amd.kernels import zoo
 
     fam, dec = CELLS[cell]
     q, k, v, g, beta = [t.to(device) if t is not None else None for t in tensors]
     sc = {n: s.to(device) for n, s in scales.items()}
     K = q.shape[-1]
-    kw = dict(eta=eta, scale=K ** -0.5, chunk_size=64, bits=bits, out_dtype=out_dtype, output_final_state=final_state,
+    kw = dict(eta=eta, scale=K ** -0.5, chunk_size=chunk, bits=bits, out_dtype=out_dtype, output_final_state=final_state,
               _debug=debug)
     if rot is not None:
         kw["rot"] = rot.to(device)
