@@ -286,12 +286,13 @@ int lq_split_rotate_quant_xBC(const lq_split_rotate_quant_xBC_args* args, hipStr
 /* replaces kronecker_hadamard_fwd, linquant/kernels/hadamard.py:141-179 (kernel :38-103):
  * y = (x * signs) . (H2 (x) H_{D/2}) per head, same dtype out, no quantization. */
 typedef struct {
-  const void* x;             /* (B,T,H,D) fp16, unit D stride */
+  const void* x;             /* (B,T,H,D) fp16 or bf16 (x_dtype), unit D stride; D a power of two, 64 .. 512 */
   int64_t x_stride_b, x_stride_t, x_stride_h;
-  void* y;                   /* (B,T,H,D) fp16 contiguous */
+  void* y;                   /* (B,T,H,D) contiguous, same dtype as x */
   const void* signs;         /* (H,D) */
   int32_t signs_dtype;
   int32_t batch, seqlen, nheads, dim;
+  int32_t x_dtype;           /* LQ_DT_F16 (0) or LQ_DT_BF16 */
 } lq_kron_hadamard_args;
 int lq_kron_hadamard(const lq_kron_hadamard_args* args, hipStream_t stream);
 

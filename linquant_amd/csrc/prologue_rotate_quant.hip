@@ -63,7 +63,8 @@ LQ_DEV void fwht_row(float* v, int sub, float hb, float kron) {
 // VEC: signs and dqk are 16-byte aligned, so a lane's eight entries are fetched as whole pieces, requested together with
 // its row piece before anything is used (element by element, behind a run-time dtype switch, they formed a chain of
 // memory round trips several times longer than the transform itself).
-template <int N, bool QUANT, bool VEC>
+// BF: the rows are bf16 in and out (stand-alone rotation only; the fused prologue rounds through fp16 by definition).
+template <int N, bool QUANT, bool VEC, bool BF = false>
 __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict__ src, int64_t s_b, int64_t s_t,
                                                      int64_t s_seg, int nseg_per_side, int64_t side_off,
                                                      void* __restrict__ dst0, void* __restrict__ dst1, _Float16* __restrict__ fp0,
@@ -84,7 +85,12 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
   const int tt = live ? t : T - 1;  // inactive rows still take part in the shuffles
 
   const _Float16* sp = src + (int64_t)b * s_b + (int64_t)tt * s_t + side * side_off + (int64_t)seg * s_seg + sub * 8;
-  const lq_v8h hv = *(const lq_v8h*)sp;
+  const lq_v4i hraw = *(const lq_v4i*)sp;
+  const lq_v8h hv = __builtin_bit_cast(lq_v8h, hraw);
+  float xin[8];  // the row piece as fp32
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    xin[i] = BF ? __uint_as_float(((uint32_t)hraw[i >> 1] >> (16 * (i & 1))) << 16) : (float)hv[i];
   float v[8];
   const float* dqk = side ? dqk1 : dqk0;
   if constexpr (VEC) {
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
     const lq_v4i s0 = *(const lq_v4i*)(es == 1 ? sgp - ((uintptr_t)sgp & 8) : sgp);          // int8: the aligned 16 bytes around the 8
     const lq_v4i s1 = *(const lq_v4i*)(es == 4 ? sgp + 16 : sgp - ((uintptr_t)sgp & 15));    // fp32: second half
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (float)hv[i];
+    for (int i = 0; i < 8; ++i) v[i] = xin[i];
     if (QUANT && dqk) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = (float)(_Float16)(v[i] * (i < 4 ? d0[i & 3] : d1[i & 3]));
@@ -117,7 +123,7 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (float)hv[i];
+    for (int i = 0; i < 8; ++i) v[i] = xin[i];
     if (QUANT && dqk) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[i] = (float)(_Float16)(v[i] * dqk[seg * N + sub * 8 + i]);
@@ -163,10 +169,20 @@ __global__ __launch_bounds__(256) void rotate_kernel(const _Float16* __restrict_
     }
   } else {
     _Float16* dp = (_Float16*)dst0 + (((int64_t)b * T + t) * nseg_per_side + seg) * N + sub * 8;
-    lq_v8h o;
+    if constexpr (BF) {
+      lq_v4i o;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = (_Float16)v[i];
-    *(lq_v8h*)dp = o;
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = __float_as_uint(bf16_round(v[2 * i])) >> 16, hi = __float_as_uint(bf16_round(v[2 * i + 1])) & 0xffff0000u;
+        o[i] = (int)(lo | hi);
+      }
+      *(lq_v4i*)dp = o;
+    } else {
+      lq_v8h o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] = (_Float16)v[i];
+      *(lq_v8h*)dp = o;
+    }
   }
 }
 
@@ -219,33 +235,34 @@ extern "C" int lq_kron_hadamard(const lq_kron_hadamard_args* a, hipStream_t stre
   if (!a || !a->x || !a->y || !a->signs) return LQ_ERR_NULL;
   const int D = a->dim, H = a->nheads;
   if (a->batch <= 0 || a->seqlen <= 0 || H <= 0) return LQ_ERR_SHAPE;
-  if (D != 64 && D != 128) return LQ_ERR_SHAPE;
+  if (D != 64 && D != 128 && D != 256 && D != 512) return LQ_ERR_SHAPE;  // a row is spread over D / 8 lanes of one wave
+  if (a->x_dtype != LQ_DT_F16 && a->x_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (a->x_stride_b % 8 || a->x_stride_t % 8 || a->x_stride_h % 8 || !al(a->x, 16) || !al(a->y, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * H > 65535) return LQ_ERR_SHAPE;
   const float hb = hblock_value(D / 2);
   const float kron = (float)(1.0 / sqrt(2.0));
   const int rpb = 256 / (D / 8);
   dim3 grid((a->seqlen + rpb - 1) / rpb, a->batch * H);
-  const bool vec = al(a->signs, 16);
-  if (D == 128 && vec)
-    hipLaunchKernelGGL((rotate_kernel<128, false, true>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
-                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
-                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron, (float*)nullptr);
-  else if (vec)
-    hipLaunchKernelGGL((rotate_kernel<64, false, true>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
-                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
-                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron, (float*)nullptr);
-  else if (D == 128)
-    hipLaunchKernelGGL((rotate_kernel<128, false, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
-                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
-                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron, (float*)nullptr);
-  else
-    hipLaunchKernelGGL((rotate_kernel<64, false, false>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b,
-                       a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs, a->signs_dtype,
-                       (const float*)nullptr, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
-                       a->seqlen, hb, kron, (float*)nullptr);
+  const bool vec = al(a->signs, 16), bf = a->x_dtype == LQ_DT_BF16;
+#define LQ_KRON_LAUNCH(NN, VV, BB)                                                                                      \
+  hipLaunchKernelGGL((rotate_kernel<NN, false, VV, BB>), grid, dim3(256), 0, stream, (const _Float16*)a->x, a->x_stride_b, \
+                     a->x_stride_t, a->x_stride_h, H, (int64_t)0, a->y, (void*)nullptr, (_Float16*)nullptr, a->signs,      \
+                     a->signs_dtype, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,                  \
+                     (const float*)nullptr, a->seqlen, hb, kron, (float*)nullptr)
+#define LQ_KRON_DISPATCH(NN)                     \
+  do {                                           \
+    if (vec && bf) LQ_KRON_LAUNCH(NN, true, true);       \
+    else if (vec) LQ_KRON_LAUNCH(NN, true, false);       \
+    else if (bf) LQ_KRON_LAUNCH(NN, false, true);        \
+    else LQ_KRON_LAUNCH(NN, false, false);               \
+  } while (0)
+  switch (D) {
+    case 64: LQ_KRON_DISPATCH(64); break;
+    case 128: LQ_KRON_DISPATCH(128); break;
+    case 256: LQ_KRON_DISPATCH(256); break;
+    default: LQ_KRON_DISPATCH(512); break;
+  }
+#undef LQ_KRON_DISPATCH
+#undef LQ_KRON_LAUNCH
   return lq_check_launch();
 }

@@ -31,17 +31,18 @@ def _resolve_kronecker_params(D, n_chunks, device):
 
 
 def kronecker_hadamard_fwd(x, signs, num_heads, n_chunks=2):
-    """x (B,T,H,D) fp16, D in {64,128}, any batch/seq/head stride (e.g. a view of xBC); signs (H,D) +-1.
-    Returns (x * signs) @ H per head, contiguous, same dtype."""
+    """x (B,T,H,D) fp16 or bf16, D a power of two from 64 to 512, any batch/seq/head stride (e.g. a view of xBC);
+    signs (H,D) +-1.  Returns (x * signs) @ H per head, contiguous, same dtype."""
     B, T, H, D = x.shape
     assert D >= 64, f"Kronecker Hadamard needs D >= 64, got {D}"
-    assert n_chunks == 2 and D in (64, 128), "two-half Kronecker rotation: D in {64, 128}"
-    assert x.dtype == torch.float16 and x.stride(3) == 1, "x must be fp16 with a dense last axis"
+    assert n_chunks == 2 and D in (64, 128, 256, 512), "two-half Kronecker rotation: D a power of two, 64 .. 512"
+    assert x.dtype in (torch.float16, torch.bfloat16) and x.stride(3) == 1, "x must be fp16 or bf16 with a dense last axis"
     signs = _signs_arg(signs)
     assert signs.numel() == H * D
     y = torch.empty((B, T, H, D), dtype=x.dtype, device=x.device)
     _lib.call("lq_kron_hadamard", x.device,
               x=_lib.ptr(x), x_stride_b=x.stride(0), x_stride_t=x.stride(1), x_stride_h=x.stride(2),
               y=_lib.ptr(y), signs=_lib.ptr(signs), signs_dtype=_SIGN_CODES[signs.dtype],
-              batch=B, seqlen=T, nheads=H, dim=D)
+              batch=B, seqlen=T, nheads=H, dim=D,
+              x_dtype=_lib.LQ_DT_BF16 if x.dtype == torch.bfloat16 else _lib.LQ_DT_F16)
     return y

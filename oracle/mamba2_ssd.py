@@ -265,9 +265,11 @@ def split_rotate_quant_xBC(xBC, r_signs, nheads, ngroups, d_state, headdim, B_in
     return x, outs[0], outs[1]
 
 
-def kron_hadamard(x, signs):
-    """x (B,T,H,D) fp16, signs (H,D) -> rotated fp16."""
-    return kron_rotate(x.astype(np.float32), np.asarray(signs, np.float32)[None, None]).astype(np.float16)
+def kron_hadamard(x, signs, bf16=False):
+    """x (B,T,H,D) fp16, signs (H,D) -> rotated fp16 (linquant/kernels/hadamard.py:81-103: the fp32 result cast to the
+    input dtype).  bf16=True: x is an fp32 array of bf16-representable values and so is the result."""
+    y = kron_rotate(x.astype(np.float32), np.asarray(signs, np.float32)[None, None])
+    return bf16_round(y) if bf16 else y.astype(np.float16)
 
 
 # ------------------------------------------------------------------------------------------ pipeline

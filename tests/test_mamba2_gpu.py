@@ -120,6 +120,36 @@ def test_prologue_and_rotation(case, cuda):
     assert np.array_equal(npy(y).view(np.uint16), ref["b_fp"].view(np.uint16))
 
 
+@pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (128, torch.bfloat16), (256, torch.float16), (256, torch.bfloat16),
+                                     (512, torch.float16), (512, torch.bfloat16)])
+def test_kronecker_hadamard_widths_and_bf16(cuda, D, dtype):
+    """kronecker_hadamard_fwd over the reference's whole domain (linquant/kernels/hadamard.py:141-152: fp16 / bf16, D a
+    power of two >= 64; here up to 512): a strided view of a wider slab, a token count that is not a multiple of the
+    rows per workgroup; bit-exact against the oracle's two-half rotation."""
+    from linquant_amd.kernels.hadamard import kronecker_hadamard_fwd
+
+    say("kron hadamard", D, dtype)
+    g = torch.Generator().manual_seed(D)
+    B, T, H = 2, 77, 3
+    slab = torch.randn(B, T, H * D + 40, generator=g).to(dtype)
+    signs = (torch.randint(0, 2, (H, D), generator=g) * 2 - 1).float()
+    view = slab.to(cuda)[..., 8:8 + H * D].view(B, T, H, D)  # row stride H*D + 40, 16-byte aligned start
+    y = kronecker_hadamard_fwd(view, signs.to(cuda), H)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and y.shape == (B, T, H, D) and y.is_contiguous()
+    x = slab[..., 8:8 + H * D].reshape(B, T, H, D)
+    if dtype == torch.bfloat16:
+        ref = O.kron_hadamard(x.float().numpy(), npy(signs), bf16=True)
+        assert np.array_equal(y.float().cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    else:
+        ref = O.kron_hadamard(npy(x), npy(signs))
+        assert np.array_equal(npy(y).view(np.uint16), ref.view(np.uint16))
+    # orthogonality: rotating twice with unit signs returns the row (H2 (x) H_{D/2} is symmetric), to half precision
+    ones = torch.ones(H, D, device=cuda)
+    back = kronecker_hadamard_fwd(kronecker_hadamard_fwd(view, ones, H), ones, H)
+    assert (back.float() - view.float()).abs().max().item() <= (0.08 if dtype == torch.bfloat16 else 0.02)
+
+
 def test_prologue_dqk_and_no_rotation(cuda):
     from linquant_amd.kernels.mamba2.fused_split_rotate_xBC import fused_split_rotate_quant_xBC, prepare_dqk
 

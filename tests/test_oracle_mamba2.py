@@ -233,7 +233,7 @@ def test_chunk_state_key_and_bmm_scalar_bruteforce():
 
 
 # ----------------------------------------------------------------------------- rotation
-@pytest.mark.parametrize("N", [64, 128])
+@pytest.mark.parametrize("N", [64, 128, 256, 512])
 def test_kron_rotation_is_signed_hadamard(N):
     rng = np.random.default_rng(N)
     Hn = scipy.linalg.hadamard(N).astype(np.float64)
