@@ -144,13 +144,15 @@ def zoo_stage_bytes(fam, dec, B, T, H, K, V):
     out = {}
     if dec != "none":
         out["cumsum"] = 2 * g + (tok if dec == "diagonal" else 0)
+        if fam == "linear" and dec == "diagonal":  # the launch also reads k, v and writes the state kernel's write operands
+            out["cumsum"] += qk + vv + qk // 2 + vv // 2 + tok
     if fam == "delta":
         # k, v, beta, g (and the log envelope) in; Hw, U, fw and the state kernel's write operands (key write codes,
         # state-read codes of W, value factor) out: W itself never leaves the chip
         out["wy_prep"] = qk + vv + tok + g + (tok if dec == "diagonal" else 0) + qk + vv + tok + qk // 2 + qk // 2 + tok
     if dec == "diagonal":
         out["gla_A"] = 2 * qk + g + A // 2 + qk // 2  # A in fp16, INT8 codes of the decayed query
-    if fam == "linear":
+    if fam == "linear" and dec != "diagonal":
         # the state stage of the reference reads the fp16 operands; the split pipeline adds the INT8 code round trip
         out["write_codes"] = qk + g + vv + (tok if dec == "diagonal" else 0) + qk // 2 + vv // 2
     out["state"] = qk // 2 + h8 + ((qk // 2 + 2 * tok + 2 * vv) if fam == "delta" else vv // 2)

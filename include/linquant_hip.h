@@ -313,6 +313,21 @@ typedef struct {
   float* logenv;             /* (B,T,H) max_k(gc_last[k] - gc[t,k]); diagonal decay only, else NULL */
   int32_t batch, seqlen, nheads, kdim; /* kdim = 0: scalar decay */
   int32_t chunk_size;
+  /* Optional (per-channel decay, linear family, chunk 64; all of them when kqT is set): the write operands of the state
+   * kernel that lq_zoo_write_codes would make from gc and logenv, made here while the chunk's decay tile is on chip:
+   * the operand preparation inside _gla_state_body (linquant/kernels/zoo/gla.py:124-141).  Same bits. */
+  const void* k;             /* (B,T,H,K) fp16/bf16 */
+  const void* v;             /* (B,T,H,V) fp16/bf16 */
+  int8_t* kqT;               /* (B,NT,H,K,C) key write codes */
+  int8_t* vqT;               /* (B,NT,H,V,C) value write codes */
+  float* ev;                 /* (B,T,H) */
+  float* gam;                /* (B,NT,H,K) */
+  const float* skw;          /* (H,K) */
+  const float* svw;          /* (H,V) */
+  float eta;
+  int32_t qmax;
+  int32_t vdim;
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16 */
 } lq_zoo_cumsum_args;
 int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
 

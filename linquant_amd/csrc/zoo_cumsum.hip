@@ -5,7 +5,7 @@
 //   logenv[b, t, h] = max_k (gc_last[k] - gc[t, k])                     (diagonal decay only)
 // One thread walks one (batch, chunk, head[, channel]) column; threads of a workgroup cover adjacent
 // channels, so every step is a coalesced row access.
-#include "lq_common.h"
+#include "zoo_common.h"
 #include "../../include/linquant_hip.h"
 
 namespace {
@@ -42,13 +42,35 @@ __global__ __launch_bounds__(256) void cumsum_scalar64_kernel(const float* __res
   }
 }
 
+// Write operands of the linear family's state kernel under per-channel decay, made by the cumsum launch from the decay
+// tile it holds (what lq_zoo_write_codes would make from the stored gc and logenv; same arithmetic, same bits):
+//   kqT[k][t] = q8(key[t][k] * exp(gk_last - gk_t - eta*le_t), 1/skw[k]),  vqT[v][t] = q8(val[t][v] * exp(eta*le_t), 1/svw[v]),
+//   ev[t] = exp(eta*le_t),  gam[k] = exp(gk_last).
+struct CumsumCodes {
+  const uint16_t* k;
+  const uint16_t* v;
+  int8_t* kqT;
+  int8_t* vqT;
+  float* ev;
+  float* gam;
+  const float* skw;
+  const float* svw;
+  float eta;
+  int qmax;
+  int V;
+  int bf;
+};
+
 // one workgroup per (batch, chunk, head); 4*K threads: thread (k, q) scans tokens q*C/4 .. of channel k (all of its
 // loads are independent and issued up front), the four partial totals are combined through LDS; LDS tile [C][K+1]
-// for the envelope reduction
+// for the envelope reduction.  CODES (chunk 64 only): a thread's 16 tokens of one channel are one 16-byte piece of that
+// channel's row of channel-major codes, so the codes go straight from registers to memory.
+template <bool CODES>
 __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restrict__ gc, float* __restrict__ logenv,
-                                   int T, int H, int K, int C) {
+                                   int T, int H, int K, int C, CumsumCodes cc) {
   extern __shared__ float tile[];           // [C][K + 1]
   double* part = (double*)(tile + C * (K + 1));  // [4][K] segment totals
+  float* le_s = (float*)(part + 4 * K);      // [C] log envelope (CODES)
   const int k = threadIdx.x % K, q = threadIdx.x / K;
   const int SEG = C / 4;                    // tokens per thread (C is a multiple of 16)
   const int h = blockIdx.x % H;
@@ -63,6 +85,14 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
     // tokens past the segment re-read its last one and count as zero
     const float x = g[base + min(t, SEG - 1) * tstride];
     v[t] = t < SEG ? x : 0.0f;
+  }
+  // CODES: this thread's 16 key values (channel k, tokens 16q ..) and its value channels' 16 values, requested now
+  uint16_t kraw[CODES ? 16 : 1];
+  float inv_skw = 0.0f;
+  if constexpr (CODES) {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) kraw[t] = cc.k[base + t * tstride];
+    inv_skw = 1.0f / cc.skw[h * K + k];
   }
   double run = 0.0, pre[16];
 #pragma unroll
@@ -96,7 +126,45 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
     for (int j = 1; j < KS; ++j) m = fmaxf(m, row[j]);
 #pragma unroll
     for (int o = 1; o < 8; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if (sub == 0) logenv[(row0 + t) * H + h] = m;
+    if (sub == 0) {
+      logenv[(row0 + t) * H + h] = m;
+      if constexpr (CODES) {
+        le_s[t] = m;
+        cc.ev[(row0 + t) * H + h] = zoo_exp(cc.eta * m);
+      }
+    }
+  }
+  if constexpr (CODES) {
+    __syncthreads();
+    const bool bf = cc.bf;
+    const int64_t cb = bc * H + h;  // (batch, chunk, head)
+    if (q == 0) cc.gam[cb * K + k] = zoo_exp(last);
+    // key write codes: 16 tokens of channel k
+    int code[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int tok = 16 * q + t;
+      const float el = cc.eta * le_s[tok];
+      const float x = zoo_dec1(kraw[t], bf) * zoo_exp(tile[tok * (K + 1) + k] - el);
+      code[t] = zoo_q8(x, inv_skw, cc.qmax);
+    }
+    lq_v4i o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) o[d] = (int)zoo_pack_codes(code[4 * d], code[4 * d + 1], code[4 * d + 2], code[4 * d + 3]);
+    *(lq_v4i*)(cc.kqT + (cb * K + k) * 64 + 16 * q) = o;
+    // value write codes: channel c = k, k + K, ... of the V value channels
+    const int V = cc.V;
+    for (int c = k; c < V; c += K) {
+      const float inv_svw = 1.0f / cc.svw[h * V + c];
+      uint16_t vraw[16];
+#pragma unroll
+      for (int t = 0; t < 16; ++t) vraw[t] = cc.v[((row0 + 16 * q + t) * H + h) * V + c];
+#pragma unroll
+      for (int t = 0; t < 16; ++t) code[t] = zoo_q8(zoo_dec1(vraw[t], bf) * zoo_exp(cc.eta * le_s[16 * q + t]), inv_svw, cc.qmax);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) o[d] = (int)zoo_pack_codes(code[4 * d], code[4 * d + 1], code[4 * d + 2], code[4 * d + 3]);
+      *(lq_v4i*)(cc.vqT + (cb * V + c) * 64 + 16 * q) = o;
+    }
   }
 }
 
@@ -118,10 +186,24 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
   } else {
     if (!a->logenv) return LQ_ERR_NULL;
     if (a->kdim > 256 || a->kdim % 16 != 0 || a->chunk_size % 16 != 0 || a->chunk_size > 64) return LQ_ERR_SHAPE;
-    const size_t lds = (size_t)a->chunk_size * (a->kdim + 1) * sizeof(float) + 4 * (size_t)a->kdim * sizeof(double);
+    const size_t lds = (size_t)a->chunk_size * (a->kdim + 1) * sizeof(float) + 4 * (size_t)a->kdim * sizeof(double) +
+                       (size_t)a->chunk_size * sizeof(float);
     if (lds > 64 * 1024) return LQ_ERR_SHAPE;
-    hipLaunchKernelGGL(cumsum_diag_kernel, dim3((unsigned)((int64_t)a->batch * NT * a->nheads)), dim3(4 * a->kdim), lds,
-                       stream, a->g, a->gc, a->logenv, a->seqlen, a->nheads, a->kdim, a->chunk_size);
+    CumsumCodes cc = {};
+    const dim3 grid((unsigned)((int64_t)a->batch * NT * a->nheads)), block(4 * a->kdim);
+    if (a->kqT) {
+      if (!a->k || !a->v || !a->vqT || !a->ev || !a->gam || !a->skw || !a->svw) return LQ_ERR_NULL;
+      if (a->chunk_size != 64 || a->vdim <= 0 || a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
+      if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
+      if (!zoo_al(a->kqT, 16) || !zoo_al(a->vqT, 16)) return LQ_ERR_SHAPE;
+      cc.k = (const uint16_t*)a->k, cc.v = (const uint16_t*)a->v, cc.kqT = a->kqT, cc.vqT = a->vqT, cc.ev = a->ev, cc.gam = a->gam;
+      cc.skw = a->skw, cc.svw = a->svw, cc.eta = a->eta, cc.qmax = a->qmax, cc.V = a->vdim, cc.bf = a->act_dtype == LQ_DT_BF16;
+      hipLaunchKernelGGL(cumsum_diag_kernel<true>, grid, block, lds, stream, a->g, a->gc, a->logenv, a->seqlen, a->nheads,
+                         a->kdim, a->chunk_size, cc);
+    } else {
+      hipLaunchKernelGGL(cumsum_diag_kernel<false>, grid, block, lds, stream, a->g, a->gc, a->logenv, a->seqlen, a->nheads,
+                         a->kdim, a->chunk_size, cc);
+    }
   }
   return lq_check_launch();
 }

@@ -134,14 +134,29 @@ def unrot_matrix(unrot, V):
     return unrot.to(torch.float16).contiguous()
 
 
-def cumsum(g, B, T, H, kdim):
-    """Chunk-local cumulative log decay (fp32) and, for per-channel decay, the log envelope."""
+def cumsum(g, B, T, H, kdim, write=None):
+    """Chunk-local cumulative log decay (fp32) and, for per-channel decay, the log envelope.  ``write`` = dict(k, v, skw,
+    svw, eta, qmax) (per-channel decay, linear family): the launch also makes the state kernel's write operands while
+    the chunk's decay tile is on chip (what ``write_codes`` would make, same bits) and returns them as a third value."""
     g = f32(g)
     gc = torch.empty_like(g)
-    logenv = torch.empty(B, T, H, dtype=torch.float32, device=g.device) if kdim else None
-    _lib.call("lq_zoo_cumsum", g.device, g=_lib.ptr(g), gc=_lib.ptr(gc), logenv=_lib.ptr(logenv), batch=B, seqlen=T,
-              nheads=H, kdim=kdim, chunk_size=CHUNK)
-    return gc, logenv
+    dev = g.device
+    logenv = torch.empty(B, T, H, dtype=torch.float32, device=dev) if kdim else None
+    if write is None:
+        _lib.call("lq_zoo_cumsum", dev, g=_lib.ptr(g), gc=_lib.ptr(gc), logenv=_lib.ptr(logenv), batch=B, seqlen=T,
+                  nheads=H, kdim=kdim, chunk_size=CHUNK)
+        return gc, logenv
+    k, v = write["k"], write["v"]
+    NT, V = T // CHUNK, v.shape[-1]
+    c = {"kqT": torch.empty(B, NT, H, kdim, CHUNK, dtype=torch.int8, device=dev),
+         "vqT": torch.empty(B, NT, H, V, CHUNK, dtype=torch.int8, device=dev), "wq": None,
+         "ev": torch.empty(B, T, H, dtype=torch.float32, device=dev),
+         "gam": torch.empty(B, NT, H, kdim, dtype=torch.float32, device=dev)}
+    _lib.call("lq_zoo_cumsum", dev, g=_lib.ptr(g), gc=_lib.ptr(gc), logenv=_lib.ptr(logenv), batch=B, seqlen=T,
+              nheads=H, kdim=kdim, chunk_size=CHUNK, k=_lib.ptr(k), v=_lib.ptr(v), kqT=_lib.ptr(c["kqT"]),
+              vqT=_lib.ptr(c["vqT"]), ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]), skw=_lib.ptr(write["skw"]),
+              svw=_lib.ptr(write["svw"]), eta=float(write["eta"]), qmax=int(write["qmax"]), vdim=V, act_dtype=act_code(k))
+    return gc, logenv, c
 
 
 def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay):

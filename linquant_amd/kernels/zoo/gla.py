@@ -29,15 +29,16 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
-    gc, logenv = C.cumsum(g, B, T, H, K)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
+    # the cumsum launch also makes the state kernel's write operands (it holds the chunk's decay tile): no pre-pass
+    gc, logenv, codes = C.cumsum(g, B, T, H, K, write=dict(k=k, v=v, skw=sc["kw"], svw=sc["vw"], eta=eta, qmax=qmax))
     A, qg = C.run_gla_A(q, k, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R)
     NT = T // C.CHUNK
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    codes = C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
-                C.DECAY_DIAGONAL, unrot=Ru)
+    C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
+                C.DECAY_DIAGONAL, unrot=Ru, codes=codes)
     C.run_output(None, None, v, h_i8, None, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
                  unrot=Ru, qg=qg)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, g=gc, logenv=logenv)

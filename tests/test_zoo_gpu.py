@@ -516,6 +516,31 @@ def test_wy_prep_also_makes_the_write_codes(cuda, cell, K, dtype, eta, bits):
     assert int(ref["kqT"].abs().max()) > qmax // 2 and int(ref["wq"].abs().max()) > 0  # the comparison is not vacuous
 
 
+@pytest.mark.parametrize("K,V,dtype,eta,bits", [(128, 128, torch.float16, 0.0, 8), (64, 128, torch.float16, 0.5, 8),
+                                                (128, 64, torch.bfloat16, 1.0, 6), (64, 192, torch.bfloat16, 0.3, 8)])
+def test_cumsum_also_makes_the_gla_write_codes(cuda, K, V, dtype, eta, bits):
+    """The per-channel cumsum launch that also emits the write operands of the linear family's state kernel gives, bit
+    for bit, what the stand-alone pre-pass makes from the stored cumulative decay and envelope; gc and logenv are the
+    same with and without the codes."""
+    from linquant_amd.kernels.zoo import _common as C
+
+    B, T, H = 2, 192, 3
+    q, k, v, g, _ = zc.cut(zc.inputs("gla", B=B, H=H, K=K, V=V, seed=27, dtype=dtype), T)
+    k, v, g = k.cuda(), v.cuda(), g.cuda()
+    gen = torch.Generator().manual_seed(3)
+    skw = (torch.rand(H, K, generator=gen) * 0.004 + 0.001).cuda()
+    svw = (torch.rand(H, V, generator=gen) * 0.02 + 0.01).cuda()
+    qmax = 2 ** (bits - 1) - 1
+    gc0, le0 = C.cumsum(g, B, T, H, K)
+    ref = C.write_codes(k, v, None, gc0, le0, skw, svw, None, eta, qmax, (B, T, H, K, V), C.FAMILY_LINEAR, C.DECAY_DIAGONAL)
+    gc1, le1, got = C.cumsum(g, B, T, H, K, write=dict(k=k, v=v, skw=skw, svw=svw, eta=eta, qmax=qmax))
+    torch.cuda.synchronize()
+    assert torch.equal(gc0, gc1) and torch.equal(le0, le1)
+    for name in ("kqT", "vqT", "ev", "gam"):
+        assert torch.equal(got[name], ref[name]), f"{name}: differs from the stand-alone pre-pass"
+    assert int(ref["kqT"].abs().max()) > qmax // 2 and int(ref["vqT"].abs().max()) > qmax // 2
+
+
 @pytest.mark.parametrize("K,dtype,rot", [(128, torch.float16, True), (64, torch.float16, False), (128, torch.bfloat16, False),
                                          (48, torch.float16, False)])
 def test_kda_applies_dqk_inside_its_kernels(cuda, K, dtype, rot):
