@@ -21,7 +21,7 @@ import sys
 import time
 
 HBM_PEAK_GBS = 8000.0
-RAMP_MS = 50.0           # untimed back-to-back launches in front of the warm-up steps
+RAMP_MS = 100.0          # untimed back-to-back launches in front of the warm-up steps
 INT8_PEAK_TOPS = 5000.0  # published dense INT8 MFMA rate of MI355X; the measured issue peak is reported next to it
 
 # source file of each stage's kernel: a counter figure from profiles/ is attached to a stage only while that file (and the
@@ -158,6 +158,21 @@ def zoo_stage_bytes(fam, dec, B, T, H, K, V):
     out["state"] = qk // 2 + h8 + ((qk // 2 + 2 * tok + 2 * vv) if fam == "delta" else vv // 2)
     out["output"] = (2 * qk + g if dec != "diagonal" else qk // 2 + A // 2) + vv + h8 + vv
     return out
+
+
+def zoo_workload_bytes(workload):
+    """{stage: algorithmic bytes} of a zoo benchmark workload as bench_zoo runs it (the linear-attention configuration
+    takes the fused operand launch: q, k, v read once, five code tensors written, the output kernel reads codes)."""
+    cell, B, T, H, K, V, _ = ZOO_WORKLOADS[workload]
+    fam, dec = ZOO_CELLS[cell]
+    nbytes = zoo_stage_bytes(fam, dec, B, T, H, K, V)
+    nbytes["prologue"] = 2 * (B * T * H * K * 2) * 2  # q and k, read and written once
+    if fam == "linear" and dec != "diagonal" and workload != "c1":
+        qk_b, vv_b = B * T * H * K * 2, B * T * H * V * 2
+        nbytes["rotate_quant"] = 2 * qk_b + vv_b + 3 * (qk_b // 2) + 2 * (vv_b // 2)
+        nbytes["output"] = 2 * (qk_b // 2) + vv_b // 2 + B * (T // 64) * H * K * V + vv_b
+        nbytes.pop("write_codes", None)
+    return nbytes
 
 
 def copy_probe(dev):
@@ -314,13 +329,7 @@ def measure_zoo(args, workload, cpu_baseline):
     finally:
         for n, f in saved.items():
             setattr(C, n, f)
-    nbytes = zoo_stage_bytes(fam, dec, B, T, H, K, V)
-    nbytes["prologue"] = 2 * (B * T * H * K * 2) * 2  # q and k, read and written once
-    if fused:  # q, k, v read once; five code tensors written; the output kernel reads codes
-        qk_b, vv_b = B * T * H * K * 2, B * T * H * V * 2
-        nbytes["rotate_quant"] = 2 * qk_b + vv_b + 3 * (qk_b // 2) + 2 * (vv_b // 2)
-        nbytes["output"] = 2 * (qk_b // 2) + vv_b // 2 + B * (T // 64) * H * K * V + vv_b
-        nbytes.pop("write_codes", None)
+    nbytes = zoo_workload_bytes(workload)
     del qs, ks
     stages = {}
     for label, evs in records.items():
@@ -357,13 +366,19 @@ def measure_zoo(args, workload, cpu_baseline):
         qz.calibrating = True
         run()
         qz.finalize()
-        t0 = time.perf_counter()
-        run()
-        t_cpu = time.perf_counter() - t0
+        # median of up to ten runs, stopping after about two seconds of CPU work (the small first configuration takes
+        # tens of milliseconds per run, the large ones tens of seconds: one run then)
+        times, spent = [], 0.0
+        while len(times) < 10 and (not times or spent < 2.0):
+            t0 = time.perf_counter()
+            run()
+            times.append(time.perf_counter() - t0)
+            spent += times[-1]
+        t_cpu = statistics.median(times)
         frac = (hs * ts_) / (B * H * T)
         cpu = {"value": round(tokens * frac / t_cpu, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
                "sample": f"float64 torch oracle on batch 1 x {hs} of {H} heads x {ts_} tokens ({frac:.5f} of the job) in "
-                         f"{t_cpu:.2f} s; value = job-equivalent tokens/s", "host_cpus": os.cpu_count(),
+                         f"{t_cpu:.3f} s (median of {len(times)} runs); value = job-equivalent tokens/s", "host_cpus": os.cpu_count(),
                "torch_threads": torch.get_num_threads()}
     line = {
         "metric": f"prefill tokens/s per layer at T={T}", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
@@ -731,9 +746,9 @@ def measure_c5(args, regime, keyside, cpu_baseline, with_graph=False):
     # from the live timing; the matrix pipeline's busy fraction and the measured issue peak from the committed counter
     # summary, attached only while the kernel's source is unchanged since they were collected)
     int8_ops = stage_int8_ops(s)
-    counters, mfma_peak = measured_counters("c5_keyside" if keyside else "c5_valueside", "c5")
-    if regime != "strong":  # the committed counters were collected on the stated recipe's data
-        counters = {}
+    # the committed counters were collected per (absorption side, decay regime)
+    ckey = ("c5_keyside" if keyside else "c5_valueside") + ("" if regime == "strong" else "_weak")
+    counters, mfma_peak = measured_counters(ckey, "c5")
     for label, st in stages.items():
         if label in int8_ops:
             # dense-equivalent: the operations of the full contraction over the stage's time, whether or not a data-dependent
