@@ -12,8 +12,9 @@
 // for both chunks.  The diagonal block factorizes the decay weight around the block's first row whenever the decay
 // spread inside the block allows it and then runs as an fp32 MFMA product; otherwise lane (i = lane & 15, j-group =
 // lane >> 4) accumulates four (i, j) pairs with one exponential per (i, j, channel).
-// Column-wise: the wave of sub-block J fetches its own rows once, hands its anchored query codes to the other waves
-// through LDS and builds its key operand once per later sub-block I (anchored at I's first row), meeting I's query codes
+// Column-wise: the wave of sub-block J fetches its own rows once (the k and g rows then stay in registers for the whole
+// chunk), hands its anchored query codes to the other waves through LDS and builds its key operand once per later
+// sub-block I (anchored at I's first row, one operand and one sweep over the rotation at a time), meeting I's query codes
 // from LDS on the INT8 MFMA; a lane's 16 INT8 slots per contraction step hold the same channels in the query and the key
 // operand, so the dot product is exact whatever the channel -> slot map.
 // With a local R_QK (rot, (K,K) fp16, x -> x.R) the anchored off-diagonal operands are rounded to fp16 and rotated
@@ -103,9 +104,10 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   // rotated query codes of sub-blocks 1..3 of both chunks: [pass][I - 1][lane][dword]
   __shared__ __align__(16) uint32_t QC[2 * 3 * 64 * (K / 16)];
   __shared__ __align__(16) float DQs[DQ ? K : 4];
+  __shared__ __align__(16) float AN[2 * 2 * K];  // first g rows of sub-blocks 2 and 3 of both chunks: [pass][I - 2][channel]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rl = lane & 15, kg = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: branches on the sub-block index are scalar
   const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
   const int H = p.H;
   const float sq = p.sq[h], sk = p.sk[h];
@@ -134,6 +136,11 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
   const int ct = 2 * blockIdx.x + pass;
   if (ct >= nchunks) break;  // uniform over the workgroup
   const int blk = pass ? 3 - wave : wave;  // sub-block of this wave in this chunk
+  // lane coordinates, made opaque per pass: left visible, every address derived from them is computed once in front of
+  // the loop over the two chunks and kept in registers through both (spilled)
+  int lane_o = lane;
+  asm volatile("" : "+v"(lane_o));
+  const int rl = lane_o & 15, kg = lane_o >> 4;
   const int i0 = 16 * blk;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
 
@@ -149,78 +156,67 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
     constexpr int KS = K / 32, MT = K / 16;
     if (ROT && pass == 0) __syncthreads();  // R^T staged
     const int64_t roff = ((t0 + i0 + rl) * H + h) * K + 8 * kg;
-    // One step (32 channels, 8 per lane) of raw operands: own rows of q / k / g and the first rows of g of two
-    // sub-blocks (anchors; the address stays inside the chunk for every sub-block <= 3).  Steps are requested one ahead
-    // of their use.
+    // One step = 32 channels, 8 per lane, requested one step ahead of its use.  The k and g rows of the sub-block stay in
+    // registers for the whole chunk (every key operand of this sub-block, one per later sub-block, is built from them); q
+    // and the own anchor row are dropped after their step.  The anchor rows of sub-blocks 2 and 3 pass through LDS (AN) to
+    // the waves that need them after the rendezvous.
+    lq_v4i kraw[KS];
+    lq_v4f gown[KS][2];
     struct Step {
-      lq_v4i q, k;
-      lq_v4f g[2], a[2], b[2];
+      lq_v4i q;
+      lq_v4f a[2];
     };
-    auto request = [&](auto with_q, int Ia, int Ib, int ks, Step& r) {
-      if constexpr (decltype(with_q)::value) r.q = *(const lq_v4i*)(p.q + roff + 32 * ks);
-      r.k = *(const lq_v4i*)(p.k + roff + 32 * ks);
+    auto request = [&](int ks, Step& r) {
+      r.q = *(const lq_v4i*)(p.q + roff + 32 * ks);
+      kraw[ks] = *(const lq_v4i*)(p.k + roff + 32 * ks);
       const float* gp = p.g + roff + 32 * ks;
-      r.g[0] = *(const lq_v4f*)gp, r.g[1] = *(const lq_v4f*)(gp + 4);
-      const float* ap = p.g + ((t0 + 16 * Ia) * H + h) * K + 32 * ks + 8 * kg;
+      gown[ks][0] = *(const lq_v4f*)gp, gown[ks][1] = *(const lq_v4f*)(gp + 4);
+      const float* ap = p.g + ((t0 + i0) * H + h) * K + 32 * ks + 8 * kg;
       r.a[0] = *(const lq_v4f*)ap, r.a[1] = *(const lq_v4f*)(ap + 4);
-      const float* bp = p.g + ((t0 + 16 * Ib) * H + h) * K + 32 * ks + 8 * kg;
-      r.b[0] = *(const lq_v4f*)bp, r.b[1] = *(const lq_v4f*)(bp + 4);
     };
     auto unpack = [&](const lq_v4i& raw, float (&o)[8]) {
 #pragma unroll
       for (int d = 0; d < 4; ++d) zoo_dec2((uint32_t)raw[d], bf, o[2 * d], o[2 * d + 1]);
     };
-    // key rows of this sub-block anchored at the first rows of sub-blocks Ia and Ib, as fp16 rotation operands (the
-    // rows are fetched again here rather than held in registers across the first sweep: they are cache hits)
-    // (without a rotation they are quantized on the spot into ca / cb)
-    auto build_k2 = [&](int Ia, int Ib, lq_v8h (&xa)[KS], lq_v8h (&xb)[KS], uint32_t (&ca)[MT], uint32_t (&cb)[MT]) {
-      Step st[2];
-      request(std::false_type{}, Ia, Ib, 0, st[0]);
+    // key rows of this sub-block anchored at the first row of a later sub-block (anchor row `an`): fp16 rotation operand
+    // x, or, without a rotation, the codes themselves
+    auto build_k = [&](auto anchor, lq_v8h (&x)[KS], uint32_t (&c)[MT]) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 1 < KS) request(std::false_type{}, Ia, Ib, ks + 1, st[(ks + 1) & 1]);
-        const Step& r = st[ks & 1];
+        lq_v4f an[2];
+        anchor(ks, an);
         float kf[8];
-        unpack(r.k, kf);
-        int ia[8], ib[8];
+        unpack(kraw[ks], kf);
+        int ic[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float gg = r.g[e >> 2][e & 3];
-          const float va = kf[e] * zoo_exp(r.a[e >> 2][e & 3] - gg), vb = kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg);
-          if constexpr (ROT) {
-            xa[ks][e] = (_Float16)va, xb[ks][e] = (_Float16)vb;
-          } else {
-            ia[e] = zoo_q8(va, inv_sk, qmax), ib[e] = zoo_q8(vb, inv_sk, qmax);
-          }
+          const float v = kf[e] * zoo_exp(an[e >> 2][e & 3] - gown[ks][e >> 2][e & 3]);
+          if constexpr (ROT)
+            x[ks][e] = (_Float16)v;
+          else
+            ic[e] = zoo_q8(v, inv_sk, qmax);
         }
         if constexpr (!ROT) {
-          ca[2 * ks] = zoo_pack_codes(ia[0], ia[1], ia[2], ia[3]), ca[2 * ks + 1] = zoo_pack_codes(ia[4], ia[5], ia[6], ia[7]);
-          cb[2 * ks] = zoo_pack_codes(ib[0], ib[1], ib[2], ib[3]), cb[2 * ks + 1] = zoo_pack_codes(ib[4], ib[5], ib[6], ib[7]);
+          c[2 * ks] = zoo_pack_codes(ic[0], ic[1], ic[2], ic[3]), c[2 * ks + 1] = zoo_pack_codes(ic[4], ic[5], ic[6], ic[7]);
           // the codes are next used after the loop: without this anchor their arithmetic sinks there and every step's
-          // raw operands stay in registers
-          asm volatile("" : "+v"(ca[2 * ks]), "+v"(ca[2 * ks + 1]), "+v"(cb[2 * ks]), "+v"(cb[2 * ks + 1]));
+          // operands stay in registers
+          asm volatile("" : "+v"(c[2 * ks]), "+v"(c[2 * ks + 1]));
         }
-        __builtin_amdgcn_sched_barrier(0);  // keeps the look-ahead at one step
+        __builtin_amdgcn_sched_barrier(0);  // one step after the other
       }
     };
-    // one sweep over R^T for one or two operands; codes of token rl, dword mt = channels 16mt + 4kg + r
-    auto sweep = [&](auto two, const lq_v8h (&x0)[KS], const lq_v8h (&x1)[KS], float inv0, float inv1, uint32_t (&c0)[MT],
-                     uint32_t (&c1)[MT]) {
-      constexpr bool kTwo = decltype(two)::value;
+    // one sweep over R^T for one operand; codes of token rl, dword mt = channels 16mt + 4kg + r
+    auto sweep = [&](const lq_v8h (&x0)[KS], float inv0, uint32_t (&c0)[MT]) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        lq_v4f r0 = {0.f, 0.f, 0.f, 0.f}, r1 = {0.f, 0.f, 0.f, 0.f};
+        lq_v4f r0 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const lq_v8h rop = *(const lq_v8h*)(RT + (16 * mt + rl) * RS + 32 * ks + 8 * kg);
           r0 = lq_mfma_f16(rop, x0[ks], r0);
-          if constexpr (kTwo) r1 = lq_mfma_f16(rop, x1[ks], r1);
         }
         c0[mt] = zoo_pack_codes(zoo_q8(r0[0], inv0, qmax), zoo_q8(r0[1], inv0, qmax), zoo_q8(r0[2], inv0, qmax),
                                 zoo_q8(r0[3], inv0, qmax));
-        if constexpr (kTwo)
-          c1[mt] = zoo_pack_codes(zoo_q8(r1[0], inv1, qmax), zoo_q8(r1[1], inv1, qmax), zoo_q8(r1[2], inv1, qmax),
-                                  zoo_q8(r1[3], inv1, qmax));
       }
     };
     const float sqk = sq * sk;
@@ -242,44 +238,42 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
     };
 
     // own rows, fetched once: state-read codes, diagonal block (factorized around the first row while the spread is
-    // measured) and the two operands of the first sweep
-    lq_v8h xq[KS], xk[KS];
+    // measured) and the query operand anchored at the sub-block's first row
+    lq_v8h x[KS];
     uint32_t cq[MT], ck[MT];
     float spread = 0.0f;
     lq_v4f dacc = {0.f, 0.f, 0.f, 0.f};
-    const int inext = blk < 3 ? blk + 1 : 3;
     Step st[2];
-    request(std::true_type{}, blk, inext, 0, st[0]);
+    request(0, st[0]);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      if (ks + 1 < KS) request(std::true_type{}, blk, inext, ks + 1, st[(ks + 1) & 1]);
+      if (ks + 1 < KS) request(ks + 1, st[(ks + 1) & 1]);
       const Step& r = st[ks & 1];
+      const lq_v4f(&aown)[2] = r.a;
       float qf[8], kf[8];
       unpack(r.q, qf);
-      unpack(r.k, kf);
+      unpack(kraw[ks], kf);
       if constexpr (DQ) {  // D_QK at load: q' = act(q * D), what the stand-alone rescaling launch would have stored
         const lq_v4f d0 = *(const lq_v4f*)(DQs + 32 * ks + 8 * kg), d1 = *(const lq_v4f*)(DQs + 32 * ks + 8 * kg + 4);
 #pragma unroll
         for (int e = 0; e < 8; ++e) qf[e] = zoo_round_act(zoo_mul_rn(qf[e], e < 4 ? d0[e & 3] : d1[e & 3]), bf);
       }
-      int cs[8], iq[8], ik[8];
+      int cs[8], iq[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float gg = r.g[e >> 2][e & 3];
-        const float d = gg - r.a[e >> 2][e & 3];
+        const float gg = gown[ks][e >> 2][e & 3];
+        const float d = gg - aown[e >> 2][e & 3];
         spread = fmaxf(spread, __builtin_fabsf(d));
         const float ed = zoo_exp(d);
         const float qh = (float)zoo_q8(qf[e] * p.scale, inv_sq, qmax) * sq;
         const float kh = (float)zoo_q8(kf[e], inv_sk, qmax) * sk;
         dacc = __builtin_amdgcn_mfma_f32_16x16x4f32(qh * ed, kh * zoo_exp(-d), dacc, 0, 0, 0);
-        float x = qf[e] * ed;
-        x = x * p.scale;
-        const float xn = kf[e] * zoo_exp(r.b[e >> 2][e & 3] - gg);
-        if constexpr (ROT) {
-          xq[ks][e] = (_Float16)x, xk[ks][e] = (_Float16)xn;
-        } else {
-          iq[e] = zoo_q8(x, inv_sq, qmax), ik[e] = zoo_q8(xn, inv_sk, qmax);
-        }
+        float xv = qf[e] * ed;
+        xv = xv * p.scale;
+        if constexpr (ROT)
+          x[ks][e] = (_Float16)xv;
+        else
+          iq[e] = zoo_q8(xv, inv_sq, qmax);
         float y = qf[e] * zoo_exp(gg);
         y = y * p.scale;
         cs[e] = zoo_q8(y, inv_sq, qmax);
@@ -292,15 +286,22 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
       }
       if constexpr (!ROT) {
         cq[2 * ks] = zoo_pack_codes(iq[0], iq[1], iq[2], iq[3]), cq[2 * ks + 1] = zoo_pack_codes(iq[4], iq[5], iq[6], iq[7]);
-        ck[2 * ks] = zoo_pack_codes(ik[0], ik[1], ik[2], ik[3]), ck[2 * ks + 1] = zoo_pack_codes(ik[4], ik[5], ik[6], ik[7]);
-        asm volatile("" : "+v"(cq[2 * ks]), "+v"(cq[2 * ks + 1]), "+v"(ck[2 * ks]), "+v"(ck[2 * ks + 1]));  // as in build_k2
+        asm volatile("" : "+v"(cq[2 * ks]), "+v"(cq[2 * ks + 1]));  // as in build_k
       }
-      __builtin_amdgcn_sched_barrier(0);  // keeps the look-ahead at one step
+      // the diagonal block's accumulator is next used at the end of the chunk: unpinned, its products sink there and
+      // their operands wait in registers
+      asm volatile("" : "+v"(dacc), "+v"(spread));  // (the running maximum of the decay spread likewise)
+      __builtin_amdgcn_sched_barrier(0);  // one step after the other
     }
-    // first sweep: query operand of this sub-block (none for sub-block 0) and key operand for sub-block blk + 1 (none
-    // for sub-block 3)
-    if constexpr (ROT) sweep(std::true_type{}, xq, xk, inv_sq, inv_sk, cq, ck);  // sub-block 0 has no use for cq, sub-block 3 none for ck
+    if (blk >= 2 && rl == 0) {  // this sub-block's first g row: the anchor of the key operands other waves build later
+      float* an = AN + ((pass * 2 + blk - 2) * K + 8 * kg);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) *(lq_v4f*)(an + 32 * ks) = gown[ks][0], *(lq_v4f*)(an + 32 * ks + 4) = gown[ks][1];
+    }
+    // before the rendezvous: the query codes of this sub-block (none for sub-block 0) go to LDS, and the key codes for
+    // the next sub-block (none for sub-block 3) are made, so that every wave arrives with about the same work done
     if (blk > 0) {
+      if constexpr (ROT) sweep(x, inv_sq, cq);
       uint32_t* qc = QC + (((pass * 3 + blk - 1) * 64 + lane) * MT);
 #pragma unroll
       for (int s = 0; s < MT / 4; ++s) {
@@ -310,14 +311,28 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
         *(lq_v4i*)(qc + 4 * s) = o;
       }
     }
+    if (blk < 3) {
+      // (anchor row from memory, one step ahead: the sub-block that owns it has not been through the rendezvous yet)
+      const float* ap = p.g + ((t0 + 16 * (blk + 1)) * H + h) * K + 8 * kg;
+      lq_v4f nx[2][2];
+      nx[0][0] = *(const lq_v4f*)ap, nx[0][1] = *(const lq_v4f*)(ap + 4);
+      build_k(
+          [&](int ks, lq_v4f (&an)[2]) {
+            if (ks + 1 < KS) nx[(ks + 1) & 1][0] = *(const lq_v4f*)(ap + 32 * (ks + 1)), nx[(ks + 1) & 1][1] = *(const lq_v4f*)(ap + 32 * (ks + 1) + 4);
+            an[0] = nx[ks & 1][0], an[1] = nx[ks & 1][1];
+          },
+          x, ck);
+      if constexpr (ROT) sweep(x, inv_sk, ck);
+    }
     __syncthreads();  // query codes of the chunk are in LDS (the two passes use separate buffers)
     if (blk < 3) meet(blk + 1, ck);
-    // second sweep: key operands for sub-blocks blk + 2 and blk + 3
-    if (blk <= 1) {
-      build_k2(2, 3, xq, xk, cq, ck);
-      if constexpr (ROT) sweep(std::true_type{}, xq, xk, inv_sk, inv_sk, cq, ck);
-      if (blk == 0) meet(2, cq);
-      meet(3, ck);
+    // key operands for the sub-blocks after the next one, from the rows still in registers
+#pragma unroll 1
+    for (int I = blk + 2; I < 4; ++I) {
+      const float* an_s = AN + ((pass * 2 + I - 2) * K + 8 * kg);
+      build_k([&](int ks, lq_v4f (&an)[2]) { an[0] = *(const lq_v4f*)(an_s + 32 * ks), an[1] = *(const lq_v4f*)(an_s + 32 * ks + 4); }, x, ck);
+      if constexpr (ROT) sweep(x, inv_sk, ck);
+      meet(I, ck);
     }
     // diagonal block, last: its rare exact path is kept away from the registers of the sweeps
     spread = wave_max(spread);
