@@ -73,8 +73,20 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
   float* le_s = (float*)(part + 4 * K);      // [C] log envelope (CODES)
   const int k = threadIdx.x % K, q = threadIdx.x / K;
   const int SEG = C / 4;                    // tokens per thread (C is a multiple of 16)
-  const int h = blockIdx.x % H;
-  const int64_t bc = blockIdx.x / H;
+  // Workgroups are dealt to the 8 XCDs round-robin in launch order and each XCD has its own L2: workgroup L = x + 8 m takes
+  // head m % H of (batch, chunk) number x + 8 (m / H), so that one XCD handles all heads of a (batch, chunk) and writes the
+  // (B, T, H) log envelope (four bytes per token and head) as whole lines
+  const uint32_t ngroups = gridDim.x / (uint32_t)H;
+  int h;
+  int64_t bc;
+  if ((ngroups & 7u) == 0) {
+    const uint32_t m = blockIdx.x >> 3;
+    h = (int)(m % (uint32_t)H);
+    bc = (int64_t)((blockIdx.x & 7u) + 8u * (m / (uint32_t)H));
+  } else {
+    h = (int)(blockIdx.x % (uint32_t)H);
+    bc = blockIdx.x / (uint32_t)H;
+  }
   const int64_t row0 = bc * C;  // global token row of the chunk start (b * T + chunk * C)
   const int64_t base = ((row0 + q * SEG) * H + h) * K + k;
   const int64_t tstride = (int64_t)H * K;

@@ -108,7 +108,23 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: branches on the sub-block index are scalar
-  const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+  // Flat grid.  Workgroups are dealt to the 8 XCDs round-robin in launch order and each XCD has its own L2.  Workgroup
+  // L = x + 8 m (x = its XCD) takes head m % H of (batch, chunk pair) number x + 8 (m / H): the workgroups resident on one
+  // XCD at a time then cover all heads of a few (batch, chunk pair)s, whose rows lie next to each other in memory, and
+  // the eight XCDs work on neighbouring chunks at the same time.
+  const int npairs = (p.T / 64 + 1) / 2;
+  const uint32_t ngroups = (uint32_t)p.B * (uint32_t)npairs;
+  uint32_t group, hh;
+  if ((ngroups & 7u) == 0) {
+    const uint32_t m = blockIdx.x >> 3;
+    hh = m % (uint32_t)p.H;
+    group = (blockIdx.x & 7u) + 8u * (m / (uint32_t)p.H);
+  } else {
+    hh = blockIdx.x % (uint32_t)p.H;
+    group = blockIdx.x / (uint32_t)p.H;
+  }
+  const int h = (int)hh;
+  const int pair = (int)(group % (uint32_t)npairs), b = (int)(group / (uint32_t)npairs);
   const int H = p.H;
   const float sq = p.sq[h], sk = p.sk[h];
   const float inv_sq = 1.0f / sq, inv_sk = 1.0f / sk;
@@ -133,7 +149,7 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
 
 #pragma unroll 1
   for (int pass = 0; pass < 2; ++pass) {
-  const int ct = 2 * blockIdx.x + pass;
+  const int ct = 2 * pair + pass;
   if (ct >= nchunks) break;  // uniform over the workgroup
   const int blk = pass ? 3 - wave : wave;  // sub-block of this wave in this chunk
   // lane coordinates, made opaque per pass: left visible, every address derived from them is computed once in front of
@@ -371,7 +387,8 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   p.dq = a->dq;
   p.sq = a->sq, p.sk = a->sk, p.rot = (const _Float16*)a->rot, p.scale = a->scale, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads;
-  dim3 grid((a->seqlen / 64 + 1) / 2, a->batch * a->nheads);
+  if ((int64_t)((a->seqlen / 64 + 1) / 2) * a->batch * a->nheads > 0x7fffffff) return LQ_ERR_SHAPE;
+  dim3 grid((uint32_t)(((a->seqlen / 64 + 1) / 2) * a->batch * a->nheads));
 #define LQ_A_LAUNCH3(KV, ROTV, BFV, QGV)                                                                   \
   do {                                                                                                     \
     if (p.dq)                                                                                              \

@@ -303,16 +303,31 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
-  const int ct = blockIdx.x;
-  const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+  // Flat grid.  Workgroups are dealt to the 8 XCDs round-robin in launch order and each XCD has its own L2.  Workgroup
+  // L = x + 8 m (x = its XCD) takes head m % H of (batch, chunk) number x + 8 (m / H): the workgroups resident on one XCD
+  // at a time then cover all heads of a few (batch, chunk)s, so the (B, T, H) tensors (beta, the log envelope, fw, ev:
+  // four bytes per token and head, a head's values 4 H bytes apart) are fetched and written as whole lines by that XCD
+  // instead of one line per value, and the eight XCDs work on neighbouring chunks at the same time.
+  const uint32_t ngroups = (uint32_t)p.B * (uint32_t)p.NT;
+  uint32_t group, hh;
+  if ((ngroups & 7u) == 0) {
+    const uint32_t m = blockIdx.x >> 3;
+    hh = m % (uint32_t)p.H;
+    group = (blockIdx.x & 7u) + 8u * (m / (uint32_t)p.H);
+  } else {
+    hh = blockIdx.x % (uint32_t)p.H;
+    group = blockIdx.x / (uint32_t)p.H;
+  }
+  const int h = (int)hh;
+  const int ct = (int)(group % (uint32_t)p.NT), b = (int)(group / (uint32_t)p.NT);
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
   const float sigma = p.sigma, tau = p.tau;
   constexpr bool bf = BF;
 
   if (DK && tid < K) {
-    dk_s[tid] = p.dk_div[blockIdx.y % p.H * K + tid];
-    dk_s[128 + tid] = p.dk_rcp[blockIdx.y % p.H * K + tid];
+    dk_s[tid] = p.dk_div[h * K + tid];
+    dk_s[128 + tid] = p.dk_rcp[h * K + tid];
   }
   // ---- per-token factors; fw is written straight out
   if (tid < 64) {
@@ -770,6 +785,7 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   p.kqT = a->kqT, p.wq = a->wq, p.ev = a->ev, p.gam = a->gam, p.logenv = a->logenv, p.skw = a->skw, p.sw = a->sw;
   p.eta = a->eta, p.qmax = a->qmax, p.NT = a->seqlen / 64;
   p.dk_div = a->dk_div, p.dk_rcp = a->dk_rcp;
-  dim3 grid(a->seqlen / 64, a->batch * a->nheads);
+  if ((int64_t)(a->seqlen / 64) * a->batch * a->nheads > 0x7fffffff) return LQ_ERR_SHAPE;
+  dim3 grid((uint32_t)((a->seqlen / 64) * a->batch * a->nheads));
   return a->kdim == 128 ? launch_decay<128>(p, a->decay, grid, stream) : launch_decay<64>(p, a->decay, grid, stream);
 }
