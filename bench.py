@@ -196,6 +196,33 @@ def hadamard_signed(n, seed, device):
     return (Hm / n ** 0.5 * signs).to(device)
 
 
+def timed_steps(step, warmup, steps):
+    """``warmup`` untimed steps, then the wall time of exactly ``steps`` steps between two synchronizations, in ms per step.
+    The interpreter's cyclic garbage collector is off for the duration (as ``timeit`` does): a full collection stops the
+    launching thread for 30-40 ms about once per 500 steps of this script, longer than the launches queued ahead of the
+    GPU last, so a timed region that happens to contain one measures that pause (seen: 50 steps at 0.27 ms each reported
+    as 0.94 ms per step)."""
+    import gc
+
+    import torch
+
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        if was_enabled:
+            gc.enable()
+
+
 def ramp(step, min_ms=RAMP_MS):
     """Runs ``step`` back to back for at least ``min_ms`` of wall time, untimed: the GPU's clocks rise under sustained
     load, and a timed region of a few milliseconds right after an idle period would measure that rise, not the kernels.
@@ -292,14 +319,7 @@ def measure_zoo(args, workload, cpu_baseline):
     if args.copy_probe:
         copy_probe(dev)
     ramp_steps = 0 if args.no_ramp else ramp(lambda: call(sc))
-    for _ in range(args.warmup):
-        call(sc)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        call(sc)
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = timed_steps(lambda: call(sc), args.warmup, args.steps)
     tokens = B * T
 
     records = {}
@@ -401,8 +421,9 @@ def bench_zoo(args):
 
 
 def ramp_note(n):
-    return (f"{n} untimed steps (at least {RAMP_MS:.0f} ms of back-to-back launches) ran before the --warmup steps, so that the "
-            "timed steps do not measure the clocks rising from idle") if n else "none"
+    gc_note = "; the interpreter's cyclic garbage collector is off during the warm-up and timed steps"
+    return ((f"{n} untimed steps (at least {RAMP_MS:.0f} ms of back-to-back launches) ran before the --warmup steps, so that the "
+             "timed steps do not measure the clocks rising from idle") if n else "none") + gc_note
 
 
 def bench_front(args):
@@ -506,14 +527,7 @@ def bench_layer(args):
     def step():
         return layer(hidden)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = timed_steps(step, args.warmup, args.steps)
 
     records = {}
 
@@ -588,14 +602,7 @@ def _stage_bench(args, stages, step_names, tokens, dtype, cpu_sample, workload):
         for name in step_names:
             stages[name][0]()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = timed_steps(step, args.warmup, args.steps)
     out = {}
     for name, (fn, nbytes) in stages.items():
         ts = []
@@ -673,14 +680,7 @@ def measure_c5(args, regime, keyside, cpu_baseline, with_graph=False):
     if args.copy_probe:
         copy_probe(dev)
     ramp_steps = 0 if args.no_ramp else ramp(step)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = timed_steps(step, args.warmup, args.steps)
     tokens = s.batch * s.seqlen
 
     # ---- per-stage durations: HIP events on the launch stream around every stage call (separate pass)
@@ -781,14 +781,7 @@ def measure_c5(args, regime, keyside, cpu_baseline, with_graph=False):
         torch.cuda.synchronize()
         with torch.cuda.graph(g):
             step()
-        for _ in range(args.warmup):
-            g.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            g.replay()
-        torch.cuda.synchronize()
-        gms = (time.perf_counter() - t0) * 1e3 / args.steps
+        gms = timed_steps(g.replay, args.warmup, args.steps)
         graph = {"ms_per_step": round(gms, 4), "tokens_per_s": round(tokens / gms * 1e3, 1)}
 
     # ---- CPU baseline: the CPU oracle on a bounded sample (batch 1 x a few heads x full length), same seeds
