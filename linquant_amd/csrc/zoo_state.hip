@@ -90,25 +90,37 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
     }
   }
 
-  auto load_step = [&](int ct, StepOps<DELTA, K, BV>& o) {
+  // part: 0 = everything, 1 = key codes and chunk decays, 2 = state-read codes and U, 3 = per-token factors (delta family)
+  auto load_part = [&](auto part_c, int ct, StepOps<DELTA, K, BV>& o) {
+    constexpr int part = decltype(part_c)::value;
     const int64_t cb = ((int64_t)b * NT + ct) * H + h;
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
+    if constexpr (part == 0 || part == 1) {
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-      const int row = KR * wave + 16 * kt;
-      o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + row + rl) * 64 + 16 * kg);
-      o.gam[kt] = *(const lq_v4f*)(p.gam + cb * K + row + 4 * kg);
+      for (int kt = 0; kt < KT; ++kt) {
+        const int row = KR * wave + 16 * kt;
+        o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + row + rl) * 64 + 16 * kg);
+        o.gam[kt] = *(const lq_v4f*)(p.gam + cb * K + row + 4 * kg);
+      }
     }
     if constexpr (!DELTA) {
+      if constexpr (part == 0 || part == 1)
 #pragma unroll
       for (int vt = 0; vt < VT; ++vt) o.vop[vt] = *(const lq_v4i*)(p.vqT + (cb * V + v0 + 16 * vt + rl) * 64 + 16 * kg);
     } else {
+      if constexpr (part == 0 || part == 2) {
 #pragma unroll
-      for (int ks = 0; ks < K / 64; ++ks)
-        o.wop[ks] = *(const lq_v4i*)(p.wq + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
+        for (int ks = 0; ks < K / 64; ++ks)
+          o.wop[ks] = *(const lq_v4i*)(p.wq + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
+      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int64_t tr = (t0 + 16 * wave + 4 * kg + r) * H + h;
+        if constexpr (part == 0 || part == 3) {
+          o.fw[r] = p.fw[tr];
+          o.ev[r] = p.ev[tr];
+        }
+        if constexpr (part == 1 || part == 3) continue;
         const _Float16* up = p.u + tr * V + v0 + NJ * rl;
         if constexpr (NJ == 4) {
           const lq_v2i uu = *(const lq_v2i*)up;
@@ -118,11 +130,10 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
         } else {
           o.u[r][0] = *(const uint16_t*)up, o.u[r][1] = 0;
         }
-        o.fw[r] = p.fw[tr];
-        o.ev[r] = p.ev[tr];
       }
     }
   };
+  auto load_step = [&](int ct, StepOps<DELTA, K, BV>& o) { load_part(std::integral_constant<int, 0>{}, ct, o); };
 
   float hc[KT][VT][4];
 #pragma unroll
@@ -151,7 +162,11 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       }
     // requested unconditionally (the last chunks re-request the final one): a branch around the loads would make the
     // compiler's count of outstanding memory operations path-dependent, and it then waits for the newest loads as well
-    load_step(min(ct + 2, NT - 1), pre);
+    const int ctn = min(ct + 2, NT - 1);
+    if constexpr (DELTA)
+      load_part(std::integral_constant<int, 1>{}, ctn, pre);  // (the delta family spreads its requests over the step, below)
+    else
+      load_step(ctn, pre);
     __syncthreads();
 
     // ---- copy the stored state out, coalesced: h_i8[b][ct][h][v0 + v][k]
@@ -185,6 +200,9 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
           const lq_v4i hop = *(const lq_v4i*)(hTb + (NJ * rl + jj) * HS + 64 * ks + 16 * kg);
           aw[jj] = lq_mfma_i8(cur.wop[ks], hop, aw[jj]);
         }
+      // the rest of chunk ct + 2's operands are requested while the matrix unit and then the vector ALU are busy: one wave
+      // per SIMD issues in order, and 18 requests in a row held it for as long as the memory pipeline took to accept them
+      load_part(std::integral_constant<int, 2>{}, ctn, pre);
       // lane holds tokens 16*wave + 4kg + r, value columns v0 + NJ*rl + jj
       uint32_t ecode[NJ][4];
 #pragma unroll
@@ -210,6 +228,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
           *(uint16_t*)(p.e_out + off) = zoo_enc1(ef[0], bf);
         }
       }
+      load_part(std::integral_constant<int, 3>{}, ctn, pre);
 #pragma unroll
       for (int jj = 0; jj < NJ; ++jj)
         *(uint32_t*)(eT + (NJ * rl + jj) * ES + 16 * wave + 4 * kg) =
