@@ -389,6 +389,10 @@ typedef struct {
   int32_t family;
   int32_t vtile;             /* value columns per workgroup: 16, 32, 64, or 0 = chosen from the grid size */
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
+  /* Optional (delta family): fw, ev and gam once more, packed per (batch, chunk, head) as 64 + 64 + K consecutive floats
+   * (what lq_zoo_wy_prep writes into its `pack`): the kernel then fetches a chunk's per-token factors and row decays
+   * from three contiguous pieces instead of 64 addresses 4 H bytes apart.  NULL: fw, ev and gam are read. */
+  const float* pack;         /* (B,NT,H,128+K) fp32 or NULL */
 } lq_zoo_state_args;
 int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
 
@@ -480,6 +484,9 @@ typedef struct {
    * write-operand codes above (kqT set). */
   const float* dk_div;       /* (H,K) fp32 D_QK, finite and positive */
   const float* dk_rcp;       /* (H,K) fp32 RN(1 / dk_div) */
+  /* Optional, with the write-operand codes: fw, ev and gam once more, packed per (batch, chunk, head) as 64 + 64 + K
+   * consecutive floats, the layout lq_zoo_state reads a chunk's factors from in three contiguous pieces. */
+  float* pack;               /* (B,NT,H,128+K) fp32 or NULL */
 } lq_zoo_wy_prep_args;
 int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* args, hipStream_t stream);
 

@@ -12,6 +12,7 @@ struct ZooStateParams {
   const float* fw;
   const float* ev;
   const float* gam;
+  const float* pack;  // fw | ev | gam per (batch, chunk, head), 64 + 64 + K floats, or nullptr
   int8_t* h_i8;
   _Float16* e_out;
   float* ht;

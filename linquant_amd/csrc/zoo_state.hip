@@ -26,11 +26,15 @@ using StateParams = ZooStateParams;
 template <bool DELTA, int K, int BV>
 struct StepOps {
   lq_v4i kop[K / 64];                  // key write codes: rows of this wave, 16 token slots of the lane's group
-  lq_v4f gam[K / 64];                  // chunk decay of the lane's 4 carry rows per row tile
+  lq_v4f gam[DELTA ? 1 : K / 64];      // linear: chunk decay of the lane's 4 carry rows per row tile
   lq_v4i vop[DELTA ? 1 : BV / 16];     // linear: value write codes
   lq_v4i wop[DELTA ? K / 64 : 1];      // delta: state-read codes of token 16*wave + (lane & 15)
   uint32_t u[DELTA ? 4 : 1][2];        // delta: U of tokens 16*wave + 4*(lane >> 4) + r, BV/16 adjacent columns
-  float fw[DELTA ? 4 : 1], ev[DELTA ? 4 : 1];
+  // delta: one value per lane of what the wave needs per token and per carry row: lanes 0..15 fw of tokens 16*wave + lane,
+  // lanes 16..31 ev of the same tokens, lanes 32.. the chunk decay of carry rows K/4*wave + lane - 32.  One request
+  // instead of ten (each of which every lane of a row group repeated); the values reach the lanes that use them through
+  // a wave-private piece of LDS.
+  float misc;
 };
 
 // BF (bf16 activations) is a template parameter: as a run-time flag every decode / encode of U and E in the chunk loop
@@ -47,6 +51,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 
   __shared__ __align__(16) unsigned char hT[(DELTA ? 1 : 2) * BV * HS];
   __shared__ __align__(16) unsigned char eT[DELTA ? BV * ES : 16];
+  __shared__ __align__(16) float misc_lds[DELTA ? 256 : 4];  // 64 floats per wave, written and read by that wave only
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -90,7 +95,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
     }
   }
 
-  // part: 0 = everything, 1 = key codes and chunk decays, 2 = state-read codes and U, 3 = per-token factors (delta family)
+  // part: 0 = everything, 1 = key codes, chunk decays and (delta family) per-token factors, 2 = state-read codes and U
   auto load_part = [&](auto part_c, int ct, StepOps<DELTA, K, BV>& o) {
     constexpr int part = decltype(part_c)::value;
     const int64_t cb = ((int64_t)b * NT + ct) * H + h;
@@ -100,7 +105,16 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       for (int kt = 0; kt < KT; ++kt) {
         const int row = KR * wave + 16 * kt;
         o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + row + rl) * 64 + 16 * kg);
-        o.gam[kt] = *(const lq_v4f*)(p.gam + cb * K + row + 4 * kg);
+        if constexpr (!DELTA) o.gam[kt] = *(const lq_v4f*)(p.gam + cb * K + row + 4 * kg);
+      }
+      if constexpr (DELTA) {
+        const int64_t tr = (t0 + 16 * wave + (lane & 15)) * H + h;
+        const float* src = lane < 16 ? p.fw + tr : lane < 32 ? p.ev + tr : p.gam + cb * K + KR * wave + min(lane - 32, KR - 1);
+        if (p.pack) {  // the same values, contiguous per (batch, chunk, head): fw[64] | ev[64] | gam[K]
+          const float* pk = p.pack + cb * (128 + K);
+          src = lane < 32 ? pk + 64 * (lane >> 4) + 16 * wave + (lane & 15) : pk + 128 + KR * wave + min(lane - 32, KR - 1);
+        }
+        o.misc = *src;
       }
     }
     if constexpr (!DELTA) {
@@ -116,11 +130,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int64_t tr = (t0 + 16 * wave + 4 * kg + r) * H + h;
-        if constexpr (part == 0 || part == 3) {
-          o.fw[r] = p.fw[tr];
-          o.ev[r] = p.ev[tr];
-        }
-        if constexpr (part == 1 || part == 3) continue;
+        if constexpr (part == 1) continue;
         const _Float16* up = p.u + tr * V + v0 + NJ * rl;
         if constexpr (NJ == 4) {
           const lq_v2i uu = *(const lq_v2i*)up;
@@ -150,6 +160,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
   auto do_step = [&](int ct, StepOps<DELTA, K, BV>& cur, StepOps<DELTA, K, BV>& pre) {
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
     unsigned char* hTb = hT + (DELTA ? 0 : (ct & 1) * BV * HS);
+    float* misc_s = misc_lds + 64 * wave;
+    if constexpr (DELTA) misc_s[lane] = cur.misc;
     // ---- stored copy of the incoming state -> LDS (V-major)
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
@@ -205,6 +217,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       load_part(std::integral_constant<int, 2>{}, ctn, pre);
       // lane holds tokens 16*wave + 4kg + r, value columns v0 + NJ*rl + jj
       uint32_t ecode[NJ][4];
+      const lq_v4f fw4 = *(const lq_v4f*)(misc_s + 4 * kg), ev4 = *(const lq_v4f*)(misc_s + 16 + 4 * kg);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + NJ * rl;
@@ -214,8 +227,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
           float ws = (float)aw[jj][r] * sw;
           ws = ws * ss_d[jj];
           const float u = zoo_dec1((cur.u[r][jj >> 1] >> (16 * (jj & 1))) & 0xffffu, bf);
-          ef[jj] = (u - ws) * cur.fw[r];
-          ecode[jj][r] = (uint32_t)zoo_q8(ef[jj] * cur.ev[r], inv_ew_d[jj], qmax);
+          ef[jj] = (u - ws) * fw4[r];
+          ecode[jj][r] = (uint32_t)zoo_q8(ef[jj] * ev4[r], inv_ew_d[jj], qmax);
         }
         if constexpr (NJ == 4) {
           lq_v2i eo;
@@ -228,7 +241,6 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
           *(uint16_t*)(p.e_out + off) = zoo_enc1(ef[0], bf);
         }
       }
-      load_part(std::integral_constant<int, 3>{}, ctn, pre);
 #pragma unroll
       for (int jj = 0; jj < NJ; ++jj)
         *(uint32_t*)(eT + (NJ * rl + jj) * ES + 16 * wave + 4 * kg) =
@@ -247,11 +259,16 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const lq_v4i a = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
+        lq_v4f gam4;
+        if constexpr (DELTA)
+          gam4 = *(const lq_v4f*)(misc_s + 32 + 16 * kt + 4 * kg);
+        else
+          gam4 = cur.gam[kt];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float prod = (float)a[r] * skw_r[kt][r];
           prod = prod * svw_c[vt];
-          hc[kt][vt][r] = hc[kt][vt][r] * cur.gam[kt][r] + prod;
+          hc[kt][vt][r] = hc[kt][vt][r] * gam4[r] + prod;
         }
       }
     }
@@ -340,6 +357,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   p.h_i8 = a->h_i8, p.e_out = (_Float16*)a->e_out, p.ht = a->ht;
   p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.ss = a->ss, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.unrot = (const _Float16*)a->unrot;
+  p.pack = a->pack;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   if (a->unrot) return zoo_state_unrot_launch(p, delta, a->kdim, a->batch, stream);
   // narrower V tiles when batch*head alone cannot fill the 256 compute units

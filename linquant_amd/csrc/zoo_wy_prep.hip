@@ -48,6 +48,7 @@ struct WyParams {
   int NT;
   const float* dk_div;  // (H,K) D_QK applied to k at load (k' = act(k / D)), with its reciprocal; or nullptr
   const float* dk_rcp;
+  float* pack;  // fw | ev | gam per (batch, chunk, head), 64 + 64 + K floats, or nullptr
 };
 
 LQ_DEV float powb(float b, float e) {
@@ -334,7 +335,11 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
     const float bt = p.beta[(t0 + tid) * H + h];
     bs_s[tid] = powb(bt, sigma);
     bh_s[tid] = powb(bt, 1.0f - sigma);
-    p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
+    const float fwv = powb(bt, (1.0f - sigma) * (1.0f - tau));
+    p.fw[(t0 + tid) * H + h] = fwv;
+    if constexpr (CODES) {
+      if (p.pack) p.pack[(((int64_t)b * p.NT + ct) * H + h) * (128 + K) + tid] = fwv;
+    }
     if (DECAY == LQ_DECAY_SCALAR) gs_s[tid] = p.g[(t0 + tid) * H + h];
   }
   if constexpr (CODES) {
@@ -344,6 +349,7 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
       if (DECAY == LQ_DECAY_SCALAR) evv = zoo_exp(p.eta * (p.g[(t0 + 63) * H + h] - p.g[(t0 + tid) * H + h]));
       if (DECAY == LQ_DECAY_DIAGONAL) evv = zoo_exp(p.eta * p.logenv[(t0 + tid) * H + h]);
       p.ev[(t0 + tid) * H + h] = evv;
+      if (p.pack) p.pack[(((int64_t)b * p.NT + ct) * H + h) * (128 + K) + 64 + tid] = evv;
     }
     if (tid < K) {
       float gm = 1.0f, gl = 0.0f;
@@ -353,6 +359,7 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
         gm = zoo_exp(gl);
       }
       p.gam[(((int64_t)b * p.NT + ct) * H + h) * K + tid] = gm;
+      if (p.pack) p.pack[(((int64_t)b * p.NT + ct) * H + h) * (128 + K) + 128 + tid] = gm;
       if (DECAY == LQ_DECAY_DIAGONAL) glast_s[tid] = gl;
       iskw_s[tid] = 1.0f / p.skw[h * K + tid];
     }
@@ -769,6 +776,7 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   if (codes && (a->qmax < 1 || a->qmax > 127)) return LQ_ERR_SHAPE;
   if (codes && (!zoo_al(a->kqT, 16) || !zoo_al(a->wq, 4) || !zoo_al(a->skw, 16))) return LQ_ERR_SHAPE;
   if ((a->dk_div != nullptr) != (a->dk_rcp != nullptr)) return LQ_ERR_NULL;
+  if (a->pack && (!codes || !zoo_al(a->pack, 16))) return LQ_ERR_SHAPE;
   if (a->dk_div && !codes) return LQ_ERR_SHAPE;  // built for the launch that also makes the write operands
   if (a->dk_div && (!zoo_al(a->dk_div, 16) || !zoo_al(a->dk_rcp, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
@@ -785,6 +793,7 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   p.kqT = a->kqT, p.wq = a->wq, p.ev = a->ev, p.gam = a->gam, p.logenv = a->logenv, p.skw = a->skw, p.sw = a->sw;
   p.eta = a->eta, p.qmax = a->qmax, p.NT = a->seqlen / 64;
   p.dk_div = a->dk_div, p.dk_rcp = a->dk_rcp;
+  p.pack = a->pack;
   if ((int64_t)(a->seqlen / 64) * a->batch * a->nheads > 0x7fffffff) return LQ_ERR_SHAPE;
   dim3 grid((uint32_t)((a->seqlen / 64) * a->batch * a->nheads));
   return a->kdim == 128 ? launch_decay<128>(p, a->decay, grid, stream) : launch_decay<64>(p, a->decay, grid, stream);

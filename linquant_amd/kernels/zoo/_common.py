@@ -186,7 +186,7 @@ def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, fa
               gam=_lib.ptr(c["gam"]), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
               svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), qmax=int(qmax), batch=B, seqlen=T, nheads=H,
               kdim=K, vdim=V, chunk_size=CHUNK, family=family, vtile=int(vtile),
-              act_dtype=act_code(value))
+              act_dtype=act_code(value), pack=_lib.ptr(c.get("pack")) if delta else None)
 
 
 def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
@@ -280,9 +280,11 @@ def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True
         c = {"kqT": torch.empty(B, NT, H, K, CHUNK, dtype=torch.int8, device=dev), "vqT": None,
              "wq": torch.empty(B, T, H, K, dtype=torch.int8, device=dev),
              "ev": torch.empty(B, T, H, dtype=torch.float32, device=dev),
-             "gam": torch.empty(B, NT, H, K, dtype=torch.float32, device=dev)}
+             "gam": torch.empty(B, NT, H, K, dtype=torch.float32, device=dev),
+             # fw | ev | gam once more, contiguous per (batch, chunk, head): what the state kernel fetches them from
+             "pack": torch.empty(B, NT, H, 128 + K, dtype=torch.float32, device=dev)}
         skw = _lib.aligned(write["skw"])
-        extra = dict(kqT=_lib.ptr(c["kqT"]), wq=_lib.ptr(c["wq"]), ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]),
+        extra = dict(kqT=_lib.ptr(c["kqT"]), wq=_lib.ptr(c["wq"]), ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]), pack=_lib.ptr(c["pack"]),
                      logenv=_lib.ptr(write["logenv"]), skw=_lib.ptr(skw), sw=_lib.ptr(write["sw"]), eta=float(write["eta"]),
                      qmax=int(write["qmax"]))
     _lib.call("lq_zoo_wy_prep", dev, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
