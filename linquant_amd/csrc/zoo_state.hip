@@ -29,7 +29,7 @@ struct StepOps {
   lq_v4f gam[DELTA ? 1 : K / 64];      // linear: chunk decay of the lane's 4 carry rows per row tile
   lq_v4i vop[DELTA ? 1 : BV / 16];     // linear: value write codes
   lq_v4i wop[DELTA ? K / 64 : 1];      // delta: state-read codes of token 16*wave + (lane & 15)
-  uint32_t u[DELTA ? 4 : 1][2];        // delta: U of tokens 16*wave + 4*(lane >> 4) + r, BV/16 adjacent columns
+  uint32_t uraw[DELTA ? BV / 8 : 1];   // delta: U of token 16*wave + (lane >> 2), columns BV/4 * (lane & 3) .. + BV/4 - 1
   // delta: one value per lane of what the wave needs per token and per carry row: lanes 0..15 fw of tokens 16*wave + lane,
   // lanes 16..31 ev of the same tokens, lanes 32.. the chunk decay of carry rows K/4*wave + lane - 32.  One request
   // instead of ten (each of which every lane of a row group repeated); the values reach the lanes that use them through
@@ -52,6 +52,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
   __shared__ __align__(16) unsigned char hT[(DELTA ? 1 : 2) * BV * HS];
   __shared__ __align__(16) unsigned char eT[DELTA ? BV * ES : 16];
   __shared__ __align__(16) float misc_lds[DELTA ? 256 : 4];  // 64 floats per wave, written and read by that wave only
+  constexpr int US = 2 * BV + 16;  // byte stride of a token row of the wave-private U / E tile (bank-conflict-free column reads)
+  __shared__ __align__(16) unsigned char ue_lds[DELTA ? 4 * 16 * US : 16];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -127,18 +129,21 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
         for (int ks = 0; ks < K / 64; ++ks)
           o.wop[ks] = *(const lq_v4i*)(p.wq + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
       }
+      if constexpr (part == 0 || part == 2) {
+        // the wave's 16 x BV tile of U, whole row pieces: lane -> token lane / 4, a quarter of the tile's columns (one request
+        // where four requests of a few bytes per lane stood); it reaches the lanes that use it through wave-private LDS
+        const _Float16* up = p.u + ((t0 + 16 * wave + (lane >> 2)) * H + h) * V + v0 + (BV / 4) * (lane & 3);
+        if constexpr (BV == 64) {
+          const lq_v4i a = *(const lq_v4i*)up, c = *(const lq_v4i*)(up + 8);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int64_t tr = (t0 + 16 * wave + 4 * kg + r) * H + h;
-        if constexpr (part == 1) continue;
-        const _Float16* up = p.u + tr * V + v0 + NJ * rl;
-        if constexpr (NJ == 4) {
-          const lq_v2i uu = *(const lq_v2i*)up;
-          o.u[r][0] = (uint32_t)uu[0], o.u[r][1] = (uint32_t)uu[1];
-        } else if constexpr (NJ == 2) {
-          o.u[r][0] = *(const uint32_t*)up, o.u[r][1] = 0;
+          for (int d = 0; d < 4; ++d) o.uraw[d] = (uint32_t)a[d], o.uraw[4 + d] = (uint32_t)c[d];
+        } else if constexpr (BV == 32) {
+          const lq_v4i a = *(const lq_v4i*)up;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) o.uraw[d] = (uint32_t)a[d];
         } else {
-          o.u[r][0] = *(const uint16_t*)up, o.u[r][1] = 0;
+          const lq_v2i a = *(const lq_v2i*)up;
+          o.uraw[0] = (uint32_t)a[0], o.uraw[1] = (uint32_t)a[1];
         }
       }
     }
@@ -161,7 +166,19 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
     unsigned char* hTb = hT + (DELTA ? 0 : (ct & 1) * BV * HS);
     float* misc_s = misc_lds + 64 * wave;
-    if constexpr (DELTA) misc_s[lane] = cur.misc;
+    unsigned char* ue_s = ue_lds + wave * 16 * US;
+    if constexpr (DELTA) {
+      misc_s[lane] = cur.misc;
+      unsigned char* ud = ue_s + (lane >> 2) * US + (BV / 2) * (lane & 3);
+      if constexpr (BV == 64) {
+        *(lq_v4i*)ud = lq_v4i{(int)cur.uraw[0], (int)cur.uraw[1], (int)cur.uraw[2], (int)cur.uraw[3]};
+        *(lq_v4i*)(ud + 16) = lq_v4i{(int)cur.uraw[4], (int)cur.uraw[5], (int)cur.uraw[6], (int)cur.uraw[7]};
+      } else if constexpr (BV == 32) {
+        *(lq_v4i*)ud = lq_v4i{(int)cur.uraw[0], (int)cur.uraw[1], (int)cur.uraw[2], (int)cur.uraw[3]};
+      } else {
+        *(lq_v2i*)ud = lq_v2i{(int)cur.uraw[0], (int)cur.uraw[1]};
+      }
+    }
     // ---- stored copy of the incoming state -> LDS (V-major)
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
@@ -220,13 +237,23 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       const lq_v4f fw4 = *(const lq_v4f*)(misc_s + 4 * kg), ev4 = *(const lq_v4f*)(misc_s + 16 + 4 * kg);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + NJ * rl;
+        // U of (token 4kg + r, columns NJ*rl ..) from the wave's tile; E goes back to the same place
+        unsigned char* cell = ue_s + (4 * kg + r) * US + 2 * NJ * rl;
+        uint32_t uw[2] = {0u, 0u};
+        if constexpr (NJ == 4) {
+          const lq_v2i uu = *(const lq_v2i*)cell;
+          uw[0] = (uint32_t)uu[0], uw[1] = (uint32_t)uu[1];
+        } else if constexpr (NJ == 2) {
+          uw[0] = *(const uint32_t*)cell;
+        } else {
+          uw[0] = *(const uint16_t*)cell;
+        }
         float ef[NJ];
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) {
           float ws = (float)aw[jj][r] * sw;
           ws = ws * ss_d[jj];
-          const float u = zoo_dec1((cur.u[r][jj >> 1] >> (16 * (jj & 1))) & 0xffffu, bf);
+          const float u = zoo_dec1((uw[jj >> 1] >> (16 * (jj & 1))) & 0xffffu, bf);
           ef[jj] = (u - ws) * fw4[r];
           ecode[jj][r] = (uint32_t)zoo_q8(ef[jj] * ev4[r], inv_ew_d[jj], qmax);
         }
@@ -234,11 +261,24 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
           lq_v2i eo;
           eo[0] = (int)zoo_enc2(ef[0], ef[1], bf);
           eo[1] = (int)zoo_enc2(ef[2], ef[3], bf);
-          *(lq_v2i*)(p.e_out + off) = eo;
+          *(lq_v2i*)cell = eo;
         } else if constexpr (NJ == 2) {
-          *(uint32_t*)(p.e_out + off) = zoo_enc2(ef[0], ef[1], bf);
+          *(uint32_t*)cell = zoo_enc2(ef[0], ef[1], bf);
         } else {
-          *(uint16_t*)(p.e_out + off) = zoo_enc1(ef[0], bf);
+          *(uint16_t*)cell = zoo_enc1(ef[0], bf);
+        }
+      }
+      {
+        // the wave's E tile leaves as whole row pieces, the way U came in
+        const unsigned char* es = ue_s + (lane >> 2) * US + (BV / 2) * (lane & 3);
+        _Float16* ep = p.e_out + ((t0 + 16 * wave + (lane >> 2)) * H + h) * V + v0 + (BV / 4) * (lane & 3);
+        if constexpr (BV == 64) {
+          *(lq_v4i*)ep = *(const lq_v4i*)es;
+          *(lq_v4i*)(ep + 8) = *(const lq_v4i*)(es + 16);
+        } else if constexpr (BV == 32) {
+          *(lq_v4i*)ep = *(const lq_v4i*)es;
+        } else {
+          *(lq_v2i*)ep = *(const lq_v2i*)es;
         }
       }
 #pragma unroll
@@ -349,7 +389,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (a->vtile != 0 && a->vtile != 16 && a->vtile != 32 && a->vtile != 64) return LQ_ERR_SHAPE;
   if (!zoo_al(a->kqT, 16) || !zoo_al(a->gam, 16) || !zoo_al(a->h_i8, 16) || (!delta && !zoo_al(a->vqT, 16)) ||
-      (delta && (!zoo_al(a->wq, 16) || !zoo_al(a->u, 8) || !zoo_al(a->e_out, 8))))
+      (delta && (!zoo_al(a->wq, 16) || !zoo_al(a->u, 16) || !zoo_al(a->e_out, 16))))
     return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   StateParams p = {};
