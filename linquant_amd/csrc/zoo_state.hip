@@ -198,8 +198,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       load_step(ctn, pre);
     __syncthreads();
 
-    // ---- copy the stored state out, coalesced: h_i8[b][ct][h][v0 + v][k]
-    {
+    // the stored state leaves coalesced: h_i8[b][ct][h][v0 + v][k]
+    auto copy_out = [&]() {
       int8_t* dst = p.h_i8 + ((((int64_t)b * NT + ct) * H + h) * V + v0) * K;
       constexpr int SEG = K / 16;
       if constexpr (BV * SEG % 256 == 0) {
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
           *(lq_v4i*)(dst + vr * K + sg * 16) = *(const lq_v4i*)(hTb + vr * HS + sg * 16);
         }
       }
-    }
+    };
 
     if constexpr (DELTA) {
       // ---- state read against the stored copy, pseudo-values E, their write codes
@@ -232,6 +232,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       // the rest of chunk ct + 2's operands are requested while the matrix unit and then the vector ALU are busy: one wave
       // per SIMD issues in order, and 18 requests in a row held it for as long as the memory pipeline took to accept them
       load_part(std::integral_constant<int, 2>{}, ctn, pre);
+      copy_out();  // behind the products and the requests: nothing in this step waits for it
       // lane holds tokens 16*wave + 4kg + r, value columns v0 + NJ*rl + jj
       uint32_t ecode[NJ][4];
       const lq_v4f fw4 = *(const lq_v4f*)(misc_s + 4 * kg), ev4 = *(const lq_v4f*)(misc_s + 16 + 4 * kg);
@@ -287,6 +288,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
             zoo_pack_codes((int)ecode[jj][0], (int)ecode[jj][1], (int)ecode[jj][2], (int)ecode[jj][3]);
       __syncthreads();
     }
+
+    if constexpr (!DELTA) copy_out();
 
     // ---- write product and carry update
 #pragma unroll
