@@ -26,12 +26,11 @@ using StateParams = ZooStateParams;
 template <bool DELTA, int K, int BV>
 struct StepOps {
   lq_v4i kop[K / 64];                  // key write codes: rows of this wave, 16 token slots of the lane's group
-  lq_v4f gam[DELTA ? 1 : K / 64];      // linear: chunk decay of the lane's 4 carry rows per row tile
   lq_v4i vop[DELTA ? 1 : BV / 16];     // linear: value write codes
   lq_v4i wop[DELTA ? K / 64 : 1];      // delta: state-read codes of token 16*wave + (lane & 15)
   uint32_t uraw[DELTA ? BV / 8 : 1];   // delta: U of token 16*wave + (lane >> 2), columns BV/4 * (lane & 3) .. + BV/4 - 1
-  // delta: one value per lane of what the wave needs per token and per carry row: lanes 0..15 fw of tokens 16*wave + lane,
-  // lanes 16..31 ev of the same tokens, lanes 32.. the chunk decay of carry rows K/4*wave + lane - 32.  One request
+  // one value per lane of what the wave needs per token and per carry row: lanes 0..15 fw of tokens 16*wave + lane, lanes
+  // 16..31 ev of the same tokens (delta family), lanes 32.. the chunk decay of carry rows K/4*wave + lane - 32.  One request
   // instead of ten (each of which every lane of a row group repeated); the values reach the lanes that use them through
   // a wave-private piece of LDS.
   float misc;
@@ -51,7 +50,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 
   __shared__ __align__(16) unsigned char hT[(DELTA ? 1 : 2) * BV * HS];
   __shared__ __align__(16) unsigned char eT[DELTA ? BV * ES : 16];
-  __shared__ __align__(16) float misc_lds[DELTA ? 256 : 4];  // 64 floats per wave, written and read by that wave only
+  __shared__ __align__(16) float misc_lds[256];  // 64 floats per wave, written and read by that wave only
   constexpr int US = 2 * BV + 16;  // byte stride of a token row of the wave-private U / E tile (bank-conflict-free column reads)
   __shared__ __align__(16) unsigned char ue_lds[DELTA ? 4 * 16 * US : 16];
 
@@ -107,8 +106,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       for (int kt = 0; kt < KT; ++kt) {
         const int row = KR * wave + 16 * kt;
         o.kop[kt] = *(const lq_v4i*)(p.kqT + (cb * K + row + rl) * 64 + 16 * kg);
-        if constexpr (!DELTA) o.gam[kt] = *(const lq_v4f*)(p.gam + cb * K + row + 4 * kg);
       }
+      if constexpr (!DELTA) o.misc = p.gam[cb * K + KR * wave + min(max(lane - 32, 0), KR - 1)];
       if constexpr (DELTA) {
         const int64_t tr = (t0 + 16 * wave + (lane & 15)) * H + h;
         const float* src = lane < 16 ? p.fw + tr : lane < 32 ? p.ev + tr : p.gam + cb * K + KR * wave + min(lane - 32, KR - 1);
@@ -167,8 +166,8 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
     unsigned char* hTb = hT + (DELTA ? 0 : (ct & 1) * BV * HS);
     float* misc_s = misc_lds + 64 * wave;
     unsigned char* ue_s = ue_lds + wave * 16 * US;
+    misc_s[lane] = cur.misc;
     if constexpr (DELTA) {
-      misc_s[lane] = cur.misc;
       unsigned char* ud = ue_s + (lane >> 2) * US + (BV / 2) * (lane & 3);
       if constexpr (BV == 64) {
         *(lq_v4i*)ud = lq_v4i{(int)cur.uraw[0], (int)cur.uraw[1], (int)cur.uraw[2], (int)cur.uraw[3]};
@@ -302,11 +301,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const lq_v4i a = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
-        lq_v4f gam4;
-        if constexpr (DELTA)
-          gam4 = *(const lq_v4f*)(misc_s + 32 + 16 * kt + 4 * kg);
-        else
-          gam4 = cur.gam[kt];
+        const lq_v4f gam4 = *(const lq_v4f*)(misc_s + 32 + 16 * kt + 4 * kg);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float prod = (float)a[r] * skw_r[kt][r];
