@@ -210,27 +210,33 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
   // without D the request goes to a valid dummy address and dsc = 0 discards it: no branch around a request
   const int8_t* rqD = p.D ? p.D + (int64_t)h0 * p.sD_h + (p.D_has_hdim ? p0 : 0) : p.states;
   const _Float16* rqX = p.x + (int64_t)b * p.sx_b + (int64_t)c * Q * p.sx_l + (int64_t)h0 * p.sx_h + p0;
-  auto request = [&](uint32_t on) {
+  // part 0: the state piece, the per-token and per-channel scalars and the first half of the x rows; part 1: the other half
+  // of the x rows; part 2: everything.  The two parts are issued at two places of a head: a wave issues in order, and the
+  // thirteen requests in a row held it for as long as the memory pipeline took to accept them (0.7 of a head's 7 us).
+  auto request = [&](uint32_t on, int part) {
     const int tid = fresh((int)threadIdx.x), lane = tid & 63;
+    if (part != 1) {
 #pragma unroll
-    for (int k = 0; k < kSPieces; ++k) {
-      const int t = tid + k * WAVES * 64;
-      // (x and the state tile are streamed: a non-temporal request keeps them from displacing the C / CB tiles that
-      // other workgroups still need)
-      spiece[k] = __builtin_nontemporal_load(at<lq_v4i>(rqS, ((uint32_t)min(t, 4 * N - 1) * 16u) & on));  // a surplus thread re-reads the last piece
+      for (int k = 0; k < kSPieces; ++k) {
+        const int t = tid + k * WAVES * 64;
+        // (x and the state tile are streamed: a non-temporal request keeps them from displacing the C / CB tiles that
+        // other workgroups still need)
+        spiece[k] = __builtin_nontemporal_load(at<lq_v4i>(rqS, ((uint32_t)min(t, 4 * N - 1) * 16u) & on));  // a surplus thread re-reads the last piece
+      }
+      const uint32_t qoff = ((uint32_t)min(tid, Q - 1) * 4u) & on;
+      dA_r = *at<float>(rqA, qoff);
+      dt_r = *at<float>(rqT, qoff);
+      ss_r = *at<float>(rqC, (__umul24((uint32_t)lane, (uint32_t)p.sss_p) * 4u) & on);
+      D_r = (int)*at<int8_t>(rqD, (p.D && p.D_has_hdim) ? ((uint32_t)lane & on) : 0u);
     }
-    const uint32_t qoff = ((uint32_t)min(tid, Q - 1) * 4u) & on;
-    dA_r = *at<float>(rqA, qoff);
-    dt_r = *at<float>(rqT, qoff);
-    ss_r = *at<float>(rqC, (__umul24((uint32_t)lane, (uint32_t)p.sss_p) * 4u) & on);
-    D_r = (int)*at<int8_t>(rqD, (p.D && p.D_has_hdim) ? ((uint32_t)lane & on) : 0u);
     // tokens 8 q .. 8 q + 7 (the four token pairs of one row of the LDS layout), channels 4 c4 .. 4 c4 + 3
     const int q8 = (tid >> 4) * 8;
     const uint32_t c4b = (uint32_t)(tid & 15) * 8u;
 #pragma unroll
     for (int r = 0; r < 8; ++r)
       // rows past the sequence end re-read its last row and are zeroed when staged (no branch around a request)
-      xr[r] = __builtin_nontemporal_load(at<lq_v2i>(rqX, (__umul24((uint32_t)min(q8 + r, limit - 1), sxl2) + c4b) & on));
+      if (part == 2 || (r < 4) == (part == 0))
+        xr[r] = __builtin_nontemporal_load(at<lq_v2i>(rqX, (__umul24((uint32_t)min(q8 + r, limit - 1), sxl2) + c4b) & on));
   };
   auto advance = [&]() {
     rqS += (int64_t)p.P * N, rqA += (int64_t)p.nchunks * Q, rqT += (int64_t)p.nchunks * Q, rqC += p.sss_h;
@@ -262,7 +268,7 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       base[2 * Q + 64 + tid] = dsc * (float)D_r;
     }
   };
-  request(0xffffffffu);
+  request(0xffffffffu, 2);
   if (nh > 1) advance();
   settle();
   write_small(0);
@@ -313,8 +319,8 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
       }
     }
     // the next head's operands travel while this one is computed
-    request(hi + 1 < nh ? 0xffffffffu : 0u);
-    if (hi + 2 < nh) advance();
+    const uint32_t on_next = hi + 1 < nh ? 0xffffffffu : 0u;
+    request(on_next, 0);
     __syncthreads();
 
     // One 16-row tile at a time, start to finish (a tile past the sequence end is processed like any other, its rows
@@ -433,8 +439,12 @@ __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4
     };
     if (rb[0] < limit) {  // else the early tile is past the sequence end, and so is the late one (wave-uniform)
       tile(0, false);
+      request(on_next, 1);
+      if (hi + 2 < nh) advance();
       tile(1, true);
     } else {
+      request(on_next, 1);
+      if (hi + 2 < nh) advance();
       settle();
       write_small((hi + 1) & 1);
     }
