@@ -196,12 +196,17 @@ def hadamard_signed(n, seed, device):
     return (Hm / n ** 0.5 * signs).to(device)
 
 
-def timed_steps(step, warmup, steps):
-    """``warmup`` untimed steps, then the wall time of exactly ``steps`` steps between two synchronizations, in ms per step.
-    The interpreter's cyclic garbage collector is off for the duration (as ``timeit`` does): a full collection stops the
-    launching thread for 30-40 ms about once per 500 steps of this script, longer than the launches queued ahead of the
-    GPU last, so a timed region that happens to contain one measures that pause (seen: 50 steps at 0.27 ms each reported
-    as 0.94 ms per step)."""
+def timed_steps(step, warmup, steps, ramp_ms=0.0):
+    """Untimed launches for at least ``ramp_ms`` of wall time, ``warmup`` untimed steps, then the wall time of exactly
+    ``steps`` steps between two synchronizations.  Returns (ms per step, number of ramp steps).
+
+    The ramp: the GPU's clocks rise under sustained load, and a timed region of a few milliseconds right after an idle
+    period measures that rise, not the kernels.  The interpreter's cyclic garbage collector runs once in front of the ramp
+    and is off from there to the end of the timed steps (as ``timeit`` does): a full collection stops the launching thread
+    for 30-40 ms about once per 500 steps of this script, longer than the launches queued ahead of the GPU last.  Inside
+    a timed region it is measured as if it were the kernels' time (seen: 50 steps at 0.27 ms each reported as 0.94 ms per
+    step); between the ramp and the warm-up steps it leaves the GPU idle long enough for the clocks to fall again (seen:
+    20 timed steps at 0.32 ms instead of 0.27)."""
     import gc
 
     import torch
@@ -210,6 +215,12 @@ def timed_steps(step, warmup, steps):
     was_enabled = gc.isenabled()
     gc.disable()
     try:
+        n, t0 = 0, time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < ramp_ms:
+            for _ in range(4):
+                step()
+            n += 4
+            torch.cuda.synchronize()
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
@@ -217,25 +228,10 @@ def timed_steps(step, warmup, steps):
         for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / steps
+        return (time.perf_counter() - t0) * 1e3 / steps, n
     finally:
         if was_enabled:
             gc.enable()
-
-
-def ramp(step, min_ms=RAMP_MS):
-    """Runs ``step`` back to back for at least ``min_ms`` of wall time, untimed: the GPU's clocks rise under sustained
-    load, and a timed region of a few milliseconds right after an idle period would measure that rise, not the kernels.
-    Returns the number of steps it ran."""
-    import torch
-
-    n, t0 = 0, time.perf_counter()
-    while (time.perf_counter() - t0) * 1e3 < min_ms:
-        for _ in range(4):
-            step()
-        n += 4
-        torch.cuda.synchronize()
-    return n
 
 
 def measure_zoo(args, workload, cpu_baseline):
@@ -318,8 +314,7 @@ def measure_zoo(args, workload, cpu_baseline):
 
     if args.copy_probe:
         copy_probe(dev)
-    ramp_steps = 0 if args.no_ramp else ramp(lambda: call(sc))
-    ms_per_step = timed_steps(lambda: call(sc), args.warmup, args.steps)
+    ms_per_step, ramp_steps = timed_steps(lambda: call(sc), args.warmup, args.steps, 0.0 if args.no_ramp else RAMP_MS)
     tokens = B * T
 
     records = {}
@@ -527,7 +522,7 @@ def bench_layer(args):
     def step():
         return layer(hidden)
 
-    ms_per_step = timed_steps(step, args.warmup, args.steps)
+    ms_per_step, _ = timed_steps(step, args.warmup, args.steps, 0.0 if args.no_ramp else RAMP_MS)
 
     records = {}
 
@@ -602,7 +597,7 @@ def _stage_bench(args, stages, step_names, tokens, dtype, cpu_sample, workload):
         for name in step_names:
             stages[name][0]()
 
-    ms_per_step = timed_steps(step, args.warmup, args.steps)
+    ms_per_step, _ = timed_steps(step, args.warmup, args.steps, 0.0 if args.no_ramp else RAMP_MS)
     out = {}
     for name, (fn, nbytes) in stages.items():
         ts = []
@@ -679,8 +674,7 @@ def measure_c5(args, regime, keyside, cpu_baseline, with_graph=False):
 
     if args.copy_probe:
         copy_probe(dev)
-    ramp_steps = 0 if args.no_ramp else ramp(step)
-    ms_per_step = timed_steps(step, args.warmup, args.steps)
+    ms_per_step, ramp_steps = timed_steps(step, args.warmup, args.steps, 0.0 if args.no_ramp else RAMP_MS)
     tokens = s.batch * s.seqlen
 
     # ---- per-stage durations: HIP events on the launch stream around every stage call (separate pass)
@@ -781,7 +775,7 @@ def measure_c5(args, regime, keyside, cpu_baseline, with_graph=False):
         torch.cuda.synchronize()
         with torch.cuda.graph(g):
             step()
-        gms = timed_steps(g.replay, args.warmup, args.steps)
+        gms, _ = timed_steps(g.replay, args.warmup, args.steps, 0.0 if args.no_ramp else RAMP_MS)
         graph = {"ms_per_step": round(gms, 4), "tokens_per_s": round(tokens / gms * 1e3, 1)}
 
     # ---- CPU baseline: the CPU oracle on a bounded sample (batch 1 x a few heads x full length), same seeds
