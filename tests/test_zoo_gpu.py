@@ -514,6 +514,52 @@ def test_wy_prep_also_makes_the_write_codes(cuda, cell, K, dtype, eta, bits):
         assert torch.equal(got[name], ref[name]), f"{cell} {name}: differs from the stand-alone pre-pass"
         assert torch.equal(got2[name], ref[name]), f"{cell} {name} (W not stored): differs from the stand-alone pre-pass"
     assert int(ref["kqT"].abs().max()) > qmax // 2 and int(ref["wq"].abs().max()) > 0  # the comparison is not vacuous
+    # the packed copy of fw | ev | gam per (batch, chunk, head) holds the same values
+    NT = T // 64
+    pack = got["pack"]
+    assert pack.shape == (B, NT, H, 128 + K)
+    assert torch.equal(pack[..., :64], fw0.view(B, NT, 64, H).transpose(2, 3))
+    assert torch.equal(pack[..., 64:128], ref["ev"].view(B, NT, 64, H).transpose(2, 3))
+    assert torch.equal(pack[..., 128:], ref["gam"])
+
+
+@pytest.mark.parametrize("cell,K,V,dtype", [("deltanet", 128, 128, torch.float16), ("gated_deltanet", 64, 64, torch.bfloat16),
+                                            ("kda", 128, 64, torch.float16)])
+def test_delta_state_kernel_takes_its_factors_packed_or_apart(cuda, cell, K, V, dtype):
+    """lq_zoo_state reads fw, ev and the chunk decays from the packed block WY prep writes or, without it, from the three
+    separate tensors: stored states, pseudo-values and the final state are the same bit for bit, at every tile width."""
+    from linquant_amd.kernels.zoo import _common as C
+
+    decay = zc.CELLS[cell][1]
+    B, T, H = 2, 256, 3
+    q, k, v, g, beta = zc.cut(zc.inputs(cell, B=B, H=H, K=K, V=V, seed=33), T)
+    dims = (B, T, H, K, V)
+    code = {"none": C.DECAY_NONE, "scalar": C.DECAY_SCALAR, "diagonal": C.DECAY_DIAGONAL}[decay]
+    k, v, beta = k.to(dtype).cuda(), v.to(dtype).cuda(), beta.cuda()
+    gc = logenv = None
+    if g is not None:
+        gc, logenv = C.cumsum(g.cuda(), B, T, H, K if decay == "diagonal" else 0)
+    gen = torch.Generator().manual_seed(5)
+    skw = (torch.rand(H, K, generator=gen) * 0.02 + 0.002).cuda()
+    sw = (torch.rand(H, generator=gen) * 0.02 + 0.004).cuda()
+    ew = (torch.rand(H, V, generator=gen) * 0.02 + 0.01).cuda()
+    ss = (torch.rand(H, V, generator=gen) * 0.01 + 0.005).cuda()
+    Hw, W, U, fw, codes = C.run_wy_prep(k, v, beta, gc, 0.5, 0.5, dims, code,
+                                        write=dict(logenv=logenv, skw=skw, sw=sw, eta=0.5, qmax=127))
+    apart = {n: t for n, t in codes.items() if n != "pack"}
+    NT = T // 64
+    for vtile in (0, 16, 32, 64):
+        outs = []
+        for c in (codes, apart):
+            h_i8 = torch.zeros(B, NT, H, V, K, dtype=torch.int8, device=cuda)
+            e_out = torch.zeros_like(v)
+            ht = torch.zeros(B, H, K, V, dtype=torch.float32, device=cuda)
+            C.state_kernel(c, U, fw, h_i8, e_out, ht, skw, ew, sw, ss, 127, dims, C.FAMILY_DELTA, vtile=vtile)
+            outs.append((h_i8, e_out, ht))
+        torch.cuda.synchronize()
+        for name, a, b_ in zip(("h_i8", "e_out", "ht"), outs[0], outs[1]):
+            assert torch.equal(a, b_), f"{cell} vtile {vtile}: {name} depends on where the factors are read from"
+        assert int(outs[0][0].abs().max()) > 20 and float(outs[0][2].abs().max()) > 0  # not vacuous
 
 
 @pytest.mark.parametrize("K,V,dtype,eta,bits", [(128, 128, torch.float16, 0.0, 8), (64, 128, torch.float16, 0.5, 8),
