@@ -138,18 +138,30 @@ def launch(fn: str, device, st):
         raise LinQuantHipError(f"{fn} failed with code {rc}: {_ERRORS.get(rc, 'unknown error')}")
 
 
+_FIELD_NAMES = {}
+
+
 def call(fn: str, device, **fields):
     """Fill ``<fn>_args`` from keyword fields and launch on the current stream of ``device``."""
-    lib = load()
-    st = STRUCTS[_SHARED_ARGS.get(fn, fn + "_args")]()
-    known = {n for n, _ in st._fields_}
+    lib = _lib if _lib is not None else load()
+    sname = _SHARED_ARGS.get(fn, fn + "_args")
+    cls = STRUCTS[sname]
+    known = _FIELD_NAMES.get(sname)
+    if known is None:
+        known = _FIELD_NAMES[sname] = frozenset(n for n, _ in cls._fields_)
+    st = cls()
     for k, v in fields.items():
         if k not in known:
             raise KeyError(f"{fn}_args has no field {k!r}")
         setattr(st, k, v)
     import torch
 
-    with torch.cuda.device(device):
-        rc = getattr(lib, fn)(ctypes.byref(st), current_stream(device))
+    # (the device guard costs several microseconds a launch: it is entered only when the tensors' device is not the current one)
+    idx = device.index if getattr(device, "index", None) is not None else torch.cuda.current_device()
+    if idx == torch.cuda.current_device():
+        rc = getattr(lib, fn)(ctypes.byref(st), torch.cuda.current_stream(idx).cuda_stream)
+    else:
+        with torch.cuda.device(device):
+            rc = getattr(lib, fn)(ctypes.byref(st), current_stream(device))
     if rc != 0:
         raise LinQuantHipError(f"{fn} failed with code {rc}: {_ERRORS.get(rc, 'unknown error')}")
