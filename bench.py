@@ -395,6 +395,23 @@ def measure_zoo(args, workload, cpu_baseline):
                "sample": f"float64 torch oracle on batch 1 x {hs} of {H} heads x {ts_} tokens ({frac:.5f} of the job) in "
                          f"{t_cpu:.3f} s (median of {len(times)} runs); value = job-equivalent tokens/s", "host_cpus": os.cpu_count(),
                "torch_threads": torch.get_num_threads()}
+    graph = None
+    if args.graph or workload == "c1":
+        # the same step captured once in a HIP graph and replayed: no host work between the launches.  The first
+        # configuration is small enough for the eager step to be bound by the launching thread (about 12 us of Python and
+        # launch per kernel); the replay shows what the kernels themselves take
+        gr = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            call(sc)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(gr):
+            call(sc)
+        gms, _ = timed_steps(gr.replay, args.warmup, args.steps, 0.0 if args.no_ramp else RAMP_MS)
+        graph = {"ms_per_step": round(gms, 4), "tokens_per_s": round(tokens / gms * 1e3, 1)}
+        del gr
     line = {
         "metric": f"prefill tokens/s per layer at T={T}", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -406,7 +423,7 @@ def measure_zoo(args, workload, cpu_baseline):
                                ("none (local R_QK inside the A kernel" +
                                 ("; D_QK (alpha 0.5) applied inside the WY prep and A kernels as they load k and q)"
                                  if dqk is not None else ")")) if rot is not None else "none"},
-        "roofline": roofline, "cpu_baseline": cpu, "stages": stages,
+        "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "hip_graph": graph,
     }
     return line
 
@@ -851,6 +868,8 @@ def compact(line, keep_cpu):
            "roofline": line["roofline"]}
     if keep_cpu:
         rec["cpu_baseline"] = line["cpu_baseline"]
+    if line.get("hip_graph"):
+        rec["hip_graph"] = line["hip_graph"]
     return rec
 
 
@@ -891,7 +910,8 @@ def main():
                     help="also run one plain device copy of 256 MiB (reference point for HBM byte counters)")
     ap.add_argument("--regime", default="strong", choices=["strong", "weak"],
                     help="c5: decay regime of the synthetic dt / A (strong = the stated recipe)")
-    ap.add_argument("--graph", action="store_true", help="c5: also time the step replayed from one captured HIP graph")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the step replayed from one captured HIP graph (always done for c1, whose eager step is bound by the launching thread)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="heads per slice of the CPU-oracle sample")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="stop the CPU-oracle sample after about this long")
     args = ap.parse_args()
