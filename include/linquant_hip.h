@@ -340,7 +340,9 @@ int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
 /* replaces the operand preparation inside the reference's state kernels (linquant/kernels/zoo/simple_gla.py:55-66,
  * gla.py:124-141, gated_delta_rule.py:85-105, kda.py:100-124): every write operand that does not depend on the
  * carried state is quantized once, in parallel over chunks, into the layout lq_zoo_state consumes.
- * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers. */
+ * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers.
+ * chunk_size is 64, or 128 (linear family, no / scalar decay; seqlen a multiple of 128): the buffers keep their 64-token
+ * layout (NT = seqlen / 64) and the decays of a chunk's first 64 tokens reach on to the end of the 128-token chunk. */
 typedef struct {
   const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16/bf16 */
   const void* val;           /* linear family: v (B,T,H,V) fp16/bf16; delta family: NULL */
@@ -367,7 +369,10 @@ int lq_zoo_write_codes(const lq_zoo_write_codes_args* args, hipStream_t stream);
  * (gla.py:102-167), _delta_state_kernel (gated_delta_rule.py:50-136) and _kda_state_kernel (kda.py:68-151):
  * sequential chunk loop with an fp32 carry, INT8 stored copy per chunk, INT8 write product (and, delta family,
  * the INT8 state read W.S and the pseudo-values E = (U - W.S) * fw, stored fp16 for the output kernel).
- * Consumes the buffers written by lq_zoo_write_codes. */
+ * Consumes the buffers written by lq_zoo_write_codes.
+ * chunk_size is 64, or 128 (linear family, rotated storage; operands from lq_zoo_write_codes with chunk_size 128): one
+ * stored state per 128 tokens, h_i8 is (B,seqlen/128,H,V,K), and the carry takes the INT8 write product summed over the
+ * 128 tokens (int32) once per chunk. */
 typedef struct {
   const int8_t* kqT;         /* (B,NT,H,K,64) */
   const int8_t* vqT;         /* linear family: (B,NT,H,V,64) */
@@ -398,7 +403,10 @@ int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
 
 /* replaces _output_kernel (linquant/kernels/zoo/simple_gla.py:98-172) and _gla_output_kernel
  * (gla.py:170-232): o = dequant(q8(q).h_i8) [* exp(g)] + (fp16(A) . fp16(q8(v))) * svl, with A computed
- * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay). */
+ * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay).
+ * chunk_size is 64, or 128 (no / scalar decay, raw q, k, v, rotated storage; h_i8 (B,seqlen/128,H,V,K) from lq_zoo_state
+ * with chunk_size 128): two launches, the first leaves the second halves' products with the first halves' tokens in
+ * `cross`, the second starts its fp32 accumulators from them. */
 typedef struct {
   const void* q;             /* no / scalar decay: (B,T,H,K) fp16/bf16; diagonal decay: NULL */
   const int8_t* qg;          /* diagonal decay: (B,T,H,K) int8 codes of q*exp(g)*scale written by lq_zoo_gla_A */
@@ -424,6 +432,7 @@ typedef struct {
   const int8_t* qc;          /* (B,T,H,K) int8 q8(q*scale, 1/sq) */
   const int8_t* kc;          /* (B,T,H,K) int8 q8(k, 1/sk) */
   const int8_t* vc;          /* (B,T,H,V) int8 q8(v, 1/svl) */
+  float* cross;              /* chunk_size 128: (B,T,H,V) fp32 workspace, 16-byte aligned (overwritten); else unused */
 } lq_zoo_output_args;
 int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
 

@@ -13,7 +13,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 HEADER = ROOT.parent / "include" / "linquant_hip.h"
 LIB_PATH = ROOT / "csrc" / "liblinquant_hip.so"
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 LQ_DT_F16, LQ_DT_F32, LQ_DT_I8, LQ_DT_BF16 = 0, 1, 2, 3
 

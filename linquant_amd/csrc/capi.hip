@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 15; }
+extern "C" int lq_abi_version(void) { return 16; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)

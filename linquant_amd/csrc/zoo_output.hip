@@ -29,14 +29,20 @@ using OutParams = ZooOutParams;
 // for both tiles)
 // CIN: the local codes of q, k, v arrive ready-made (lq_zoo_rotate_quant made them): they are copied into the same LDS
 // tiles instead of being quantized here.
-template <bool GLA, bool USE_G, int K, bool BF, int NV, bool CIN>
+// CROSS (128-token chunks, which run as pairs of 64-token halves): this launch makes, for the second half of every chunk,
+// the part of the local product that reaches back into the first half -- fp16(Af[i][j]) . fp16(q8(v_j)) over the 64 tokens j
+// of the first half, no causal mask, no state read -- and leaves it as fp32 in p.cross; the ordinary launch that follows
+// starts its local accumulators from it (one fp32 accumulation over the 128 tokens, oldest first, as a 128-token tile has).
+template <bool GLA, bool USE_G, int K, bool BF, int NV, bool CIN, bool CROSS = false>
 __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
+  static_assert(!CROSS || (!GLA && !CIN), "the cross launch exists for the no / scalar decay kernels on raw operands");
   constexpr int QS = K + 16;  // byte stride of a code row
   __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) _Float16 Afl[GLA ? 8 : 64 * kAS];
   __shared__ __align__(16) uint32_t vP[NV * 32 * kVW];
   __shared__ float g_s[64];
+  __shared__ float gk_s[CROSS ? 64 : 1];  // cross launch: cumulative log decay of the first half's tokens
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -53,10 +59,12 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       bh = vid / (nv * gridDim.y);
     }
   }
+  if constexpr (CROSS) ct = 2 * ct + 1;  // the grid walks the chunks; the rows are those of the second half
   const int v0 = vtile * BV * NV;
   const int b = bh / p.H, h = bh % p.H;
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
+  const int64_t tk0 = CROSS ? t0 - 64 : t0;  // first token of the keys / values this launch contracts against
   const float sq = p.sq[h];
   const float inv_sq = 1.0f / sq;
   const float sk = GLA ? 1.0f : p.sk[h];
@@ -76,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       const int t = it / (K / 8), c8 = it % (K / 8);
       const int64_t off = ((t0 + t) * H + h) * K + 8 * c8;
       qraw[i] = *(const lq_v4i*)(p.q + off);
-      kraw[i] = *(const lq_v4i*)(p.k + off);
+      kraw[i] = *(const lq_v4i*)(p.k + off + (tk0 - t0) * H * K);
     }
   }
   if constexpr (!GLA && CIN) {  // 16 codes per piece: half as many pieces
@@ -90,7 +98,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
     }
   }
   const int tp = tid >> 3, c8v = tid & 7;  // value tile: 32 token pairs x 8 groups of 8 channels
-  const int64_t voff = ((t0 + 2 * tp) * H + h) * V + v0 + 8 * c8v;
+  const int64_t voff = ((tk0 + 2 * tp) * H + h) * V + v0 + 8 * c8v;
   lq_v4i va_raw[NV], vb_raw[NV];
   lq_v4f sv0[NV], sv1[NV];
 #pragma unroll
@@ -104,16 +112,20 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
     }
   }
   const float g_raw = (USE_G && !GLA) ? p.g[(t0 + (tid & 63)) * H + h] : 0.0f;
-  const int8_t* hp = p.h_i8 + ((((int64_t)b * p.NT + ct) * H + h) * V + v0) * K;
-  lq_v4i hop[NV][K / 64][4];
+  const float gk_raw = (USE_G && CROSS) ? p.g[(tk0 + (tid & 63)) * H + h] : 0.0f;
+  // (128-token chunks: one stored state per chunk, read by both halves)
+  const int8_t* hp = p.h_i8 + ((((int64_t)b * (p.NT >> p.hshift) + (ct >> p.hshift)) * H + h) * V + v0) * K;
+  lq_v4i hop[CROSS ? 1 : NV][K / 64][4];
   lq_v4i qgop[GLA ? K / 64 : 1];
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
     if constexpr (GLA) qgop[ks] = *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
+    if constexpr (!CROSS) {
 #pragma unroll
-    for (int n = 0; n < NV; ++n)
+      for (int n = 0; n < NV; ++n)
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) hop[n][ks][jj] = *(const lq_v4i*)(hp + (BV * n + 4 * rl + jj) * K + 64 * ks + 16 * kg);
+        for (int jj = 0; jj < 4; ++jj) hop[n][ks][jj] = *(const lq_v4i*)(hp + (BV * n + 4 * rl + jj) * K + 64 * ks + 16 * kg);
+    }
   }
   lq_v4f ss4[NV], svl4[NV];
 #pragma unroll
@@ -183,14 +195,17 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
     *(lq_v4i*)(vP + (32 * n + tp) * kVW + 8 * c8v + 4) = o1;
   }
   if (USE_G && !GLA) g_s[tid & 63] = g_raw;  // four threads per token write the same value
+  if constexpr (USE_G && CROSS) gk_s[tid & 63] = gk_raw;
   __syncthreads();
 
   // ---- phase 2: INT8 contractions of this wave's 16 rows
-  lq_v4i o32[NV][4];
+  lq_v4i o32[CROSS ? 1 : NV][4];
+  if constexpr (!CROSS) {
 #pragma unroll
-  for (int n = 0; n < NV; ++n)
+    for (int n = 0; n < NV; ++n)
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) o32[n][jj] = lq_v4i{0, 0, 0, 0};
+      for (int jj = 0; jj < 4; ++jj) o32[n][jj] = lq_v4i{0, 0, 0, 0};
+  }
   lq_v4i a32[4];
 #pragma unroll
   for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
@@ -201,14 +216,16 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       qop = qgop[ks];
     else
       qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
+    if constexpr (!CROSS) {
 #pragma unroll
-    for (int n = 0; n < NV; ++n)
+      for (int n = 0; n < NV; ++n)
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) o32[n][jj] = lq_mfma_i8(qop, hop[n][ks][jj], o32[n][jj]);
+        for (int jj = 0; jj < 4; ++jj) o32[n][jj] = lq_mfma_i8(qop, hop[n][ks][jj], o32[n][jj]);
+    }
     if (!GLA) {
 #pragma unroll
       for (int jt = 0; jt < 4; ++jt) {
-        if (jt > wave) continue;  // strictly above the diagonal (wave-uniform)
+        if (!CROSS && jt > wave) continue;  // strictly above the diagonal (wave-uniform)
         const lq_v4i kop = *(const lq_v4i*)(kc + (16 * jt + rl) * QS + 64 * ks + 16 * kg);
         a32[jt] = lq_mfma_i8(qop, kop, a32[jt]);
       }
@@ -216,30 +233,35 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
 
   // ---- phase 3: dequantize; A -> fp16 in operand layout
-  float of[NV][4][4];  // [tile][jj][r]: rows 16w + 4kg + r, channels v0 + 64 tile + 4rl + jj
+  float of[CROSS ? 1 : NV][4][4];  // [tile][jj][r]: rows 16w + 4kg + r, channels v0 + 64 tile + 4rl + jj
+  if constexpr (!CROSS) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + 4 * kg + r]) : 1.0f;
+    for (int r = 0; r < 4; ++r) {
+      const float eg = (USE_G && !GLA) ? zoo_exp(g_s[16 * wave + 4 * kg + r]) : 1.0f;
 #pragma unroll
-    for (int n = 0; n < NV; ++n)
+      for (int n = 0; n < NV; ++n)
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        float x = (float)o32[n][jj][r] * sq;
-        x = x * ss4[n][jj];
-        of[n][jj][r] = (USE_G && !GLA) ? x * eg : x;
-      }
+        for (int jj = 0; jj < 4; ++jj) {
+          float x = (float)o32[n][jj][r] * sq;
+          x = x * ss4[n][jj];
+          of[n][jj][r] = (USE_G && !GLA) ? x * eg : x;
+        }
+    }
   }
   if (!GLA) {
     const float sqk = sq * sk;
 #pragma unroll
     for (int jt = 0; jt < 4; ++jt) {
-      if (jt > wave + 1) continue;
+      if (!CROSS && jt > wave + 1) continue;
       const int j = 16 * jt + rl;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * wave + 4 * kg + r;
         float x = 0.0f;
-        if (jt <= wave && j <= i) {
+        if constexpr (CROSS) {  // every token of the first half precedes every row: the whole block, its decay from gk_s
+          x = (float)a32[jt][r] * sqk;
+          if (USE_G) x = x * zoo_exp(g_s[i] - gk_s[j]);
+        } else if (jt <= wave && j <= i) {
           x = (float)a32[jt][r] * sqk;
           if (USE_G) x = x * zoo_exp(g_s[i] - g_s[j]);
         }
@@ -255,7 +277,19 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   for (int n = 0; n < NV; ++n)
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) loc[n][jj] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-  const int nslab = (16 * wave + 15) / 32 + 1;
+  if constexpr (!GLA && !CROSS) {
+    if (p.cross && (ct & 1)) {  // second half of a 128-token chunk: what the cross launch left for these rows
+#pragma unroll
+      for (int n = 0; n < NV; ++n)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const lq_v4f c4 = *(const lq_v4f*)(p.cross + ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + BV * n + 4 * rl);
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) loc[n][jj][r] = c4[jj];
+        }
+    }
+  }
+  const int nslab = CROSS ? 2 : (16 * wave + 15) / 32 + 1;
   for (int js = 0; js < nslab; ++js) {
     lq_v8h aop;
     if (GLA) {
@@ -281,22 +315,37 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int64_t off = ((t0 + 16 * wave + 4 * kg + r) * H + h) * V + v0 + BV * n + 4 * rl;
-    float res[4];
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) res[jj] = of[n][jj][r] + loc[n][jj][r] * svl4[n][jj];
-    if (p.o_is_f32) {
-      __builtin_nontemporal_store(lq_v4f{res[0], res[1], res[2], res[3]}, (lq_v4f*)((float*)p.o + off));
+    if constexpr (CROSS) {
+      *(lq_v4f*)(p.cross + off) = lq_v4f{loc[n][0][r], loc[n][1][r], loc[n][2][r], loc[n][3][r]};
     } else {
-      lq_v2i w;
-      w[0] = (int)zoo_enc2(res[0], res[1], bf);
-      w[1] = (int)zoo_enc2(res[2], res[3], bf);
-      __builtin_nontemporal_store(w, (lq_v2i*)((_Float16*)p.o + off));
+      float res[4];
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) res[jj] = of[n][jj][r] + loc[n][jj][r] * svl4[n][jj];
+      if (p.o_is_f32) {
+        __builtin_nontemporal_store(lq_v4f{res[0], res[1], res[2], res[3]}, (lq_v4f*)((float*)p.o + off));
+      } else {
+        lq_v2i w;
+        w[0] = (int)zoo_enc2(res[0], res[1], bf);
+        w[1] = (int)zoo_enc2(res[2], res[3], bf);
+        __builtin_nontemporal_store(w, (lq_v2i*)((_Float16*)p.o + off));
+      }
     }
   }
 }
 
+template <bool USE_G, int K, int NV>
+void launch_cross(const OutParams& p, dim3 grid, hipStream_t stream) {
+  if (p.bf)
+    hipLaunchKernelGGL((zoo_output_kernel<false, USE_G, K, true, NV, false, true>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_output_kernel<false, USE_G, K, false, NV, false, true>), grid, dim3(256), 0, stream, p);
+}
+
 template <bool GLA, bool USE_G, int K, int NV>
 void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
+  if constexpr (!GLA) {
+    if (p.cross) launch_cross<USE_G, K, NV>(p, dim3(grid.x, grid.y / 2, grid.z), stream);
+  }
   if constexpr (!GLA) {
     if (p.qc) {  // ready-made codes: the activation dtype only matters for a 16-bit output
       if (p.bf)
@@ -344,7 +393,12 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
+  // 128-token chunks (no / scalar decay, raw operands, rotated storage) run as pairs of 64-token halves
+  const bool pair = a->chunk_size == 128;
+  if (pair && (gla || cin || a->unrot)) return LQ_ERR_SHAPE;
+  if (pair && !a->cross) return LQ_ERR_NULL;
+  if (pair && !zoo_al(a->cross, 16)) return LQ_ERR_SHAPE;
+  if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
@@ -359,6 +413,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   p.unrot = (const _Float16*)a->unrot;
   p.qc = a->qc, p.kc = a->kc, p.vc = a->vc;
+  p.cross = pair ? a->cross : nullptr, p.hshift = pair ? 1 : 0;
   if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
   if (gla) return launch<true, true>(p, a->kdim, stream);
   if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, stream);

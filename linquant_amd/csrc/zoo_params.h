@@ -48,6 +48,8 @@ struct ZooOutParams {
   int qmax;
   int bf;  // activations (and a 16-bit output) are bf16
   int B, T, H, V, NT;
+  float* cross;  // 128-token chunks: fp32 (B,T,H,V) partial local products of the second halves, else nullptr
+  int hshift;    // log2 of the 64-token halves per stored state (1 for 128-token chunks)
 };
 
 // canonical storage: one workgroup spans all V value channels (V = 64 or 128); defined in zoo_unrot.hip

@@ -38,8 +38,13 @@ struct StepOps {
 
 // BF (bf16 activations) is a template parameter: as a run-time flag every decode / encode of U and E in the chunk loop
 // became a branch of its own.
-template <bool DELTA, int K, int BV, bool BF>
+// PAIR (linear family, 128-token chunks): the chunk loop still walks 64-token halves, whose operands the pre-pass wrote
+// with the decay to the end of the 128-token chunk.  The state is quantized and stored at the first half only (index
+// ct / 2), the INT8 write product of the first half stays in the accumulators that the second half's product adds to, and
+// the carry takes decay and product once per chunk: the integer sum over 128 tokens that one 128-token tile gives.
+template <bool DELTA, int K, int BV, bool BF, bool PAIR = false>
 __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StateParams p) {
+  static_assert(!PAIR || !DELTA, "128-token chunks exist for the linear family");
   constexpr int KR = K / 4;     // carry rows per wave
   constexpr int KT = KR / 16;   // 16-row tiles per wave (= K / 64)
   constexpr int VT = BV / 16;   // 16-col tiles
@@ -161,9 +166,11 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
   // retire in issue order, loads and stores alike, so a load issued behind the stores of the previous step is not seen
   // complete before those stores are acknowledged: with one step of look-ahead that acknowledgement sat on the critical
   // path of every step, with two it has a whole step to arrive.
+  lq_v4i pend[PAIR ? KT : 1][PAIR ? VT : 1];  // PAIR: the first half's write product
   auto do_step = [&](int ct, StepOps<DELTA, K, BV>& cur, StepOps<DELTA, K, BV>& pre) {
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
-    unsigned char* hTb = hT + (DELTA ? 0 : (ct & 1) * BV * HS);
+    const bool second = PAIR && (ct & 1);  // PAIR: second half of a chunk (nothing stored, the carry is updated)
+    unsigned char* hTb = hT + (DELTA ? 0 : ((PAIR ? ct >> 1 : ct) & 1) * BV * HS);
     float* misc_s = misc_lds + 64 * wave;
     unsigned char* ue_s = ue_lds + wave * 16 * US;
     misc_s[lane] = cur.misc;
@@ -179,15 +186,17 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       }
     }
     // ---- stored copy of the incoming state -> LDS (V-major)
+    if (!second) {
 #pragma unroll
-    for (int kt = 0; kt < KT; ++kt)
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-      for (int vt = 0; vt < VT; ++vt) {
-        int cd[4];
+        for (int vt = 0; vt < VT; ++vt) {
+          int cd[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) cd[r] = zoo_q8(hc[kt][vt][r], inv_ss_c[vt], 127);
-        *(uint32_t*)(hTb + (16 * vt + rl) * HS + KR * wave + 16 * kt + 4 * kg) = zoo_pack_codes(cd[0], cd[1], cd[2], cd[3]);
-      }
+          for (int r = 0; r < 4; ++r) cd[r] = zoo_q8(hc[kt][vt][r], inv_ss_c[vt], 127);
+          *(uint32_t*)(hTb + (16 * vt + rl) * HS + KR * wave + 16 * kt + 4 * kg) = zoo_pack_codes(cd[0], cd[1], cd[2], cd[3]);
+        }
+    }
     // requested unconditionally (the last chunks re-request the final one): a branch around the loads would make the
     // compiler's count of outstanding memory operations path-dependent, and it then waits for the newest loads as well
     const int ctn = min(ct + 2, NT - 1);
@@ -199,7 +208,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 
     // the stored state leaves coalesced: h_i8[b][ct][h][v0 + v][k]
     auto copy_out = [&]() {
-      int8_t* dst = p.h_i8 + ((((int64_t)b * NT + ct) * H + h) * V + v0) * K;
+      int8_t* dst = p.h_i8 + ((((int64_t)b * (PAIR ? NT >> 1 : NT) + (PAIR ? ct >> 1 : ct)) * H + h) * V + v0) * K;
       constexpr int SEG = K / 16;
       if constexpr (BV * SEG % 256 == 0) {
 #pragma unroll
@@ -288,7 +297,9 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       __syncthreads();
     }
 
-    if constexpr (!DELTA) copy_out();
+    if constexpr (!DELTA) {
+      if (!second) copy_out();
+    }
 
     // ---- write product and carry update
 #pragma unroll
@@ -300,7 +311,16 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
         bop = cur.vop[vt];
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
-        const lq_v4i a = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
+        lq_v4i a;
+        if constexpr (PAIR) {
+          if (!second) {
+            pend[kt][vt] = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
+            continue;
+          }
+          a = lq_mfma_i8(cur.kop[kt], bop, pend[kt][vt]);
+        } else {
+          a = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
+        }
         const lq_v4f gam4 = *(const lq_v4f*)(misc_s + 32 + 16 * kt + 4 * kg);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -351,11 +371,17 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 }
 
 template <bool DELTA, int K>
-int launch_bv(const StateParams& p, int BV, int B, hipStream_t stream) {
+int launch_bv(const StateParams& p, int BV, int B, hipStream_t stream, bool pair = false) {
   dim3 grid(p.V / BV, B * p.H);
   constexpr bool D = DELTA;  // the linear family touches no half-precision tensor: one instantiation serves both dtypes
 #define LQ_STATE_LAUNCH(BVV)                                                                                  \
   do {                                                                                                        \
+    if constexpr (!D) {                                                                                       \
+      if (pair) {                                                                                             \
+        hipLaunchKernelGGL((zoo_state_kernel<false, K, BVV, false, true>), grid, dim3(256), 0, stream, p);    \
+        break;                                                                                                \
+      }                                                                                                       \
+    }                                                                                                         \
     if (D && p.bf)                                                                                            \
       hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, BVV, D>), grid, dim3(256), 0, stream, p);                \
     else                                                                                                      \
@@ -381,7 +407,10 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (!delta && !a->vqT) return LQ_ERR_NULL;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
+  // 128-token chunks (linear family, rotated storage) run as pairs of 64-token halves
+  const bool pair = a->chunk_size == 128;
+  if (pair && (delta || a->unrot)) return LQ_ERR_SHAPE;
+  if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
@@ -410,5 +439,5 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
       BV = wg64 >= 1024 ? 64 : (wg64 >= 512 ? 32 : 16);
   }
   if (delta) return a->kdim == 128 ? launch_bv<true, 128>(p, BV, a->batch, stream) : launch_bv<true, 64>(p, BV, a->batch, stream);
-  return a->kdim == 128 ? launch_bv<false, 128>(p, BV, a->batch, stream) : launch_bv<false, 64>(p, BV, a->batch, stream);
+  return a->kdim == 128 ? launch_bv<false, 128>(p, BV, a->batch, stream, pair) : launch_bv<false, 64>(p, BV, a->batch, stream, pair);
 }

@@ -33,6 +33,7 @@ struct CodesParams {
   int qmax;
   int bf;
   int T, H, V, NT;
+  int span;  // tokens per chunk: 64, or 128 (two workgroups per chunk, the decays reach to the end of the chunk)
 };
 
 template <int DECAY, int K, bool BF>
@@ -48,6 +49,8 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   const int H = p.H, V = p.V, T = p.T;
   const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
   const int64_t cb = ((int64_t)b * p.NT + ct) * H + h;  // (batch, chunk, head) index
+  // last token of the chunk: of these 64 tokens, or, when they are one half of a 128-token chunk, of that chunk
+  const int64_t tlast = t0 + 63 + (p.span == 128 && !(ct & 1) ? 64 : 0);
   const float eta = p.eta;
   const int qmax = p.qmax;
   constexpr bool bf = BF;
@@ -55,7 +58,7 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   if (tid < 64) {
     float ekv = 1.0f, evv = 1.0f;
     if (DECAY == LQ_DECAY_SCALAR) {
-      const float d = p.g[(t0 + 63) * H + h] - p.g[(t0 + tid) * H + h];
+      const float d = p.g[tlast * H + h] - p.g[(t0 + tid) * H + h];
       ekv = zoo_exp((1.0f - eta) * d);
       evv = zoo_exp(eta * d);
     } else if (DECAY == LQ_DECAY_DIAGONAL) {
@@ -69,8 +72,8 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   }
   if (tid < K) {
     float gm = 1.0f;
-    if (DECAY == LQ_DECAY_SCALAR) gm = zoo_exp(p.g[(t0 + 63) * H + h]);
-    if (DECAY == LQ_DECAY_DIAGONAL) gm = zoo_exp(p.g[((t0 + 63) * H + h) * K + tid]);
+    if (DECAY == LQ_DECAY_SCALAR) gm = zoo_exp(p.g[tlast * H + h]);
+    if (DECAY == LQ_DECAY_DIAGONAL) gm = zoo_exp(p.g[(tlast * H + h) * K + tid]);
     p.gam[cb * K + tid] = gm;
   }
   __syncthreads();
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
     }
     if (DECAY == LQ_DECAY_DIAGONAL) {
 #pragma unroll
-      for (int d = 0; d < CK / 4; ++d) glast[d] = *(const gf_t*)(p.g + ((t0 + 63) * H + h) * K + CK * cg + 4 * d);
+      for (int d = 0; d < CK / 4; ++d) glast[d] = *(const gf_t*)(p.g + (tlast * H + h) * K + CK * cg + 4 * d);
     }
     if (p.w) {
 #pragma unroll
@@ -214,7 +217,10 @@ extern "C" int lq_zoo_write_codes(const lq_zoo_write_codes_args* a, hipStream_t 
   if (a->decay != LQ_DECAY_NONE && !a->g) return LQ_ERR_NULL;
   if (a->decay == LQ_DECAY_DIAGONAL && !a->logenv) return LQ_ERR_NULL;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
+  // 128-token chunks (linear family, no / scalar decay): the state kernel walks them as pairs of 64-token halves
+  const bool pair = a->chunk_size == 128;
+  if (pair && (a->decay == LQ_DECAY_DIAGONAL || a->w || !a->val)) return LQ_ERR_SHAPE;
+  if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
@@ -227,6 +233,7 @@ extern "C" int lq_zoo_write_codes(const lq_zoo_write_codes_args* a, hipStream_t 
   p.g = a->g, p.logenv = a->logenv, p.kqT = a->kqT, p.vqT = a->vqT, p.wq = a->wq, p.ev = a->ev, p.gam = a->gam;
   p.skw = a->skw, p.svw = a->svw, p.sw = a->sw, p.eta = a->eta, p.qmax = a->qmax, p.bf = a->act_dtype == LQ_DT_BF16;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
+  p.span = a->chunk_size;
   dim3 grid(p.NT, a->batch * a->nheads);
   return a->kdim == 128 ? launch<128>(p, a->decay, grid, stream) : launch<64>(p, a->decay, grid, stream);
 }

@@ -46,7 +46,7 @@ def pad_chunks(chunk_size, q, k, v, g=None, beta=None):
     triangular inverse is the identity there), and the sub-block anchoring of the per-channel decay (16-token sub-blocks
     from the start of the chunk) is the reference's own for C a multiple of 16; the state is quantized at every chunk
     boundary as before, i.e. every C real tokens.  Returns (q, k, v, g, beta, restore) with ``restore`` cutting an
-    output back to the caller's tokens.  Chunk sizes above 64 are not built."""
+    output back to the caller's tokens.  (128-token chunks: the no / scalar decay wrapper runs them as pairs of halves.)"""
     T = q.shape[1]
     assert T % chunk_size == 0, f"T={T} must be a multiple of the chunk size {chunk_size}"
     assert 1 <= chunk_size <= CHUNK, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {CHUNK} tokens"
@@ -134,8 +134,8 @@ def unrot_matrix(unrot, V):
     return unrot.to(torch.float16).contiguous()
 
 
-def cumsum(g, B, T, H, kdim, write=None):
-    """Chunk-local cumulative log decay (fp32) and, for per-channel decay, the log envelope.  ``write`` = dict(k, v, skw,
+def cumsum(g, B, T, H, kdim, write=None, span=CHUNK):
+    """Chunk-local cumulative log decay (fp32) over chunks of ``span`` tokens and, for per-channel decay, the log envelope.  ``write`` = dict(k, v, skw,
     svw, eta, qmax) (per-channel decay, linear family): the launch also makes the state kernel's write operands while
     the chunk's decay tile is on chip (what ``write_codes`` would make, same bits) and returns them as a third value."""
     g = f32(g)
@@ -144,8 +144,9 @@ def cumsum(g, B, T, H, kdim, write=None):
     logenv = torch.empty(B, T, H, dtype=torch.float32, device=dev) if kdim else None
     if write is None:
         _lib.call("lq_zoo_cumsum", dev, g=_lib.ptr(g), gc=_lib.ptr(gc), logenv=_lib.ptr(logenv), batch=B, seqlen=T,
-                  nheads=H, kdim=kdim, chunk_size=CHUNK)
+                  nheads=H, kdim=kdim, chunk_size=span)
         return gc, logenv
+    assert span == CHUNK
     k, v = write["k"], write["v"]
     NT, V = T // CHUNK, v.shape[-1]
     c = {"kqT": torch.empty(B, NT, H, kdim, CHUNK, dtype=torch.int8, device=dev),
@@ -159,8 +160,9 @@ def cumsum(g, B, T, H, kdim, write=None):
     return gc, logenv, c
 
 
-def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay):
-    """Write-operand pre-pass: INT8 codes (and decay factors) of everything that does not depend on the carry."""
+def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay, span=CHUNK):
+    """Write-operand pre-pass: INT8 codes (and decay factors) of everything that does not depend on the carry.
+    ``span`` = tokens per chunk (64, or 128 for the linear family: same buffers, decays to the end of the 128-token chunk)."""
     B, T, H, K, V = dims
     dev, NT = key.device, T // CHUNK
     delta = family == FAMILY_DELTA
@@ -173,11 +175,11 @@ def write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family,
               g=_lib.ptr(g), logenv=_lib.ptr(logenv), kqT=_lib.ptr(c["kqT"]), vqT=_lib.ptr(c["vqT"]), wq=_lib.ptr(c["wq"]),
               ev=_lib.ptr(c["ev"]), gam=_lib.ptr(c["gam"]), skw=_lib.ptr(skw), svw=None if delta else _lib.ptr(svw),
               sw=_lib.ptr(sw), eta=float(eta), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K, vdim=V,
-              chunk_size=CHUNK, decay=decay, act_dtype=act_code(key))
+              chunk_size=span, decay=decay, act_dtype=act_code(key))
     return c
 
 
-def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile=0, unrot=None):
+def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile=0, unrot=None, span=CHUNK):
     """Sequential chunk recurrence over the pre-quantized operands ``c`` (see write_codes)."""
     B, T, H, K, V = dims
     delta = family == FAMILY_DELTA
@@ -185,32 +187,35 @@ def state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, fa
               u=_lib.ptr(value) if delta else None, fw=_lib.ptr(fw), ev=_lib.ptr(c["ev"]) if delta else None,
               gam=_lib.ptr(c["gam"]), h_i8=_lib.ptr(h_i8), e_out=_lib.ptr(e_out), ht=_lib.ptr(ht), skw=_lib.ptr(skw),
               svw=_lib.ptr(svw), sw=_lib.ptr(sw), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), qmax=int(qmax), batch=B, seqlen=T, nheads=H,
-              kdim=K, vdim=V, chunk_size=CHUNK, family=family, vtile=int(vtile),
+              kdim=K, vdim=V, chunk_size=span, family=family, vtile=int(vtile),
               act_dtype=act_code(value), pack=_lib.ptr(c.get("pack")) if delta else None)
 
 
 def run_state(key, value, g, logenv, h_i8, ht, skw, svw, ss, eta, qmax, dims, family, decay, w=None, fw=None, e_out=None,
-              sw=None, vtile=0, unrot=None, codes=None):
+              sw=None, vtile=0, unrot=None, codes=None, span=CHUNK):
     """``value`` is v (linear family) or U (delta family); ``codes``: write-operand codes that ``run_wy_prep`` already made
     (no pre-pass then)."""
-    c = codes if codes is not None else write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay)
-    state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile, unrot)
+    c = codes if codes is not None else write_codes(key, value, w, g, logenv, skw, svw, sw, eta, qmax, dims, family, decay, span)
+    state_kernel(c, value, fw, h_i8, e_out, ht, skw, svw, sw, ss, qmax, dims, family, vtile, unrot, span)
     return c
 
 
 def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims, decay, unrot=None, qg=None, local=None,
-               act=None):
+               act=None, span=CHUNK):
     """``A`` (fp16) and ``qg`` (INT8 codes of the decayed query) come from run_gla_A under per-channel decay; q and key
     are only read under no / scalar decay.  ``local`` = (qc, kc, vc): ready-made local codes from ``rotate_quant`` (q,
     key and value are then not read; ``act`` names the activation dtype code)."""
     B, T, H, K, V = dims
     svl, ss = _lib.aligned(svl), _lib.aligned(ss)
     qc, kc, vc = local if local is not None else (None, None, None)
+    # 128-token chunks: workspace for the second halves' products with the first halves' tokens
+    cross = torch.empty(B, T, H, V, dtype=torch.float32, device=h_i8.device) if span != CHUNK else None
     _lib.call("lq_zoo_output", h_i8.device, q=_lib.ptr(q), qg=_lib.ptr(qg), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
               g=_lib.ptr(g), A=_lib.ptr(A), o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), sq=_lib.ptr(sq),
               sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay,
-              act_dtype=act if act is not None else act_code(value), qc=_lib.ptr(qc), kc=_lib.ptr(kc), vc=_lib.ptr(vc))
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=span, decay=decay,
+              act_dtype=act if act is not None else act_code(value), qc=_lib.ptr(qc), kc=_lib.ptr(kc), vc=_lib.ptr(vc),
+              cross=_lib.ptr(cross))
 
 
 def rotate_quant(q, k, v, g, sq, sk, svl, skw, svw, eta, scale, qmax, dims, signs_qk=None, signs_v=None, dqk=None,

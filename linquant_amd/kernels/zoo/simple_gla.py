@@ -20,8 +20,15 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     the model produced them, and the persistent rotations R_QK / R_V (``rotation_signs`` of a signed Hadamard matrix) and
     the D_QK rescaling are applied in the launch that also quantizes the operands: the result of calling
     ``rotate_qkv(q, k, v, ...)`` first and this function on its outputs, bit for bit, in one launch fewer and without the
-    rotated activations ever reaching memory (K, V in {64, 128}, rotated storage)."""
-    if prologue is not None and (q.shape[-1] not in (64, 128) or v.shape[-1] not in (64, 128) or unrot is not None):
+    rotated activations ever reaching memory (K, V in {64, 128}, rotated storage).
+    ``chunk_size``: up to 64 (smaller chunks are padded to 64 tokens), or 128 with rotated storage: the kernels then walk
+    every chunk as two 64-token halves, with one stored state, one carry update (the INT8 write product summed over the 128
+    tokens) and one fp32 local accumulation per chunk."""
+    span = 2 * C.CHUNK if chunk_size == 2 * C.CHUNK else C.CHUNK
+    if span != C.CHUNK:
+        assert unrot is None, "128-token chunks are built for rotated storage"
+        assert q.shape[1] % span == 0, f"T={q.shape[1]} must be a multiple of the chunk size {chunk_size}"
+    if prologue is not None and (q.shape[-1] not in (64, 128) or v.shape[-1] not in (64, 128) or unrot is not None or span != C.CHUNK):
         from .prologue import rotate_qkv  # shapes the fused launch is not built for: rotate up front
 
         K, V = q.shape[-1], v.shape[-1]
@@ -35,7 +42,7 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
         if do_v:
             v = rv
         prologue = None
-    q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g)
+    q, k, v, g, _, restore = C.pad_chunks(C.CHUNK if span != C.CHUNK else chunk_size, q, k, v, g)
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
@@ -48,8 +55,8 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     gg = None
     if g is not None:
         assert g.shape == (B, T, H)
-        gg, _ = C.cumsum(g, B, T, H, 0)
-    NT = T // C.CHUNK
+        gg, _ = C.cumsum(g, B, T, H, 0, span=span)
+    NT = T // span
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
@@ -63,7 +70,8 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
                      local=local, act=C.act_code(v))
         C.export_debug(_debug, h_i8, codes, g=gg, local=local, rotated=rotated)
         return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
-    codes = C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru)
-    C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
+    codes = C.run_state(k, v, gg, None, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR, decay, unrot=Ru,
+                        span=span)
+    C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru, span=span)
     C.export_debug(_debug, h_i8, codes, g=gg)
     return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -85,6 +85,35 @@ def test_one_call_forward_validates_every_stage_limit_before_the_first_launch():
         assert entry(ctypes.byref(args(D=ctypes.addressof(buf), D_scale=None)), None) == -14
 
 
+def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
+    """128-token chunks exist for the linear family with no / scalar decay on raw operands in rotated storage: the three
+    entry points refuse every other combination on the host (the buffers here are host memory: a call that passed
+    validation would launch, so only refusals are exercised)."""
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    a = ctypes.addressof(buf)
+    dims = dict(batch=1, seqlen=256, nheads=1, kdim=64, vdim=64, qmax=127, act_dtype=_lib.LQ_DT_F16)
+
+    def rc(fn, **kw):
+        return getattr(lib, fn)(ctypes.byref(_lib.fill(fn + "_args", **{**dims, **kw})), None)
+
+    wc = dict(key=a, kqT=a, ev=a, gam=a, skw=a, val=a, vqT=a, svw=a, g=a, chunk_size=128)
+    assert rc("lq_zoo_write_codes", **wc, decay=2, logenv=a) == -22                 # per-channel decay
+    assert rc("lq_zoo_write_codes", **wc, decay=1, w=a, wq=a, sw=a) == -22          # delta family operands
+    assert rc("lq_zoo_write_codes", **{**wc, "seqlen": 192}, decay=1) == -22        # not a whole number of chunks
+    assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 256}, decay=1) == -22
+    stt = dict(kqT=a, gam=a, h_i8=a, skw=a, svw=a, ss=a, vqT=a, chunk_size=128)
+    assert rc("lq_zoo_state", **stt, family=1, wq=a, u=a, fw=a, ev=a, e_out=a, sw=a) == -22   # delta family
+    assert rc("lq_zoo_state", **stt, family=0, unrot=a) == -22                                # canonical storage
+    assert rc("lq_zoo_state", **{**stt, "seqlen": 192}, family=0) == -22
+    out = dict(h_i8=a, o=a, sq=a, svl=a, ss=a, q=a, k=a, v=a, sk=a, g=a, chunk_size=128, scale=1.0)
+    assert rc("lq_zoo_output", **out, decay=1) == -14                                         # no cross workspace
+    assert rc("lq_zoo_output", **out, decay=2, A=a, qg=a, cross=a) == -22                     # per-channel decay
+    assert rc("lq_zoo_output", **out, decay=1, cross=a, qc=a, kc=a, vc=a) == -22              # ready-made codes
+    assert rc("lq_zoo_output", **out, decay=1, cross=a, unrot=a) == -22                       # canonical storage
+    assert rc("lq_zoo_output", **{**out, "seqlen": 192}, decay=1, cross=a) == -22
+
+
 def test_every_entry_point_rejects_an_empty_argument_struct():
     """A zeroed argument struct (every pointer NULL, every size 0) and a NULL struct pointer come back as an error code
     from every entry point: nothing is launched and no device is touched."""

@@ -76,6 +76,38 @@ def test_chunk_sizes_below_64(cuda, cell, chunk):
     assert (last - codes[-1]).abs().max().item() <= (2 if cell == "deltanet" else 1)
 
 
+@pytest.mark.parametrize("cell,eta", [("linear_none", 1.0), ("mamba2", 1.0), ("mamba2", 0.0), ("mamba2", 0.5)])
+@pytest.mark.parametrize("K,V,dtype", [(64, 64, torch.float16), (128, 128, torch.float16), (64, 192, torch.bfloat16)])
+def test_chunk_size_128_no_and_scalar_decay(cuda, cell, eta, K, V, dtype):
+    """128-token chunks of the no / scalar decay kernels (linquant/kernels/zoo/simple_gla.py:184: BT = chunk_size is free
+    there): the kernels walk a chunk as two 64-token halves.  Against the oracle run with C = 128: outputs by the
+    reference's criterion, one stored state per 128 tokens with codes within one step of the oracle's (equal but for rare
+    rounding ties), the final carry close to the oracle's last state; and the state entering the second chunk is NOT the one
+    a 64-token chunking stores there (the carry is quantized half as often)."""
+    T = 512
+    tensors = zc.inputs(cell, B=2, T=T, H=3, K=K, V=V, seed=31, dtype=dtype)
+    qz, run = zc.calibrated(cell, tensors, eta=eta, chunk=128)
+    scales = qz.kernel_scales(0, 3, K, V)
+    dbg = {}
+    out, ht = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=128, final_state=True, debug=dbg)
+    torch.cuda.synchronize()
+    assert out.shape == tensors[2].shape and out.dtype == dtype and dbg["h_i8"].shape[1] == T // 128
+    zc.check(out, run, qz, f"{cell} chunk 128 eta={eta}")
+    codes = zc.state_codes(qz, run)                      # (NT, B, H, K, V): state after each chunk
+    got = dbg["h_i8"].cpu()                              # (B, NT, H, K, V): state entering each chunk
+    NT = codes.shape[0]
+    assert NT == T // 128 and (got[:, 0] == 0).all()
+    d = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
+    assert int(d.max()) <= 1 and (d != 0).float().mean().item() < 2e-3, (int(d.max()), (d != 0).float().mean().item())
+    last = torch.round(ht.cpu() / scales["state"][None, :, None, :]).clamp(-127, 127)
+    assert (last - codes[-1]).abs().max().item() <= 1
+    # the same inputs and scales in 64-token chunks: same tokens seen by the state entering token 128, other arithmetic
+    out64, _ = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=64)
+    assert not torch.equal(out64[:, 64:128], out[:, 64:128])  # second half of the first chunk: stored state vs local product
+    if tensors[3] is None:
+        assert torch.equal(out64[:, :64], out[:, :64])        # first half: the same arithmetic either way
+
+
 @pytest.mark.parametrize("cell,eta", [("mamba2", 0.0), ("mamba2", 0.5), ("gla", 0.5), ("gla", 1.0),
                                       ("gated_deltanet", 0.0), ("gated_deltanet", 0.5), ("kda", 0.5), ("kda", 1.0)])
 def test_eta_split(cuda, cell, eta):
