@@ -24,21 +24,25 @@ __global__ __launch_bounds__(256) void cumsum_scalar_kernel(const float* __restr
   }
 }
 
-// The same scan for the chunk size every caller uses: all 64 values of a thread are requested before the first is added
-// (the loop above waits for each load in turn: 64 round trips), summed in the same order.
-__global__ __launch_bounds__(256) void cumsum_scalar64_kernel(const float* __restrict__ g, float* __restrict__ gc, int H,
-                                                              int64_t total) {
+// The same scan for the chunk sizes the callers use (C = 64 or 128): 64 values of a thread are requested before the first
+// is added (the loop above waits for each load in turn: C round trips), summed in the same order.
+template <int C>
+__global__ __launch_bounds__(256) void cumsum_scalar_fixed_kernel(const float* __restrict__ g, float* __restrict__ gc, int H,
+                                                                  int64_t total) {
   const int64_t idx = min((int64_t)blockIdx.x * 256 + threadIdx.x, total - 1);  // (b, chunk, h); the tail repeats the last
   const int h = idx % H;
-  const int64_t base = (idx / H) * 64 * H + h;
-  float v[64];
-#pragma unroll
-  for (int t = 0; t < 64; ++t) v[t] = g[base + (int64_t)t * H];
+  const int64_t base = (idx / H) * C * H + h;
   double run = 0.0;
+#pragma unroll 1
+  for (int t0 = 0; t0 < C; t0 += 64) {
+    float v[64];
 #pragma unroll
-  for (int t = 0; t < 64; ++t) {
-    run += (double)v[t];
-    gc[base + (int64_t)t * H] = (float)run;
+    for (int t = 0; t < 64; ++t) v[t] = g[base + (int64_t)(t0 + t) * H];
+#pragma unroll
+    for (int t = 0; t < 64; ++t) {
+      run += (double)v[t];
+      gc[base + (int64_t)(t0 + t) * H] = (float)run;
+    }
   }
 }
 
@@ -190,8 +194,11 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
   if (a->kdim == 0) {
     const int64_t total = (int64_t)a->batch * NT * a->nheads;
     if (a->chunk_size == 64)
-      hipLaunchKernelGGL(cumsum_scalar64_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g, a->gc,
-                         a->nheads, total);
+      hipLaunchKernelGGL(cumsum_scalar_fixed_kernel<64>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g,
+                         a->gc, a->nheads, total);
+    else if (a->chunk_size == 128)
+      hipLaunchKernelGGL(cumsum_scalar_fixed_kernel<128>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g,
+                         a->gc, a->nheads, total);
     else
       hipLaunchKernelGGL(cumsum_scalar_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g, a->gc,
                          a->seqlen, a->nheads, a->chunk_size, total);
