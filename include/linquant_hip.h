@@ -341,7 +341,7 @@ int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
  * gla.py:124-141, gated_delta_rule.py:85-105, kda.py:100-124): every write operand that does not depend on the
  * carried state is quantized once, in parallel over chunks, into the layout lq_zoo_state consumes.
  * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers.
- * chunk_size is 64, or 128 (linear family, no / scalar decay; seqlen a multiple of 128): the buffers keep their 64-token
+ * chunk_size is 64, or 128 (linear family; seqlen a multiple of 128): the buffers keep their 64-token
  * layout (NT = seqlen / 64) and the decays of a chunk's first 64 tokens reach on to the end of the 128-token chunk. */
 typedef struct {
   const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16/bf16 */
@@ -404,9 +404,9 @@ int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
 /* replaces _output_kernel (linquant/kernels/zoo/simple_gla.py:98-172) and _gla_output_kernel
  * (gla.py:170-232): o = dequant(q8(q).h_i8) [* exp(g)] + (fp16(A) . fp16(q8(v))) * svl, with A computed
  * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay).
- * chunk_size is 64, or 128 (no / scalar decay, raw q, k, v, rotated storage; h_i8 (B,seqlen/128,H,V,K) from lq_zoo_state
- * with chunk_size 128): two launches, the first leaves the second halves' products with the first halves' tokens in
- * `cross`, the second starts its fp32 accumulators from them. */
+ * chunk_size is 64, or 128 (raw q, k, v, rotated storage; h_i8 (B,seqlen/128,H,V,K) from lq_zoo_state with chunk_size
+ * 128; under diagonal decay A and A_cross from lq_zoo_gla_A with chunk_size 128): two launches, the first leaves the
+ * second halves' products with the first halves' tokens in `cross`, the second starts its fp32 accumulators from them. */
 typedef struct {
   const void* q;             /* no / scalar decay: (B,T,H,K) fp16/bf16; diagonal decay: NULL */
   const int8_t* qg;          /* diagonal decay: (B,T,H,K) int8 codes of q*exp(g)*scale written by lq_zoo_gla_A */
@@ -433,12 +433,14 @@ typedef struct {
   const int8_t* kc;          /* (B,T,H,K) int8 q8(k, 1/sk) */
   const int8_t* vc;          /* (B,T,H,V) int8 q8(v, 1/svl) */
   float* cross;              /* chunk_size 128: (B,T,H,V) fp32 workspace, 16-byte aligned (overwritten); else unused */
+  const void* A_cross;       /* chunk_size 128, diagonal decay: (B,T,H,64) fp16 written by lq_zoo_gla_A; else unused */
 } lq_zoo_output_args;
 int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
 
 /* replaces _gla_A_inter + _gla_A_intra (linquant/kernels/zoo/gla.py:27-99): intra-chunk product under
  * per-channel decay, 16-token sub-blocks: INT8 dots on anchor-rescaled operands off the diagonal, fp32
- * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows, zeros above
+ * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows (C = 64; chunk_size 128:
+ * two (64,64) tensors, see A_cross), zeros above
  * the diagonal, and the INT8 codes of the decayed query (gla.py:188-190 computes them in the output kernel). */
 typedef struct {
   const void* q;             /* (B,T,H,K) fp16/bf16 */
@@ -455,6 +457,9 @@ typedef struct {
   int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16: dtype of every 16-bit activation tensor of the call */
   const float* dq;           /* optional (H,K) fp32 D_QK (linquant/harness.py:68-88) applied to q as it is loaded:
                                 q' = act(q * dq), exactly what lq_zoo_rotate_qkv would have stored; NULL: q as it is */
+  void* A_cross;             /* chunk_size 128 (g cumulated over 128 tokens): (B,T,H,64) fp16; rows of the second halves
+                                receive their blocks with the first halves' tokens (column j = token j of the chunk), A
+                                the blocks inside either half, as for chunk_size 64; else unused */
 } lq_zoo_gla_A_args;
 int lq_zoo_gla_A(const lq_zoo_gla_A_args* args, hipStream_t stream);
 

@@ -69,11 +69,16 @@ struct CumsumCodes {
 // loads are independent and issued up front), the four partial totals are combined through LDS; LDS tile [C][K+1]
 // for the envelope reduction.  CODES (chunk 64 only): a thread's 16 tokens of one channel are one 16-byte piece of that
 // channel's row of channel-major codes, so the codes go straight from registers to memory.
-template <bool CODES>
+// SM = tokens per thread at most: 16 (chunks up to 64 tokens), or 32 (128-token chunks: the envelope tile then holds one half
+// of the chunk at a time, so that the workgroup's LDS stays what a 64-token chunk takes).
+template <bool CODES, int SM = 16>
 __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restrict__ gc, float* __restrict__ logenv,
                                    int T, int H, int K, int C, CumsumCodes cc) {
-  extern __shared__ float tile[];           // [C][K + 1]
-  double* part = (double*)(tile + C * (K + 1));  // [4][K] segment totals
+  static_assert(!CODES || SM == 16, "the write codes are made for 64-token chunks");
+  constexpr int PH = SM / 16;               // passes over the envelope tile
+  const int CT = C / PH;                    // tokens the tile holds at a time
+  extern __shared__ float tile[];           // [CT][K + 1]
+  double* part = (double*)(tile + CT * (K + 1));  // [4][K] segment totals
   float* le_s = (float*)(part + 4 * K);      // [C] log envelope (CODES)
   const int k = threadIdx.x % K, q = threadIdx.x / K;
   const int SEG = C / 4;                    // tokens per thread (C is a multiple of 16)
@@ -94,9 +99,9 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
   const int64_t row0 = bc * C;  // global token row of the chunk start (b * T + chunk * C)
   const int64_t base = ((row0 + q * SEG) * H + h) * K + k;
   const int64_t tstride = (int64_t)H * K;
-  float v[16];
+  float v[SM];
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
+  for (int t = 0; t < SM; ++t) {
     // requested without a branch (a load under `t < SEG` is waited for inside its branch: sixteen round trips in a row);
     // tokens past the segment re-read its last one and count as zero
     const float x = g[base + min(t, SEG - 1) * tstride];
@@ -110,9 +115,9 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
     for (int t = 0; t < 16; ++t) kraw[t] = cc.k[base + t * tstride];
     inv_skw = 1.0f / cc.skw[h * K + k];
   }
-  double run = 0.0, pre[16];
+  double run = 0.0, pre[SM];
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
+  for (int t = 0; t < SM; ++t) {
     run += (double)v[t];
     pre[t] = run;
   }
@@ -127,26 +132,31 @@ __global__ void cumsum_diag_kernel(const float* __restrict__ g, float* __restric
   }
   const float last = (float)total;
 #pragma unroll
-  for (int t = 0; t < 16; ++t)
-    if (t < SEG) {
-      const float c = (float)(off + pre[t]);
-      gc[base + t * tstride] = c;
-      tile[(q * SEG + t) * (K + 1) + k] = last - c;
-    }
-  __syncthreads();
-  // envelope: 8 lanes per token, each over a contiguous K/8 slice, then a max over the 8 lanes
-  const int sub = threadIdx.x & 7, KS = K / 8;
-  for (int t = threadIdx.x >> 3; t < C; t += blockDim.x >> 3) {
-    const float* row = tile + t * (K + 1) + sub * KS;
-    float m = row[0];
-    for (int j = 1; j < KS; ++j) m = fmaxf(m, row[j]);
+  for (int t = 0; t < SM; ++t)
+    if (t < SEG) gc[base + t * tstride] = (float)(off + pre[t]);
+#pragma unroll 1
+  for (int ph = 0; ph < PH; ++ph) {
+    if (ph) __syncthreads();  // the previous pass has been read
 #pragma unroll
-    for (int o = 1; o < 8; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
-    if (sub == 0) {
-      logenv[(row0 + t) * H + h] = m;
-      if constexpr (CODES) {
-        le_s[t] = m;
-        cc.ev[(row0 + t) * H + h] = zoo_exp(cc.eta * m);
+    for (int t = 0; t < SM; ++t) {
+      const int tok = q * SEG + t - ph * CT;  // row of the tile
+      if (t < SEG && tok >= 0 && tok < CT) tile[tok * (K + 1) + k] = last - (float)(off + pre[t]);
+    }
+    __syncthreads();
+    // envelope: 8 lanes per token, each over a contiguous K/8 slice, then a max over the 8 lanes
+    const int sub = threadIdx.x & 7, KS = K / 8;
+    for (int t = threadIdx.x >> 3; t < CT; t += blockDim.x >> 3) {
+      const float* row = tile + t * (K + 1) + sub * KS;
+      float m = row[0];
+      for (int j = 1; j < KS; ++j) m = fmaxf(m, row[j]);
+#pragma unroll
+      for (int o = 1; o < 8; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
+      if (sub == 0) {
+        logenv[(row0 + ph * CT + t) * H + h] = m;
+        if constexpr (CODES) {
+          le_s[t] = m;
+          cc.ev[(row0 + t) * H + h] = zoo_exp(cc.eta * m);
+        }
       }
     }
   }
@@ -204,9 +214,12 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
                          a->seqlen, a->nheads, a->chunk_size, total);
   } else {
     if (!a->logenv) return LQ_ERR_NULL;
-    if (a->kdim > 256 || a->kdim % 16 != 0 || a->chunk_size % 16 != 0 || a->chunk_size > 64) return LQ_ERR_SHAPE;
-    const size_t lds = (size_t)a->chunk_size * (a->kdim + 1) * sizeof(float) + 4 * (size_t)a->kdim * sizeof(double) +
-                       (size_t)a->chunk_size * sizeof(float);
+    const bool big = a->chunk_size == 128;  // two passes over an envelope tile of 64 tokens
+    if (a->kdim > 256 || a->kdim % 16 != 0 || a->chunk_size % 16 != 0 || (a->chunk_size > 64 && !big)) return LQ_ERR_SHAPE;
+    if (big && a->kqT) return LQ_ERR_SHAPE;
+    const int ctile = big ? 64 : a->chunk_size;
+    const size_t lds = (size_t)ctile * (a->kdim + 1) * sizeof(float) + 4 * (size_t)a->kdim * sizeof(double) +
+                       (size_t)ctile * sizeof(float);
     if (lds > 64 * 1024) return LQ_ERR_SHAPE;
     CumsumCodes cc = {};
     const dim3 grid((unsigned)((int64_t)a->batch * NT * a->nheads)), block(4 * a->kdim);
@@ -219,6 +232,9 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
       cc.skw = a->skw, cc.svw = a->svw, cc.eta = a->eta, cc.qmax = a->qmax, cc.V = a->vdim, cc.bf = a->act_dtype == LQ_DT_BF16;
       hipLaunchKernelGGL(cumsum_diag_kernel<true>, grid, block, lds, stream, a->g, a->gc, a->logenv, a->seqlen, a->nheads,
                          a->kdim, a->chunk_size, cc);
+    } else if (big) {
+      hipLaunchKernelGGL((cumsum_diag_kernel<false, 32>), grid, block, lds, stream, a->g, a->gc, a->logenv, a->seqlen,
+                         a->nheads, a->kdim, a->chunk_size, cc);
     } else {
       hipLaunchKernelGGL(cumsum_diag_kernel<false>, grid, block, lds, stream, a->g, a->gc, a->logenv, a->seqlen, a->nheads,
                          a->kdim, a->chunk_size, cc);

@@ -22,7 +22,7 @@
 // blocks are never rotated.
 #include <type_traits>
 
-#include "zoo_common.h"
+#include "zoo_params.h"
 #include "../../include/linquant_hip.h"
 
 namespace {
@@ -373,7 +373,12 @@ __global__ __launch_bounds__(256, 3) void zoo_gla_A_kernel(AParams p) {
 extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
   if (!a || !a->q || !a->k || !a->g || !a->A || !a->sq || !a->sk) return LQ_ERR_NULL;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
+  // 128-token chunks: the blocks inside either half are those of 64-token chunks (g cumulated over the 128 tokens), the
+  // blocks between the halves come from a second launch into A_cross
+  const bool pair = a->chunk_size == 128;
+  if (pair && !a->A_cross) return LQ_ERR_NULL;
+  if (pair && !zoo_al(a->A_cross, 16)) return LQ_ERR_SHAPE;
+  if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if (a->kdim != 64 && a->kdim != 128) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
@@ -421,5 +426,13 @@ extern "C" int lq_zoo_gla_A(const lq_zoo_gla_A_args* a, hipStream_t stream) {
 #undef LQ_A_LAUNCH3
 #undef LQ_A_LAUNCH2
 #undef LQ_A_LAUNCH
+  if (pair) {
+    const int rc = lq_check_launch();
+    if (rc) return rc;
+    ZooACrossParams c = {};
+    c.q = p.q, c.k = p.k, c.g = p.g, c.Ax = (_Float16*)a->A_cross, c.sq = p.sq, c.sk = p.sk, c.rot = p.rot, c.dq = p.dq;
+    c.scale = p.scale, c.qmax = p.qmax, c.bf = p.bf, c.B = p.B, c.T = p.T, c.H = p.H;
+    return zoo_gla_A_cross_launch(c, a->kdim, stream);
+  }
   return lq_check_launch();
 }

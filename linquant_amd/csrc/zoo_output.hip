@@ -31,11 +31,11 @@ using OutParams = ZooOutParams;
 // tiles instead of being quantized here.
 // CROSS (128-token chunks, which run as pairs of 64-token halves): this launch makes, for the second half of every chunk,
 // the part of the local product that reaches back into the first half -- fp16(Af[i][j]) . fp16(q8(v_j)) over the 64 tokens j
-// of the first half, no causal mask, no state read -- and leaves it as fp32 in p.cross; the ordinary launch that follows
+// of the first half, no causal mask, no state read; under per-channel decay Af comes from p.Ax -- and leaves it as fp32 in p.cross; the ordinary launch that follows
 // starts its local accumulators from it (one fp32 accumulation over the 128 tokens, oldest first, as a 128-token tile has).
 template <bool GLA, bool USE_G, int K, bool BF, int NV, bool CIN, bool CROSS = false>
 __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
-  static_assert(!CROSS || (!GLA && !CIN), "the cross launch exists for the no / scalar decay kernels on raw operands");
+  static_assert(!CROSS || !CIN, "the cross launch exists for raw operands");
   constexpr int QS = K + 16;  // byte stride of a code row
   __shared__ __align__(16) unsigned char qc[GLA ? 16 : 64 * QS];
   __shared__ __align__(16) unsigned char kc[GLA ? 16 : 64 * QS];
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   lq_v4i qgop[GLA ? K / 64 : 1];
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
-    if constexpr (GLA) qgop[ks] = *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
+    if constexpr (GLA && !CROSS) qgop[ks] = *(const lq_v4i*)(p.qg + ((t0 + 16 * wave + rl) * H + h) * K + 64 * ks + 16 * kg);
     if constexpr (!CROSS) {
 #pragma unroll
       for (int n = 0; n < NV; ++n)
@@ -211,8 +211,10 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   for (int jt = 0; jt < 4; ++jt) a32[jt] = lq_v4i{0, 0, 0, 0};
 #pragma unroll
   for (int ks = 0; ks < K / 64; ++ks) {
-    lq_v4i qop;
-    if constexpr (GLA)
+    lq_v4i qop = {0, 0, 0, 0};
+    if constexpr (GLA && CROSS)
+      break;  // nothing to contract: A arrives ready-made, the state is not read
+    else if constexpr (GLA)
       qop = qgop[ks];
     else
       qop = *(const lq_v4i*)(qc + (16 * wave + rl) * QS + 64 * ks + 16 * kg);
@@ -277,7 +279,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   for (int n = 0; n < NV; ++n)
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) loc[n][jj] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-  if constexpr (!GLA && !CROSS) {
+  if constexpr (!CROSS) {
     if (p.cross && (ct & 1)) {  // second half of a 128-token chunk: what the cross launch left for these rows
 #pragma unroll
       for (int n = 0; n < NV; ++n)
@@ -293,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   for (int js = 0; js < nslab; ++js) {
     lq_v8h aop;
     if (GLA) {
-      aop = *(const lq_v8h*)(p.A + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg);
+      aop = *(const lq_v8h*)((CROSS ? p.Ax : p.A) + ((t0 + 16 * wave + rl) * H + h) * 64 + 32 * js + 8 * kg);
     } else {
       aop = *(const lq_v8h*)(Afl + (16 * wave + rl) * kAS + 32 * js + 8 * kg);
     }
@@ -333,19 +335,17 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   }
 }
 
-template <bool USE_G, int K, int NV>
+template <bool GLA, bool USE_G, int K, int NV>
 void launch_cross(const OutParams& p, dim3 grid, hipStream_t stream) {
   if (p.bf)
-    hipLaunchKernelGGL((zoo_output_kernel<false, USE_G, K, true, NV, false, true>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, true, NV, false, true>), grid, dim3(256), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_output_kernel<false, USE_G, K, false, NV, false, true>), grid, dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false, NV, false, true>), grid, dim3(256), 0, stream, p);
 }
 
 template <bool GLA, bool USE_G, int K, int NV>
 void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
-  if constexpr (!GLA) {
-    if (p.cross) launch_cross<USE_G, K, NV>(p, dim3(grid.x, grid.y / 2, grid.z), stream);
-  }
+  if (p.cross) launch_cross<GLA, USE_G, K, NV>(p, dim3(grid.x, grid.y / 2, grid.z), stream);
   if constexpr (!GLA) {
     if (p.qc) {  // ready-made codes: the activation dtype only matters for a 16-bit output
       if (p.bf)
@@ -393,11 +393,11 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks (no / scalar decay, raw operands, rotated storage) run as pairs of 64-token halves
+  // 128-token chunks (raw operands, rotated storage) run as pairs of 64-token halves
   const bool pair = a->chunk_size == 128;
-  if (pair && (gla || cin || a->unrot)) return LQ_ERR_SHAPE;
-  if (pair && !a->cross) return LQ_ERR_NULL;
-  if (pair && !zoo_al(a->cross, 16)) return LQ_ERR_SHAPE;
+  if (pair && (cin || a->unrot)) return LQ_ERR_SHAPE;
+  if (pair && (!a->cross || (gla && !a->A_cross))) return LQ_ERR_NULL;
+  if (pair && (!zoo_al(a->cross, 16) || (gla && !zoo_al(a->A_cross, 16)))) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
@@ -414,6 +414,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.unrot = (const _Float16*)a->unrot;
   p.qc = a->qc, p.kc = a->kc, p.vc = a->vc;
   p.cross = pair ? a->cross : nullptr, p.hshift = pair ? 1 : 0;
+  p.Ax = pair ? (const _Float16*)a->A_cross : nullptr;
   if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
   if (gla) return launch<true, true>(p, a->kdim, stream);
   if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, stream);

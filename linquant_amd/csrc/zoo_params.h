@@ -48,9 +48,27 @@ struct ZooOutParams {
   int qmax;
   int bf;  // activations (and a 16-bit output) are bf16
   int B, T, H, V, NT;
+  const _Float16* Ax;  // 128-token chunks under per-channel decay: (B,T,H,64) fp16 from the cross launch of the A kernel
   float* cross;  // 128-token chunks: fp32 (B,T,H,V) partial local products of the second halves, else nullptr
   int hshift;    // log2 of the 64-token halves per stored state (1 for 128-token chunks)
 };
+
+// 128-token chunks under per-channel decay: the second halves' blocks of the intra-chunk product with the first halves' tokens
+struct ZooACrossParams {
+  const _Float16* q;
+  const _Float16* k;
+  const float* g;
+  _Float16* Ax;  // (B,T,H,64) fp16, rows of the second halves
+  const float* sq;
+  const float* sk;
+  const _Float16* rot;
+  const float* dq;
+  float scale;
+  int qmax;
+  int bf;
+  int B, T, H;
+};
+int zoo_gla_A_cross_launch(const ZooACrossParams& p, int K, hipStream_t stream);  // defined in zoo_gla_A_cross.hip
 
 // canonical storage: one workgroup spans all V value channels (V = 64 or 128); defined in zoo_unrot.hip
 int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, hipStream_t stream);

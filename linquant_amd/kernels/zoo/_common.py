@@ -208,6 +208,7 @@ def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims,
     B, T, H, K, V = dims
     svl, ss = _lib.aligned(svl), _lib.aligned(ss)
     qc, kc, vc = local if local is not None else (None, None, None)
+    A, Ax = A if isinstance(A, tuple) else (A, None)
     # 128-token chunks: workspace for the second halves' products with the first halves' tokens
     cross = torch.empty(B, T, H, V, dtype=torch.float32, device=h_i8.device) if span != CHUNK else None
     _lib.call("lq_zoo_output", h_i8.device, q=_lib.ptr(q), qg=_lib.ptr(qg), k=_lib.ptr(key), v=_lib.ptr(value), h_i8=_lib.ptr(h_i8),
@@ -215,7 +216,7 @@ def run_output(q, key, value, h_i8, g, A, o, sq, sk, svl, ss, scale, qmax, dims,
               sk=_lib.ptr(sk), svl=_lib.ptr(svl), ss=_lib.ptr(ss), unrot=_lib.ptr(unrot), scale=float(scale), qmax=int(qmax),
               batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=span, decay=decay,
               act_dtype=act if act is not None else act_code(value), qc=_lib.ptr(qc), kc=_lib.ptr(kc), vc=_lib.ptr(vc),
-              cross=_lib.ptr(cross))
+              cross=_lib.ptr(cross), A_cross=_lib.ptr(Ax))
 
 
 def rotate_quant(q, k, v, g, sq, sk, svl, skw, svw, eta, scale, qmax, dims, signs_qk=None, signs_v=None, dqk=None,
@@ -255,17 +256,19 @@ def dqk_tables(dqk, H, K):
     return d, _lib.aligned((1.0 / d).contiguous())
 
 
-def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None, dq=None):
+def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None, dq=None, span=CHUNK):
     """Returns (A fp16 (B,T,H,64), qg int8 (B,T,H,K)): the intra-chunk product and the codes of q*exp(g)*scale.
-    ``dq`` (H,K): q is multiplied by it (and rounded to the activation dtype) as it is loaded."""
+    ``dq`` (H,K): q is multiplied by it (and rounded to the activation dtype) as it is loaded.  ``span`` = 128: A is a pair
+    (A, A_cross), the blocks inside the 64-token halves and the second halves' blocks with the first halves' tokens."""
     B, T, H, K, _ = dims
     A = torch.empty(B, T, H, CHUNK, dtype=torch.float16, device=q.device)
+    Ax = torch.empty(B, T, H, CHUNK, dtype=torch.float16, device=q.device) if span != CHUNK else None
     qg = torch.empty(B, T, H, K, dtype=torch.int8, device=q.device)
     assert rot is None or tuple(rot.shape) == (K, K), "rot: (K, K) R_QK"
     _lib.call("lq_zoo_gla_A", q.device, q=_lib.ptr(q), k=_lib.ptr(key), g=_lib.ptr(gc), A=_lib.ptr(A), qg=_lib.ptr(qg), rot=_lib.ptr(rot),
               sq=_lib.ptr(sq), sk=_lib.ptr(sk), scale=float(scale), qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K,
-              chunk_size=CHUNK, act_dtype=act_code(q), dq=_lib.ptr(dq))
-    return A, qg
+              chunk_size=span, act_dtype=act_code(q), dq=_lib.ptr(dq), A_cross=_lib.ptr(Ax))
+    return (A if Ax is None else (A, Ax)), qg
 
 
 def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True, dk=(None, None)):

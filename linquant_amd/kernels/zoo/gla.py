@@ -16,9 +16,14 @@ BC = 16  # secondary chunk
 def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, output_final_state=False, unrot=None,
                    rot=None, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
-    Returns (o, final fp32 state or None)."""
+    Returns (o, final fp32 state or None).  ``chunk_size``: a multiple of 16 up to 64, or 128 with rotated storage (the
+    kernels walk such a chunk as two 64-token halves; the sub-block anchoring over its eight sub-blocks is the reference's)."""
     assert g.shape == q.shape
-    q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g)
+    span = 2 * C.CHUNK if chunk_size == 2 * C.CHUNK else C.CHUNK
+    if span != C.CHUNK:
+        assert unrot is None, "128-token chunks are built for rotated storage"
+        assert q.shape[1] % span == 0, f"T={q.shape[1]} must be a multiple of the chunk size {chunk_size}"
+    q, k, v, g, _, restore = C.pad_chunks(C.CHUNK if span != C.CHUNK else chunk_size, q, k, v, g)
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
@@ -31,15 +36,18 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     qmax = 2 ** (bits - 1) - 1
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
     # the cumsum launch also makes the state kernel's write operands (it holds the chunk's decay tile): no pre-pass
-    gc, logenv, codes = C.cumsum(g, B, T, H, K, write=dict(k=k, v=v, skw=sc["kw"], svw=sc["vw"], eta=eta, qmax=qmax))
-    A, qg = C.run_gla_A(q, k, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R)
-    NT = T // C.CHUNK
+    if span == C.CHUNK:
+        gc, logenv, codes = C.cumsum(g, B, T, H, K, write=dict(k=k, v=v, skw=sc["kw"], svw=sc["vw"], eta=eta, qmax=qmax))
+    else:
+        (gc, logenv), codes = C.cumsum(g, B, T, H, K, span=span), None
+    A, qg = C.run_gla_A(q, k, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R, span=span)
+    NT = T // span
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
-                C.DECAY_DIAGONAL, unrot=Ru, codes=codes)
+    codes = C.run_state(k, v, gc, logenv, h_i8, ht, sc["kw"], sc["vw"], sc["state"], eta, qmax, dims, C.FAMILY_LINEAR,
+                        C.DECAY_DIAGONAL, unrot=Ru, codes=codes, span=span)
     C.run_output(None, None, v, h_i8, None, A, o, sc["q"], None, sc["vl"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
-                 unrot=Ru, qg=qg)
+                 unrot=Ru, qg=qg, span=span)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, g=gc, logenv=logenv)
     return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -86,8 +86,8 @@ def test_one_call_forward_validates_every_stage_limit_before_the_first_launch():
 
 
 def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
-    """128-token chunks exist for the linear family with no / scalar decay on raw operands in rotated storage: the three
-    entry points refuse every other combination on the host (the buffers here are host memory: a call that passed
+    """128-token chunks exist for the linear family on raw operands in rotated storage: the entry points refuse every
+    other combination on the host (the buffers here are host memory: a call that passed
     validation would launch, so only refusals are exercised)."""
     lib = _lib.load()
     buf = (ctypes.c_char * 4096)()
@@ -95,10 +95,10 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
     dims = dict(batch=1, seqlen=256, nheads=1, kdim=64, vdim=64, qmax=127, act_dtype=_lib.LQ_DT_F16)
 
     def rc(fn, **kw):
-        return getattr(lib, fn)(ctypes.byref(_lib.fill(fn + "_args", **{**dims, **kw})), None)
+        known = {n for n, _ in _lib.STRUCTS[fn + "_args"]._fields_}
+        return getattr(lib, fn)(ctypes.byref(_lib.fill(fn + "_args", **{k: v for k, v in {**dims, **kw}.items() if k in known})), None)
 
     wc = dict(key=a, kqT=a, ev=a, gam=a, skw=a, val=a, vqT=a, svw=a, g=a, chunk_size=128)
-    assert rc("lq_zoo_write_codes", **wc, decay=2, logenv=a) == -22                 # per-channel decay
     assert rc("lq_zoo_write_codes", **wc, decay=1, w=a, wq=a, sw=a) == -22          # delta family operands
     assert rc("lq_zoo_write_codes", **{**wc, "seqlen": 192}, decay=1) == -22        # not a whole number of chunks
     assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 256}, decay=1) == -22
@@ -108,10 +108,16 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
     assert rc("lq_zoo_state", **{**stt, "seqlen": 192}, family=0) == -22
     out = dict(h_i8=a, o=a, sq=a, svl=a, ss=a, q=a, k=a, v=a, sk=a, g=a, chunk_size=128, scale=1.0)
     assert rc("lq_zoo_output", **out, decay=1) == -14                                         # no cross workspace
-    assert rc("lq_zoo_output", **out, decay=2, A=a, qg=a, cross=a) == -22                     # per-channel decay
+    assert rc("lq_zoo_output", **out, decay=2, A=a, qg=a, cross=a) == -14                     # per-channel decay: no A_cross
     assert rc("lq_zoo_output", **out, decay=1, cross=a, qc=a, kc=a, vc=a) == -22              # ready-made codes
     assert rc("lq_zoo_output", **out, decay=1, cross=a, unrot=a) == -22                       # canonical storage
     assert rc("lq_zoo_output", **{**out, "seqlen": 192}, decay=1, cross=a) == -22
+    ga = dict(q=a, k=a, g=a, A=a, sq=a, sk=a, chunk_size=128, scale=1.0)
+    assert rc("lq_zoo_gla_A", **ga) == -14                                                    # no A_cross
+    assert rc("lq_zoo_gla_A", **{**ga, "seqlen": 192}, A_cross=a) == -22
+    cs = dict(g=a, gc=a, logenv=a, chunk_size=128)
+    assert rc("lq_zoo_cumsum", **cs, kqT=a, k=a, v=a, vqT=a, ev=a, gam=a, skw=a, svw=a) == -22   # no write codes at 128
+    assert rc("lq_zoo_cumsum", **{**cs, "chunk_size": 96}) == -22
 
 
 def test_every_entry_point_rejects_an_empty_argument_struct():

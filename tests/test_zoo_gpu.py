@@ -76,20 +76,25 @@ def test_chunk_sizes_below_64(cuda, cell, chunk):
     assert (last - codes[-1]).abs().max().item() <= (2 if cell == "deltanet" else 1)
 
 
-@pytest.mark.parametrize("cell,eta", [("linear_none", 1.0), ("mamba2", 1.0), ("mamba2", 0.0), ("mamba2", 0.5)])
+@pytest.mark.parametrize("cell,eta,rot", [("linear_none", 1.0, False), ("mamba2", 1.0, False), ("mamba2", 0.0, False),
+                                          ("mamba2", 0.5, False), ("gla", 0.0, False), ("gla", 0.5, False), ("gla", 1.0, True)])
 @pytest.mark.parametrize("K,V,dtype", [(64, 64, torch.float16), (128, 128, torch.float16), (64, 192, torch.bfloat16)])
-def test_chunk_size_128_no_and_scalar_decay(cuda, cell, eta, K, V, dtype):
-    """128-token chunks of the no / scalar decay kernels (linquant/kernels/zoo/simple_gla.py:184: BT = chunk_size is free
-    there): the kernels walk a chunk as two 64-token halves.  Against the oracle run with C = 128: outputs by the
-    reference's criterion, one stored state per 128 tokens with codes within one step of the oracle's (equal but for rare
-    rounding ties), the final carry close to the oracle's last state; and the state entering the second chunk is NOT the one
-    a 64-token chunking stores there (the carry is quantized half as often)."""
+def test_chunk_size_128_linear_family(cuda, cell, eta, rot, K, V, dtype):
+    """128-token chunks of the linear family (linquant/kernels/zoo/simple_gla.py:184, gla.py:244-246: BT = chunk_size is
+    free there; under per-channel decay the eight 16-token sub-blocks of a chunk are anchored as gla.py:27-63 does, with
+    or without the local R_QK): the kernels walk a chunk as two 64-token halves.  Against the oracle run with C = 128:
+    outputs by the reference's criterion, one stored state per 128 tokens with codes within one step of the oracle's (equal
+    but for rare rounding ties), the final carry close to the oracle's last state; and the second half of the first chunk
+    differs from what a 64-token chunking gives there (a stored state read against a local product)."""
     T = 512
     tensors = zc.inputs(cell, B=2, T=T, H=3, K=K, V=V, seed=31, dtype=dtype)
-    qz, run = zc.calibrated(cell, tensors, eta=eta, chunk=128)
+    from oracle.zoo_reference import signed_hadamard
+
+    R = signed_hadamard(K, 3) if rot else None
+    qz, run = zc.calibrated(cell, tensors, eta=eta, chunk=128, rot_qk=R)
     scales = qz.kernel_scales(0, 3, K, V)
     dbg = {}
-    out, ht = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=128, final_state=True, debug=dbg)
+    out, ht = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=128, final_state=True, debug=dbg, rot=R)
     torch.cuda.synchronize()
     assert out.shape == tensors[2].shape and out.dtype == dtype and dbg["h_i8"].shape[1] == T // 128
     zc.check(out, run, qz, f"{cell} chunk 128 eta={eta}")
@@ -102,10 +107,43 @@ def test_chunk_size_128_no_and_scalar_decay(cuda, cell, eta, K, V, dtype):
     last = torch.round(ht.cpu() / scales["state"][None, :, None, :]).clamp(-127, 127)
     assert (last - codes[-1]).abs().max().item() <= 1
     # the same inputs and scales in 64-token chunks: same tokens seen by the state entering token 128, other arithmetic
-    out64, _ = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=64)
+    out64, _ = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=64, rot=R)
     assert not torch.equal(out64[:, 64:128], out[:, 64:128])  # second half of the first chunk: stored state vs local product
     if tensors[3] is None:
         assert torch.equal(out64[:, :64], out[:, :64])        # first half: the same arithmetic either way
+
+
+@pytest.mark.parametrize("K,rot", [(64, False), (128, False), (64, True), (128, True)])
+def test_chunk_128_cross_blocks_equal_the_64_token_kernel_on_a_shifted_window(cuda, K, rot):
+    """The blocks of the intra-chunk product that pair a row of a 128-token chunk's second half with a token of its first
+    half (gla.py:27-63 with BT = 128) come from a kernel of their own.  Tokens 32..95 of the chunk, taken as one 64-token
+    chunk, have the same sub-blocks, anchors and decay differences: the 64-token kernel (checked against the oracle
+    elsewhere) must give the same entries there, up to the last-bit difference that cumulating g from another token leaves
+    in a decay difference (a changed code on a rounding tie; with a rotation the fp16 rounding in front of it sees that
+    bit too: a few entries in a thousand move by one code step)."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.inputs("gla", B=2, T=256, H=3, K=K, V=64, seed=5)
+    R = signed_hadamard(K, 3) if rot else None
+    qz, _ = zc.calibrated("gla", tensors, eta=0.5, chunk=128, rot_qk=R)
+    scales = qz.kernel_scales(0, 3, K, 64)
+    dbg, dwin = {}, {}
+    zc.run_kernel("gla", tensors, scales, eta=0.5, chunk=128, debug=dbg, rot=R)
+    window = [t[:, 32:96].contiguous() if t is not None else None for t in tensors]
+    zc.run_kernel("gla", window, scales, eta=0.5, chunk=64, debug=dwin, rot=R)
+    A, Ax = dbg["A"]
+    for c in (0, 1):  # both chunks of the 128-token run have such a window; the second one's is tokens 160..223
+        if c == 1:
+            window = [t[:, 160:224].contiguous() if t is not None else None for t in tensors]
+            dwin = {}
+            zc.run_kernel("gla", window, scales, eta=0.5, chunk=64, debug=dwin, rot=R)
+        want = dwin["A"][:, 32:64, :, 0:32].float().cpu()
+        got = Ax[:, 128 * c + 64:128 * c + 96, :, 32:64].float().cpu()
+        top = want.abs().max().item()
+        d = (got - want).abs()
+        assert top > 0 and d.max().item() <= 0.02 * top and (d != 0).float().mean().item() <= 1e-2, (c, top, d.max().item())
+        inside = (A[:, 128 * c + 64:128 * c + 96, :, 0:32].float().cpu() - dwin["A"][:, 32:64, :, 32:64].float().cpu()).abs()
+        assert inside.max().item() <= 0.02 * top
 
 
 @pytest.mark.parametrize("cell,eta", [("mamba2", 0.0), ("mamba2", 0.5), ("gla", 0.5), ("gla", 1.0),
