@@ -154,14 +154,16 @@ def test_eta_split(cuda, cell, eta):
     zc.check(out, run, qz, f"{cell} eta={eta}")
 
 
-@pytest.mark.parametrize("name", list(zc.CONFIGS))
-def test_full_size_slices(cuda, name):
+@pytest.mark.parametrize("name,chunk", [(n, 64) for n in zc.CONFIGS] + [("c2_la", 128), ("c2_gla", 128)],
+                         ids=list(zc.CONFIGS) + ["c2_la-chunk128", "c2_gla-chunk128"])
+def test_full_size_slices(cuda, name, chunk):
     """The benchmark configurations as they are stated, at full size (K = V = 128, chunk 64): c2 linear attention and
     GLA under kernel_pt with N(0,1) queries, c3 DeltaNet / Gated DeltaNet under kernel_ptk with the write gate at
     sigma = 0.5, c4 KDA under per-channel static scales with D_QK (alpha = 0.5) and the local R_QK; static scales from a
     separate seed-1 batch.  Every (batch row, head) is an independent recurrence, so the full-size launch must reproduce,
     bit for bit, a launch on one batch row and two non-adjacent heads cut out of the same inputs; that cut is small
-    enough for the float64 oracle and is held to the reference's criterion over the whole 64- or 128-chunk horizon."""
+    enough for the float64 oracle and is held to the reference's criterion over the whole 64- or 128-chunk horizon.
+    The two linear-family configurations also run in 128-token chunks (oracle at C = 128)."""
     import sys
 
     from linquant_amd.calibration import dqk_from_absmax
@@ -181,12 +183,13 @@ def test_full_size_slices(cuda, name):
     part = [t[b:b + 1, :, hs].contiguous() if t is not None else None for t in tensors]
     fam, dec = zc.CELLS[cell]
     eta, rho = cfg["eta"], cfg["rho"]
-    qz, run = zc.calibrated(cell, part, policy=cfg["policy"], eta=eta, rho=rho, rot_qk=rot, calib_tensors=calib)
+    qz, run = zc.calibrated(cell, part, policy=cfg["policy"], eta=eta, rho=rho, rot_qk=rot, calib_tensors=calib, chunk=chunk)
     sc = qz.kernel_scales(0, 2, K, V, delta=fam == "delta")
     pick = torch.zeros(H, dtype=torch.long)
     pick[hs[1]] = 1                                                  # every other head borrows the first cut head's scales
-    out_full, _ = zc.run_kernel(cell, tensors, {n: s[pick].contiguous() for n, s in sc.items()}, eta=eta, rho=rho, rot=rot)
-    out_part, _ = zc.run_kernel(cell, part, sc, eta=eta, rho=rho, rot=rot)
+    out_full, _ = zc.run_kernel(cell, tensors, {n: s[pick].contiguous() for n, s in sc.items()}, eta=eta, rho=rho, rot=rot,
+                                chunk=chunk)
+    out_part, _ = zc.run_kernel(cell, part, sc, eta=eta, rho=rho, rot=rot, chunk=chunk)
     torch.cuda.synchronize()
     assert torch.isfinite(out_full).all()
     assert torch.equal(out_full[b:b + 1][:, :, hs], out_part), f"{name}: the full-size launch differs from the launch on its cut"
