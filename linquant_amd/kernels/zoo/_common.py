@@ -39,8 +39,15 @@ def pad_keys(q, k, g, scales, rot=None):
     return q, k, g, scales, rot, K
 
 
-def pad_chunks(chunk_size, q, k, v, g=None, beta=None):
-    """Chunk sizes below 64 run on the 64-token kernels: every chunk of C tokens is followed by 64 - C padding tokens with
+def chunk_span(chunk_size):
+    """Tokens per chunk as the linear-family kernels run it: 64, or 128 for chunk sizes above 64 (pad_chunks fills up)."""
+    assert 1 <= chunk_size <= 2 * CHUNK, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {2 * CHUNK} tokens"
+    return CHUNK if chunk_size <= CHUNK else 2 * CHUNK
+
+
+def pad_chunks(chunk_size, q, k, v, g=None, beta=None, span=CHUNK):
+    """Chunk sizes below ``span`` (64; 128 where the kernels walk a chunk as two halves) run on the ``span``-token kernels:
+    every chunk of C tokens is followed by span - C padding tokens with
     q = k = v = 0, log decay 0 and beta = 1.  Padding tokens add nothing to any product (their codes are zero), leave the
     decay accumulated over the chunk and hence the carried state unchanged, their Gram rows and columns are zero (the
     triangular inverse is the identity there), and the sub-block anchoring of the per-channel decay (16-token sub-blocks
@@ -49,20 +56,20 @@ def pad_chunks(chunk_size, q, k, v, g=None, beta=None):
     output back to the caller's tokens.  (128-token chunks: the no / scalar decay wrapper runs them as pairs of halves.)"""
     T = q.shape[1]
     assert T % chunk_size == 0, f"T={T} must be a multiple of the chunk size {chunk_size}"
-    assert 1 <= chunk_size <= CHUNK, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {CHUNK} tokens"
-    if chunk_size == CHUNK:
+    assert 1 <= chunk_size <= span, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {span} tokens"
+    if chunk_size == span:
         return q, k, v, g, beta, lambda o: o
-    NT, pad = T // chunk_size, CHUNK - chunk_size
+    NT, pad = T // chunk_size, span - chunk_size
 
     def widen(t, value=0.0):
         if t is None:
             return None
         x = t.reshape(t.shape[0], NT, chunk_size, *t.shape[2:])
         x = torch.nn.functional.pad(x, (0, 0) * (x.dim() - 3) + (0, pad), value=value)
-        return x.reshape(t.shape[0], NT * CHUNK, *t.shape[2:])
+        return x.reshape(t.shape[0], NT * span, *t.shape[2:])
 
     def restore(o):
-        x = o.reshape(o.shape[0], NT, CHUNK, *o.shape[2:])[:, :, :chunk_size]
+        x = o.reshape(o.shape[0], NT, span, *o.shape[2:])[:, :, :chunk_size]
         return x.reshape(o.shape[0], T, *o.shape[2:]).contiguous()
 
     return widen(q), widen(k), widen(v), widen(g), widen(beta, 1.0), restore

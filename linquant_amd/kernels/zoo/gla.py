@@ -16,14 +16,12 @@ BC = 16  # secondary chunk
 def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, output_final_state=False, unrot=None,
                    rot=None, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
-    Returns (o, final fp32 state or None).  ``chunk_size``: a multiple of 16 up to 64, or 128 with rotated storage (the
-    kernels walk such a chunk as two 64-token halves; the sub-block anchoring over its eight sub-blocks is the reference's)."""
+    Returns (o, final fp32 state or None).  ``chunk_size``: a multiple of 16 up to 64, or up to 128 with rotated storage (the
+    kernels walk a chunk of more than 64 tokens as two 64-token halves, padded to 128 tokens; the sub-block anchoring over its eight sub-blocks is the reference's)."""
     assert g.shape == q.shape
-    span = 2 * C.CHUNK if chunk_size == 2 * C.CHUNK else C.CHUNK
-    if span != C.CHUNK:
-        assert unrot is None, "128-token chunks are built for rotated storage"
-        assert q.shape[1] % span == 0, f"T={q.shape[1]} must be a multiple of the chunk size {chunk_size}"
-    q, k, v, g, _, restore = C.pad_chunks(C.CHUNK if span != C.CHUNK else chunk_size, q, k, v, g)
+    span = C.chunk_span(chunk_size)
+    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
+    q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g, span=span)
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()

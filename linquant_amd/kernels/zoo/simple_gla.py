@@ -21,13 +21,11 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     the D_QK rescaling are applied in the launch that also quantizes the operands: the result of calling
     ``rotate_qkv(q, k, v, ...)`` first and this function on its outputs, bit for bit, in one launch fewer and without the
     rotated activations ever reaching memory (K, V in {64, 128}, rotated storage).
-    ``chunk_size``: up to 64 (smaller chunks are padded to 64 tokens), or 128 with rotated storage: the kernels then walk
-    every chunk as two 64-token halves, with one stored state, one carry update (the INT8 write product summed over the 128
+    ``chunk_size``: up to 64 (smaller chunks are padded to 64 tokens), or up to 128 with rotated storage (padded to 128): the
+    kernels then walk every chunk as two 64-token halves, with one stored state, one carry update (the INT8 write product summed over the 128
     tokens) and one fp32 local accumulation per chunk."""
-    span = 2 * C.CHUNK if chunk_size == 2 * C.CHUNK else C.CHUNK
-    if span != C.CHUNK:
-        assert unrot is None, "128-token chunks are built for rotated storage"
-        assert q.shape[1] % span == 0, f"T={q.shape[1]} must be a multiple of the chunk size {chunk_size}"
+    span = C.chunk_span(chunk_size)
+    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
     if prologue is not None and (q.shape[-1] not in (64, 128) or v.shape[-1] not in (64, 128) or unrot is not None or span != C.CHUNK):
         from .prologue import rotate_qkv  # shapes the fused launch is not built for: rotate up front
 
@@ -42,7 +40,7 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
         if do_v:
             v = rv
         prologue = None
-    q, k, v, g, _, restore = C.pad_chunks(C.CHUNK if span != C.CHUNK else chunk_size, q, k, v, g)
+    q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g, span=span)
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()

@@ -113,6 +113,31 @@ def test_chunk_size_128_linear_family(cuda, cell, eta, rot, K, V, dtype):
         assert torch.equal(out64[:, :64], out[:, :64])        # first half: the same arithmetic either way
 
 
+@pytest.mark.parametrize("cell", ["linear_none", "mamba2", "gla"])
+@pytest.mark.parametrize("chunk", [80, 96, 112])
+def test_chunk_sizes_between_64_and_128(cuda, cell, chunk):
+    """Multiples of 16 between the two built tile counts (the reference takes any, gla.py:246): the wrappers lay such a
+    chunk out as a 128-token chunk whose tail is padding (zero operands, zero log decay).  Against the oracle at that
+    chunk size: outputs, one stored state per chunk with codes within one step, final state."""
+    T = 3 * chunk
+    tensors = zc.inputs(cell, B=1, T=T, H=2, K=64, V=64, seed=29)
+    eta = DEFAULT_ETA[cell]
+    qz, run = zc.calibrated(cell, tensors, eta=eta, chunk=chunk)
+    scales = qz.kernel_scales(0, 2, 64, 64)
+    dbg = {}
+    out, ht = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=chunk, final_state=True, debug=dbg)
+    torch.cuda.synchronize()
+    assert out.shape == tensors[2].shape and dbg["h_i8"].shape[1] == 3
+    zc.check(out, run, qz, f"{cell} chunk {chunk}")
+    codes = zc.state_codes(qz, run)
+    got = dbg["h_i8"].cpu()
+    assert codes.shape[0] == 3 and (got[:, 0] == 0).all()
+    d = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[:2].int()).abs()
+    assert int(d.max()) <= 1 and (d != 0).float().mean().item() < 2e-3, (int(d.max()), (d != 0).float().mean().item())
+    last = torch.round(ht.cpu() / scales["state"][None, :, None, :]).clamp(-127, 127)
+    assert (last - codes[-1]).abs().max().item() <= 1
+
+
 @pytest.mark.parametrize("K,rot", [(64, False), (128, False), (64, True), (128, True)])
 def test_chunk_128_cross_blocks_equal_the_64_token_kernel_on_a_shifted_window(cuda, K, rot):
     """The blocks of the intra-chunk product that pair a row of a 128-token chunk's second half with a token of its first
