@@ -150,3 +150,23 @@ def test_fused_prologue_falls_back_for_widths_it_is_not_built_for(cuda):
     o1, _ = zoo.chunk_simple_gla_int8(dev(q), dev(k), dev(v), dev(g), sc, prologue=dict(signs_v=sv))
     torch.cuda.synchronize()
     assert torch.equal(o0, o1)
+
+
+def test_fused_prologue_with_128_token_chunks_rotates_up_front(cuda):
+    """The one-launch rotation + quantization is built for 64-token chunks; with chunk_size = 128 the call rotates up front
+    and gives, bit for bit, what rotate_qkv followed by the call gives."""
+    from linquant_amd.kernels import zoo
+
+    q, k, v, g, _ = zc.cut(zc.inputs("mamba2", B=1, H=2, K=64, V=64, seed=6), 256)
+    sq, sv = (zoo.rotation_signs(Z.signed_hadamard(64, s).to(cuda)) for s in (1, 2))
+    sc = {"q": torch.full((2,), 0.002), "k": torch.full((2,), 0.01), "kw": torch.full((2, 64), 0.01),
+          "vw": torch.full((2, 64), 0.03), "vl": torch.full((2, 64), 0.03), "state": torch.full((2, 64), 0.05)}
+    sc = {n: t.to(cuda) for n, t in sc.items()}
+    dev = lambda t: t.to(cuda)  # noqa: E731
+    qr, kr, vr = zoo.rotate_qkv(dev(q), dev(k), dev(v), signs_qk=sq, signs_v=sv)
+    o0, h0 = zoo.chunk_simple_gla_int8(qr, kr, vr, dev(g), sc, chunk_size=128, output_final_state=True)
+    o1, h1 = zoo.chunk_simple_gla_int8(dev(q), dev(k), dev(v), dev(g), sc, chunk_size=128, output_final_state=True,
+                                       prologue=dict(signs_qk=sq, signs_v=sv))
+    o64, _ = zoo.chunk_simple_gla_int8(qr, kr, vr, dev(g), sc, chunk_size=64)
+    torch.cuda.synchronize()
+    assert torch.equal(o0, o1) and torch.equal(h0, h1) and not torch.equal(o0, o64)
