@@ -341,7 +341,7 @@ int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
  * gla.py:124-141, gated_delta_rule.py:85-105, kda.py:100-124): every write operand that does not depend on the
  * carried state is quantized once, in parallel over chunks, into the layout lq_zoo_state consumes.
  * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers.
- * chunk_size is 64, or 128 (linear family; seqlen a multiple of 128): the buffers keep their 64-token
+ * chunk_size is 64, or 128 (seqlen a multiple of 128): the buffers keep their 64-token
  * layout (NT = seqlen / 64) and the decays of a chunk's first 64 tokens reach on to the end of the 128-token chunk. */
 typedef struct {
   const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16/bf16 */
@@ -370,9 +370,9 @@ int lq_zoo_write_codes(const lq_zoo_write_codes_args* args, hipStream_t stream);
  * sequential chunk loop with an fp32 carry, INT8 stored copy per chunk, INT8 write product (and, delta family,
  * the INT8 state read W.S and the pseudo-values E = (U - W.S) * fw, stored fp16 for the output kernel).
  * Consumes the buffers written by lq_zoo_write_codes.
- * chunk_size is 64, or 128 (linear family, rotated storage; operands from lq_zoo_write_codes with chunk_size 128): one
- * stored state per 128 tokens, h_i8 is (B,seqlen/128,H,V,K), and the carry takes the INT8 write product summed over the
- * 128 tokens (int32) once per chunk. */
+ * chunk_size is 64, or 128 (rotated storage; operands from lq_zoo_write_codes with chunk_size 128, delta family: W and U
+ * from lq_zoo_wy_prep with chunk_size 128): one stored state per 128 tokens, h_i8 is (B,seqlen/128,H,V,K), both halves of
+ * a chunk read it, and the carry takes the INT8 write product summed over the 128 tokens (int32) once per chunk. */
 typedef struct {
   const int8_t* kqT;         /* (B,NT,H,K,64) */
   const int8_t* vqT;         /* linear family: (B,NT,H,V,64) */
@@ -466,7 +466,9 @@ int lq_zoo_gla_A(const lq_zoo_gla_A_args* args, hipStream_t stream);
 /* replaces the WY / UT prep of the delta family (linquant/kernels/zoo/gated_delta_rule.py:20-47 and
  * kda.py:22-53; the reference's default sigma=tau=1 route through fla-core's prep kernels is replaced by
  * the same native prep): fp32 Gram with decay, unit-lower-triangular inverse, W = T.(L*exp(g)),
- * U = T.(beta^sigma v), Hw = beta^((1-sigma)tau) k, fw = beta^((1-sigma)(1-tau)). */
+ * U = T.(beta^sigma v), Hw = beta^((1-sigma)tau) k, fw = beta^((1-sigma)(1-tau)).
+ * chunk_size is 64, or 128 (g cumulated over 128 tokens; 128 x 128 Gram matrix and inverse in a kernel of its own,
+ * which stores Hw, W, U, fw only: kqT, dk_div and pack must be NULL, lq_zoo_write_codes makes the write codes). */
 typedef struct {
   const void* k;             /* (B,T,H,K) fp16/bf16 */
   const void* v;             /* (B,T,H,V) fp16/bf16 */

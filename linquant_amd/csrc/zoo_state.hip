@@ -38,13 +38,13 @@ struct StepOps {
 
 // BF (bf16 activations) is a template parameter: as a run-time flag every decode / encode of U and E in the chunk loop
 // became a branch of its own.
-// PAIR (linear family, 128-token chunks): the chunk loop still walks 64-token halves, whose operands the pre-pass wrote
-// with the decay to the end of the 128-token chunk.  The state is quantized and stored at the first half only (index
-// ct / 2), the INT8 write product of the first half stays in the accumulators that the second half's product adds to, and
-// the carry takes decay and product once per chunk: the integer sum over 128 tokens that one 128-token tile gives.
+// PAIR (128-token chunks): the chunk loop still walks 64-token halves, whose operands the pre-pass wrote with the decay
+// to the end of the 128-token chunk.  The state is quantized and stored at the first half only (index ct / 2; the delta
+// family's second half reads that same stored copy: its W and U come from a WY transform over the 128 tokens), the INT8
+// write product of the first half stays in the accumulators that the second half's product adds to, and the carry takes
+// decay and product once per chunk: the integer sum over 128 tokens that one 128-token tile gives.
 template <bool DELTA, int K, int BV, bool BF, bool PAIR = false>
 __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StateParams p) {
-  static_assert(!PAIR || !DELTA, "128-token chunks exist for the linear family");
   constexpr int KR = K / 4;     // carry rows per wave
   constexpr int KT = KR / 16;   // 16-row tiles per wave (= K / 64)
   constexpr int VT = BV / 16;   // 16-col tiles
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       // the rest of chunk ct + 2's operands are requested while the matrix unit and then the vector ALU are busy: one wave
       // per SIMD issues in order, and 18 requests in a row held it for as long as the memory pipeline took to accept them
       load_part(std::integral_constant<int, 2>{}, ctn, pre);
-      copy_out();  // behind the products and the requests: nothing in this step waits for it
+      if (!second) copy_out();  // behind the products and the requests: nothing in this step waits for it
       // lane holds tokens 16*wave + 4kg + r, value columns v0 + NJ*rl + jj
       uint32_t ecode[NJ][4];
       const lq_v4f fw4 = *(const lq_v4f*)(misc_s + 4 * kg), ev4 = *(const lq_v4f*)(misc_s + 16 + 4 * kg);
@@ -376,11 +376,12 @@ int launch_bv(const StateParams& p, int BV, int B, hipStream_t stream, bool pair
   constexpr bool D = DELTA;  // the linear family touches no half-precision tensor: one instantiation serves both dtypes
 #define LQ_STATE_LAUNCH(BVV)                                                                                  \
   do {                                                                                                        \
-    if constexpr (!D) {                                                                                       \
-      if (pair) {                                                                                             \
-        hipLaunchKernelGGL((zoo_state_kernel<false, K, BVV, false, true>), grid, dim3(256), 0, stream, p);    \
-        break;                                                                                                \
-      }                                                                                                       \
+    if (pair) {                                                                                               \
+      if (D && p.bf)                                                                                          \
+        hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, BVV, D, true>), grid, dim3(256), 0, stream, p);        \
+      else                                                                                                    \
+        hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, BVV, false, true>), grid, dim3(256), 0, stream, p);    \
+      break;                                                                                                  \
     }                                                                                                         \
     if (D && p.bf)                                                                                            \
       hipLaunchKernelGGL((zoo_state_kernel<DELTA, K, BVV, D>), grid, dim3(256), 0, stream, p);                \
@@ -407,9 +408,9 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (!delta && !a->vqT) return LQ_ERR_NULL;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks (linear family, rotated storage) run as pairs of 64-token halves
+  // 128-token chunks (rotated storage) run as pairs of 64-token halves
   const bool pair = a->chunk_size == 128;
-  if (pair && (delta || a->unrot)) return LQ_ERR_SHAPE;
+  if (pair && a->unrot) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
@@ -438,6 +439,6 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
     else
       BV = wg64 >= 1024 ? 64 : (wg64 >= 512 ? 32 : 16);
   }
-  if (delta) return a->kdim == 128 ? launch_bv<true, 128>(p, BV, a->batch, stream) : launch_bv<true, 64>(p, BV, a->batch, stream);
+  if (delta) return a->kdim == 128 ? launch_bv<true, 128>(p, BV, a->batch, stream, pair) : launch_bv<true, 64>(p, BV, a->batch, stream, pair);
   return a->kdim == 128 ? launch_bv<false, 128>(p, BV, a->batch, stream, pair) : launch_bv<false, 64>(p, BV, a->batch, stream, pair);
 }

@@ -217,9 +217,8 @@ extern "C" int lq_zoo_write_codes(const lq_zoo_write_codes_args* a, hipStream_t 
   if (a->decay != LQ_DECAY_NONE && !a->g) return LQ_ERR_NULL;
   if (a->decay == LQ_DECAY_DIAGONAL && !a->logenv) return LQ_ERR_NULL;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks (linear family): the state kernel walks them as pairs of 64-token halves
+  // 128-token chunks: the state kernel walks them as pairs of 64-token halves
   const bool pair = a->chunk_size == 128;
-  if (pair && (a->w || !a->val)) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;

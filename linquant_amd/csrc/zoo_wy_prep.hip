@@ -152,18 +152,18 @@ LQ_DEV lq_v4f tx_tile(const uint32_t* Xt, const lq_v4i (&th)[2], const lq_v4i (&
 // the decay spread over the whole chunk is too large for one anchor): operands straight from global memory, lane
 // (rl, kg) supplies 16 contiguous channels of token rl per 64-channel pass; off-diagonal blocks: both factors <= 1;
 // diagonal block: only when the spread inside the block is small, otherwise one exponential per (i, j, channel).
-template <int DECAY, int K, bool BF, bool DK>
-LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, const float* bh_s, const float* gs_s, int wave,
+// NB = row blocks of the chunk (4, or 8 for the 128-token kernel), GS = floats per row of the G tile.
+template <int DECAY, int K, bool BF, bool DK, int NB = 4, int GS = kGS>
+LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, const float* bh_s, const float* gs_s, int I,
                           int rl, int kg, int64_t t0, int h, const float* dk_s) {
   const int H = p.H;
   constexpr bool bf = BF;
-    const int I = wave;
     const int64_t irow = ((t0 + 16 * I + rl) * H + h) * K;
     const int64_t arow = ((t0 + 16 * I) * H + h) * K;
     const float bs_i = bs_s[16 * I + rl];
-    lq_v4f acc[4];
+    lq_v4f acc[NB];
 #pragma unroll
-    for (int J = 0; J < 4; ++J) acc[J] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+    for (int J = 0; J < NB; ++J) acc[J] = lq_v4f{0.f, 0.f, 0.f, 0.f};
     bool exact_diag = false;
     if (DECAY == LQ_DECAY_DIAGONAL) {
       float spread = 0.0f;
@@ -204,7 +204,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
         }
       }
 #pragma unroll
-      for (int J = 0; J < 4; ++J) {
+      for (int J = 0; J < NB; ++J) {
         if (J > I) continue;
         if (DECAY == LQ_DECAY_DIAGONAL && J == I && exact_diag) continue;
         const int64_t jrow = ((t0 + 16 * J + rl) * H + h) * K;
@@ -232,7 +232,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
     }
     // lane holds column j = rl of block J, rows i = 4kg + r of block I
 #pragma unroll
-    for (int J = 0; J < 4; ++J) {
+    for (int J = 0; J < NB; ++J) {
       if (J > I) continue;
       if (DECAY == LQ_DECAY_DIAGONAL && J == I && exact_diag) continue;
 #pragma unroll
@@ -243,7 +243,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
           v = acc[J][r];
           if (DECAY == LQ_DECAY_SCALAR) v = v * zoo_exp(gs_s[i] - gs_s[j]);
         }
-        G_s[i * kGS + j] = v;
+        G_s[i * GS + j] = v;
       }
     }
     if (DECAY == LQ_DECAY_DIAGONAL && exact_diag) {
@@ -272,7 +272,7 @@ LQ_DEV void gram_rowblock(const WyParams& p, float* G_s, const float* bs_s, cons
         }
       }
 #pragma unroll
-      for (int jj = 0; jj < 4; ++jj) G_s[(16 * I + rl) * kGS + 16 * I + 4 * kg + jj] = (rl > 4 * kg + jj) ? sacc[jj] : 0.0f;
+      for (int jj = 0; jj < 4; ++jj) G_s[(16 * I + rl) * GS + 16 * I + 4 * kg + jj] = (rl > 4 * kg + jj) ? sacc[jj] : 0.0f;
     }
 }
 
@@ -739,6 +739,188 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
   }
 }
 
+// ---- 128-token chunks: the same transform over a 128 x 128 Gram matrix (gated_delta_rule.py:20-47, kda.py:22-53 with
+// chunk_size = 128), written for reach, not for speed: one workgroup per (chunk, batch*head) with the G and T tiles in LDS
+// (134 KB: one workgroup per compute unit), everything on the fp32 MFMA.
+//   Gram: wave w takes row blocks w and 7 - w (equal numbers of 16 x 16 blocks), per-channel decay anchored at the row
+//     block's first row (both factors <= 1), operands straight from global memory (gram_rowblock).
+//   Inverse: the eight diagonal blocks by forward substitution, then block rows 1..7.
+//   W, U: T . X with X staged as fp32 in LDS 32 columns at a time (over the dead G tile).
+// No write codes (lq_zoo_write_codes makes them from the stored Hw and W), no D_QK at load.
+constexpr int kGS2 = 134;  // floats per row of the 128-row G / T tiles (2 mod 4, as kGS)
+constexpr int kXS2 = 48;   // floats per token row of the X slab (16 mod 32: the two halves of a wave's read hit disjoint banks)
+
+template <int DECAY, int K, bool BF>
+__global__ __launch_bounds__(256) void zoo_wy_prep128_kernel(WyParams p) {
+  __shared__ __align__(16) float G_s[128 * kGS2];
+  __shared__ __align__(16) float T_s[128 * kGS2];
+  __shared__ float gs_s[128], bs_s[128], bh_s[128], bw_s[128];
+  static_assert(128 * kXS2 <= 128 * kGS2, "the X slab overlays the G tile");
+  float* X_s = G_s;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rl = lane & 15, kg = lane >> 4;
+  const int H = p.H, V = p.V;
+  const int h = blockIdx.x % H;
+  const int64_t grp = blockIdx.x / H;  // b * (T / 128) + chunk
+  const int64_t t0 = grp * 128;        // (b * T + chunk * 128: T is a multiple of 128)
+  const float sigma = p.sigma, tau = p.tau;
+  constexpr bool bf = BF;
+
+  if (tid < 128) {
+    const float bt = p.beta[(t0 + tid) * H + h];
+    bs_s[tid] = powb(bt, sigma);
+    bh_s[tid] = powb(bt, 1.0f - sigma);
+    bw_s[tid] = powb(bt, (1.0f - sigma) * tau);
+    p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
+    gs_s[tid] = DECAY == LQ_DECAY_SCALAR ? p.g[(t0 + tid) * H + h] : 0.0f;
+  }
+  // T starts as zero: the blocks right of the diagonal are read as part of whole rows below
+  for (int it = tid; it < 128 * kGS2; it += 256) T_s[it] = 0.0f;
+  __syncthreads();
+
+  // ---- Gram
+#pragma unroll 1
+  for (int u = 0; u < 2; ++u)
+    gram_rowblock<DECAY, K, BF, false, 8, kGS2>(p, G_s, bs_s, bh_s, gs_s, u ? 7 - wave : wave, rl, kg, t0, h, nullptr);
+  __syncthreads();
+
+  // ---- T = (I + G)^-1: diagonal blocks (wave w: blocks w and w + 4; lane c < 16 holds column c)
+  if (lane < 16) {
+#pragma unroll 1
+    for (int u = 0; u < 2; ++u) {
+      const int o = 16 * (wave + 4 * u);
+      float tc[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float a = (i == lane) ? 1.0f : 0.0f;
+#pragma unroll
+        for (int j = 0; j < i; ++j) a = fmaf(-G_s[(o + i) * kGS2 + o + j], tc[j], a);
+        tc[i] = a;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) T_s[(o + i) * kGS2 + o + lane] = tc[i];
+    }
+  }
+  __syncthreads();
+  // block rows 1..7: T_IJ = -T_II . sum_{J <= M < I} G_IM . T_MJ, the J of a row dealt to the waves
+#pragma unroll 1
+  for (int I = 1; I < 8; ++I) {
+#pragma unroll 1
+    for (int J = wave; J < I; J += 4) {
+      lq_v4f sacc = {0.f, 0.f, 0.f, 0.f};
+      for (int M = J; M < I; ++M)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const int m = 16 * M + 4 * s + kg;
+          sacc = mfma_f32(G_s[(16 * I + rl) * kGS2 + m], T_s[m * kGS2 + 16 * J + rl], sacc);
+        }
+      // sacc: lane (rl = column, kg) holds rows 4kg + r, which is contraction index 4kg + s of the next product
+      lq_v4f tacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) tacc = mfma_f32(T_s[(16 * I + rl) * kGS2 + 16 * I + 4 * kg + s], sacc[s], tacc);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) T_s[(16 * I + 4 * kg + r) * kGS2 + 16 * J + rl] = -tacc[r];
+    }
+    __syncthreads();
+  }
+
+  // ---- W = T . X (X = beta^sigma k exp(g)) and U = T . (beta^sigma v), 32 columns at a time; Hw goes straight out.
+  // Staging: thread (token = tid / 2, half = tid % 2) forms 16 columns of its token.
+  const int tok = tid >> 1, hf = tid & 1;
+  const int nslab = (K + V) / 32;
+#pragma unroll 1
+  for (int sl = 0; sl < nslab; ++sl) {
+    const bool isk = sl < K / 32;
+    const int c0 = (isk ? 32 * sl : 32 * sl - K) + 16 * hf;  // first column of this thread in k (or v)
+    __syncthreads();  // the slab (first pass: the G tile) is no longer read
+    {
+      float x[16];
+      if (isk) {
+        const int64_t off = ((t0 + tok) * H + h) * K + c0;
+        float kk[16];
+        zoo_ld8(p.k + off, bf, *(float(*)[8])kk);
+        zoo_ld8(p.k + off + 8, bf, *(float(*)[8])(kk + 8));
+        float bl = bs_s[tok];
+        if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(gs_s[tok]);
+        const float bw = bw_s[tok];
+        float hw[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          x[e] = bl * kk[e];
+          hw[e] = bw * kk[e];
+        }
+        if (DECAY == LQ_DECAY_DIAGONAL) {
+#pragma unroll
+          for (int e4 = 0; e4 < 4; ++e4) {
+            const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[4 * e4 + e] = x[4 * e4 + e] * zoo_exp(g4[e]);
+          }
+        }
+        lq_v4i o0, o1;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          o0[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+          o1[d] = (int)zoo_enc2(hw[8 + 2 * d], hw[8 + 2 * d + 1], bf);
+        }
+        *(lq_v4i*)(p.Hw + off) = o0;
+        *(lq_v4i*)(p.Hw + off + 8) = o1;
+      } else {
+        const int64_t off = ((t0 + tok) * H + h) * V + c0;
+        float vv[16];
+        zoo_ld8(p.v + off, bf, *(float(*)[8])vv);
+        zoo_ld8(p.v + off + 8, bf, *(float(*)[8])(vv + 8));
+        const float bsr = bs_s[tok];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) x[e] = bsr * vv[e];
+      }
+#pragma unroll
+      for (int e4 = 0; e4 < 4; ++e4)
+        *(lq_v4f*)(X_s + tok * kXS2 + 16 * hf + 4 * e4) = lq_v4f{x[4 * e4], x[4 * e4 + 1], x[4 * e4 + 2], x[4 * e4 + 3]};
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int u = 0; u < 2; ++u) {
+      const int I = u ? 7 - wave : wave;
+      lq_v4f acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+      for (int s = 0; s < 4 * (I + 1); ++s) {
+        const float t = T_s[(16 * I + rl) * kGS2 + 4 * s + kg];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) acc[nt] = mfma_f32(t, X_s[(4 * s + kg) * kXS2 + 16 * nt + rl], acc[nt]);
+      }
+      // lane holds column 16nt + rl of the slab, rows 16I + 4kg + r
+      _Float16* dst = isk ? p.W : p.U;
+      const int C = isk ? K : V, cc = isk ? 32 * sl : 32 * sl - K;
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          *(uint16_t*)(dst + ((t0 + 16 * I + 4 * kg + r) * H + h) * C + cc + 16 * nt + rl) = (uint16_t)zoo_enc1(acc[nt][r], bf);
+    }
+  }
+}
+
+template <int DECAY, int K>
+int launch128(const WyParams& p, hipStream_t stream) {
+  const dim3 grid((uint32_t)((int64_t)(p.T / 128) * p.B * p.H));
+  if (p.bf)
+    hipLaunchKernelGGL((zoo_wy_prep128_kernel<DECAY, K, true>), grid, dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((zoo_wy_prep128_kernel<DECAY, K, false>), grid, dim3(256), 0, stream, p);
+  return lq_check_launch();
+}
+
+template <int K>
+int launch128_decay(const WyParams& p, int decay, hipStream_t stream) {
+  switch (decay) {
+    case LQ_DECAY_NONE: return launch128<LQ_DECAY_NONE, K>(p, stream);
+    case LQ_DECAY_SCALAR: return launch128<LQ_DECAY_SCALAR, K>(p, stream);
+    case LQ_DECAY_DIAGONAL: return launch128<LQ_DECAY_DIAGONAL, K>(p, stream);
+  }
+  return LQ_ERR_SHAPE;
+}
+
 template <int DECAY, int K, bool CODES, bool DK>
 int launch_c(const WyParams& p, dim3 grid, hipStream_t stream) {
   if (p.bf)
@@ -780,10 +962,14 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   if (a->dk_div && !codes) return LQ_ERR_SHAPE;  // built for the launch that also makes the write operands
   if (a->dk_div && (!zoo_al(a->dk_div, 16) || !zoo_al(a->dk_rcp, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  if (a->chunk_size != 64 || a->seqlen % 64 != 0) return LQ_ERR_SHAPE;
+  // 128-token chunks: a kernel of their own, without the write codes and without D_QK at load
+  const bool big = a->chunk_size == 128;
+  if (big && (codes || a->dk_div || !a->W)) return LQ_ERR_SHAPE;
+  if ((a->chunk_size != 64 && !big) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->act_dtype != LQ_DT_F16 && a->act_dtype != LQ_DT_BF16) return LQ_ERR_SHAPE;
   if (!zoo_al(a->k, 16) || !zoo_al(a->v, 16) || !zoo_al(a->Hw, 16)) return LQ_ERR_SHAPE;
+  if (a->decay == LQ_DECAY_DIAGONAL && !zoo_al(a->g, 16)) return LQ_ERR_SHAPE;
   if ((int64_t)a->batch * a->nheads > 65535) return LQ_ERR_SHAPE;
   WyParams p = {};
   p.k = (const _Float16*)a->k, p.v = (const _Float16*)a->v, p.beta = a->beta, p.g = a->g;
@@ -795,6 +981,7 @@ extern "C" int lq_zoo_wy_prep(const lq_zoo_wy_prep_args* a, hipStream_t stream) 
   p.dk_div = a->dk_div, p.dk_rcp = a->dk_rcp;
   p.pack = a->pack;
   if ((int64_t)(a->seqlen / 64) * a->batch * a->nheads > 0x7fffffff) return LQ_ERR_SHAPE;
+  if (big) return a->kdim == 128 ? launch128_decay<128>(p, a->decay, stream) : launch128_decay<64>(p, a->decay, stream);
   dim3 grid((uint32_t)((a->seqlen / 64) * a->batch * a->nheads));
   return a->kdim == 128 ? launch_decay<128>(p, a->decay, grid, stream) : launch_decay<64>(p, a->decay, grid, stream);
 }

@@ -278,12 +278,14 @@ def run_gla_A(q, key, gc, sq, sk, scale, qmax, dims, rot=None, dq=None, span=CHU
     return (A if Ax is None else (A, Ax)), qg
 
 
-def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True, dk=(None, None)):
+def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True, dk=(None, None), span=CHUNK):
     """Returns (Hw, W, U, fw, codes): operands of the delta state kernel in the activation dtype and the value-side share
     of beta.  ``write`` = dict(logenv, skw, sw, eta, qmax): the launch also makes the state kernel's write-operand codes
     (what ``write_codes`` would make from the stored Hw and W, same bits) and returns them as ``codes``; W itself is
     then stored only when ``keep_W``.  ``dk`` = (D, 1 / D) from ``dqk_tables``: k is divided by D (and rounded to the
-    activation dtype) as it is loaded; needs ``write``."""
+    activation dtype) as it is loaded; needs ``write``.  ``span`` = 128: the transform over 128-token chunks (a kernel of
+    its own; neither ``write`` nor ``dk``)."""
+    assert span == CHUNK or (write is None and dk[0] is None)
     B, T, H, K, V = dims
     dev, NT = k.device, T // CHUNK
     Hw = torch.empty_like(k)
@@ -304,7 +306,7 @@ def run_wy_prep(k, v, beta, gc, sigma, tau, dims, decay, write=None, keep_W=True
                      qmax=int(write["qmax"]))
     _lib.call("lq_zoo_wy_prep", dev, k=_lib.ptr(k), v=_lib.ptr(v), beta=_lib.ptr(beta), g=_lib.ptr(gc),
               Hw=_lib.ptr(Hw), W=_lib.ptr(W), U=_lib.ptr(U), fw=_lib.ptr(fw), sigma=float(sigma), tau=float(tau),
-              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=CHUNK, decay=decay, act_dtype=act_code(k),
+              batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=span, decay=decay, act_dtype=act_code(k),
               dk_div=_lib.ptr(dk[0]), dk_rcp=_lib.ptr(dk[1]), **extra)
     return Hw, W, U, fw, c
 

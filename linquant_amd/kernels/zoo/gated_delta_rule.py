@@ -15,8 +15,12 @@ from . import _common as C
 def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, scale=None, chunk_size=64,
                      output_final_state=False, unrot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None (DeltaNet), beta [B,T,H].
-    scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None)."""
-    q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta)
+    scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None).
+    ``chunk_size``: up to 64 (padded to 64 tokens), or up to 128 with rotated storage (padded to 128: the WY transform then
+    runs over 128 x 128 Gram matrices in a kernel of its own, the state and output kernels walk a chunk as two halves)."""
+    span = C.chunk_span(chunk_size)
+    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
+    q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta, span=span)
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
@@ -30,19 +34,23 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     gg = None
     if g is not None:
         assert g.shape == (B, T, H)
-        gg, _ = C.cumsum(g, B, T, H, 0)
+        gg, _ = C.cumsum(g, B, T, H, 0, span=span)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
     # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
-    Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay,
-                                        write=dict(logenv=None, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
-                                        keep_W=_debug is not None)
-    NT = T // C.CHUNK
+    if span == C.CHUNK:
+        Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay,
+                                            write=dict(logenv=None, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
+                                            keep_W=_debug is not None)
+    else:  # the write-operand codes come from the pre-pass launch
+        Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay, span=span)
+    NT = T // span
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
-                w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes)
-    C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay, unrot=Ru)
+    codes = C.run_state(Hw, U, gg, None, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA, decay,
+                        w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes, span=span)
+    C.run_output(q, Hw, e_out, h_i8, gg, None, o, sc["q"], sc["k"], sc["el"], sc["state"], scale, qmax, dims, decay, unrot=Ru,
+                 span=span)
     C.export_debug(_debug, h_i8, codes, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -19,14 +19,17 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None).
     ``dqk`` (H,K) fp32, not in the reference's signature: the diagonal rescaling D_QK of linquant/harness.py:68-88
     (q' = q D, k' = k / D, rounded to the activation dtype) applied inside the kernels as they load q and k, with the
-    result of calling ``rotate_qkv(q, k, None, dqk=dqk)`` first, bit for bit, and without that launch."""
+    result of calling ``rotate_qkv(q, k, None, dqk=dqk)`` first, bit for bit, and without that launch.
+    ``chunk_size``: a multiple of 16 up to 64, or up to 128 with rotated storage (as ``chunk_delta_int8``)."""
     assert g.shape == q.shape
-    if dqk is not None and q.shape[-1] not in (64, 128):
+    span = C.chunk_span(chunk_size)
+    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
+    if dqk is not None and (q.shape[-1] not in (64, 128) or span != C.CHUNK):
         # widths the kernels widen with zero channels: rescale up front (same roundings: one fp32 product, one quotient)
         d = dqk.to(q.device)
         q, k = (q.float() * d.float()).to(q.dtype), (k.double() / d.double()).float().to(k.dtype)
         dqk = None
-    q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta)
+    q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta, span=span)
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)
     q, k, v, beta = q.contiguous(), k.contiguous(), v.contiguous(), beta.contiguous()
@@ -37,22 +40,25 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
-    gc, logenv = C.cumsum(g, B, T, H, K)
+    gc, logenv = C.cumsum(g, B, T, H, K, span=span)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
     # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
     dq, dq_rcp = C.dqk_tables(dqk, H, K)
-    Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL,
-                                        write=dict(logenv=logenv, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
-                                        keep_W=_debug is not None, dk=(dq, dq_rcp))
-    A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R, dq=dq)
-    NT = T // C.CHUNK
+    if span == C.CHUNK:
+        Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL,
+                                            write=dict(logenv=logenv, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),
+                                            keep_W=_debug is not None, dk=(dq, dq_rcp))
+    else:  # (D_QK was applied up front; the write-operand codes come from the pre-pass launch)
+        Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL, span=span)
+    A, qg = C.run_gla_A(q, Hw, gc, sc["q"], sc["k"], scale, qmax, dims, rot=R, dq=dq, span=span)
+    NT = T // span
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
     e_out = torch.empty_like(v)
     ht = torch.empty(B, H, K, V, dtype=torch.float32, device=q.device) if output_final_state else None
     o = C.out_buffer(v, out_dtype)
-    C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
-                C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes)
+    codes = C.run_state(Hw, U, gc, logenv, h_i8, ht, sc["kw"], sc["ew"], sc["state"], eta, qmax, dims, C.FAMILY_DELTA,
+                        C.DECAY_DIAGONAL, w=W, fw=fw, e_out=e_out, sw=sc["w"], unrot=Ru, codes=codes, span=span)
     C.run_output(None, None, e_out, h_i8, None, A, o, sc["q"], None, sc["el"], sc["state"], scale, qmax, dims, C.DECAY_DIAGONAL,
-                 unrot=Ru, qg=qg)
+                 unrot=Ru, qg=qg, span=span)
     C.export_debug(_debug, h_i8, codes, A=A, qg=qg, Hw=Hw, W=W, U=U, fw=fw, e_out=e_out)
     return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -86,8 +86,7 @@ def test_one_call_forward_validates_every_stage_limit_before_the_first_launch():
 
 
 def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
-    """128-token chunks exist for the linear family on raw operands in rotated storage: the entry points refuse every
-    other combination on the host (the buffers here are host memory: a call that passed
+    """128-token chunks exist for raw operands in rotated storage: the entry points refuse every other combination on the host (the buffers here are host memory: a call that passed
     validation would launch, so only refusals are exercised)."""
     lib = _lib.load()
     buf = (ctypes.c_char * 4096)()
@@ -99,11 +98,9 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
         return getattr(lib, fn)(ctypes.byref(_lib.fill(fn + "_args", **{k: v for k, v in {**dims, **kw}.items() if k in known})), None)
 
     wc = dict(key=a, kqT=a, ev=a, gam=a, skw=a, val=a, vqT=a, svw=a, g=a, chunk_size=128)
-    assert rc("lq_zoo_write_codes", **wc, decay=1, w=a, wq=a, sw=a) == -22          # delta family operands
     assert rc("lq_zoo_write_codes", **{**wc, "seqlen": 192}, decay=1) == -22        # not a whole number of chunks
     assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 256}, decay=1) == -22
     stt = dict(kqT=a, gam=a, h_i8=a, skw=a, svw=a, ss=a, vqT=a, chunk_size=128)
-    assert rc("lq_zoo_state", **stt, family=1, wq=a, u=a, fw=a, ev=a, e_out=a, sw=a) == -22   # delta family
     assert rc("lq_zoo_state", **stt, family=0, unrot=a) == -22                                # canonical storage
     assert rc("lq_zoo_state", **{**stt, "seqlen": 192}, family=0) == -22
     out = dict(h_i8=a, o=a, sq=a, svl=a, ss=a, q=a, k=a, v=a, sk=a, g=a, chunk_size=128, scale=1.0)
@@ -115,6 +112,10 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
     ga = dict(q=a, k=a, g=a, A=a, sq=a, sk=a, chunk_size=128, scale=1.0)
     assert rc("lq_zoo_gla_A", **ga) == -14                                                    # no A_cross
     assert rc("lq_zoo_gla_A", **{**ga, "seqlen": 192}, A_cross=a) == -22
+    wy = dict(k=a, v=a, beta=a, Hw=a, W=a, U=a, fw=a, g=a, chunk_size=128, decay=1)
+    assert rc("lq_zoo_wy_prep", **wy, kqT=a, wq=a, ev=a, gam=a, skw=a, sw=a) == -22           # no write codes at 128
+    assert rc("lq_zoo_wy_prep", **{**wy, "W": None}) == -14
+    assert rc("lq_zoo_wy_prep", **{**wy, "seqlen": 192}) == -22
     cs = dict(g=a, gc=a, logenv=a, chunk_size=128)
     assert rc("lq_zoo_cumsum", **cs, kqT=a, k=a, v=a, vqT=a, ev=a, gam=a, skw=a, svw=a) == -22   # no write codes at 128
     assert rc("lq_zoo_cumsum", **{**cs, "chunk_size": 96}) == -22
