@@ -440,6 +440,26 @@ def test_stored_state_codes_and_final_state(cuda, cell, seed):
     assert (last - codes[-1]).abs().max().item() <= limit
 
 
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+def test_chunk_128_with_widened_widths_int6_codes_and_fp32_output(cuda, cell):
+    """What the wrappers do around the kernels composes with 128-token chunks: a key width of 48 and a value width of 96
+    (widened with zero channels), INT6 codes in INT8 containers, an fp32 output."""
+    tensors = zc.cut(zc.inputs(cell, B=1, H=2, K=48, V=96, seed=11), 256)
+    dbg = {}
+    qz, run = zc.calibrated(cell, tensors, bits=6, eta=DEFAULT_ETA[cell], rho=0.5, tau=0.5, chunk=128, out_dtype=torch.float32)
+    scales = qz.kernel_scales(0, 2, 48, 96, delta=zc.CELLS[cell][0] == "delta")
+    out, ht = zc.run_kernel(cell, tensors, scales, eta=DEFAULT_ETA[cell], rho=0.5, tau=0.5, bits=6, chunk=128,
+                            out_dtype=torch.float32, final_state=True, debug=dbg)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float32 and out.shape == (1, 256, 2, 96) and ht.shape == (1, 2, 48, 96)
+    zc.check(out, run, qz, f"{cell} chunk 128, K=48, V=96, INT6, fp32 out")
+    codes = zc.state_codes(qz, run)
+    got = dbg["h_i8"].cpu()
+    assert got.shape[1] == 2 and (got[..., 48:, :] == 0).all() and (got[..., 96:] == 0).all()
+    d = (got[:, 1, :, :48, :96].int() - codes[0].int()).abs()
+    assert d.max().item() <= (2 if cell == "deltanet" else 1) and (d != 0).float().mean().item() < 2e-3
+
+
 @pytest.mark.parametrize("K", [16, 32, 48, 96])
 @pytest.mark.parametrize("cell", list(zc.CELLS))
 def test_key_widths_between_the_built_ones(cuda, cell, K):
