@@ -265,7 +265,8 @@ def measure_zoo(args, workload, cpu_baseline):
         dqk = dqk_from_absmax(cq.half().float(), ck.half().float(), 0.5).to(dev)
     # linear family: the rotation is part of the call's own operand launch (prologue=...); delta family: a launch of its own.
     # D_QK is applied inside the KDA kernels as they load q and k
-    fused = persistent and fam == "linear"
+    chunk = getattr(args, "zoo_chunk", 64)
+    fused = persistent and fam == "linear" and chunk == 64  # (the one-launch rotation + quantization is built for 64-token chunks)
     has_prologue = persistent and not fused
     qr, kr = (torch.empty_like(q0), torch.empty_like(k0)) if has_prologue else (None, None)
 
@@ -281,6 +282,7 @@ def measure_zoo(args, workload, cpu_baseline):
     eta = 0.0 if dec == "diagonal" else 1.0
 
     def kernels(sc, **kw):
+        kw["chunk_size"] = chunk
         if fam == "linear" and dec == "diagonal":
             return zoo.chunk_gla_int8(q, k, v, g, sc, eta=eta, scale=scale, rot=rot, **kw)
         if fam == "linear":
@@ -350,16 +352,17 @@ def measure_zoo(args, workload, cpu_baseline):
     for label, evs in records.items():
         ts = sorted(a.elapsed_time(b) for a, b in evs)
         med = statistics.median(ts)
-        stages[label] = {"ms": round(med, 4), "p25": round(ts[len(ts) // 4], 4), "p75": round(ts[(3 * len(ts)) // 4], 4),
-                         "MB": round(nbytes[label] / 1e6, 1), "GBps": round(nbytes[label] / 1e6 / med, 1),
-                         "hbm_frac": round(nbytes[label] / 1e6 / med / HBM_PEAK_GBS, 4)}
-    dom = max(stages, key=lambda n: stages[n]["ms"])
+        stages[label] = {"ms": round(med, 4), "p25": round(ts[len(ts) // 4], 4), "p75": round(ts[(3 * len(ts)) // 4], 4)}
+        if chunk == 64:  # (the byte model below is that of the 64-token route)
+            stages[label].update({"MB": round(nbytes[label] / 1e6, 1), "GBps": round(nbytes[label] / 1e6 / med, 1),
+                                  "hbm_frac": round(nbytes[label] / 1e6 / med / HBM_PEAK_GBS, 4)})
+    dom = max((n for n in stages if n in nbytes), key=lambda n: stages[n]["ms"])
     avg_dom = statistics.mean(a.elapsed_time(b) for a, b in records[dom])
     achieved = nbytes[dom] / 1e6 / avg_dom
     roofline = {"kernel": "zoo_" + dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "avg_ms": round(avg_dom, 4),
                 "algorithmic_MB": round(nbytes[dom] / 1e6, 1)}
-    counters, mfma_peak = measured_counters(workload, "zoo")
+    counters, mfma_peak = measured_counters(workload, "zoo") if chunk == 64 else ({}, None)
     for label, rec in counters.items():
         if label in stages:
             stages[label].update({k: v for k, v in rec.items() if k in ("traffic_MB", "mfma_busy_frac")})
@@ -376,7 +379,7 @@ def measure_zoo(args, workload, cpu_baseline):
         cut = lambda t: None if t is None else t[:1, :ts_, :hs].cpu()  # noqa: E731
         qz = Z.ZooQuantizer.kernel_profile("kernel_static", 8)
         run = lambda: Z.chunk_forward(cut(q), cut(k), cut(v), cut(g), cut(beta), family=fam, decay=dec, scale=scale, qz=qz,  # noqa: E731
-                                      eta=eta, rho=sigma, tau=1.0, read_post=True, C=64,
+                                      eta=eta, rho=sigma, tau=1.0, read_post=True, C=chunk,
                                       rot_qk=None if rot is None else rot.cpu())
         qz.calibrating = True
         run()
@@ -416,7 +419,8 @@ def measure_zoo(args, workload, cpu_baseline):
         "metric": f"prefill tokens/s per layer at T={T}", "value": round(tokens / ms_per_step * 1e3, 1), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"{workload} = BASELINE.json {desc}; fp16 activations, static absmax scales",
+        "config": {"workload": f"{workload} = BASELINE.json {desc}; fp16 activations, static absmax scales"
+                               + ("" if chunk == 64 else f"; run in {chunk}-token chunks instead of the configuration's 64"),
                    "tokens_per_step": tokens, "ramp": ramp_note(ramp_steps),
                    "prologue": "in the timed step: R_QK on q, k" if has_prologue else
                                "R_QK on q, k inside the call's operand launch (rotate + quantize in one)" if fused else
@@ -912,6 +916,9 @@ def main():
                     help="c5: decay regime of the synthetic dt / A (strong = the stated recipe)")
     ap.add_argument("--graph", action="store_true",
                     help="also time the step replayed from one captured HIP graph (always done for c1, whose eager step is bound by the launching thread)")
+    ap.add_argument("--zoo-chunk", type=int, default=64,
+                    help="zoo workloads: tokens per chunk (the configurations say 64; up to 128 is built, without the launch "
+                         "fusions of the 64-token route and without per-stage byte figures)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="heads per slice of the CPU-oracle sample")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="stop the CPU-oracle sample after about this long")
     args = ap.parse_args()

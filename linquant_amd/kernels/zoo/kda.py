@@ -24,7 +24,12 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     assert g.shape == q.shape
     span = C.chunk_span(chunk_size)
     assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
-    if dqk is not None and (q.shape[-1] not in (64, 128) or span != C.CHUNK):
+    if dqk is not None and q.shape[-1] in (64, 128) and span != C.CHUNK:
+        from .prologue import rotate_qkv  # (the 128-token WY kernel does not rescale at load: one launch up front)
+
+        q, k, _ = rotate_qkv(q.contiguous(), k.contiguous(), None, dqk=dqk)
+        dqk = None
+    if dqk is not None and q.shape[-1] not in (64, 128):
         # widths the kernels widen with zero channels: rescale up front (same roundings: one fp32 product, one quotient)
         d = dqk.to(q.device)
         q, k = (q.float() * d.float()).to(q.dtype), (k.double() / d.double()).float().to(k.dtype)
