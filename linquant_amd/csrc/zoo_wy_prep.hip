@@ -740,23 +740,23 @@ __global__ __launch_bounds__(256, 4) void zoo_wy_prep_kernel(WyParams p) {
 }
 
 // ---- 128-token chunks: the same transform over a 128 x 128 Gram matrix (gated_delta_rule.py:20-47, kda.py:22-53 with
-// chunk_size = 128), written for reach, not for speed: one workgroup per (chunk, batch*head) with the G and T tiles in LDS
-// (134 KB: one workgroup per compute unit), everything on the fp32 MFMA.
+// chunk_size = 128), written for reach, not for speed: one workgroup per (chunk, batch*head) with the G tile in 67 KB of LDS
+// (two workgroups per compute unit), inverted in place, everything on the fp32 MFMA.
 //   Gram: wave w takes row blocks w and 7 - w (equal numbers of 16 x 16 blocks), per-channel decay anchored at the row
 //     block's first row (both factors <= 1), operands straight from global memory (gram_rowblock).
-//   Inverse: the eight diagonal blocks by forward substitution, then block rows 1..7.
-//   W, U: T . X with X staged as fp32 in LDS 32 columns at a time (over the dead G tile).
+//   Inverse, in place (row I of the tile holds G until block row I is done, T after): the eight diagonal blocks by forward
+//     substitution, then block rows 1..7, every block of a row formed in registers before the row is overwritten.
+//   W, U: T . X with X staged as fp32 in LDS 16 columns at a time.
 // No write codes (lq_zoo_write_codes makes them from the stored Hw and W), no D_QK at load.
-constexpr int kGS2 = 134;  // floats per row of the 128-row G / T tiles (2 mod 4, as kGS)
-constexpr int kXS2 = 48;   // floats per token row of the X slab (16 mod 32: the two halves of a wave's read hit disjoint banks)
+constexpr int kGS2 = 130;  // floats per row of the 128-row G / T tile (2 mod 4, as kGS)
+constexpr int kXS2 = 20;   // floats per token row of the X slab (16 columns + pad); with the tile and the tables 77 KB
 
 template <int DECAY, int K, bool BF>
-__global__ __launch_bounds__(256) void zoo_wy_prep128_kernel(WyParams p) {
+__global__ __launch_bounds__(256, 2) void zoo_wy_prep128_kernel(WyParams p) {
   __shared__ __align__(16) float G_s[128 * kGS2];
-  __shared__ __align__(16) float T_s[128 * kGS2];
+  __shared__ __align__(16) float X_s[128 * kXS2];
   __shared__ float gs_s[128], bs_s[128], bh_s[128], bw_s[128];
-  static_assert(128 * kXS2 <= 128 * kGS2, "the X slab overlays the G tile");
-  float* X_s = G_s;
+  float* T_s = G_s;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rl = lane & 15, kg = lane >> 4;
@@ -775,8 +775,6 @@ __global__ __launch_bounds__(256) void zoo_wy_prep128_kernel(WyParams p) {
     p.fw[(t0 + tid) * H + h] = powb(bt, (1.0f - sigma) * (1.0f - tau));
     gs_s[tid] = DECAY == LQ_DECAY_SCALAR ? p.g[(t0 + tid) * H + h] : 0.0f;
   }
-  // T starts as zero: the blocks right of the diagonal are read as part of whole rows below
-  for (int it = tid; it < 128 * kGS2; it += 256) T_s[it] = 0.0f;
   __syncthreads();
 
   // ---- Gram
@@ -806,8 +804,13 @@ __global__ __launch_bounds__(256) void zoo_wy_prep128_kernel(WyParams p) {
   // block rows 1..7: T_IJ = -T_II . sum_{J <= M < I} G_IM . T_MJ, the J of a row dealt to the waves
 #pragma unroll 1
   for (int I = 1; I < 8; ++I) {
-#pragma unroll 1
-    for (int J = wave; J < I; J += 4) {
+    lq_v4f tnew[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) tnew[u] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int J = wave + 4 * u;
+      if (J >= I) continue;
       lq_v4f sacc = {0.f, 0.f, 0.f, 0.f};
       for (int M = J; M < I; ++M)
 #pragma unroll
@@ -819,84 +822,77 @@ __global__ __launch_bounds__(256) void zoo_wy_prep128_kernel(WyParams p) {
       lq_v4f tacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s) tacc = mfma_f32(T_s[(16 * I + rl) * kGS2 + 16 * I + 4 * kg + s], sacc[s], tacc);
+      tnew[u] = tacc;
+    }
+    __syncthreads();  // every wave has read what it needs of row I's G blocks
 #pragma unroll
-      for (int r = 0; r < 4; ++r) T_s[(16 * I + 4 * kg + r) * kGS2 + 16 * J + rl] = -tacc[r];
+    for (int u = 0; u < 2; ++u) {
+      const int J = wave + 4 * u;
+      if (J < I) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) T_s[(16 * I + 4 * kg + r) * kGS2 + 16 * J + rl] = -tnew[u][r];
+      }
     }
     __syncthreads();
   }
 
-  // ---- W = T . X (X = beta^sigma k exp(g)) and U = T . (beta^sigma v), 32 columns at a time; Hw goes straight out.
-  // Staging: thread (token = tid / 2, half = tid % 2) forms 16 columns of its token.
+  // ---- W = T . X (X = beta^sigma k exp(g)) and U = T . (beta^sigma v), 16 columns at a time; Hw goes straight out.
+  // Staging: thread (token = tid / 2, half = tid % 2) forms 8 columns of its token.
   const int tok = tid >> 1, hf = tid & 1;
-  const int nslab = (K + V) / 32;
+  const int nslab = (K + V) / 16;
 #pragma unroll 1
   for (int sl = 0; sl < nslab; ++sl) {
-    const bool isk = sl < K / 32;
-    const int c0 = (isk ? 32 * sl : 32 * sl - K) + 16 * hf;  // first column of this thread in k (or v)
-    __syncthreads();  // the slab (first pass: the G tile) is no longer read
+    const bool isk = sl < K / 16;
+    const int cc = isk ? 16 * sl : 16 * sl - K;  // first column of the slab in k (or v)
+    const int c0 = cc + 8 * hf;                  // first column of this thread
+    __syncthreads();  // the slab is no longer read
     {
-      float x[16];
+      float x[8];
       if (isk) {
         const int64_t off = ((t0 + tok) * H + h) * K + c0;
-        float kk[16];
-        zoo_ld8(p.k + off, bf, *(float(*)[8])kk);
-        zoo_ld8(p.k + off + 8, bf, *(float(*)[8])(kk + 8));
+        float kk[8];
+        zoo_ld8(p.k + off, bf, kk);
         float bl = bs_s[tok];
         if (DECAY == LQ_DECAY_SCALAR) bl = bl * zoo_exp(gs_s[tok]);
         const float bw = bw_s[tok];
-        float hw[16];
+        float hw[8];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
+        for (int e = 0; e < 8; ++e) {
           x[e] = bl * kk[e];
           hw[e] = bw * kk[e];
         }
         if (DECAY == LQ_DECAY_DIAGONAL) {
+          const lq_v4f g0 = *(const lq_v4f*)(p.g + off), g1 = *(const lq_v4f*)(p.g + off + 4);
 #pragma unroll
-          for (int e4 = 0; e4 < 4; ++e4) {
-            const lq_v4f g4 = *(const lq_v4f*)(p.g + off + 4 * e4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x[4 * e4 + e] = x[4 * e4 + e] * zoo_exp(g4[e]);
-          }
+          for (int e = 0; e < 4; ++e) x[e] = x[e] * zoo_exp(g0[e]), x[4 + e] = x[4 + e] * zoo_exp(g1[e]);
         }
-        lq_v4i o0, o1;
+        lq_v4i o;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          o0[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
-          o1[d] = (int)zoo_enc2(hw[8 + 2 * d], hw[8 + 2 * d + 1], bf);
-        }
-        *(lq_v4i*)(p.Hw + off) = o0;
-        *(lq_v4i*)(p.Hw + off + 8) = o1;
+        for (int d = 0; d < 4; ++d) o[d] = (int)zoo_enc2(hw[2 * d], hw[2 * d + 1], bf);
+        *(lq_v4i*)(p.Hw + off) = o;
       } else {
-        const int64_t off = ((t0 + tok) * H + h) * V + c0;
-        float vv[16];
-        zoo_ld8(p.v + off, bf, *(float(*)[8])vv);
-        zoo_ld8(p.v + off + 8, bf, *(float(*)[8])(vv + 8));
+        float vv[8];
+        zoo_ld8(p.v + ((t0 + tok) * H + h) * V + c0, bf, vv);
         const float bsr = bs_s[tok];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) x[e] = bsr * vv[e];
+        for (int e = 0; e < 8; ++e) x[e] = bsr * vv[e];
       }
-#pragma unroll
-      for (int e4 = 0; e4 < 4; ++e4)
-        *(lq_v4f*)(X_s + tok * kXS2 + 16 * hf + 4 * e4) = lq_v4f{x[4 * e4], x[4 * e4 + 1], x[4 * e4 + 2], x[4 * e4 + 3]};
+      *(lq_v4f*)(X_s + tok * kXS2 + 8 * hf) = lq_v4f{x[0], x[1], x[2], x[3]};
+      *(lq_v4f*)(X_s + tok * kXS2 + 8 * hf + 4) = lq_v4f{x[4], x[5], x[6], x[7]};
     }
     __syncthreads();
+    _Float16* dst = isk ? p.W : p.U;
+    const int C = isk ? K : V;
 #pragma unroll 1
     for (int u = 0; u < 2; ++u) {
       const int I = u ? 7 - wave : wave;
-      lq_v4f acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-      for (int s = 0; s < 4 * (I + 1); ++s) {
-        const float t = T_s[(16 * I + rl) * kGS2 + 4 * s + kg];
+      lq_v4f acc = {0.f, 0.f, 0.f, 0.f};
+      for (int s = 0; s < 4 * (I + 1); ++s)
+        acc = mfma_f32(T_s[(16 * I + rl) * kGS2 + 4 * s + kg], X_s[(4 * s + kg) * kXS2 + rl], acc);
+      // lane holds column rl of the slab, rows 16I + 4kg + r
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) acc[nt] = mfma_f32(t, X_s[(4 * s + kg) * kXS2 + 16 * nt + rl], acc[nt]);
-      }
-      // lane holds column 16nt + rl of the slab, rows 16I + 4kg + r
-      _Float16* dst = isk ? p.W : p.U;
-      const int C = isk ? K : V, cc = isk ? 32 * sl : 32 * sl - K;
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          *(uint16_t*)(dst + ((t0 + 16 * I + 4 * kg + r) * H + h) * C + cc + 16 * nt + rl) = (uint16_t)zoo_enc1(acc[nt][r], bf);
+      for (int r = 0; r < 4; ++r)
+        *(uint16_t*)(dst + ((t0 + 16 * I + 4 * kg + r) * H + h) * C + cc + rl) = (uint16_t)zoo_enc1(acc[r], bf);
     }
   }
 }
