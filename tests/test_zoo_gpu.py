@@ -441,6 +441,27 @@ def test_stored_state_codes_and_final_state(cuda, cell, seed):
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))
+@pytest.mark.parametrize("B,H,T,K,V", [(1, 1, 128, 64, 64), (3, 5, 384, 64, 128), (8, 8, 256, 128, 128)])
+def test_chunk_128_grid_shapes(cuda, cell, B, H, T, K, V):
+    """128-token chunks on grids of other shapes than the tests above use: a single chunk of a single head, batch x chunk
+    counts that are not a multiple of eight (the kernels renumber their workgroups over the eight XCDs only when they are),
+    and one that is."""
+    tensors = zc.inputs(cell, B=B, T=T, H=H, K=K, V=V, seed=100 * B + H)
+    eta = DEFAULT_ETA[cell]
+    qz, run = zc.calibrated(cell, tensors, eta=eta, rho=0.5, tau=0.5, chunk=128)
+    scales = qz.kernel_scales(0, H, K, V, delta=zc.CELLS[cell][0] == "delta")
+    dbg = {}
+    out, _ = zc.run_kernel(cell, tensors, scales, eta=eta, rho=0.5, tau=0.5, chunk=128, debug=dbg)
+    torch.cuda.synchronize()
+    zc.check(out, run, qz, f"{cell} chunk 128 {(B, H, T, K, V)}")
+    codes, got = zc.state_codes(qz, run), dbg["h_i8"].cpu()
+    NT = codes.shape[0]
+    if NT > 1:
+        d = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
+        assert int(d.max()) <= (2 if cell == "deltanet" else 1)
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
 def test_chunk_128_with_widened_widths_int6_codes_and_fp32_output(cuda, cell):
     """What the wrappers do around the kernels composes with 128-token chunks: a key width of 48 and a value width of 96
     (widened with zero channels), INT6 codes in INT8 containers, an fp32 output."""
