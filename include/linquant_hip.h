@@ -370,7 +370,7 @@ int lq_zoo_write_codes(const lq_zoo_write_codes_args* args, hipStream_t stream);
  * sequential chunk loop with an fp32 carry, INT8 stored copy per chunk, INT8 write product (and, delta family,
  * the INT8 state read W.S and the pseudo-values E = (U - W.S) * fw, stored fp16 for the output kernel).
  * Consumes the buffers written by lq_zoo_write_codes.
- * chunk_size is 64, or 128 (rotated storage; operands from lq_zoo_write_codes with chunk_size 128, delta family: W and U
+ * chunk_size is 64, or 128 (operands from lq_zoo_write_codes with chunk_size 128, delta family: W and U
  * from lq_zoo_wy_prep with chunk_size 128): one stored state per 128 tokens, h_i8 is (B,seqlen/128,H,V,K), both halves of
  * a chunk read it, and the carry takes the INT8 write product summed over the 128 tokens (int32) once per chunk. */
 typedef struct {
@@ -404,7 +404,7 @@ int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
 /* replaces _output_kernel (linquant/kernels/zoo/simple_gla.py:98-172) and _gla_output_kernel
  * (gla.py:170-232): o = dequant(q8(q).h_i8) [* exp(g)] + (fp16(A) . fp16(q8(v))) * svl, with A computed
  * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay).
- * chunk_size is 64, or 128 (raw q, k, v, rotated storage; h_i8 (B,seqlen/128,H,V,K) from lq_zoo_state with chunk_size
+ * chunk_size is 64, or 128 (raw q, k, v; h_i8 (B,seqlen/128,H,V,K) from lq_zoo_state with chunk_size
  * 128; under diagonal decay A and A_cross from lq_zoo_gla_A with chunk_size 128): two launches, the first leaves the
  * second halves' products with the first halves' tokens in `cross`, the second starts its fp32 accumulators from them. */
 typedef struct {

@@ -361,6 +361,20 @@ void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
     hipLaunchKernelGGL((zoo_output_kernel<GLA, USE_G, K, false, NV, false>), grid, dim3(256), 0, stream, p);
 }
 
+// the cross launch alone (canonical storage: the local product is formed in the rotated basis there too, so its first-half
+// part comes from this kernel and the un-rotating kernel starts from it)
+template <bool GLA, bool USE_G>
+int launch_cross_only(const OutParams& p, int K, hipStream_t stream) {
+  const bool two = p.V % (2 * BV) == 0;
+  const dim3 grid(p.V / (two ? 2 * BV : BV), p.NT / 2, p.B * p.H);
+  if (K == 128) {
+    if (two) launch_cross<GLA, USE_G, 128, 2>(p, grid, stream); else launch_cross<GLA, USE_G, 128, 1>(p, grid, stream);
+  } else {
+    if (two) launch_cross<GLA, USE_G, 64, 2>(p, grid, stream); else launch_cross<GLA, USE_G, 64, 1>(p, grid, stream);
+  }
+  return lq_check_launch();
+}
+
 template <bool GLA, bool USE_G>
 int launch(const OutParams& p, int K, hipStream_t stream) {
   const bool two = p.V % (2 * BV) == 0;  // two V tiles per workgroup
@@ -393,9 +407,9 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks (raw operands, rotated storage) run as pairs of 64-token halves
+  // 128-token chunks (raw operands) run as pairs of 64-token halves
   const bool pair = a->chunk_size == 128;
-  if (pair && (cin || a->unrot)) return LQ_ERR_SHAPE;
+  if (pair && cin) return LQ_ERR_SHAPE;
   if (pair && (!a->cross || (gla && !a->A_cross))) return LQ_ERR_NULL;
   if (pair && (!zoo_al(a->cross, 16) || (gla && !zoo_al(a->A_cross, 16)))) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
@@ -415,7 +429,15 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.qc = a->qc, p.kc = a->kc, p.vc = a->vc;
   p.cross = pair ? a->cross : nullptr, p.hshift = pair ? 1 : 0;
   p.Ax = pair ? (const _Float16*)a->A_cross : nullptr;
-  if (a->unrot) return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
+  if (a->unrot) {
+    if (pair) {
+      const int rc = gla ? launch_cross_only<true, true>(p, a->kdim, stream)
+                         : (a->decay == LQ_DECAY_SCALAR ? launch_cross_only<false, true>(p, a->kdim, stream)
+                                                        : launch_cross_only<false, false>(p, a->kdim, stream));
+      if (rc) return rc;
+    }
+    return zoo_output_unrot_launch(p, a->decay, a->kdim, stream);
+  }
   if (gla) return launch<true, true>(p, a->kdim, stream);
   if (a->decay == LQ_DECAY_SCALAR) return launch<false, true>(p, a->kdim, stream);
   return launch<false, false>(p, a->kdim, stream);

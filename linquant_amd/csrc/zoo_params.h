@@ -71,5 +71,5 @@ struct ZooACrossParams {
 int zoo_gla_A_cross_launch(const ZooACrossParams& p, int K, hipStream_t stream);  // defined in zoo_gla_A_cross.hip
 
 // canonical storage: one workgroup spans all V value channels (V = 64 or 128); defined in zoo_unrot.hip
-int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, hipStream_t stream);
+int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, bool pair, hipStream_t stream);
 int zoo_output_unrot_launch(const ZooOutParams& p, int decay, int K, hipStream_t stream);

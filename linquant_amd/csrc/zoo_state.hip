@@ -408,9 +408,8 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (!delta && !a->vqT) return LQ_ERR_NULL;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks (rotated storage) run as pairs of 64-token halves
+  // 128-token chunks run as pairs of 64-token halves
   const bool pair = a->chunk_size == 128;
-  if (pair && a->unrot) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
@@ -427,7 +426,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   p.unrot = (const _Float16*)a->unrot;
   p.pack = a->pack;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
-  if (a->unrot) return zoo_state_unrot_launch(p, delta, a->kdim, a->batch, stream);
+  if (a->unrot) return zoo_state_unrot_launch(p, delta, a->kdim, a->batch, pair, stream);
   // narrower V tiles when batch*head alone cannot fill the 256 compute units
   int BV = a->vtile;
   if (BV == 0) {

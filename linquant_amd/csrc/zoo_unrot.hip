@@ -87,7 +87,10 @@ struct UStepOps {
 // back into the basis of U contracts over all canonical channels) and each rotates it into, and finishes E for, one half
 // of the value channels.  The delta family's single workgroup per (batch, head) runs one dependent chain of chunk steps,
 // so halving what a wave does per step is what shortens it.
-template <bool DELTA, int K, int V, int KP, int VS = 1, int NW = 4>
+// PAIR: 128-token chunks walked as two 64-token halves: the state is quantized and stored at the first half only (both
+// halves of the delta family read that copy), the INT8 write product of the first half stays in the accumulators the second
+// half's product adds to, and the sum over the 128 tokens is dequantized, un-rotated and added to the carry once.
+template <bool DELTA, int K, int V, int KP, int VS = 1, int NW = 4, bool PAIR = false>
 __global__ __launch_bounds__(NW * 64) void zoo_state_unrot_kernel(ZooStateParams p) {
   static_assert(KP == 1 || !DELTA, "the delta family needs all of K in one workgroup");
   static_assert(VS == 1 || !DELTA, "the delta family needs all of V in one workgroup");
@@ -164,24 +167,28 @@ __global__ __launch_bounds__(NW * 64) void zoo_state_unrot_kernel(ZooStateParams
   nxt = cur;
   __syncthreads();
 
+  lq_v4i pend[PAIR ? KT : 1][PAIR ? VT : 1];  // PAIR: the first half's write product
   for (int ct = 0; ct < NT; ++ct) {
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
+    const bool second = PAIR && (ct & 1);  // wave-uniform
     // the next step's operands are requested first and without a condition (the last step asks for its own again): a
     // request inside a branch is waited for where the paths join, in front of the products below
     load_step(min(ct + 1, NT - 1), nxt);
     // ---- stored copy of the incoming state -> LDS (V-major), one byte per (v, k)
+    if (!second) {
 #pragma unroll
-    for (int vt = 0; vt < VOT; ++vt) {
-      const lq_v4f is4 = *(const lq_v4f*)(inv_ss_s + v0 + 16 * vt + 4 * kg);
+      for (int vt = 0; vt < VOT; ++vt) {
+        const lq_v4f is4 = *(const lq_v4f*)(inv_ss_s + v0 + 16 * vt + 4 * kg);
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt)
+        for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          hT[(16 * vt + 4 * kg + r) * HS + KR * wave + 16 * kt + rl] = (unsigned char)zoo_q8(hc[vt][kt][r], is4[r], 127);
+          for (int r = 0; r < 4; ++r)
+            hT[(16 * vt + 4 * kg + r) * HS + KR * wave + 16 * kt + rl] = (unsigned char)zoo_q8(hc[vt][kt][r], is4[r], 127);
+      }
     }
     __syncthreads();
-    {
-      int8_t* dst = p.h_i8 + ((((int64_t)b * NT + ct) * H + h) * V + v0) * K + kb;
+    if (!second) {
+      int8_t* dst = p.h_i8 + ((((int64_t)b * (PAIR ? NT >> 1 : NT) + (PAIR ? ct >> 1 : ct)) * H + h) * V + v0) * K + kb;
       constexpr int SEG = KW / 16;
       for (int it = tid; it < VO * SEG; it += NTHR) {
         const int vr = it / SEG, sg = it % SEG;
@@ -230,6 +237,20 @@ __global__ __launch_bounds__(NW * 64) void zoo_state_unrot_kernel(ZooStateParams
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
       float d[VT][4];
+      if constexpr (PAIR) {
+        if (!second) {  // first half: the product waits for the second half's
+#pragma unroll
+          for (int vt = 0; vt < VT; ++vt) {
+            lq_v4i aop;
+            if constexpr (DELTA)
+              aop = *(const lq_v4i*)(eT + (16 * vt + rl) * ES + 16 * kg);
+            else
+              aop = cur.vop[vt];
+            pend[kt][vt] = lq_mfma_i8(aop, cur.kop[kt], lq_v4i{0, 0, 0, 0});
+          }
+          continue;
+        }
+      }
 #pragma unroll
       for (int vt = 0; vt < VT; ++vt) {
         lq_v4i aop;
@@ -237,7 +258,7 @@ __global__ __launch_bounds__(NW * 64) void zoo_state_unrot_kernel(ZooStateParams
           aop = *(const lq_v4i*)(eT + (16 * vt + rl) * ES + 16 * kg);
         else
           aop = cur.vop[vt];
-        const lq_v4i a = lq_mfma_i8(aop, cur.kop[kt], lq_v4i{0, 0, 0, 0});
+        const lq_v4i a = lq_mfma_i8(aop, cur.kop[kt], PAIR ? pend[kt][vt] : lq_v4i{0, 0, 0, 0});
         const lq_v4f w4 = *(const lq_v4f*)(svw_s + 16 * vt + 4 * kg);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -292,7 +313,8 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
 
   // state-read operands (and the stored query codes) are requested first: they are not needed before phase 2 and
   // arrive while phase 1 stages the codes
-  const int8_t* hp = p.h_i8 + (((int64_t)b * p.NT + ct) * H + h) * V * K;
+  // (128-token chunks: one stored state per chunk, read by both halves)
+  const int8_t* hp = p.h_i8 + (((int64_t)b * (p.NT >> p.hshift) + (ct >> p.hshift)) * H + h) * V * K;
   lq_v4i hop[K / 64][VT];
   lq_v4i qgop[GLA ? K / 64 : 1];
 #pragma unroll
@@ -403,6 +425,13 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
     lq_v4f loc[VT];
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) loc[vt] = lq_v4f{0.f, 0.f, 0.f, 0.f};
+    if (p.cross && (ct & 1)) {
+      // second half of a 128-token chunk: the local product with the first half's tokens, left by the cross launch of the
+      // rotated-storage output kernel (the local product is in the rotated basis either way); lane (rl = token, kg) holds
+      // channels 16vt + 4kg + r
+#pragma unroll
+      for (int vt = 0; vt < VT; ++vt) loc[vt] = *(const lq_v4f*)(p.cross + ((t0 + 16 * wave + rl) * H + h) * V + 16 * vt + 4 * kg);
+    }
     const int nslab = (16 * wave + 15) / 32 + 1;
     for (int js = 0; js < nslab; ++js) {
       lq_v8h aop;
@@ -452,7 +481,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
   }
 }
 
-template <bool DELTA, int K>
+template <bool DELTA, int K, bool PAIR>
 int launch_state(const ZooStateParams& p, int batch, hipStream_t stream) {
   constexpr int KP = (!DELTA && K == 128) ? 2 : 1;
   // canonical value slices of 32 (V = 128) or 16 (V = 64) channels; measured at B4 T4096 H16 K = V = 128, no decay: one
@@ -462,9 +491,9 @@ int launch_state(const ZooStateParams& p, int batch, hipStream_t stream) {
   constexpr int NW = (DELTA && K == 128) ? 8 : 4;
   dim3 grid(batch * p.H, KP, VS);
   if (p.V == 128)
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP, VS, NW>), grid, dim3(NW * 64), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 128, KP, VS, NW, PAIR>), grid, dim3(NW * 64), 0, stream, p);
   else
-    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP, VS, NW>), grid, dim3(NW * 64), 0, stream, p);
+    hipLaunchKernelGGL((zoo_state_unrot_kernel<DELTA, K, 64, KP, VS, NW, PAIR>), grid, dim3(NW * 64), 0, stream, p);
   return lq_check_launch();
 }
 
@@ -480,10 +509,14 @@ int launch_output(const ZooOutParams& p, hipStream_t stream) {
 
 }  // namespace
 
-int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, hipStream_t stream) {
+int zoo_state_unrot_launch(const ZooStateParams& p, bool delta, int K, int batch, bool pair, hipStream_t stream) {
   if (p.V != 64 && p.V != 128) return LQ_ERR_SHAPE;
-  if (delta) return K == 128 ? launch_state<true, 128>(p, batch, stream) : launch_state<true, 64>(p, batch, stream);
-  return K == 128 ? launch_state<false, 128>(p, batch, stream) : launch_state<false, 64>(p, batch, stream);
+  if (pair) {
+    if (delta) return K == 128 ? launch_state<true, 128, true>(p, batch, stream) : launch_state<true, 64, true>(p, batch, stream);
+    return K == 128 ? launch_state<false, 128, true>(p, batch, stream) : launch_state<false, 64, true>(p, batch, stream);
+  }
+  if (delta) return K == 128 ? launch_state<true, 128, false>(p, batch, stream) : launch_state<true, 64, false>(p, batch, stream);
+  return K == 128 ? launch_state<false, 128, false>(p, batch, stream) : launch_state<false, 64, false>(p, batch, stream);
 }
 
 int zoo_output_unrot_launch(const ZooOutParams& p, int decay, int K, hipStream_t stream) {

@@ -16,10 +16,9 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
                      output_final_state=False, unrot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None (DeltaNet), beta [B,T,H].
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None).
-    ``chunk_size``: up to 64 (padded to 64 tokens), or up to 128 with rotated storage (padded to 128: the WY transform then
+    ``chunk_size``: up to 64 (padded to 64 tokens), or up to 128 (padded to 128: the WY transform then
     runs over 128 x 128 Gram matrices in a kernel of its own, the state and output kernels walk a chunk as two halves)."""
     span = C.chunk_span(chunk_size)
-    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
     q, k, v, g, beta, restore = C.pad_chunks(chunk_size, q, k, v, g, beta, span=span)
     q, k, g, scales, _, K0 = C.pad_keys(q, k, g, scales)
     v, scales, V0 = C.pad_values(v, scales, unrot)

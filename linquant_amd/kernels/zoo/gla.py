@@ -16,11 +16,10 @@ BC = 16  # secondary chunk
 def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, output_final_state=False, unrot=None,
                    rot=None, bits=8, out_dtype=None, _debug=None):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
-    Returns (o, final fp32 state or None).  ``chunk_size``: a multiple of 16 up to 64, or up to 128 with rotated storage (the
+    Returns (o, final fp32 state or None).  ``chunk_size``: a multiple of 16 up to 64, or up to 128 (the
     kernels walk a chunk of more than 64 tokens as two 64-token halves, padded to 128 tokens; the sub-block anchoring over its eight sub-blocks is the reference's)."""
     assert g.shape == q.shape
     span = C.chunk_span(chunk_size)
-    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
     q, k, v, g, _, restore = C.pad_chunks(chunk_size, q, k, v, g, span=span)
     q, k, g, scales, rot, K0 = C.pad_keys(q, k, g, scales, rot)
     v, scales, V0 = C.pad_values(v, scales, unrot)

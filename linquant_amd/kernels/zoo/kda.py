@@ -20,10 +20,9 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     ``dqk`` (H,K) fp32, not in the reference's signature: the diagonal rescaling D_QK of linquant/harness.py:68-88
     (q' = q D, k' = k / D, rounded to the activation dtype) applied inside the kernels as they load q and k, with the
     result of calling ``rotate_qkv(q, k, None, dqk=dqk)`` first, bit for bit, and without that launch.
-    ``chunk_size``: a multiple of 16 up to 64, or up to 128 with rotated storage (as ``chunk_delta_int8``)."""
+    ``chunk_size``: a multiple of 16 up to 64, or up to 128 (as ``chunk_delta_int8``)."""
     assert g.shape == q.shape
     span = C.chunk_span(chunk_size)
-    assert span == C.CHUNK or unrot is None, "chunks of more than 64 tokens are built for rotated storage"
     if dqk is not None and q.shape[-1] in (64, 128) and span != C.CHUNK:
         from .prologue import rotate_qkv  # (the 128-token WY kernel does not rescale at load: one launch up front)
 

@@ -86,7 +86,7 @@ def test_one_call_forward_validates_every_stage_limit_before_the_first_launch():
 
 
 def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
-    """128-token chunks exist for raw operands in rotated storage: the entry points refuse every other combination on the host (the buffers here are host memory: a call that passed
+    """128-token chunks exist for raw operands: the entry points refuse every other combination on the host (the buffers here are host memory: a call that passed
     validation would launch, so only refusals are exercised)."""
     lib = _lib.load()
     buf = (ctypes.c_char * 4096)()
@@ -101,13 +101,11 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
     assert rc("lq_zoo_write_codes", **{**wc, "seqlen": 192}, decay=1) == -22        # not a whole number of chunks
     assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 256}, decay=1) == -22
     stt = dict(kqT=a, gam=a, h_i8=a, skw=a, svw=a, ss=a, vqT=a, chunk_size=128)
-    assert rc("lq_zoo_state", **stt, family=0, unrot=a) == -22                                # canonical storage
     assert rc("lq_zoo_state", **{**stt, "seqlen": 192}, family=0) == -22
     out = dict(h_i8=a, o=a, sq=a, svl=a, ss=a, q=a, k=a, v=a, sk=a, g=a, chunk_size=128, scale=1.0)
     assert rc("lq_zoo_output", **out, decay=1) == -14                                         # no cross workspace
     assert rc("lq_zoo_output", **out, decay=2, A=a, qg=a, cross=a) == -14                     # per-channel decay: no A_cross
     assert rc("lq_zoo_output", **out, decay=1, cross=a, qc=a, kc=a, vc=a) == -22              # ready-made codes
-    assert rc("lq_zoo_output", **out, decay=1, cross=a, unrot=a) == -22                       # canonical storage
     assert rc("lq_zoo_output", **{**out, "seqlen": 192}, decay=1, cross=a) == -22
     ga = dict(q=a, k=a, g=a, A=a, sq=a, sk=a, chunk_size=128, scale=1.0)
     assert rc("lq_zoo_gla_A", **ga) == -14                                                    # no A_cross

@@ -22,7 +22,7 @@ DEFAULT_ETA = {"linear_none": 1.0, "mamba2": 1.0, "gla": 0.0, "deltanet": 1.0, "
 def _go(cell, tensors, *, policy="kernel_static", bits=8, eta=None, rho=1.0, tau=1.0, label=None, rot=None, rot_v=None, **kw):
     eta = DEFAULT_ETA[cell] if eta is None else eta
     qz, run = zc.calibrated(cell, tensors, policy=policy, bits=bits, eta=eta, rho=rho, tau=tau, rot_qk=rot, rot_v=rot_v,
-                            out_dtype=kw.get("out_dtype"))
+                            out_dtype=kw.get("out_dtype"), chunk=kw.get("chunk", 64))
     if rot_v is not None:  # the kernel receives the rotated value operand, materialized in the activation dtype
         q_, k_, v_, g_, b_ = tensors
         tensors = (q_, k_, (v_.double() @ rot_v).to(v_.dtype), g_, b_)
@@ -357,6 +357,33 @@ def test_canonical_storage_rv(cuda, cell, n, K, V):
     tensors = zc.cut(zc.inputs(cell, K=K, V=V, H=2 if K == 128 else 4), n)
     out, _, qz, run = _go(cell, tensors, eta=1.0, rot_v=signed_hadamard(V, 7))
     zc.check(out, run, qz, f"{cell} canonical R_V T={n} K={K} V={V}")
+
+
+@pytest.mark.parametrize("cell", list(zc.CELLS))
+@pytest.mark.parametrize("n,K,V,chunk,rho", [(512, 64, 128, 128, 1.0), (384, 128, 64, 128, 0.0), (512, 128, 128, 128, 0.5),
+                                             (288, 64, 64, 96, 1.0)])
+def test_canonical_storage_rv_above_64_tokens(cuda, cell, n, K, V, chunk, rho):
+    """Canonical R_V storage in 128-token chunks (and 96, padded): the un-rotating state kernel keeps the first half's INT8
+    write product for the second half's and un-rotates their sum once, the un-rotating output kernel starts its local
+    product from the cross launch's.  Against the oracle at that chunk size, with the write gate on either side."""
+    from oracle.zoo_reference import signed_hadamard
+
+    tensors = zc.cut(zc.inputs(cell, K=K, V=V, H=2 if K == 128 else 3, seed=9), n)
+    dbg = {}
+    out, ht, qz, run = _go(cell, tensors, eta=1.0, rho=rho, tau=1.0, rot_v=signed_hadamard(V, 7), chunk=chunk, final_state=True,
+                           debug=dbg)
+    zc.check(out, run, qz, f"{cell} canonical R_V T={n} K={K} V={V} chunk {chunk}")
+    codes, got = zc.state_codes(qz, run), dbg["h_i8"].cpu()
+    NT = codes.shape[0]
+    assert got.shape[1] == NT == n // chunk
+    d = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[: NT - 1].int()).abs()
+    if cell == "deltanet":
+        # the undecayed state under canonical storage: every write passes through an fp16 un-rotation whose rounding ties
+        # the kernel and the oracle break differently, and nothing decays the difference away (measured here: up to three
+        # steps, 6 % of the codes one step apart; in 64-token chunks 15 %)
+        assert int(d.max()) <= 3 and (d > 1).float().mean().item() < 1e-2
+    else:
+        assert int(d.max()) <= 1 and (d != 0).float().mean().item() < 5e-3
 
 
 @pytest.mark.parametrize("cell", list(zc.CELLS))
