@@ -299,7 +299,8 @@ int lq_kron_hadamard(const lq_kron_hadamard_args* args, hipStream_t stream);
 /* ------------------------------------------------------------------------------------------
  * Zoo chunk kernels: linear attention (no / scalar decay), GLA, DeltaNet / Gated DeltaNet, KDA.
  * q,k (B,T,H,K) and v (B,T,H,V) fp16/bf16 contiguous, T a multiple of the chunk size, K in {64,128},
- * V a multiple of 64.  g holds the chunk-local cumulative log decay (lq_zoo_cumsum).  Scales are
+ * V a multiple of 64.  The chunk size is 64; every entry point but lq_zoo_rotate_quant also takes 128 (the kernels then
+ * walk a chunk as two 64-token halves; see each entry).  g holds the chunk-local cumulative log decay (lq_zoo_cumsum).  Scales are
  * fp32: q,k,w (H,), kw (H,K), vw,vl,el,ew,state (H,V).  h_i8 is the per-chunk INT8 stored state in
  * V-major layout (B,NT,H,V,K): an internal buffer shared by the state and output kernels.
  * qmax is 127 (INT8) or 31 (INT6 codes in INT8 containers); the stored state always uses 127.
@@ -312,7 +313,7 @@ typedef struct {
   float* gc;                 /* same shape */
   float* logenv;             /* (B,T,H) max_k(gc_last[k] - gc[t,k]); diagonal decay only, else NULL */
   int32_t batch, seqlen, nheads, kdim; /* kdim = 0: scalar decay */
-  int32_t chunk_size;
+  int32_t chunk_size;        /* scalar decay: any divisor of seqlen; per-channel decay: a multiple of 16 up to 64, or 128 */
   /* Optional (per-channel decay, linear family, chunk 64; all of them when kqT is set): the write operands of the state
    * kernel that lq_zoo_write_codes would make from gc and logenv, made here while the chunk's decay tile is on chip:
    * the operand preparation inside _gla_state_body (linquant/kernels/zoo/gla.py:124-141).  Same bits. */
