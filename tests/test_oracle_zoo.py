@@ -105,9 +105,10 @@ def test_unquantized_matches_token_recurrence(cell):
     q, k, v, g, beta = make_inputs(cell, seed=5)
     ref = _token_recurrence(q, k, v, g, beta, fam, dec, K ** -0.5)
     noq = Z.ZooQuantizer("none")
-    for kw in (dict(), dict(eta=0.5), dict(rho=0.5, tau=0.5), dict(read_post=True), dict(C=32)):
+    for kw in (dict(), dict(eta=0.5), dict(rho=0.5, tau=0.5), dict(read_post=True), dict(C=32), dict(C=16), dict(C=128),
+               dict(C=128, eta=0.5, rho=0.5, tau=0.5)):
         if dec == "none" and "eta" in kw:
-            continue
+            kw = {n: x for n, x in kw.items() if n != "eta"}
         o = Z.chunk_forward(q, k, v, g, beta, family=fam, decay=dec, scale=K ** -0.5, qz=noq, out_dtype=torch.float64, **kw)
         assert (o - ref).abs().max() / ref.abs().max() < 1e-9, (cell, kw)
 
