@@ -342,8 +342,8 @@ int lq_zoo_cumsum(const lq_zoo_cumsum_args* args, hipStream_t stream);
  * gla.py:124-141, gated_delta_rule.py:85-105, kda.py:100-124): every write operand that does not depend on the
  * carried state is quantized once, in parallel over chunks, into the layout lq_zoo_state consumes.
  * kqT/vqT are channel-major inside each 64-token chunk; all five outputs are internal buffers of the wrappers.
- * chunk_size is 64, or 128 (seqlen a multiple of 128): the buffers keep their 64-token
- * layout (NT = seqlen / 64) and the decays of a chunk's first 64 tokens reach on to the end of the 128-token chunk. */
+ * chunk_size is 64, or 128 (linear family with no / scalar decay: also 192, 256; seqlen a multiple of it): the buffers keep
+ * their 64-token layout (NT = seqlen / 64) and the decays of a chunk's earlier tokens reach on to the end of the chunk. */
 typedef struct {
   const void* key;           /* key operand of the write: k (linear) or Hw (delta), (B,T,H,K) fp16/bf16 */
   const void* val;           /* linear family: v (B,T,H,V) fp16/bf16; delta family: NULL */
@@ -373,7 +373,8 @@ int lq_zoo_write_codes(const lq_zoo_write_codes_args* args, hipStream_t stream);
  * Consumes the buffers written by lq_zoo_write_codes.
  * chunk_size is 64, or 128 (operands from lq_zoo_write_codes with chunk_size 128, delta family: W and U
  * from lq_zoo_wy_prep with chunk_size 128): one stored state per 128 tokens, h_i8 is (B,seqlen/128,H,V,K), both halves of
- * a chunk read it, and the carry takes the INT8 write product summed over the 128 tokens (int32) once per chunk. */
+ * a chunk read it, and the carry takes the INT8 write product summed over the 128 tokens (int32) once per chunk.  The linear
+ * family in rotated storage also takes 192 and 256 (h_i8 (B,seqlen/chunk_size,H,V,K)). */
 typedef struct {
   const int8_t* kqT;         /* (B,NT,H,K,64) */
   const int8_t* vqT;         /* linear family: (B,NT,H,V,64) */
@@ -407,7 +408,8 @@ int lq_zoo_state(const lq_zoo_state_args* args, hipStream_t stream);
  * in-kernel from q8(q).q8(k)^T (no / scalar decay) or read from the fp32 A tensor (diagonal decay).
  * chunk_size is 64, or 128 (raw q, k, v; h_i8 (B,seqlen/128,H,V,K) from lq_zoo_state with chunk_size
  * 128; under diagonal decay A and A_cross from lq_zoo_gla_A with chunk_size 128): two launches, the first leaves the
- * second halves' products with the first halves' tokens in `cross`, the second starts its fp32 accumulators from them. */
+ * second halves' products with the first halves' tokens in `cross`, the second starts its fp32 accumulators from them.
+ * No / scalar decay in rotated storage also takes 192 and 256 (one such launch per earlier 64-token piece). */
 typedef struct {
   const void* q;             /* no / scalar decay: (B,T,H,K) fp16/bf16; diagonal decay: NULL */
   const int8_t* qg;          /* diagonal decay: (B,T,H,K) int8 codes of q*exp(g)*scale written by lq_zoo_gla_A */
@@ -433,7 +435,7 @@ typedef struct {
   const int8_t* qc;          /* (B,T,H,K) int8 q8(q*scale, 1/sq) */
   const int8_t* kc;          /* (B,T,H,K) int8 q8(k, 1/sk) */
   const int8_t* vc;          /* (B,T,H,V) int8 q8(v, 1/svl) */
-  float* cross;              /* chunk_size 128: (B,T,H,V) fp32 workspace, 16-byte aligned (overwritten); else unused */
+  float* cross;              /* chunk_size above 64: (B,T,H,V) fp32 workspace, 16-byte aligned (overwritten); else unused */
   const void* A_cross;       /* chunk_size 128, diagonal decay: (B,T,H,64) fp16 written by lq_zoo_gla_A; else unused */
 } lq_zoo_output_args;
 int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);

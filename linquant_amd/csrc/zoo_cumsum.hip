@@ -24,7 +24,7 @@ __global__ __launch_bounds__(256) void cumsum_scalar_kernel(const float* __restr
   }
 }
 
-// The same scan for the chunk sizes the callers use (C = 64 or 128): 64 values of a thread are requested before the first
+// The same scan for the chunk sizes the callers use (C = 64, 128, 192 or 256): 64 values of a thread are requested before the first
 // is added (the loop above waits for each load in turn: C round trips), summed in the same order.
 template <int C>
 __global__ __launch_bounds__(256) void cumsum_scalar_fixed_kernel(const float* __restrict__ g, float* __restrict__ gc, int H,
@@ -208,6 +208,12 @@ extern "C" int lq_zoo_cumsum(const lq_zoo_cumsum_args* a, hipStream_t stream) {
                          a->gc, a->nheads, total);
     else if (a->chunk_size == 128)
       hipLaunchKernelGGL(cumsum_scalar_fixed_kernel<128>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g,
+                         a->gc, a->nheads, total);
+    else if (a->chunk_size == 192)
+      hipLaunchKernelGGL(cumsum_scalar_fixed_kernel<192>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g,
+                         a->gc, a->nheads, total);
+    else if (a->chunk_size == 256)
+      hipLaunchKernelGGL(cumsum_scalar_fixed_kernel<256>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g,
                          a->gc, a->nheads, total);
     else
       hipLaunchKernelGGL(cumsum_scalar_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a->g, a->gc,

@@ -29,7 +29,9 @@ using OutParams = ZooOutParams;
 // for both tiles)
 // CIN: the local codes of q, k, v arrive ready-made (lq_zoo_rotate_quant made them): they are copied into the same LDS
 // tiles instead of being quantized here.
-// CROSS (128-token chunks, which run as pairs of 64-token halves): this launch makes, for the second half of every chunk,
+// CROSS (chunks of S = 2..4 pieces of 64 tokens; described for S = 2, where it runs once: launch j of S - 1 gives piece
+// s >= j its product with the tokens of piece j - 1, adding to what launch j - 1 left, oldest tokens first): this launch
+// makes, for the second half of every chunk,
 // the part of the local product that reaches back into the first half -- fp16(Af[i][j]) . fp16(q8(v_j)) over the 64 tokens j
 // of the first half, no causal mask, no state read; under per-channel decay Af comes from p.Ax -- and leaves it as fp32 in p.cross; the ordinary launch that follows
 // starts its local accumulators from it (one fp32 accumulation over the 128 tokens, oldest first, as a 128-token tile has).
@@ -59,12 +61,16 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
       bh = vid / (nv * gridDim.y);
     }
   }
-  if constexpr (CROSS) ct = 2 * ct + 1;  // the grid walks the chunks; the rows are those of the second half
+  const int piece = ct % p.S;  // which 64-token piece of its chunk
+  if constexpr (CROSS) {
+    if (piece < p.cross_j) return;  // (uniform over the workgroup, in front of every barrier)
+  }
   const int v0 = vtile * BV * NV;
   const int b = bh / p.H, h = bh % p.H;
   const int H = p.H, V = p.V;
   const int64_t t0 = (int64_t)b * p.T + (int64_t)ct * 64;
-  const int64_t tk0 = CROSS ? t0 - 64 : t0;  // first token of the keys / values this launch contracts against
+  // first token of the keys / values this launch contracts against
+  const int64_t tk0 = CROSS ? t0 - (int64_t)(piece - p.cross_j + 1) * 64 : t0;
   const float sq = p.sq[h];
   const float inv_sq = 1.0f / sq;
   const float sk = GLA ? 1.0f : p.sk[h];
@@ -114,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   const float g_raw = (USE_G && !GLA) ? p.g[(t0 + (tid & 63)) * H + h] : 0.0f;
   const float gk_raw = (USE_G && CROSS) ? p.g[(tk0 + (tid & 63)) * H + h] : 0.0f;
   // (128-token chunks: one stored state per chunk, read by both halves)
-  const int8_t* hp = p.h_i8 + ((((int64_t)b * (p.NT >> p.hshift) + (ct >> p.hshift)) * H + h) * V + v0) * K;
+  const int8_t* hp = p.h_i8 + ((((int64_t)b * (p.NT / p.S) + ct / p.S) * H + h) * V + v0) * K;
   lq_v4i hop[CROSS ? 1 : NV][K / 64][4];
   lq_v4i qgop[GLA ? K / 64 : 1];
 #pragma unroll
@@ -279,8 +285,9 @@ __global__ __launch_bounds__(256, 2) void zoo_output_kernel(OutParams p) {
   for (int n = 0; n < NV; ++n)
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) loc[n][jj] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-  if constexpr (!CROSS) {
-    if (p.cross && (ct & 1)) {  // second half of a 128-token chunk: what the cross launch left for these rows
+  {
+    // later piece of a chunk: what the cross launch(es) left for these rows
+    if (CROSS ? p.cross_j > 1 : (p.cross != nullptr && piece != 0)) {
 #pragma unroll
       for (int n = 0; n < NV; ++n)
 #pragma unroll
@@ -345,7 +352,10 @@ void launch_cross(const OutParams& p, dim3 grid, hipStream_t stream) {
 
 template <bool GLA, bool USE_G, int K, int NV>
 void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
-  if (p.cross) launch_cross<GLA, USE_G, K, NV>(p, dim3(grid.x, grid.y / 2, grid.z), stream);
+  if (p.cross) {
+    OutParams c = p;
+    for (c.cross_j = 1; c.cross_j < p.S; ++c.cross_j) launch_cross<GLA, USE_G, K, NV>(c, grid, stream);
+  }
   if constexpr (!GLA) {
     if (p.qc) {  // ready-made codes: the activation dtype only matters for a 16-bit output
       if (p.bf)
@@ -366,11 +376,13 @@ void launch_bf(const OutParams& p, dim3 grid, hipStream_t stream) {
 template <bool GLA, bool USE_G>
 int launch_cross_only(const OutParams& p, int K, hipStream_t stream) {
   const bool two = p.V % (2 * BV) == 0;
-  const dim3 grid(p.V / (two ? 2 * BV : BV), p.NT / 2, p.B * p.H);
+  const dim3 grid(p.V / (two ? 2 * BV : BV), p.NT, p.B * p.H);
+  OutParams c = p;
+  c.cross_j = 1;  // (canonical storage: two pieces per chunk)
   if (K == 128) {
-    if (two) launch_cross<GLA, USE_G, 128, 2>(p, grid, stream); else launch_cross<GLA, USE_G, 128, 1>(p, grid, stream);
+    if (two) launch_cross<GLA, USE_G, 128, 2>(c, grid, stream); else launch_cross<GLA, USE_G, 128, 1>(c, grid, stream);
   } else {
-    if (two) launch_cross<GLA, USE_G, 64, 2>(p, grid, stream); else launch_cross<GLA, USE_G, 64, 1>(p, grid, stream);
+    if (two) launch_cross<GLA, USE_G, 64, 2>(c, grid, stream); else launch_cross<GLA, USE_G, 64, 1>(c, grid, stream);
   }
   return lq_check_launch();
 }
@@ -407,9 +419,11 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   if (a->decay < 0 || a->decay > 2) return LQ_ERR_SHAPE;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks (raw operands) run as pairs of 64-token halves
-  const bool pair = a->chunk_size == 128;
+  // chunks of 128 tokens (raw operands) run as pairs of 64-token halves; no / scalar decay in rotated storage also as
+  // three or four pieces (192, 256 tokens)
+  const bool pair = a->chunk_size == 128 || a->chunk_size == 192 || a->chunk_size == 256;
   if (pair && cin) return LQ_ERR_SHAPE;
+  if (a->chunk_size > 128 && (gla || a->unrot)) return LQ_ERR_SHAPE;
   if (pair && (!a->cross || (gla && !a->A_cross))) return LQ_ERR_NULL;
   if (pair && (!zoo_al(a->cross, 16) || (gla && !zoo_al(a->A_cross, 16)))) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
@@ -427,7 +441,7 @@ extern "C" int lq_zoo_output(const lq_zoo_output_args* a, hipStream_t stream) {
   p.B = a->batch, p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
   p.unrot = (const _Float16*)a->unrot;
   p.qc = a->qc, p.kc = a->kc, p.vc = a->vc;
-  p.cross = pair ? a->cross : nullptr, p.hshift = pair ? 1 : 0;
+  p.cross = pair ? a->cross : nullptr, p.S = a->chunk_size / 64, p.cross_j = 0;
   p.Ax = pair ? (const _Float16*)a->A_cross : nullptr;
   if (a->unrot) {
     if (pair) {

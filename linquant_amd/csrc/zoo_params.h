@@ -24,6 +24,7 @@ struct ZooStateParams {
   int qmax;
   int bf;  // activations are bf16
   int T, H, V, NT;
+  int S;  // 64-token pieces per chunk (1; 2..4 in the kernels' PAIR mode)
 };
 
 struct ZooOutParams {
@@ -49,8 +50,9 @@ struct ZooOutParams {
   int bf;  // activations (and a 16-bit output) are bf16
   int B, T, H, V, NT;
   const _Float16* Ax;  // 128-token chunks under per-channel decay: (B,T,H,64) fp16 from the cross launch of the A kernel
-  float* cross;  // 128-token chunks: fp32 (B,T,H,V) partial local products of the second halves, else nullptr
-  int hshift;    // log2 of the 64-token halves per stored state (1 for 128-token chunks)
+  float* cross;  // chunks of S > 1 pieces: fp32 (B,T,H,V) partial local products of the later pieces, else nullptr
+  int S;         // 64-token pieces per chunk (and per stored state): 1, or 2..4
+  int cross_j;   // cross launch j = 1 .. S-1: piece s >= j of a chunk takes its product with the tokens of piece j - 1
 };
 
 // 128-token chunks under per-channel decay: the second halves' blocks of the intra-chunk product with the first halves' tokens

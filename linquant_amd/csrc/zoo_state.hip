@@ -38,8 +38,9 @@ struct StepOps {
 
 // BF (bf16 activations) is a template parameter: as a run-time flag every decode / encode of U and E in the chunk loop
 // became a branch of its own.
-// PAIR (128-token chunks): the chunk loop still walks 64-token halves, whose operands the pre-pass wrote with the decay
-// to the end of the 128-token chunk.  The state is quantized and stored at the first half only (index ct / 2; the delta
+// PAIR (chunks of S = 2 pieces of 64 tokens; the linear family also S = 3, 4, where "first half" below reads "first piece"
+// and "second half" "last piece", the pieces between only adding their product): the chunk loop still walks 64-token halves,
+// whose operands the pre-pass wrote with the decay to the end of the chunk.  The state is quantized and stored at the first half only (index ct / 2; the delta
 // family's second half reads that same stored copy: its W and U come from a WY transform over the 128 tokens), the INT8
 // write product of the first half stays in the accumulators that the second half's product adds to, and the carry takes
 // decay and product once per chunk: the integer sum over 128 tokens that one 128-token tile gives.
@@ -169,8 +170,11 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
   lq_v4i pend[PAIR ? KT : 1][PAIR ? VT : 1];  // PAIR: the first half's write product
   auto do_step = [&](int ct, StepOps<DELTA, K, BV>& cur, StepOps<DELTA, K, BV>& pre) {
     const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
-    const bool second = PAIR && (ct & 1);  // PAIR: second half of a chunk (nothing stored, the carry is updated)
-    unsigned char* hTb = hT + (DELTA ? 0 : ((PAIR ? ct >> 1 : ct) & 1) * BV * HS);
+    const int S = PAIR ? p.S : 1;
+    const int piece = PAIR ? ct % S : 0;
+    const bool second = piece != 0;       // PAIR: a later piece of a chunk (nothing is stored)
+    const bool last = piece == S - 1;     // PAIR: the piece after which the carry is updated
+    unsigned char* hTb = hT + (DELTA ? 0 : ((PAIR ? ct / S : ct) & 1) * BV * HS);
     float* misc_s = misc_lds + 64 * wave;
     unsigned char* ue_s = ue_lds + wave * 16 * US;
     misc_s[lane] = cur.misc;
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
 
     // the stored state leaves coalesced: h_i8[b][ct][h][v0 + v][k]
     auto copy_out = [&]() {
-      int8_t* dst = p.h_i8 + ((((int64_t)b * (PAIR ? NT >> 1 : NT) + (PAIR ? ct >> 1 : ct)) * H + h) * V + v0) * K;
+      int8_t* dst = p.h_i8 + ((((int64_t)b * (PAIR ? NT / S : NT) + (PAIR ? ct / S : ct)) * H + h) * V + v0) * K;
       constexpr int SEG = K / 16;
       if constexpr (BV * SEG % 256 == 0) {
 #pragma unroll
@@ -313,11 +317,11 @@ __global__ __launch_bounds__(256, DELTA ? 1 : 2) void zoo_state_kernel(StatePara
       for (int kt = 0; kt < KT; ++kt) {
         lq_v4i a;
         if constexpr (PAIR) {
-          if (!second) {
-            pend[kt][vt] = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
+          a = lq_mfma_i8(cur.kop[kt], bop, second ? pend[kt][vt] : lq_v4i{0, 0, 0, 0});
+          if (!last) {
+            pend[kt][vt] = a;
             continue;
           }
-          a = lq_mfma_i8(cur.kop[kt], bop, pend[kt][vt]);
         } else {
           a = lq_mfma_i8(cur.kop[kt], bop, lq_v4i{0, 0, 0, 0});
         }
@@ -408,8 +412,9 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   if (!delta && !a->vqT) return LQ_ERR_NULL;
   if (a->unrot && ((a->vdim != 64 && a->vdim != 128) || !zoo_al(a->unrot, 16))) return LQ_ERR_SHAPE;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks run as pairs of 64-token halves
-  const bool pair = a->chunk_size == 128;
+  // 128-token chunks run as pairs of 64-token halves; the linear family in rotated storage also takes 192 and 256 tokens
+  const bool pair = a->chunk_size == 128 || a->chunk_size == 192 || a->chunk_size == 256;
+  if (a->chunk_size > 128 && (delta || a->unrot)) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;
@@ -426,6 +431,7 @@ extern "C" int lq_zoo_state(const lq_zoo_state_args* a, hipStream_t stream) {
   p.unrot = (const _Float16*)a->unrot;
   p.pack = a->pack;
   p.T = a->seqlen, p.H = a->nheads, p.V = a->vdim, p.NT = a->seqlen / 64;
+  p.S = a->chunk_size / 64;
   if (a->unrot) return zoo_state_unrot_launch(p, delta, a->kdim, a->batch, pair, stream);
   // narrower V tiles when batch*head alone cannot fill the 256 compute units
   int BV = a->vtile;

@@ -314,7 +314,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
   // state-read operands (and the stored query codes) are requested first: they are not needed before phase 2 and
   // arrive while phase 1 stages the codes
   // (128-token chunks: one stored state per chunk, read by both halves)
-  const int8_t* hp = p.h_i8 + (((int64_t)b * (p.NT >> p.hshift) + (ct >> p.hshift)) * H + h) * V * K;
+  const int8_t* hp = p.h_i8 + (((int64_t)b * (p.NT / p.S) + ct / p.S) * H + h) * V * K;
   lq_v4i hop[K / 64][VT];
   lq_v4i qgop[GLA ? K / 64 : 1];
 #pragma unroll
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void zoo_output_unrot_kernel(ZooOutParams p
     lq_v4f loc[VT];
 #pragma unroll
     for (int vt = 0; vt < VT; ++vt) loc[vt] = lq_v4f{0.f, 0.f, 0.f, 0.f};
-    if (p.cross && (ct & 1)) {
+    if (p.cross && (ct % p.S) != 0) {
       // second half of a 128-token chunk: the local product with the first half's tokens, left by the cross launch of the
       // rotated-storage output kernel (the local product is in the rotated basis either way); lane (rl = token, kg) holds
       // channels 16vt + 4kg + r

@@ -49,8 +49,9 @@ __global__ __launch_bounds__(256) void zoo_write_codes_kernel(CodesParams p) {
   const int H = p.H, V = p.V, T = p.T;
   const int64_t t0 = (int64_t)b * T + (int64_t)ct * 64;
   const int64_t cb = ((int64_t)b * p.NT + ct) * H + h;  // (batch, chunk, head) index
-  // last token of the chunk: of these 64 tokens, or, when they are one half of a 128-token chunk, of that chunk
-  const int64_t tlast = t0 + 63 + (p.span == 128 && !(ct & 1) ? 64 : 0);
+  // last token of the chunk: of these 64 tokens, or, when they are one piece of a chunk of 128 .. 256 tokens, of that chunk
+  const int pieces = p.span / 64;
+  const int64_t tlast = t0 + 63 + (int64_t)(pieces - 1 - ct % pieces) * 64;
   const float eta = p.eta;
   const int qmax = p.qmax;
   constexpr bool bf = BF;
@@ -217,8 +218,9 @@ extern "C" int lq_zoo_write_codes(const lq_zoo_write_codes_args* a, hipStream_t 
   if (a->decay != LQ_DECAY_NONE && !a->g) return LQ_ERR_NULL;
   if (a->decay == LQ_DECAY_DIAGONAL && !a->logenv) return LQ_ERR_NULL;
   if (a->batch <= 0 || a->seqlen <= 0 || a->nheads <= 0) return LQ_ERR_SHAPE;
-  // 128-token chunks: the state kernel walks them as pairs of 64-token halves
-  const bool pair = a->chunk_size == 128;
+  // 128-token chunks: the state kernel walks them as pairs of 64-token halves (linear family, no / scalar decay: also 192, 256)
+  const bool pair = a->chunk_size == 128 || a->chunk_size == 192 || a->chunk_size == 256;
+  if (a->chunk_size > 128 && (a->w || a->decay == LQ_DECAY_DIAGONAL)) return LQ_ERR_SHAPE;
   if ((a->chunk_size != 64 && !pair) || a->seqlen % a->chunk_size != 0) return LQ_ERR_SHAPE;
   if ((a->kdim != 64 && a->kdim != 128) || a->vdim % 64 != 0 || a->vdim <= 0) return LQ_ERR_SHAPE;
   if (a->qmax < 1 || a->qmax > 127) return LQ_ERR_SHAPE;

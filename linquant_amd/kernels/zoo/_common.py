@@ -39,10 +39,10 @@ def pad_keys(q, k, g, scales, rot=None):
     return q, k, g, scales, rot, K
 
 
-def chunk_span(chunk_size):
-    """Tokens per chunk as the linear-family kernels run it: 64, or 128 for chunk sizes above 64 (pad_chunks fills up)."""
-    assert 1 <= chunk_size <= 2 * CHUNK, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {2 * CHUNK} tokens"
-    return CHUNK if chunk_size <= CHUNK else 2 * CHUNK
+def chunk_span(chunk_size, pieces=2):
+    """Tokens per chunk as the kernels run it: the next multiple of 64 (pad_chunks fills up), at most ``pieces`` x 64."""
+    assert 1 <= chunk_size <= pieces * CHUNK, f"chunk_size={chunk_size}: the HIP kernels hold chunks of at most {pieces * CHUNK} tokens"
+    return -(-chunk_size // CHUNK) * CHUNK
 
 
 def pad_chunks(chunk_size, q, k, v, g=None, beta=None, span=CHUNK):

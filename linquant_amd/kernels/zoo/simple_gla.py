@@ -21,10 +21,10 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     the D_QK rescaling are applied in the launch that also quantizes the operands: the result of calling
     ``rotate_qkv(q, k, v, ...)`` first and this function on its outputs, bit for bit, in one launch fewer and without the
     rotated activations ever reaching memory (K, V in {64, 128}, rotated storage).
-    ``chunk_size``: up to 64 (smaller chunks are padded to 64 tokens), or up to 128 (padded to 128): the
-    kernels then walk every chunk as two 64-token halves, with one stored state, one carry update (the INT8 write product summed over the 128
-    tokens) and one fp32 local accumulation per chunk."""
-    span = C.chunk_span(chunk_size)
+    ``chunk_size``: up to 256 in rotated storage, up to 128 in canonical storage (padded to the next multiple of 64):
+    above 64 the kernels walk every chunk as two to four 64-token pieces, with one stored state, one carry update (the INT8
+    write product summed over the chunk's tokens) and one fp32 local accumulation per chunk."""
+    span = C.chunk_span(chunk_size, pieces=2 if unrot is not None else 4)
     if prologue is not None and (q.shape[-1] not in (64, 128) or v.shape[-1] not in (64, 128) or unrot is not None or span != C.CHUNK):
         from .prologue import rotate_qkv  # shapes the fused launch is not built for: rotate up front
 

@@ -99,7 +99,8 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
 
     wc = dict(key=a, kqT=a, ev=a, gam=a, skw=a, val=a, vqT=a, svw=a, g=a, chunk_size=128)
     assert rc("lq_zoo_write_codes", **{**wc, "seqlen": 192}, decay=1) == -22        # not a whole number of chunks
-    assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 256}, decay=1) == -22
+    assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 320, "seqlen": 640}, decay=1) == -22
+    assert rc("lq_zoo_write_codes", **{**wc, "chunk_size": 256, "seqlen": 512}, decay=2, logenv=a) == -22   # per-channel decay: up to 128
     stt = dict(kqT=a, gam=a, h_i8=a, skw=a, svw=a, ss=a, vqT=a, chunk_size=128)
     assert rc("lq_zoo_state", **{**stt, "seqlen": 192}, family=0) == -22
     out = dict(h_i8=a, o=a, sq=a, svl=a, ss=a, q=a, k=a, v=a, sk=a, g=a, chunk_size=128, scale=1.0)
@@ -107,6 +108,10 @@ def test_zoo_chunk_size_128_is_taken_where_it_is_built_and_refused_elsewhere():
     assert rc("lq_zoo_output", **out, decay=2, A=a, qg=a, cross=a) == -14                     # per-channel decay: no A_cross
     assert rc("lq_zoo_output", **out, decay=1, cross=a, qc=a, kc=a, vc=a) == -22              # ready-made codes
     assert rc("lq_zoo_output", **{**out, "seqlen": 192}, decay=1, cross=a) == -22
+    # 192 and 256 tokens: linear family with no / scalar decay in rotated storage only
+    assert rc("lq_zoo_state", **{**stt, "chunk_size": 256, "seqlen": 512}, family=1, wq=a, u=a, fw=a, ev=a, e_out=a, sw=a) == -22
+    assert rc("lq_zoo_output", **{**out, "chunk_size": 192, "seqlen": 384}, decay=2, A=a, qg=a, cross=a, A_cross=a) == -22
+    assert rc("lq_zoo_output", **{**out, "chunk_size": 256, "seqlen": 512}, decay=1, cross=a, unrot=a) == -22
     ga = dict(q=a, k=a, g=a, A=a, sq=a, sk=a, chunk_size=128, scale=1.0)
     assert rc("lq_zoo_gla_A", **ga) == -14                                                    # no A_cross
     assert rc("lq_zoo_gla_A", **{**ga, "seqlen": 192}, A_cross=a) == -22

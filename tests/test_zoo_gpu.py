@@ -151,6 +151,32 @@ def test_chunk_sizes_above_64_delta_family(cuda, cell, K, V, dtype, chunk, rho, 
     assert dl.max().item() <= lim + bf and (dl > lim).float().mean().item() < (1e-3 if bf else 1e-4), dl.max().item()
 
 
+@pytest.mark.parametrize("cell,eta", [("linear_none", 1.0), ("mamba2", 1.0), ("mamba2", 0.25)])
+@pytest.mark.parametrize("chunk,K,V,dtype", [(192, 64, 64, torch.float16), (256, 128, 128, torch.float16), (256, 64, 192, torch.bfloat16),
+                                             (160, 64, 64, torch.float16)])
+def test_chunk_sizes_up_to_256_no_and_scalar_decay(cuda, cell, eta, chunk, K, V, dtype):
+    """Chunks of three and four 64-token pieces (linquant/kernels/zoo/simple_gla.py:184 takes any chunk size that divides
+    T; 256 is the Mamba-2 mixer's own): one stored state and one carry update per chunk, a cross launch per earlier piece
+    adding into the fp32 local accumulation, oldest tokens first.  Against the oracle at that chunk size: outputs, stored
+    state codes within one step, final state; 160 runs as a padded 192-token chunk."""
+    T = 3 * chunk
+    tensors = zc.inputs(cell, B=2, T=T, H=3, K=K, V=V, seed=41, dtype=dtype)
+    qz, run = zc.calibrated(cell, tensors, eta=eta, chunk=chunk)
+    scales = qz.kernel_scales(0, 3, K, V)
+    dbg = {}
+    out, ht = zc.run_kernel(cell, tensors, scales, eta=eta, chunk=chunk, final_state=True, debug=dbg)
+    torch.cuda.synchronize()
+    assert out.shape == tensors[2].shape and out.dtype == dtype and dbg["h_i8"].shape[1] == 3
+    zc.check(out, run, qz, f"{cell} chunk {chunk} eta={eta}")
+    codes = zc.state_codes(qz, run)
+    got = dbg["h_i8"].cpu()
+    assert codes.shape[0] == 3 and (got[:, 0] == 0).all()
+    d = (got[:, 1:].permute(1, 0, 2, 3, 4).int() - codes[:2].int()).abs()
+    assert int(d.max()) <= 1 and (d != 0).float().mean().item() < 2e-3, (int(d.max()), (d != 0).float().mean().item())
+    last = torch.round(ht.cpu() / scales["state"][None, :, None, :]).clamp(-127, 127)
+    assert (last - codes[-1]).abs().max().item() <= 1
+
+
 @pytest.mark.parametrize("cell", ["linear_none", "mamba2", "gla"])
 @pytest.mark.parametrize("chunk", [80, 96, 112])
 def test_chunk_sizes_between_64_and_128(cuda, cell, chunk):
