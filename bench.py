@@ -30,7 +30,8 @@ STAGE_SOURCES = {
     "c5": {"prologue": "prologue_rotate_quant.hip", "chunk_cumsum": "mamba2_cumsum.hip", "chunk_state": "mamba2_chunk_state.hip",
            "state_passing": "mamba2_state_passing.hip", "bmm_chunk": "mamba2_bmm_chunk.hip", "chunk_scan": "mamba2_chunk_scan.hip"},
     "zoo": {"prologue": "zoo_rotate.hip", "cumsum": "zoo_cumsum.hip", "wy_prep": "zoo_wy_prep.hip", "gla_A": "zoo_gla_A.hip",
-            "write_codes": "zoo_write_codes.hip", "state": "zoo_state.hip", "output": "zoo_output.hip"},
+            "write_codes": "zoo_write_codes.hip", "state": "zoo_state.hip", "output": "zoo_output.hip",
+            "rotate_quant": "zoo_rotate_quant.hip"},
 }
 COUNTER_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic_and_mfma_counters.md")
 
