@@ -440,6 +440,37 @@ typedef struct {
 } lq_zoo_output_args;
 int lq_zoo_output(const lq_zoo_output_args* args, hipStream_t stream);
 
+/* replaces chunk_simple_gla_int8 as a whole (linquant/kernels/zoo/simple_gla.py:175-212; rotated storage, raw operands):
+ * lq_zoo_cumsum (scalar decay only), lq_zoo_write_codes, lq_zoo_state and lq_zoo_output launched back to back on `stream`
+ * over one caller-supplied workspace that holds the intermediates (cumulative decay, write codes, per-token factors, stored
+ * states, and for chunk sizes above 64 the cross workspace).  Same kernels and bits as the four calls; one foreign call and
+ * one allocation per forward, which is what bounds small shapes.  Field meanings as in the per-stage structs. */
+typedef struct {
+  const void* q;             /* (B,T,H,K) fp16/bf16 */
+  const void* k;             /* (B,T,H,K) */
+  const void* v;             /* (B,T,H,V) */
+  const float* g;            /* (B,T,H) fp32 log decay per token (not cumulated), or NULL: no decay */
+  void* o;                   /* (B,T,H,V) fp16/bf16, or fp32 when o_is_f32 */
+  int32_t o_is_f32;
+  float* ht;                 /* (B,H,K,V) fp32 final state, or NULL */
+  const float* sq;           /* (H,) */
+  const float* sk;           /* (H,) */
+  const float* skw;          /* (H,K) */
+  const float* svw;          /* (H,V) */
+  const float* svl;          /* (H,V), 16-byte aligned */
+  const float* ss;           /* (H,V), 16-byte aligned */
+  float eta, scale;
+  int32_t qmax;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size; /* K in {64,128}, V a multiple of 64, chunk 64, 128, 192 or 256 */
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16 */
+  void* workspace;           /* device memory, 256-byte aligned, lq_zoo_simple_gla_workspace_bytes() bytes; contents undefined
+                                on entry and on return */
+  int64_t workspace_bytes;
+} lq_zoo_simple_gla_args;
+int lq_zoo_simple_gla(const lq_zoo_simple_gla_args* args, hipStream_t stream);
+/* workspace size for the dims in `args` (pointers are not read), written to *bytes */
+int lq_zoo_simple_gla_workspace_bytes(const lq_zoo_simple_gla_args* args, int64_t* bytes);
+
 /* replaces _gla_A_inter + _gla_A_intra (linquant/kernels/zoo/gla.py:27-99): intra-chunk product under
  * per-channel decay, 16-token sub-blocks: INT8 dots on anchor-rescaled operands off the diagonal, fp32
  * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows (C = 64; chunk_size 128:

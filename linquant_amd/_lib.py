@@ -13,7 +13,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 HEADER = ROOT.parent / "include" / "linquant_hip.h"
 LIB_PATH = ROOT / "csrc" / "liblinquant_hip.so"
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 LQ_DT_F16, LQ_DT_F32, LQ_DT_I8, LQ_DT_BF16 = 0, 1, 2, 3
 
@@ -56,7 +56,8 @@ STRUCTS = {name: type(name, (ctypes.Structure,), {"_fields_": fields}) for name,
 FUNCTIONS = tuple(_funcs)
 
 # entry points whose first argument is another function's args struct
-_SHARED_ARGS = {"lq_ssd_combined_static": "lq_ssd_combined_args", "lq_ssd_combined_workspace_bytes": "lq_ssd_combined_args"}
+_SHARED_ARGS = {"lq_ssd_combined_static": "lq_ssd_combined_args", "lq_ssd_combined_workspace_bytes": "lq_ssd_combined_args",
+                "lq_zoo_simple_gla_workspace_bytes": "lq_zoo_simple_gla_args"}
 
 _lib = None
 

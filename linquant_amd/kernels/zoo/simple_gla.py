@@ -49,9 +49,13 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     decay = C.DECAY_NONE if g is None else C.DECAY_SCALAR
+    assert g is None or g.shape == (B, T, H)
+    if prologue is None and unrot is None and _debug is None:
+        # the whole forward as one C call over one workspace (same kernels and bits as the stage-by-stage route below)
+        o, ht = _one_call(q, k, v, g, scales, eta, scale, qmax, dims, span, output_final_state, out_dtype)
+        return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
     gg = None
     if g is not None:
-        assert g.shape == (B, T, H)
         gg, _ = C.cumsum(g, B, T, H, 0, span=span)
     NT = T // span
     h_i8 = torch.empty(B, NT, H, V, K, dtype=torch.int8, device=q.device)
@@ -72,3 +76,37 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     C.run_output(q, k, v, h_i8, gg, None, o, sc["q"], sc["k"], sc["vl"], sc["state"], scale, qmax, dims, decay, unrot=Ru, span=span)
     C.export_debug(_debug, h_i8, codes, g=gg)
     return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
+
+
+def _one_call(q, k, v, g, scales, eta, scale, qmax, dims, span, final_state, out_dtype):
+    """lq_zoo_simple_gla: cumsum, write-operand pre-pass, state recurrence and output from one foreign call."""
+    import ctypes
+
+    from ... import _lib
+
+    B, T, H, K, V = dims
+    dev = q.device
+    sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
+    svl, ss = _lib.aligned(sc["vl"]), _lib.aligned(sc["state"])
+    gf = None if g is None else C.f32(g)
+    key = (B, T, H, K, V, span)
+    nbytes = _WS_BYTES.get(key)
+    if nbytes is None:
+        st = _lib.fill("lq_zoo_simple_gla_args", batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=span)
+        n = ctypes.c_int64(0)
+        rc = _lib.load().lq_zoo_simple_gla_workspace_bytes(ctypes.byref(st), ctypes.byref(n))
+        if rc != 0:
+            raise _lib.LinQuantHipError(f"lq_zoo_simple_gla_workspace_bytes failed with code {rc}")
+        nbytes = _WS_BYTES[key] = n.value
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    o = C.out_buffer(v, out_dtype)
+    ht = torch.empty(B, H, K, V, dtype=torch.float32, device=dev) if final_state else None
+    _lib.call("lq_zoo_simple_gla", dev, q=_lib.ptr(q), k=_lib.ptr(k), v=_lib.ptr(v), g=_lib.ptr(gf), o=_lib.ptr(o),
+              o_is_f32=int(o.dtype == torch.float32), ht=_lib.ptr(ht), sq=_lib.ptr(sc["q"]), sk=_lib.ptr(sc["k"]),
+              skw=_lib.ptr(sc["kw"]), svw=_lib.ptr(sc["vw"]), svl=_lib.ptr(svl), ss=_lib.ptr(ss), eta=float(eta), scale=float(scale),
+              qmax=int(qmax), batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=span, act_dtype=C.act_code(v),
+              workspace=_lib.ptr(ws), workspace_bytes=nbytes)
+    return o, ht
+
+
+_WS_BYTES = {}

@@ -113,6 +113,31 @@ def test_chunk_size_128_linear_family(cuda, cell, eta, rot, K, V, dtype):
         assert torch.equal(out64[:, :64], out[:, :64])        # first half: the same arithmetic either way
 
 
+@pytest.mark.parametrize("cell", ["linear_none", "mamba2"])
+@pytest.mark.parametrize("chunk,K,V,dtype,out_dtype", [(64, 64, 64, torch.float16, None), (64, 128, 128, torch.bfloat16, None),
+                                                       (32, 48, 96, torch.float16, torch.float32), (128, 128, 64, torch.float16, None),
+                                                       (256, 64, 128, torch.float16, None)])
+def test_one_call_forward_equals_the_stage_by_stage_route(cuda, cell, chunk, K, V, dtype, out_dtype):
+    """chunk_simple_gla_int8 issues its stages from one C call over one workspace (lq_zoo_simple_gla) unless a caller asks
+    for the intermediates; both routes run the same kernels on the same operands: outputs and final states are equal bit
+    for bit, for every chunk size, with widened widths and an fp32 output."""
+    from linquant_amd.kernels import zoo
+
+    T = 4 * max(chunk, 64)
+    q, k, v, g, _ = [t.to(cuda) if t is not None else None for t in zc.inputs(cell, B=2, T=T, H=3, K=K, V=V, seed=43, dtype=dtype)]
+    gen = torch.Generator().manual_seed(5)
+    sc = {"q": torch.rand(3, generator=gen) * 0.002 + 0.001, "k": torch.rand(3, generator=gen) * 0.005 + 0.005,
+          "kw": torch.rand(3, K, generator=gen) * 0.01 + 0.005, "vw": torch.rand(3, V, generator=gen) * 0.02 + 0.02,
+          "vl": torch.rand(3, V, generator=gen) * 0.02 + 0.02, "state": torch.rand(3, V, generator=gen) * 0.05 + 0.02}
+    sc = {n: t.to(cuda) for n, t in sc.items()}
+    kw = dict(eta=0.5, chunk_size=chunk, output_final_state=True, out_dtype=out_dtype)
+    o1, h1 = zoo.chunk_simple_gla_int8(q, k, v, g, sc, **kw)
+    o0, h0 = zoo.chunk_simple_gla_int8(q, k, v, g, sc, _debug={}, **kw)
+    torch.cuda.synchronize()
+    assert o1.shape == v.shape and o1.dtype == (out_dtype or dtype) and h1.shape == (2, 3, K, V)
+    assert torch.equal(o0, o1) and torch.equal(h0, h1) and float(o1.float().abs().max()) > 0
+
+
 @pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet", "kda"])
 @pytest.mark.parametrize("K,V,dtype,chunk", [(64, 64, torch.float16, 128), (128, 128, torch.float16, 128),
                                              (64, 192, torch.bfloat16, 128), (64, 64, torch.float16, 96)])
