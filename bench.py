@@ -342,7 +342,7 @@ def measure_zoo(args, workload, cpu_baseline):
         for _ in range(max(10, args.steps)):
             if has_prologue:
                 tp()
-            kernels(sc, _debug={})  # (asks for the stage-by-stage route where the call would issue its stages from one C call)
+            kernels(sc, _staged=True)  # (the stage-by-stage route, where the call would issue its stages from one C call)
         torch.cuda.synchronize()
     finally:
         for n, f in saved.items():

@@ -471,6 +471,45 @@ int lq_zoo_simple_gla(const lq_zoo_simple_gla_args* args, hipStream_t stream);
 /* workspace size for the dims in `args` (pointers are not read), written to *bytes */
 int lq_zoo_simple_gla_workspace_bytes(const lq_zoo_simple_gla_args* args, int64_t* bytes);
 
+/* replaces chunk_gla_int8 (linquant/kernels/zoo/gla.py:235-279), chunk_delta_int8 (gated_delta_rule.py:159-203) and
+ * chunk_kda_int8 (kda.py:154-203) as a whole (rotated storage): the stage entry points above in the order the wrappers
+ * issue them -- cumsum, WY prep (delta family), write-codes pre-pass (128-token chunks; 64-token chunks make them in the
+ * cumsum / WY launch), A kernel (per-channel decay), state recurrence, output -- on `stream` over one caller-supplied
+ * workspace that holds every intermediate.  Same kernels and bits as the separate calls; one foreign call and one
+ * allocation per forward.  family x decay: linear x diagonal = GLA; delta x none = DeltaNet, delta x scalar = Gated
+ * DeltaNet, delta x diagonal = KDA (linear x none / scalar: lq_zoo_simple_gla).  Field meanings as in the per-stage structs. */
+typedef struct {
+  const void* q;             /* (B,T,H,K) fp16/bf16 */
+  const void* k;             /* (B,T,H,K) */
+  const void* v;             /* (B,T,H,V) */
+  const float* g;            /* log decay per token, not cumulated: (B,T,H) scalar, (B,T,H,K) diagonal, NULL none */
+  const float* beta;         /* delta family: (B,T,H) fp32 */
+  void* o;                   /* (B,T,H,V) fp16/bf16, or fp32 when o_is_f32 */
+  int32_t o_is_f32;
+  float* ht;                 /* (B,H,K,V) fp32 final state, or NULL */
+  const float* sq;           /* (H,) */
+  const float* sk;           /* (H,) */
+  const float* sw;           /* delta family: (H,) */
+  const float* skw;          /* (H,K) */
+  const float* svw;          /* (H,V) value write scale: vw (linear) or ew (delta) */
+  const float* svl;          /* (H,V) local value scale: vl (linear) or el (delta); 16-byte aligned */
+  const float* ss;           /* (H,V), 16-byte aligned */
+  const void* rot;           /* diagonal decay: (K,K) fp16 local R_QK, or NULL */
+  const float* dq;           /* KDA, 64-token chunks: (H,K) D_QK applied to q and k as they are loaded, or NULL */
+  const float* dq_rcp;       /* (H,K) RN(1 / dq), with dq */
+  float sigma, tau, eta, scale;
+  int32_t qmax;
+  int32_t family, decay;
+  int32_t batch, seqlen, nheads, kdim, vdim, chunk_size; /* K in {64,128}, V a multiple of 64, chunk 64 or 128 */
+  int32_t act_dtype;         /* LQ_DT_F16 or LQ_DT_BF16 */
+  void* workspace;           /* device memory, 256-byte aligned, lq_zoo_chunk_forward_workspace_bytes() bytes; contents
+                                undefined on entry and on return */
+  int64_t workspace_bytes;
+} lq_zoo_chunk_forward_args;
+int lq_zoo_chunk_forward(const lq_zoo_chunk_forward_args* args, hipStream_t stream);
+/* workspace size for the dims, family, decay and chunk size in `args` (pointers are not read), written to *bytes */
+int lq_zoo_chunk_forward_workspace_bytes(const lq_zoo_chunk_forward_args* args, int64_t* bytes);
+
 /* replaces _gla_A_inter + _gla_A_intra (linquant/kernels/zoo/gla.py:27-99): intra-chunk product under
  * per-channel decay, 16-token sub-blocks: INT8 dots on anchor-rescaled operands off the diagonal, fp32
  * reduction over the dequantized codes on the diagonal blocks.  Writes the full (C,C) rows (C = 64; chunk_size 128:

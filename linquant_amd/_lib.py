@@ -13,7 +13,7 @@ from pathlib import Path
 ROOT = Path(__file__).resolve().parent
 HEADER = ROOT.parent / "include" / "linquant_hip.h"
 LIB_PATH = ROOT / "csrc" / "liblinquant_hip.so"
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 LQ_DT_F16, LQ_DT_F32, LQ_DT_I8, LQ_DT_BF16 = 0, 1, 2, 3
 
@@ -57,7 +57,8 @@ FUNCTIONS = tuple(_funcs)
 
 # entry points whose first argument is another function's args struct
 _SHARED_ARGS = {"lq_ssd_combined_static": "lq_ssd_combined_args", "lq_ssd_combined_workspace_bytes": "lq_ssd_combined_args",
-                "lq_zoo_simple_gla_workspace_bytes": "lq_zoo_simple_gla_args"}
+                "lq_zoo_simple_gla_workspace_bytes": "lq_zoo_simple_gla_args",
+                "lq_zoo_chunk_forward_workspace_bytes": "lq_zoo_chunk_forward_args"}
 
 _lib = None
 

@@ -4,7 +4,7 @@
 #include "lq_common.h"
 #include "../../include/linquant_hip.h"
 
-extern "C" int lq_abi_version(void) { return 17; }
+extern "C" int lq_abi_version(void) { return 18; }
 
 #define LQ_SIZE_OF(T) \
   if (strcmp(name, #T) == 0) return (int)sizeof(T)
@@ -32,6 +32,7 @@ extern "C" int lq_args_size(const char* name) {
   LQ_SIZE_OF(lq_zoo_state_args);
   LQ_SIZE_OF(lq_zoo_output_args);
   LQ_SIZE_OF(lq_zoo_simple_gla_args);
+  LQ_SIZE_OF(lq_zoo_chunk_forward_args);
   LQ_SIZE_OF(lq_zoo_gla_A_args);
   LQ_SIZE_OF(lq_zoo_wy_prep_args);
   LQ_SIZE_OF(lq_zoo_rotate_qkv_args);

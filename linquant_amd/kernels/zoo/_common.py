@@ -327,3 +327,40 @@ def export_debug(debug, h_i8, codes=None, **extra):
             tok = lambda t: None if t is None else t.permute(0, 1, 4, 2, 3).reshape(B, NT * CHUNK, H, t.shape[3])  # noqa: E731
             debug.update(kq=tok(codes["kqT"]), vq=tok(codes["vqT"]), wq=codes["wq"])
         debug.update(extra)
+
+
+_FORWARD_WS = {}
+
+
+def one_call_forward(family, decay, q, k, v, g, beta, sc, dims, span, *, sigma=1.0, tau=1.0, eta, scale, qmax, final_state,
+                     out_dtype, rot=None, dq=None, dq_rcp=None):
+    """lq_zoo_chunk_forward: every stage of a chunk forward (GLA, DeltaNet, Gated DeltaNet, KDA; rotated storage) from one
+    foreign call over one workspace.  ``sc``: fp32 scales by role ('q','k','w','kw', value write 'vw' / 'ew', value local
+    'vl' / 'el', 'state').  Returns (o, final fp32 state or None)."""
+    import ctypes
+
+    B, T, H, K, V = dims
+    dev = q.device
+    delta = family == FAMILY_DELTA
+    svw, svl = (sc["ew"], sc["el"]) if delta else (sc["vw"], sc["vl"])
+    svl, ss, skw = _lib.aligned(svl), _lib.aligned(sc["state"]), _lib.aligned(sc["kw"])
+    key = (family, decay, B, T, H, K, V, span)
+    nbytes = _FORWARD_WS.get(key)
+    if nbytes is None:
+        st = _lib.fill("lq_zoo_chunk_forward_args", family=family, decay=decay, batch=B, seqlen=T, nheads=H, kdim=K, vdim=V,
+                       chunk_size=span)
+        n = ctypes.c_int64(0)
+        rc = _lib.load().lq_zoo_chunk_forward_workspace_bytes(ctypes.byref(st), ctypes.byref(n))
+        if rc != 0:
+            raise _lib.LinQuantHipError(f"lq_zoo_chunk_forward_workspace_bytes failed with code {rc}")
+        nbytes = _FORWARD_WS[key] = n.value
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    o = out_buffer(v, out_dtype)
+    ht = torch.empty(B, H, K, V, dtype=torch.float32, device=dev) if final_state else None
+    _lib.call("lq_zoo_chunk_forward", dev, q=_lib.ptr(q), k=_lib.ptr(k), v=_lib.ptr(v), g=_lib.ptr(g), beta=_lib.ptr(beta),
+              o=_lib.ptr(o), o_is_f32=int(o.dtype == torch.float32), ht=_lib.ptr(ht), sq=_lib.ptr(sc["q"]), sk=_lib.ptr(sc["k"]),
+              sw=_lib.ptr(sc.get("w")), skw=_lib.ptr(skw), svw=_lib.ptr(svw), svl=_lib.ptr(svl), ss=_lib.ptr(ss), rot=_lib.ptr(rot),
+              dq=_lib.ptr(dq), dq_rcp=_lib.ptr(dq_rcp), sigma=float(sigma), tau=float(tau), eta=float(eta), scale=float(scale),
+              qmax=int(qmax), family=family, decay=decay, batch=B, seqlen=T, nheads=H, kdim=K, vdim=V, chunk_size=span,
+              act_dtype=act_code(v), workspace=_lib.ptr(ws), workspace_bytes=nbytes)
+    return o, ht

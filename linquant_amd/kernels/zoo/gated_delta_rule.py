@@ -13,7 +13,7 @@ from . import _common as C
 
 
 def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, scale=None, chunk_size=64,
-                     output_final_state=False, unrot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None):
+                     output_final_state=False, unrot=None, fla_prep=True, bits=8, out_dtype=None, _debug=None, _staged=False):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None (DeltaNet), beta [B,T,H].
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None).
     ``chunk_size``: up to 64 (padded to 64 tokens), or up to 128 (padded to 128: the WY transform then
@@ -30,11 +30,17 @@ def chunk_delta_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=1.0, s
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     decay = C.DECAY_NONE if g is None else C.DECAY_SCALAR
+    assert g is None or g.shape == (B, T, H)
+    sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
+    if unrot is None and _debug is None and not _staged:
+        # the whole forward as one C call over one workspace (same kernels and bits as the stage-by-stage route below)
+        o, ht = C.one_call_forward(C.FAMILY_DELTA, decay, q, k, v, None if g is None else C.f32(g), C.f32(beta), sc, dims, span,
+                                   sigma=sigma, tau=tau, eta=eta, scale=scale, qmax=qmax, final_state=output_final_state,
+                                   out_dtype=out_dtype)
+        return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
     gg = None
     if g is not None:
-        assert g.shape == (B, T, H)
         gg, _ = C.cumsum(g, B, T, H, 0, span=span)
-    sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
     # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
     if span == C.CHUNK:
         Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gg, sigma, tau, dims, decay,

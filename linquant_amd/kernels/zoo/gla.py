@@ -14,7 +14,7 @@ BC = 16  # secondary chunk
 
 
 def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, output_final_state=False, unrot=None,
-                   rot=None, bits=8, out_dtype=None, _debug=None):
+                   rot=None, bits=8, out_dtype=None, _debug=None, _staged=False):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay. scales as chunk_simple_gla_int8.
     Returns (o, final fp32 state or None).  ``chunk_size``: a multiple of 16 up to 64, or up to 128 (the
     kernels walk a chunk of more than 64 tokens as two 64-token halves, padded to 128 tokens; the sub-block anchoring over its eight sub-blocks is the reference's)."""
@@ -32,6 +32,11 @@ def chunk_gla_int8(q, k, v, g, scales, *, eta=0.0, scale=None, chunk_size=64, ou
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "kw", "vw", "vl", "state")}
+    if unrot is None and _debug is None and not _staged:
+        # the whole forward as one C call over one workspace (same kernels and bits as the stage-by-stage route below)
+        o, ht = C.one_call_forward(C.FAMILY_LINEAR, C.DECAY_DIAGONAL, q, k, v, C.f32(g), None, sc, dims, span, eta=eta, scale=scale,
+                                   qmax=qmax, final_state=output_final_state, out_dtype=out_dtype, rot=R)
+        return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
     # the cumsum launch also makes the state kernel's write operands (it holds the chunk's decay tile): no pre-pass
     if span == C.CHUNK:
         gc, logenv, codes = C.cumsum(g, B, T, H, K, write=dict(k=k, v=v, skw=sc["kw"], svw=sc["vw"], eta=eta, qmax=qmax))

@@ -14,7 +14,7 @@ from .gla import BC
 
 def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, scale=None, chunk_size=64,
                    output_final_state=False, unrot=None, rot=None, fla_prep=True, bits=8, out_dtype=None, dqk=None,
-                   _debug=None):
+                   _debug=None, _staged=False):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H,K] fp32 per-channel log decay, beta [B,T,H].
     scales: 'q','k','w' (H,), 'kw' (H,K), 'el','ew','state' (H,V). Returns (o, final fp32 state or None).
     ``dqk`` (H,K) fp32, not in the reference's signature: the diagonal rescaling D_QK of linquant/harness.py:68-88
@@ -44,10 +44,16 @@ def chunk_kda_int8(q, k, v, g, beta, scales, *, sigma=1.0, tau=1.0, eta=0.0, sca
     R = None if rot is None else rot.to(torch.float16).contiguous()
     scale = K0 ** -0.5 if scale is None else scale
     qmax = 2 ** (bits - 1) - 1
-    gc, logenv = C.cumsum(g, B, T, H, K, span=span)
     sc = {n: C.f32(scales[n]) for n in ("q", "k", "w", "kw", "el", "ew", "state")}
-    # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
     dq, dq_rcp = C.dqk_tables(dqk, H, K)
+    if unrot is None and _debug is None and not _staged:
+        # the whole forward as one C call over one workspace (same kernels and bits as the stage-by-stage route below)
+        o, ht = C.one_call_forward(C.FAMILY_DELTA, C.DECAY_DIAGONAL, q, k, v, C.f32(g), C.f32(beta), sc, dims, span, sigma=sigma,
+                                   tau=tau, eta=eta, scale=scale, qmax=qmax, final_state=output_final_state, out_dtype=out_dtype,
+                                   rot=R, dq=dq, dq_rcp=dq_rcp)
+        return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)
+    gc, logenv = C.cumsum(g, B, T, H, K, span=span)
+    # one launch makes Hw, U, fw and the state kernel's write-operand codes; W leaves the chip only for a caller that asks
     if span == C.CHUNK:
         Hw, W, U, fw, codes = C.run_wy_prep(k, v, C.f32(beta), gc, sigma, tau, dims, C.DECAY_DIAGONAL,
                                             write=dict(logenv=logenv, skw=sc["kw"], sw=sc["w"], eta=eta, qmax=qmax),

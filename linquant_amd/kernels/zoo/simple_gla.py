@@ -13,7 +13,7 @@ from . import _common as C
 
 
 def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size=64, output_final_state=False,
-                          unrot=None, bits=8, out_dtype=None, prologue=None, _debug=None):
+                          unrot=None, bits=8, out_dtype=None, prologue=None, _debug=None, _staged=False):
     """q,k [B,T,H,K], v [B,T,H,V] fp16, g [B,T,H] fp32 log decay or None. scales: 'q','k' (H,), 'kw' (H,K),
     'vw','vl','state' (H,V) fp32. Returns (o [B,T,H,V] in v.dtype or out_dtype, final fp32 state [B,H,K,V] or None).
     ``prologue`` (not in the reference's signature) = dict(signs_qk=, signs_v=, dqk=), each optional: q, k, v arrive as
@@ -50,7 +50,7 @@ def chunk_simple_gla_int8(q, k, v, g, scales, *, eta=1.0, scale=None, chunk_size
     qmax = 2 ** (bits - 1) - 1
     decay = C.DECAY_NONE if g is None else C.DECAY_SCALAR
     assert g is None or g.shape == (B, T, H)
-    if prologue is None and unrot is None and _debug is None:
+    if prologue is None and unrot is None and _debug is None and not _staged:
         # the whole forward as one C call over one workspace (same kernels and bits as the stage-by-stage route below)
         o, ht = _one_call(q, k, v, g, scales, eta, scale, qmax, dims, span, output_final_state, out_dtype)
         return C.cut_values(restore(o), C.cut_keys(ht, K0), V0)

@@ -138,6 +138,45 @@ def test_one_call_forward_equals_the_stage_by_stage_route(cuda, cell, chunk, K, 
     assert torch.equal(o0, o1) and torch.equal(h0, h1) and float(o1.float().abs().max()) > 0
 
 
+@pytest.mark.parametrize("cell", ["gla", "deltanet", "gated_deltanet", "kda"])
+@pytest.mark.parametrize("chunk,K,V,dtype,out_dtype,extras", [(64, 64, 64, torch.float16, None, False), (64, 128, 128, torch.bfloat16, None, True),
+                                                              (32, 48, 96, torch.float16, torch.float32, False),
+                                                              (128, 128, 64, torch.float16, None, True), (96, 64, 128, torch.float16, None, False)])
+def test_one_call_forward_equals_the_stage_by_stage_route_other_cells(cuda, cell, chunk, K, V, dtype, out_dtype, extras):
+    """chunk_gla_int8, chunk_delta_int8 and chunk_kda_int8 issue their stages from one C call over one workspace
+    (lq_zoo_chunk_forward) unless a caller asks for canonical storage or the intermediates; both routes run the same kernels
+    on the same operands: outputs and final states are equal bit for bit.  ``extras``: the local R_QK (per-channel decay)
+    and D_QK (KDA) as well."""
+    from linquant_amd.kernels import zoo
+    from oracle.zoo_reference import signed_hadamard
+
+    T = 4 * max(chunk, 64)
+    H = 3
+    q, k, v, g, beta = [t.to(cuda) if t is not None else None for t in zc.inputs(cell, B=2, T=T, H=H, K=K, V=V, seed=47, dtype=dtype)]
+    gen = torch.Generator().manual_seed(6)
+    r = lambda *shape, lo, hi: (torch.rand(*shape, generator=gen) * (hi - lo) + lo).to(cuda)  # noqa: E731
+    sc = {"q": r(H, lo=0.001, hi=0.003), "k": r(H, lo=0.005, hi=0.01), "w": r(H, lo=0.02, hi=0.04), "kw": r(H, K, lo=0.005, hi=0.015),
+          "vw": r(H, V, lo=0.02, hi=0.04), "vl": r(H, V, lo=0.02, hi=0.04), "el": r(H, V, lo=0.04, hi=0.06),
+          "ew": r(H, V, lo=0.04, hi=0.06), "state": r(H, V, lo=0.02, hi=0.07)}
+    fam, dec = zc.CELLS[cell]
+    kw = dict(eta=0.25, chunk_size=chunk, output_final_state=True, out_dtype=out_dtype)
+    if dec == "diagonal" and extras and K in (64, 128):
+        kw["rot"] = signed_hadamard(K, 2).float().to(cuda)
+    if cell == "kda" and extras:
+        kw["dqk"] = r(H, K, lo=0.25, hi=1.75)
+    if fam == "delta":
+        kw.update(sigma=0.5, tau=0.5)
+        fn = zoo.chunk_kda_int8 if dec == "diagonal" else zoo.chunk_delta_int8
+        call = lambda **x: fn(q, k, v, g, beta, sc, **kw, **x)  # noqa: E731
+    else:
+        call = lambda **x: zoo.chunk_gla_int8(q, k, v, g, sc, **kw, **x)  # noqa: E731
+    o1, h1 = call()
+    o0, h0 = call(_debug={})
+    torch.cuda.synchronize()
+    assert o1.shape == v.shape and o1.dtype == (out_dtype or dtype) and h1.shape == (2, H, K, V)
+    assert torch.equal(o0, o1) and torch.equal(h0, h1) and float(o1.float().abs().max()) > 0
+
+
 @pytest.mark.parametrize("cell", ["deltanet", "gated_deltanet", "kda"])
 @pytest.mark.parametrize("K,V,dtype,chunk", [(64, 64, torch.float16, 128), (128, 128, torch.float16, 128),
                                              (64, 192, torch.bfloat16, 128), (64, 64, torch.float16, 96)])
